@@ -1,0 +1,369 @@
+/*
+ * sah.h — C ABI of libsah_mi355.so: the MI355X (gfx950) kernels behind the
+ * ResearchAttention decode path of sparse-attention-hub.
+ *
+ * The reference implementation is pure Python on torch and has no FFI of its
+ * own; every entry point below therefore cites the reference *Python* function
+ * whose body it replaces (paths relative to the reference checkout,
+ * sparse_attention_hub/sparse_attention/...).
+ *
+ * Conventions
+ *   - every pointer is a device pointer unless its comment says "host";
+ *   - every call is asynchronous on `stream` (a hipStream_t passed as void*),
+ *     never synchronises, never allocates, never frees;
+ *   - return value 0 = success, negative = SAH_E* argument error (nothing was
+ *     launched), positive = hipError_t from the launch;
+ *   - sah_last_error() returns a thread-local description of the last failure;
+ *   - tensors are addressed by element strides, the innermost (head_dim)
+ *     stride must be 1.
+ *
+ * Native sparse-mask layout ("rows"): the reference Mask
+ * (utils/mask.py:10) is a dense (B,Hq,Lq,Lk) weight tensor or a flat int64
+ * indices/ptr/data triple. The kernels use one row per (b, h, q):
+ *     cols  [n_rows, cap]   int32  key columns of the active entries (unordered)
+ *     cnt   [n_rows]        int32  number of valid entries of the row
+ *     w     [n_rows, cap]   float  weight of each entry, or NULL (all 1.0)
+ *     bitmap[n_rows, n_words] uint32  bit j of the row set <=> column j active
+ * n_words = ceil(n_keys / 32). The Python Mask facade converts this to the
+ * reference's flat int64 indices / ptr / data or to a dense tensor on demand.
+ */
+#ifndef SAH_H
+#define SAH_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SAH_VERSION 1
+
+enum {
+  SAH_OK = 0,
+  SAH_EINVAL = -1,      /* bad argument value / combination            */
+  SAH_ENULL = -2,       /* required pointer is NULL                    */
+  SAH_ESHAPE = -3,      /* shape the kernels do not support            */
+  SAH_ECAPACITY = -4,   /* rows.cap or a workspace is too small        */
+  SAH_EDTYPE = -5       /* unsupported dtype code                      */
+};
+
+/* element type codes */
+enum { SAH_F32 = 0, SAH_BF16 = 1, SAH_F16 = 2 };
+
+/* activation codes of the signature MLP (hashattention_top_k.py:210-215) */
+enum { SAH_ACT_RELU = 0, SAH_ACT_SILU = 1, SAH_ACT_GELU = 2, SAH_ACT_TANH = 3 };
+
+typedef struct sah_rows {
+  int32_t* cols;
+  int32_t* cnt;
+  float* w;          /* may be NULL */
+  uint32_t* bitmap;
+  int32_t n_rows;    /* B * Hq * Lq */
+  int32_t cap;       /* row pitch of cols / w */
+  int32_t n_keys;    /* Lk */
+  int32_t n_words;   /* row pitch of bitmap = ceil(Lk/32) */
+} sah_rows;
+
+int sah_version(void);
+const char* sah_last_error(void);
+
+/* ---------------------------------------------------------------------------
+ * Fused Sink + Local builder. Replaces SinkMasker.get_updated_mask_dense
+ * (maskers/fixed/implementations/basic_fixed.py:354-363) and
+ * LocalMasker.update_core (basic_fixed.py:48-67): columns [0, sink) and, for
+ * query row q of Lq, columns [Lk-Lq-window+1+q, Lk-Lq+q]. Either part may be
+ * switched off with 0. With fresh != 0 the rows are taken to be empty and are
+ * initialised (cnt, bitmap and cols all written); otherwise the ranges are
+ * merged into the existing rows (already-active columns keep their entry, and
+ * a weighted entry that falls inside a range has its weight raised to 1.0 as
+ * the reference's dense assignment `mask[...] = 1.0` does).
+ * With clear_future != 0 every entry with column > Lk-Lq+q is removed first
+ * (basic_fixed.py:60-66); a no-op when Lq == 1.
+ * ------------------------------------------------------------------------- */
+typedef struct sah_sink_local_args {
+  sah_rows rows;
+  int32_t lq;            /* query rows per (b,h): row r has q = r % lq */
+  int32_t sink;          /* sink size, 0 = skip                         */
+  int32_t window;        /* local window, 0 = skip                      */
+  int32_t fresh;
+  int32_t clear_future;
+  void* stream;
+} sah_sink_local_args;
+int sah_sink_local_indices(const sah_sink_local_args* a);
+
+/* ---------------------------------------------------------------------------
+ * Dense <-> rows conversion. Replaces Mask.get_index_mask's dense scan
+ * (utils/mask.py:553-573) and Mask.get_dense_mask's scatter (:595-609).
+ * dense is [n_rows, n_keys] contiguous in `dtype`; an entry is active iff its
+ * weight != 0. rows.w may be NULL for from_dense (weights dropped: caller
+ * asserts they are all 1.0) and for to_dense (ones are written).
+ * from_dense writes columns in ascending order and returns SAH_ECAPACITY
+ * nowhere: rows whose population exceeds cap are truncated and their cnt is
+ * still the true population, so the caller can detect it (cnt > cap).
+ * ------------------------------------------------------------------------- */
+typedef struct sah_dense_rows_args {
+  sah_rows rows;
+  void* dense;
+  int32_t dtype;
+  void* stream;
+} sah_dense_rows_args;
+int sah_rows_from_dense(const sah_dense_rows_args* a);
+int sah_rows_to_dense(const sah_dense_rows_args* a);
+
+/* ---------------------------------------------------------------------------
+ * Hash signatures. Replaces HashAttentionTopKMasker._get_signatures /
+ * _apply_single_layer (hashattention_top_k.py:203-253): per query head h,
+ * x <- act(x W_i + b_i) for all but the last layer, x <- x W_L + b_L, then
+ * sign(x) in {-1, 0, +1}. A signature is stored as a pair of uint32 planes
+ * ("code", 8 bytes): bit e of word 0 = (x_e > 0), bit e of word 1 = (x_e != 0),
+ * LSB first; at most 32 signature bits. (Exact zeros are common in bf16, and
+ * the reference scores such a bit as 0.)
+ * x is [B, Hx, L, D] with element strides; head h reads x head h / group
+ * (group = Hq / Hx; keys pass Hx = Hkv, queries pass Hx = Hq, group = 1).
+ * Layer i has W_i [Hq, d_in_i, d_out_i] and b_i [Hq, d_out_i], contiguous, in
+ * `dtype`. With dtype = SAH_BF16 / SAH_F16 every layer output, bias add and
+ * activation is rounded to that type exactly where torch would round it.
+ * codes[((b*Hq + h) * code_pitch + code_offset + l) * 2 + {0,1}] receives
+ * vector l (code_pitch and code_offset count codes, not words).
+ * ------------------------------------------------------------------------- */
+#define SAH_MAX_MLP_LAYERS 4
+typedef struct sah_hash_sig_args {
+  const void* x;
+  int64_t xs_b, xs_h, xs_l;
+  int32_t dtype;
+  int32_t B, Hq, group, L, D;
+  int32_t n_layers;
+  const void* W[SAH_MAX_MLP_LAYERS];
+  const void* bias[SAH_MAX_MLP_LAYERS];
+  int32_t d_out[SAH_MAX_MLP_LAYERS];  /* d_in of layer 0 is D */
+  int32_t act;
+  uint32_t* codes;
+  int64_t code_pitch;
+  int64_t code_offset;
+  void* stream;
+} sah_hash_sig_args;
+int sah_hash_signatures(const sah_hash_sig_args* a);
+
+/* ---------------------------------------------------------------------------
+ * Signature top-k. Replaces the score half of
+ * HashAttentionTopKMasker._compute_hashattention_score
+ * (hashattention_top_k.py:365-370: scores = q_sig @ k_sig^T, already-active
+ * columns pushed to the bottom),
+ * TopKMasker._get_topk_indices_from_inactive_positions (fixed/base.py:74-85)
+ * and the dense scatter + clamp-add merge that follows
+ * (maskers/base.py:128-150, utils/mask.py:875-877).
+ * With nz = q.nonzero & k.nonzero the score is
+ *     popcount(nz) - 2 * popcount((q.positive ^ k.positive) & nz)
+ * (= bits - 2 * Hamming distance when no signature entry is zero).
+ * For row r = (b,h,q): rank columns j < n_keys by descending score of
+ * qcodes[r] against kcodes[(b*Hq+h)*code_pitch + j], ties by lowest j,
+ * columns whose bitmap bit is set ranking below every other column; the first
+ * k of that order which are not yet active are appended to the row (ascending
+ * j) with weight 1.0 and their bits are set.
+ * ------------------------------------------------------------------------- */
+typedef struct sah_hamming_topk_args {
+  sah_rows rows;
+  const uint32_t* kcodes;   /* 2 words per code */
+  int64_t code_pitch;       /* in codes */
+  const uint32_t* qcodes;   /* [n_rows] codes */
+  int32_t lq;               /* row r uses key-code stream r / lq */
+  int32_t k;
+  void* stream;
+} sah_hamming_topk_args;
+int sah_hamming_topk(const sah_hamming_topk_args* a);
+
+/* Signature scores with an additive attention mask
+ * (hashattention_top_k.py:365-369): key of round_to_dtype(float(score) +
+ * amask[b, h|0, q, j]) in the sortable-key form of sah_qk_scores, written at
+ * keys_out[r * key_pitch + j]; feed sah_select_topk with the key of -inf as
+ * excluded_key (fixed/base.py:80). amask may be NULL. */
+typedef struct sah_hamming_scores_args {
+  const uint32_t* kcodes;
+  int64_t code_pitch;
+  const uint32_t* qcodes;
+  int32_t B, Hq, Lq, n_keys;
+  const void* amask; int64_t ms_b, ms_h, ms_l;
+  int32_t dtype;
+  void* keys_out;
+  int64_t key_pitch;
+  void* stream;
+} sah_hamming_scores_args;
+int sah_hamming_scores(const sah_hamming_scores_args* a);
+
+/* ---------------------------------------------------------------------------
+ * Exact QK scores as sortable keys. Replaces OracleTopK.update_core's
+ * `matmul(queries, keys^T)` (+ attention_mask) (oracle_top_k.py:70-72) without
+ * repeat_kv: score = round_to_dtype(q[b,h,q,:] . K[b,h/group,j,:]), un-scaled,
+ * then (+ amask, rounded again). Scores are written as order-preserving
+ * unsigned keys (larger score => larger key; -0 == +0): uint16 for bf16/f16,
+ * uint32 for f32, at keys_out[r * key_pitch + j].
+ * amask is NULL or an additive mask [B, 1|Hq, Lq, >=Lk] in `dtype` with
+ * element strides (stride 0 for a broadcast head).
+ * ------------------------------------------------------------------------- */
+typedef struct sah_qk_scores_args {
+  const void* q;  int64_t qs_b, qs_h, qs_l;
+  const void* k;  int64_t ks_b, ks_h, ks_l;
+  const void* amask; int64_t ms_b, ms_h, ms_l;
+  int32_t dtype;
+  int32_t B, Hq, Hkv, Lq, Lk, D;
+  void* keys_out;
+  int64_t key_pitch;
+  void* stream;
+} sah_qk_scores_args;
+int sah_qk_scores(const sah_qk_scores_args* a);
+
+/* ---------------------------------------------------------------------------
+ * Generic top-k over sortable keys. Replaces `scores[prev != 0] = min;
+ * torch.topk; scatter_(1.0)` (oracle_top_k.py:73-79, pq_top_k.py:513-537,
+ * fixed/base.py:74-85) with the canonical tie rule "lowest column first".
+ * Row r ranks candidates c in [0, n_cand) (column j = c + col_offset) by
+ * descending key; active columns take `excluded_key` as their key. The first k
+ * in that order that are not active are appended (ascending j), weight 1.0.
+ * key_bits is 16 or 32. lds/work: none beyond static LDS.
+ * ------------------------------------------------------------------------- */
+typedef struct sah_select_topk_args {
+  sah_rows rows;
+  const void* keys;
+  int64_t key_pitch;
+  int32_t key_bits;
+  int32_t n_cand;
+  int32_t col_offset;
+  int32_t k;
+  uint32_t excluded_key;
+  void* stream;
+} sah_select_topk_args;
+int sah_select_topk(const sah_select_topk_args* a);
+
+/* ---------------------------------------------------------------------------
+ * Product quantisation (PQCache). A "group" is g = (b*Hkv + hk)*n_sub + s: one
+ * sub-space s of one KV head; its vectors are K[b, hk, key_offset + n,
+ * s*d_sub : (s+1)*d_sub] for n in [0, n_keys), read in `dtype`, used as fp32.
+ * d_sub <= 16, n_cent <= 256 (codes are uint8).
+ *
+ * sah_pq_kmeans_assign: replaces pairwise_distance_batched + argmin
+ * (maskers/fixed/implementations/utils/pq_utils.py:220-257, :353):
+ * code = argmin_c sum_d (x[d] - centre[g,c,d])^2 in fp32, first minimum wins.
+ * centres fp32 [n_groups, n_cent, d_sub]; codes uint8 laid out
+ * [B, Hkv, code_pitch, n_sub], key n written at index code_offset + n.
+ * With sums/counts non-NULL it also accumulates the per-centre fp32 sums
+ * [n_groups, n_cent, d_sub] and int32 counts [n_groups, n_cent] of this
+ * assignment (the one-hot sums of pq_utils.py:360-381; caller zeroes them).
+ * With round_dist != 0 the distance follows PQCache._quantize_new_keys
+ * (pq_top_k.py:388-404) instead, which works in the key dtype: each difference
+ * and each square is rounded to `dtype`, the sum is accumulated in fp32 and
+ * rounded to `dtype` (centres must already hold `dtype`-representable values).
+ * skip_flag (optional): if *skip_flag != 0 the kernel does nothing; this is
+ * how the Lloyd loop stops early without a host round trip.
+ *
+ * sah_pq_kmeans_update: replaces the centre update, empty-cluster reseed and
+ * convergence test (pq_utils.py:372-432): centre = sum / max(count, 1); an
+ * empty cluster takes vector reseed_idx[g*n_cent + c] of its group (the
+ * reference draws these with torch.randint); shift2[g] = (sum_c ||new-old||)^2.
+ * state is int32[4], zeroed by the caller before the first iteration:
+ * when every group has shift2 < tol the kernel sets state[2] = 1 (the
+ * skip_flag of later launches). centres are updated in place.
+ *
+ * sah_pq_adc_scores: replaces PQCache._compute_pq_scores
+ * (pq_top_k.py:406-490): LUT[s][c] = round_to_dtype(q_sub . centre[g,c,:d_sub])
+ * and score(n) = round_to_dtype(sum_s LUT[s][code[n,s]]) with fp32
+ * accumulation; emitted as sortable keys like sah_qk_scores for candidates
+ * n in [0, n_cand) at keys_out[r * key_pitch + n]. centres are the fp32
+ * widening of the stored (`dtype`-rounded) centroids, [n_groups, n_cent, d_sub].
+ * ------------------------------------------------------------------------- */
+typedef struct sah_pq_assign_args {
+  const void* k; int64_t ks_b, ks_h, ks_l;
+  int32_t dtype;
+  int32_t B, Hkv, n_sub, d_sub, n_cent;
+  int32_t key_offset, n_keys;
+  const float* centres;
+  uint8_t* codes; int64_t code_pitch; int64_t code_offset;
+  float* sums; int32_t* counts;
+  int32_t round_dist;
+  const int32_t* skip_flag;
+  void* stream;
+} sah_pq_assign_args;
+int sah_pq_kmeans_assign(const sah_pq_assign_args* a);
+
+typedef struct sah_pq_update_args {
+  const void* k; int64_t ks_b, ks_h, ks_l;
+  int32_t dtype;
+  int32_t B, Hkv, n_sub, d_sub, n_cent;
+  int32_t key_offset;
+  float* centres;
+  const float* sums; const int32_t* counts;
+  const int32_t* reseed_idx;
+  float* shift2;       /* [n_groups] */
+  float tol;
+  int32_t* state;      /* int32[4]: converged count, ticket, done flag, pending verdict */
+  void* stream;
+} sah_pq_update_args;
+int sah_pq_kmeans_update(const sah_pq_update_args* a);
+
+typedef struct sah_pq_adc_args {
+  const void* q; int64_t qs_b, qs_h, qs_l;
+  int32_t dtype;
+  int32_t B, Hq, Hkv, Lq, n_sub, d_sub, n_cent;
+  const float* centres;
+  const uint8_t* codes; int64_t code_pitch;
+  int32_t n_cand;
+  void* keys_out; int64_t key_pitch;
+  void* stream;
+} sah_pq_adc_args;
+int sah_pq_adc_scores(const sah_pq_adc_args* a);
+
+/* ---------------------------------------------------------------------------
+ * Masked-softmax attention over the gathered rows. Replaces
+ * get_masked_attention_output (utils/mask_attention_utils.py:406-491):
+ * z[j] = q.K[j] * scaling (+amask) in fp32, e[j] = exp(z[j] - m) / (w[j]+1e-6)
+ * (unit_inv_w when rows.w is NULL), out = sum e V / (sum e [+ sink term,
+ * apply_sink_bias :357-402]), written as out[b, q, h, :] in `dtype`
+ * (contiguous (B, Lq, Hq, D)). With dense != 0 the rows are ignored and every
+ * column j < Lk is used with weight 1 (the reference's treatment of an empty
+ * or full Mask, utils/mask.py:733-735).
+ * work: fp32 scratch of sah_sparse_attention_work_floats(...) floats.
+ * logits_out (optional, fp32 [n_rows, cap]) receives z[j] per entry and
+ * stats_out (optional, fp32 [n_rows, 2]) the final (m, den) so that the dense
+ * attention-weight tensor can be produced by sah_attention_weights.
+ * ------------------------------------------------------------------------- */
+typedef struct sah_attention_args {
+  sah_rows rows;
+  const void* q;  int64_t qs_b, qs_h, qs_l;
+  const void* k;  int64_t ks_b, ks_h, ks_l;
+  const void* v;  int64_t vs_b, vs_h, vs_l;
+  const void* amask; int64_t ms_b, ms_h, ms_l;
+  const float* sinks;     /* [Hq] fp32 or NULL */
+  int32_t dtype;
+  int32_t B, Hq, Hkv, Lq, Lk, D;
+  float scaling;
+  float unit_inv_w;
+  int32_t dense;
+  int32_t max_cnt;        /* upper bound of cnt[r] the grid is sized for */
+  void* out;
+  float* work; int64_t work_floats;
+  float* logits_out;
+  float* stats_out;
+  void* stream;
+} sah_attention_args;
+int64_t sah_sparse_attention_work_floats(int32_t n_rows, int32_t max_cnt, int32_t D);
+int sah_sparse_attention(const sah_attention_args* a);
+
+/* Dense attention probabilities (the second return value of
+ * get_masked_attention_output, utils/mask_attention_utils.py:482-489):
+ * weights[r, j] = round_to_dtype(exp(z - m) * inv_w / den) at the row's
+ * entries; the caller zero-fills weights [n_rows, Lk] first. */
+typedef struct sah_attention_weights_args {
+  sah_rows rows;
+  const float* logits;   /* [n_rows, cap] */
+  const float* stats;    /* [n_rows, 2]   */
+  float unit_inv_w;
+  int32_t dense;         /* rows ignored: entry i is column i, pitch n_keys */
+  int32_t dtype;
+  void* weights;
+  void* stream;
+} sah_attention_weights_args;
+int sah_attention_weights(const sah_attention_weights_args* a);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SAH_H */

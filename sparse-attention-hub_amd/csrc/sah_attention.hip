@@ -1,0 +1,401 @@
+// Masked-softmax attention over gathered KV rows (flash-decoding layout).
+//
+// HBM-bound: every selected key costs one K row and one V row (D * elem bytes
+// each). A wavefront reads 64/LPK rows per load instruction, LPK = D/8 lanes per
+// row with 8 elements (16 B for bf16, 32 B for fp32) per lane, so each row is
+// one fully coalesced segment. grid = (splits, mask rows); each workgroup
+// (4 waves) walks its slice of the row's column list in chunks of 256 keys with
+// a two-phase softmax per chunk (all K loads, block max, all V loads) and an
+// online rescale between chunks, then writes (m, l, acc[D]) to the workspace.
+// A second small kernel merges the splits, applies the optional sink logit and
+// writes out[b, q, h, :].
+#include "sah_common.h"
+
+#define ATT_NT 256
+#define ATT_NW (ATT_NT / SAH_WAVE)
+#define ATT_CHUNK (ATT_NT)  // keys per workgroup iteration: 64 per wave
+
+struct att_params {
+  sah_rows rows;
+  const void* q; int64_t qs_b, qs_h, qs_l;
+  const void* k; int64_t ks_b, ks_h, ks_l;
+  const void* v; int64_t vs_b, vs_h, vs_l;
+  const void* amask; int64_t ms_b, ms_h, ms_l;
+  int Hq, Hkv, Lq, Lk;
+  float scaling, unit_inv_w;
+  int dense;
+  int kps;      // keys per split (multiple of ATT_CHUNK)
+  int n_split;
+  float* work;
+  float* logits_out;
+  int64_t logits_pitch;
+};
+
+// exact expf for fp32 storage (1e-5 output tolerance), hardware exp2 path otherwise
+template <int DT>
+__device__ __forceinline__ float att_exp(float x) {
+  return DT == SAH_F32 ? expf(x) : __expf(x);
+}
+
+template <int LPK>
+__device__ __forceinline__ float att_group_sum(float v) {
+  // sum over each aligned group of LPK lanes (LPK in {2,4,8,16})
+  v += sah_dpp<0xB1>(v);
+  if (LPK >= 4) v += sah_dpp<0x4E>(v);
+  if (LPK >= 8) v += sah_dpp<0x141>(v);
+  if (LPK >= 16) v += sah_dpp<0x140>(v);
+  return v;
+}
+
+template <int DT, int D>
+__global__ __launch_bounds__(ATT_NT) void k_sparse_attn(att_params P) {
+  constexpr int LPK = D / 8;            // lanes per key
+  constexpr int KPI = SAH_WAVE / LPK;   // keys per wave iteration
+  constexpr int IT = SAH_WAVE / KPI;    // iterations per 64-key wave chunk (== LPK)
+  constexpr int UB = (DT == SAH_F32) ? (IT < 4 ? IT : 4) : (IT < 8 ? IT : 8);  // loads in flight per batch
+
+  __shared__ float s_max[ATT_NW];
+  __shared__ float s_l[ATT_NW];
+  __shared__ float s_acc[ATT_NW][D];
+
+  const int split = blockIdx.x;
+  const int r = blockIdx.y;
+  const int tid = threadIdx.x;
+  const int lane = tid & (SAH_WAVE - 1);
+  const int wave = tid / SAH_WAVE;
+  const int sub = lane % LPK;   // which 8-element slice of the row
+  const int grp = lane / LPK;   // which key of the iteration
+
+  const int qi = r % P.Lq;
+  const int h = (r / P.Lq) % P.Hq;
+  const int b = r / (P.Lq * P.Hq);
+  const int hk = h / (P.Hq / P.Hkv);
+
+  int cnt = P.dense ? P.Lk : P.rows.cnt[r];
+  if (!P.dense && cnt > P.rows.cap) cnt = P.rows.cap;
+  const int begin = split * P.kps;
+  int end = begin + P.kps;
+  if (end > cnt) end = cnt;
+
+  float* wout = P.work + ((int64_t)r * P.n_split + split) * (D + 2);
+  if (begin >= end) {
+    if (tid == 0) {
+      wout[0] = -INFINITY;
+      wout[1] = 0.f;
+    }
+    return;
+  }
+
+  const int* cols = P.dense ? nullptr : P.rows.cols + (int64_t)r * P.rows.cap;
+  const float* wts = (!P.dense && P.rows.w) ? P.rows.w + (int64_t)r * P.rows.cap : nullptr;
+  const char* kbase = (const char*)P.k;
+  const char* vbase = (const char*)P.v;
+  constexpr int ES = (DT == SAH_F32) ? 4 : 2;
+  const int64_t koff = ((int64_t)b * P.ks_b + (int64_t)hk * P.ks_h) * ES;
+  const int64_t voff = ((int64_t)b * P.vs_b + (int64_t)hk * P.vs_h) * ES;
+  const int64_t moff = P.amask ? ((int64_t)b * P.ms_b + (int64_t)h * P.ms_h + (int64_t)qi * P.ms_l) : 0;
+
+  float qv[8];
+  sah_load8<DT>(P.q, (int64_t)b * P.qs_b + (int64_t)h * P.qs_h + (int64_t)qi * P.qs_l + sub * 8, qv);
+
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  float l_run = 0.f;
+  float m_run = -INFINITY;
+
+  for (int cbase = begin; cbase < end; cbase += ATT_CHUNK) {
+    // one column (and its inverse weight) per lane: this wave's 64 keys
+    const int my = cbase + wave * SAH_WAVE + lane;
+    int idx_l = -1;
+    float invw_l = P.unit_inv_w;
+    if (my < end) {
+      idx_l = P.dense ? my : cols[my];
+      // the reference evaluates 1/(w + 1e-6) in the mask dtype (utils/mask.py:737-740)
+      if (wts) invw_l = sah_round<DT>(1.0f / sah_round<DT>(wts[my] + 1e-6f));
+      if (idx_l < 0 || idx_l >= P.Lk) idx_l = -1;
+    }
+
+    // ---- phase 1: logits of this wave's keys -----------------------------
+    float z[IT];
+#pragma unroll
+    for (int ib = 0; ib < IT; ib += UB) {
+      float kv[UB][8];
+      int id[UB];
+#pragma unroll
+      for (int u = 0; u < UB; ++u) {
+        id[u] = __shfl(idx_l, (ib + u) * KPI + grp);
+        if (id[u] >= 0) {
+          sah_load8<DT>(kbase + koff + (int64_t)id[u] * P.ks_l * ES, sub * 8, kv[u]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) kv[u][e] = 0.f;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < UB; ++u) {
+        float d = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) d = fmaf(qv[e], kv[u][e], d);
+        d = att_group_sum<LPK>(d) * P.scaling;
+        if (id[u] >= 0) {
+          if (P.amask) d += sah_load<DT>(P.amask, moff + id[u]);
+        } else {
+          d = -INFINITY;
+        }
+        z[ib + u] = d;
+      }
+    }
+    if (P.logits_out && sub == 0) {
+#pragma unroll
+      for (int it = 0; it < IT; ++it) {
+        const int pos = cbase + wave * SAH_WAVE + it * KPI + grp;
+        if (pos < end) {
+          const int64_t at = P.dense ? (int64_t)pos : (int64_t)pos;
+          P.logits_out[(int64_t)r * P.logits_pitch + at] = z[it];
+        }
+      }
+    }
+
+    float m_loc = z[0];
+#pragma unroll
+    for (int it = 1; it < IT; ++it) m_loc = fmaxf(m_loc, z[it]);
+    m_loc = sah_wave_max(m_loc);
+    __syncthreads();  // s_max free (previous chunk's readers are done)
+    if (lane == 0) s_max[wave] = m_loc;
+    __syncthreads();
+    float m_new = m_run;
+#pragma unroll
+    for (int wv = 0; wv < ATT_NW; ++wv) m_new = fmaxf(m_new, s_max[wv]);
+
+    const float rescale = (m_run == -INFINITY) ? 0.f : att_exp<DT>(m_run - m_new);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] *= rescale;
+    l_run *= rescale;
+    m_run = m_new;
+
+    // ---- phase 2: weighted sum of this wave's value rows -------------------
+#pragma unroll
+    for (int ib = 0; ib < IT; ib += UB) {
+      float vv[UB][8];
+      int id[UB];
+#pragma unroll
+      for (int u = 0; u < UB; ++u) {
+        id[u] = __shfl(idx_l, (ib + u) * KPI + grp);
+        if (id[u] >= 0) {
+          sah_load8<DT>(vbase + voff + (int64_t)id[u] * P.vs_l * ES, sub * 8, vv[u]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) vv[u][e] = 0.f;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < UB; ++u) {
+        const float iw = __shfl(invw_l, (ib + u) * KPI + grp);
+        float p = 0.f;
+        if (id[u] >= 0 && z[ib + u] != -INFINITY) p = att_exp<DT>(z[ib + u] - m_new) * iw;
+        l_run += p;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] = fmaf(p, vv[u][e], acc[e]);
+      }
+    }
+  }
+
+  // ---- reduce the KPI lane groups of the wave, then the waves -----------------
+#pragma unroll
+  for (int o = LPK; o < SAH_WAVE; o <<= 1) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] += __shfl_xor(acc[e], o);
+    l_run += __shfl_xor(l_run, o);
+  }
+  if (lane < LPK) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s_acc[wave][sub * 8 + e] = acc[e];
+  }
+  if (lane == 0) s_l[wave] = l_run;
+  __syncthreads();
+  if (tid < D) {
+    float a = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < ATT_NW; ++wv) a += s_acc[wv][tid];
+    wout[2 + tid] = a;
+  }
+  if (tid == 0) {
+    float l = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < ATT_NW; ++wv) l += s_l[wv];
+    wout[0] = m_run;
+    wout[1] = l;
+  }
+}
+
+// merge the splits of one row: out = sum_s acc_s e^(m_s-M) / sum_s l_s e^(m_s-M)
+template <int DT, int D>
+__global__ __launch_bounds__(D < 64 ? 64 : D) void k_attn_combine(const float* work, int n_split, int Hq, int Lq,
+                                                                  const float* sinks, void* out, float* stats) {
+  const int r = blockIdx.x;
+  const int d = threadIdx.x;
+  const float* w = work + (int64_t)r * n_split * (D + 2);
+  float M = -INFINITY;
+  for (int s = 0; s < n_split; ++s) M = fmaxf(M, w[(int64_t)s * (D + 2)]);
+  float L = 0.f, a = 0.f;
+  for (int s = 0; s < n_split; ++s) {
+    const float* ws = w + (int64_t)s * (D + 2);
+    const float ms = ws[0];
+    if (ms == -INFINITY) continue;
+    const float sc = att_exp<DT>(ms - M);
+    L = fmaf(ws[1], sc, L);
+    if (d < D) a = fmaf(ws[2 + d], sc, a);
+  }
+  const int qi = r % Lq;
+  const int h = (r / Lq) % Hq;
+  const int b = r / (Lq * Hq);
+  float Mf = M, den = L;
+  if (sinks) {
+    const float sk = sinks[h];
+    Mf = fmaxf(M, sk);
+    const float sc = (M == -INFINITY) ? 0.f : att_exp<DT>(M - Mf);
+    a *= sc;
+    den = L * sc + att_exp<DT>(sk - Mf);
+  }
+  if (d < D) sah_store<DT>(out, (((int64_t)b * Lq + qi) * Hq + h) * D + d, a / den);
+  if (stats && d == 0) {
+    stats[2 * (int64_t)r] = Mf;
+    stats[2 * (int64_t)r + 1] = den;
+  }
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void k_attn_weights(sah_rows R, const float* logits, int64_t pitch,
+                                                      const float* stats, float unit_inv_w, int dense, void* weights) {
+  const int r = blockIdx.y;
+  const float m = stats[2 * (int64_t)r];
+  const float den = stats[2 * (int64_t)r + 1];
+  int cnt = dense ? R.n_keys : R.cnt[r];
+  if (!dense && cnt > R.cap) cnt = R.cap;
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= cnt) return;
+  int c = i;
+  float iw = unit_inv_w;
+  if (!dense) {
+    c = R.cols[(int64_t)r * R.cap + i];
+    if (R.w) iw = sah_round<DT>(1.0f / sah_round<DT>(R.w[(int64_t)r * R.cap + i] + 1e-6f));
+    if (c < 0 || c >= R.n_keys) return;
+  }
+  const float z = logits[(int64_t)r * pitch + i];
+  const float p = (z == -INFINITY) ? 0.f : att_exp<DT>(z - m) * iw / den;
+  sah_store<DT>(weights, (int64_t)r * R.n_keys + c, p);
+}
+
+static int att_pick_split(int n_rows, int max_cnt, int* kps_out) {
+  // enough workgroups to cover 256 CUs several times, at least one chunk each
+  int chunks = (max_cnt + ATT_CHUNK - 1) / ATT_CHUNK;
+  if (chunks < 1) chunks = 1;
+  int want = (4096 + n_rows - 1) / n_rows;  // target ~4096 workgroups
+  if (want < 1) want = 1;
+  int n_split = chunks < want ? chunks : want;
+  if (n_split > 64) n_split = 64;
+  int cps = (chunks + n_split - 1) / n_split;  // chunks per split
+  n_split = (chunks + cps - 1) / cps;
+  *kps_out = cps * ATT_CHUNK;
+  return n_split;
+}
+
+extern "C" int64_t sah_sparse_attention_work_floats(int32_t n_rows, int32_t max_cnt, int32_t D) {
+  if (n_rows <= 0 || max_cnt < 0 || D <= 0) return 0;
+  int kps;
+  int n_split = att_pick_split(n_rows, max_cnt, &kps);
+  return (int64_t)n_rows * n_split * (D + 2);
+}
+
+template <int DT, int D>
+static int att_launch(const sah_attention_args* a, const att_params& P) {
+  hipStream_t st = (hipStream_t)a->stream;
+  hipLaunchKernelGGL((k_sparse_attn<DT, D>), dim3(P.n_split, a->rows.n_rows), dim3(ATT_NT), 0, st, P);
+  int rc = sah_launch_status("sah_sparse_attention");
+  if (rc) return rc;
+  hipLaunchKernelGGL((k_attn_combine<DT, D>), dim3(a->rows.n_rows), dim3(D < 64 ? 64 : D), 0, st,
+                     (const float*)a->work, P.n_split, a->Hq, a->Lq, a->sinks, a->out, a->stats_out);
+  return sah_launch_status("sah_sparse_attention(combine)");
+}
+
+template <int DT>
+static int att_dispatch_d(const sah_attention_args* a, const att_params& P) {
+  switch (a->D) {
+    case 16: return att_launch<DT, 16>(a, P);
+    case 32: return att_launch<DT, 32>(a, P);
+    case 64: return att_launch<DT, 64>(a, P);
+    case 128: return att_launch<DT, 128>(a, P);
+    default: return sah_fail(SAH_ESHAPE, "sah_sparse_attention: head_dim %d not in {16,32,64,128}", a->D);
+  }
+}
+
+extern "C" int sah_sparse_attention(const sah_attention_args* a) {
+  if (!a) return sah_fail(SAH_ENULL, "sah_sparse_attention: args is NULL");
+  if (!a->q || !a->k || !a->v || !a->out || !a->work) return sah_fail(SAH_ENULL, "sah_sparse_attention: NULL tensor");
+  if (a->B <= 0 || a->Hq <= 0 || a->Hkv <= 0 || a->Lq <= 0 || a->Lk <= 0)
+    return sah_fail(SAH_EINVAL, "sah_sparse_attention: non-positive dimension");
+  if (a->Hq % a->Hkv) return sah_fail(SAH_EINVAL, "sah_sparse_attention: Hq %% Hkv != 0");
+  if (a->rows.n_rows != a->B * a->Hq * a->Lq || a->rows.n_keys != a->Lk)
+    return sah_fail(SAH_EINVAL, "sah_sparse_attention: rows shape does not match B*Hq*Lq x Lk");
+  if (!a->dense) {
+    int rc = sah_check_rows(a->rows, "sah_sparse_attention");
+    if (rc) return rc;
+  }
+  const int es = a->dtype == SAH_F32 ? 4 : 2;
+  const int64_t align = 8;  // elements: 8-element vector loads
+  if (a->qs_b % align || a->qs_h % align || a->qs_l % align || a->ks_b % align || a->ks_h % align ||
+      a->ks_l % align || a->vs_b % align || a->vs_h % align || a->vs_l % align)
+    return sah_fail(SAH_ESHAPE, "sah_sparse_attention: strides must be multiples of 8 elements");
+  if (((uintptr_t)a->q | (uintptr_t)a->k | (uintptr_t)a->v) % (8 * es))
+    return sah_fail(SAH_ESHAPE, "sah_sparse_attention: q/k/v base pointers must be %d-byte aligned", 8 * es);
+  int max_cnt = a->dense ? a->Lk : a->max_cnt;
+  if (max_cnt <= 0) return sah_fail(SAH_EINVAL, "sah_sparse_attention: max_cnt must be > 0");
+  if (!a->dense && max_cnt > a->rows.cap) max_cnt = a->rows.cap;
+
+  att_params P;
+  P.rows = a->rows;
+  P.q = a->q; P.qs_b = a->qs_b; P.qs_h = a->qs_h; P.qs_l = a->qs_l;
+  P.k = a->k; P.ks_b = a->ks_b; P.ks_h = a->ks_h; P.ks_l = a->ks_l;
+  P.v = a->v; P.vs_b = a->vs_b; P.vs_h = a->vs_h; P.vs_l = a->vs_l;
+  P.amask = a->amask; P.ms_b = a->ms_b; P.ms_h = a->ms_h; P.ms_l = a->ms_l;
+  P.Hq = a->Hq; P.Hkv = a->Hkv; P.Lq = a->Lq; P.Lk = a->Lk;
+  P.scaling = a->scaling; P.unit_inv_w = a->unit_inv_w;
+  P.dense = a->dense ? 1 : 0;
+  P.n_split = att_pick_split(a->rows.n_rows, max_cnt, &P.kps);
+  P.work = a->work;
+  P.logits_out = a->logits_out;
+  P.logits_pitch = a->dense ? a->Lk : a->rows.cap;
+  const int64_t need = (int64_t)a->rows.n_rows * P.n_split * (a->D + 2);
+  if (a->work_floats < need)
+    return sah_fail(SAH_ECAPACITY, "sah_sparse_attention: work has %lld floats, need %lld", (long long)a->work_floats,
+                    (long long)need);
+  switch (a->dtype) {
+    case SAH_F32: return att_dispatch_d<SAH_F32>(a, P);
+    case SAH_BF16: return att_dispatch_d<SAH_BF16>(a, P);
+    case SAH_F16: return att_dispatch_d<SAH_F16>(a, P);
+    default: return sah_fail(SAH_EDTYPE, "sah_sparse_attention: dtype %d", a->dtype);
+  }
+}
+
+extern "C" int sah_attention_weights(const sah_attention_weights_args* a) {
+  if (!a) return sah_fail(SAH_ENULL, "sah_attention_weights: args is NULL");
+  if (!a->logits || !a->stats || !a->weights) return sah_fail(SAH_ENULL, "sah_attention_weights: NULL tensor");
+  if (a->rows.n_rows <= 0 || a->rows.n_keys <= 0) return sah_fail(SAH_EINVAL, "sah_attention_weights: empty rows");
+  const int dense = a->dense ? 1 : 0;
+  if (!dense) {
+    int rc = sah_check_rows(a->rows, "sah_attention_weights");
+    if (rc) return rc;
+  }
+  const int max_cnt = dense ? a->rows.n_keys : a->rows.cap;
+  const int64_t pitch = dense ? a->rows.n_keys : a->rows.cap;
+  dim3 g((max_cnt + 255) / 256, a->rows.n_rows), b(256);
+  hipStream_t st = (hipStream_t)a->stream;
+  switch (a->dtype) {
+    case SAH_F32: hipLaunchKernelGGL(k_attn_weights<SAH_F32>, g, b, 0, st, a->rows, a->logits, pitch, a->stats, a->unit_inv_w, dense, a->weights); break;
+    case SAH_BF16: hipLaunchKernelGGL(k_attn_weights<SAH_BF16>, g, b, 0, st, a->rows, a->logits, pitch, a->stats, a->unit_inv_w, dense, a->weights); break;
+    case SAH_F16: hipLaunchKernelGGL(k_attn_weights<SAH_F16>, g, b, 0, st, a->rows, a->logits, pitch, a->stats, a->unit_inv_w, dense, a->weights); break;
+    default: return sah_fail(SAH_EDTYPE, "sah_attention_weights: dtype %d", a->dtype);
+  }
+  return sah_launch_status("sah_attention_weights");
+}

@@ -1,0 +1,222 @@
+// Shared device/host helpers for the gfx950 kernels of libsah_mi355.so.
+// Wavefront = 64 lanes; a DPP "row" = 16 lanes; LDS = 160 KB per CU.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+#include <type_traits>
+
+#include "../../include/sah.h"
+
+#define SAH_WAVE 64
+
+// ---------------------------------------------------------------------------
+// host side: error reporting
+// ---------------------------------------------------------------------------
+char* sah_err_buf();  // thread-local, 512 bytes
+
+static inline int sah_fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(sah_err_buf(), 512, fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+static inline int sah_launch_status(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    return sah_fail((int)e, "%s: launch failed: %s", what, hipGetErrorString(e));
+  }
+  return SAH_OK;
+}
+
+static inline int sah_check_rows(const sah_rows& r, const char* what, bool need_cols = true) {
+  if (r.n_rows <= 0 || r.n_keys <= 0) return sah_fail(SAH_EINVAL, "%s: rows.n_rows/n_keys must be > 0", what);
+  if (r.n_words != (r.n_keys + 31) / 32) return sah_fail(SAH_EINVAL, "%s: rows.n_words != ceil(n_keys/32)", what);
+  if (!r.cnt || !r.bitmap) return sah_fail(SAH_ENULL, "%s: rows.cnt / rows.bitmap is NULL", what);
+  if (need_cols && (!r.cols || r.cap <= 0)) return sah_fail(SAH_ENULL, "%s: rows.cols is NULL or cap <= 0", what);
+  return SAH_OK;
+}
+
+// ---------------------------------------------------------------------------
+// device side: dtype helpers (bf16 / f16 handled as raw bits, fp32 arithmetic)
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float sah_bits_to_float(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t sah_float_to_bits(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+__device__ __forceinline__ float sah_bf16_to_float(uint16_t h) { return sah_bits_to_float(((uint32_t)h) << 16); }
+
+// round-to-nearest-even fp32 -> bf16 (what torch's .to(bfloat16) does)
+__device__ __forceinline__ uint16_t sah_float_to_bf16(float f) {
+  uint32_t u = sah_float_to_bits(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);  // NaN stays NaN
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float sah_f16_to_float(uint16_t h) {
+  return (float)__builtin_bit_cast(_Float16, h);
+}
+__device__ __forceinline__ uint16_t sah_float_to_f16(float f) {
+  return __builtin_bit_cast(uint16_t, (_Float16)f);
+}
+
+// value of `f` after a round trip through storage type DT
+template <int DT>
+__device__ __forceinline__ float sah_round(float f) {
+  if (DT == SAH_BF16) return sah_bf16_to_float(sah_float_to_bf16(f));
+  if (DT == SAH_F16) return sah_f16_to_float(sah_float_to_f16(f));
+  return f;
+}
+
+template <int DT>
+__device__ __forceinline__ float sah_load(const void* p, int64_t i) {
+  if (DT == SAH_BF16) return sah_bf16_to_float(((const uint16_t*)p)[i]);
+  if (DT == SAH_F16) return sah_f16_to_float(((const uint16_t*)p)[i]);
+  return ((const float*)p)[i];
+}
+
+template <int DT>
+__device__ __forceinline__ void sah_store(void* p, int64_t i, float f) {
+  if (DT == SAH_BF16) ((uint16_t*)p)[i] = sah_float_to_bf16(f);
+  else if (DT == SAH_F16) ((uint16_t*)p)[i] = sah_float_to_f16(f);
+  else ((float*)p)[i] = f;
+}
+
+// 8 consecutive elements starting at element index i (i % 8 == 0, 16-byte
+// aligned for 2-byte types, 32-byte for fp32) -> 8 floats
+template <int DT>
+__device__ __forceinline__ void sah_load8(const void* p, int64_t i, float (&o)[8]) {
+  if (DT == SAH_F32) {
+    const float4* f = (const float4*)((const float*)p + i);
+    float4 a = f[0], b = f[1];
+    o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+    o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+  } else {
+    uint4 u = *(const uint4*)((const uint16_t*)p + i);
+    uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      if (DT == SAH_BF16) {
+        o[2 * t] = sah_bits_to_float(w[t] << 16);
+        o[2 * t + 1] = sah_bits_to_float(w[t] & 0xffff0000u);
+      } else {
+        o[2 * t] = sah_f16_to_float((uint16_t)(w[t] & 0xffffu));
+        o[2 * t + 1] = sah_f16_to_float((uint16_t)(w[t] >> 16));
+      }
+    }
+  }
+}
+
+// order-preserving key of a score already rounded to DT: larger score => larger
+// unsigned key; -0 and +0 map to the same key (torch compares them equal).
+template <int DT>
+__device__ __forceinline__ uint32_t sah_sort_key(float score) {
+  if (DT == SAH_F32) {
+    uint32_t u = sah_float_to_bits(score);
+    if (u == 0x80000000u) u = 0;
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+  } else {
+    uint32_t u = (DT == SAH_BF16) ? sah_float_to_bf16(score) : sah_float_to_f16(score);
+    if (u == 0x8000u) u = 0;
+    return (u & 0x8000u) ? ((~u) & 0xffffu) : (u | 0x8000u);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// device side: cross-lane helpers
+// ---------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float sah_dpp(float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+
+// sum over each aligned group of 16 lanes (one DPP row); every lane gets the sum
+__device__ __forceinline__ float sah_row16_sum(float v) {
+  v += sah_dpp<0xB1>(v);   // quad_perm [1,0,3,2]
+  v += sah_dpp<0x4E>(v);   // quad_perm [2,3,0,1]
+  v += sah_dpp<0x141>(v);  // row_half_mirror
+  v += sah_dpp<0x140>(v);  // row_mirror
+  return v;
+}
+
+__device__ __forceinline__ float sah_wave_sum(float v) {
+  v = sah_row16_sum(v);
+  v += __shfl_xor(v, 16);
+  v += __shfl_xor(v, 32);
+  return v;
+}
+
+__device__ __forceinline__ float sah_wave_max(float v) {
+  v = fmaxf(v, sah_dpp<0xB1>(v));
+  v = fmaxf(v, sah_dpp<0x4E>(v));
+  v = fmaxf(v, sah_dpp<0x141>(v));
+  v = fmaxf(v, sah_dpp<0x140>(v));
+  v = fmaxf(v, __shfl_xor(v, 16));
+  v = fmaxf(v, __shfl_xor(v, 32));
+  return v;
+}
+
+__device__ __forceinline__ int sah_wave_sum_i(int v) {
+#pragma unroll
+  for (int o = 1; o < SAH_WAVE; o <<= 1) v += __shfl_xor(v, o);
+  return v;
+}
+
+// number of set bits of `m` at lane positions below the calling lane
+__device__ __forceinline__ int sah_lane_prefix(uint64_t m) {
+  return __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0));
+}
+
+// inclusive scan of one int per lane across the wave
+__device__ __forceinline__ int sah_wave_incl_scan(int v) {
+  const int lane = threadIdx.x & (SAH_WAVE - 1);
+#pragma unroll
+  for (int o = 1; o < SAH_WAVE; o <<= 1) {
+    int t = __shfl_up(v, o);
+    if (lane >= o) v += t;
+  }
+  return v;
+}
+
+// Exclusive scan of one int per thread across a block of NT threads
+// (NT % 64 == 0, NT <= 1024). `wsum` is LDS scratch of NT/64 + 1 ints. All
+// threads must call. Returns the exclusive prefix; *total receives the sum.
+template <int NT>
+__device__ __forceinline__ int sah_block_excl_scan(int v, int* wsum, int* total) {
+  constexpr int NW = NT / SAH_WAVE;
+  const int lane = threadIdx.x & (SAH_WAVE - 1);
+  const int wave = threadIdx.x / SAH_WAVE;
+  int incl = sah_wave_incl_scan(v);
+  __syncthreads();  // protect wsum from a previous use
+  if (lane == SAH_WAVE - 1) wsum[wave] = incl;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int i = 0; i < NW; ++i) {
+      int t = wsum[i];
+      wsum[i] = run;
+      run += t;
+    }
+    wsum[NW] = run;
+  }
+  __syncthreads();
+  *total = wsum[NW];
+  return wsum[wave] + incl - v;
+}
+
+// bits of 32-bit word `wi` that fall inside column range [lo, hi)
+__device__ __forceinline__ uint32_t sah_range_bits(int wi, int lo, int hi) {
+  int base = wi * 32;
+  int a = lo - base, b = hi - base;
+  if (b <= 0 || a >= 32) return 0u;
+  if (a < 0) a = 0;
+  if (b > 32) b = 32;
+  uint32_t upto_b = (b == 32) ? 0xffffffffu : ((1u << b) - 1u);
+  uint32_t upto_a = (a == 0) ? 0u : ((1u << a) - 1u);
+  return upto_b & ~upto_a;
+}

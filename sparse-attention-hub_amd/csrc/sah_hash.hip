@@ -1,0 +1,147 @@
+// HashAttention bit signatures: per query head a small MLP (D -> hidden ... ->
+// bits) followed by sign(), packed LSB-first into two uint32 planes per vector:
+// "positive" and "non-zero" (in bf16 an exact zero is not rare, and the reference
+// scores such a bit as 0, so it has to be representable).
+//
+// k_hash_sig_tile: one workgroup per (b, h, tile of TL vectors). The tile lives
+// in LDS as fp32; thread e owns output feature e and streams W[h][:, e] (coalesced
+// across threads) once per tile, so weight traffic is amortised over TL vectors.
+// Rounding follows torch op by op when the storage type is 16-bit: the layer
+// output, the bias add and the activation are each rounded to that type.
+#include "sah_common.h"
+
+#define SIG_NT 128
+#define SIG_TL 16        // vectors per tile
+#define SIG_MAXD 256     // widest layer supported
+
+struct sig_params {
+  const void* x; int64_t xs_b, xs_h, xs_l;
+  int B, Hq, group, L, D;
+  int n_layers;
+  const void* W[SAH_MAX_MLP_LAYERS];
+  const void* bias[SAH_MAX_MLP_LAYERS];
+  int d_out[SAH_MAX_MLP_LAYERS];
+  int act;
+  uint32_t* codes; int64_t code_pitch, code_offset;
+};
+
+__device__ __forceinline__ float sig_act(int act, float v) {
+  switch (act) {
+    case SAH_ACT_RELU: return v > 0.f ? v : 0.f;
+    case SAH_ACT_SILU: return v / (1.0f + expf(-v));
+    case SAH_ACT_GELU: return 0.5f * v * (1.0f + erff(v * 0.70710678118654752440f));
+    default: return tanhf(v);
+  }
+}
+
+template <int DT>
+__global__ __launch_bounds__(SIG_NT) void k_hash_sig_tile(sig_params P) {
+  __shared__ float s_a[SIG_TL][SIG_MAXD];
+  __shared__ float s_b[SIG_TL][SIG_MAXD];
+  const int tid = threadIdx.x;
+  const int tile = blockIdx.x;
+  const int bh = blockIdx.y;
+  const int h = bh % P.Hq;
+  const int b = bh / P.Hq;
+  const int hx = h / P.group;
+  const int l0 = tile * SIG_TL;
+  int nl = P.L - l0;
+  if (nl > SIG_TL) nl = SIG_TL;
+
+  // stage the tile (zero rows beyond nl keep the arithmetic finite)
+  for (int i = tid; i < SIG_TL * P.D; i += SIG_NT) {
+    const int t = i / P.D, d = i % P.D;
+    float v = 0.f;
+    if (t < nl) v = sah_load<DT>(P.x, (int64_t)b * P.xs_b + (int64_t)hx * P.xs_h + (int64_t)(l0 + t) * P.xs_l + d);
+    s_a[t][d] = v;
+  }
+  __syncthreads();
+
+  float (*cur)[SIG_MAXD] = s_a;
+  float (*nxt)[SIG_MAXD] = s_b;
+  int din = P.D;
+  for (int layer = 0; layer < P.n_layers; ++layer) {
+    const int dout = P.d_out[layer];
+    const bool last = (layer == P.n_layers - 1);
+    const int64_t wbase = (int64_t)h * din * dout;
+    for (int e = tid; e < dout; e += SIG_NT) {
+      float acc[SIG_TL];
+#pragma unroll
+      for (int t = 0; t < SIG_TL; ++t) acc[t] = 0.f;
+      for (int d = 0; d < din; ++d) {
+        const float wv = sah_load<DT>(P.W[layer], wbase + (int64_t)d * dout + e);
+#pragma unroll
+        for (int t = 0; t < SIG_TL; ++t) acc[t] = fmaf(cur[t][d], wv, acc[t]);
+      }
+      const float bv = sah_load<DT>(P.bias[layer], (int64_t)h * dout + e);
+#pragma unroll
+      for (int t = 0; t < SIG_TL; ++t) {
+        float y = sah_round<DT>(acc[t]);
+        y = sah_round<DT>(y + bv);
+        if (!last) y = sah_round<DT>(sig_act(P.act, y));
+        nxt[t][e] = y;
+      }
+    }
+    __syncthreads();
+    float (*tmp)[SIG_MAXD] = cur;
+    cur = nxt;
+    nxt = tmp;
+    din = dout;
+  }
+
+  // pack two planes per vector: bit e of .x = (y_e > 0), bit e of .y = (y_e != 0);
+  // the first wave ballots one vector at a time
+  if (tid < SAH_WAVE) {
+    const int bits = din;  // <= 32, checked on the host
+    for (int t = 0; t < nl; ++t) {
+      const float y = (tid < bits) ? cur[t][tid] : 0.f;
+      const uint64_t pos = __ballot(y > 0.f);
+      const uint64_t nz = __ballot(y != 0.f);
+      if (tid == 0) {
+        uint2 c;
+        c.x = (uint32_t)pos;
+        c.y = (uint32_t)nz;
+        ((uint2*)P.codes)[(int64_t)bh * P.code_pitch + P.code_offset + l0 + t] = c;
+      }
+    }
+  }
+}
+
+extern "C" int sah_hash_signatures(const sah_hash_sig_args* a) {
+  if (!a) return sah_fail(SAH_ENULL, "sah_hash_signatures: args is NULL");
+  if (!a->x || !a->codes) return sah_fail(SAH_ENULL, "sah_hash_signatures: x / codes is NULL");
+  if (a->B <= 0 || a->Hq <= 0 || a->group <= 0 || a->D <= 0 || a->Hq % a->group)
+    return sah_fail(SAH_EINVAL, "sah_hash_signatures: bad B/Hq/group/D");
+  if (a->L <= 0) return SAH_OK;  // nothing to hash
+  if (a->n_layers < 1 || a->n_layers > SAH_MAX_MLP_LAYERS)
+    return sah_fail(SAH_ESHAPE, "sah_hash_signatures: n_layers %d not in [1, %d]", a->n_layers, SAH_MAX_MLP_LAYERS);
+  if (a->D > SIG_MAXD) return sah_fail(SAH_ESHAPE, "sah_hash_signatures: D %d > %d", a->D, SIG_MAXD);
+  for (int i = 0; i < a->n_layers; ++i) {
+    if (!a->W[i] || !a->bias[i]) return sah_fail(SAH_ENULL, "sah_hash_signatures: layer %d weights are NULL", i);
+    if (a->d_out[i] <= 0 || a->d_out[i] > SIG_MAXD)
+      return sah_fail(SAH_ESHAPE, "sah_hash_signatures: layer %d width %d not in [1, %d]", i, a->d_out[i], SIG_MAXD);
+  }
+  if (a->d_out[a->n_layers - 1] > 32)
+    return sah_fail(SAH_ESHAPE, "sah_hash_signatures: %d signature bits do not fit one uint32 code", a->d_out[a->n_layers - 1]);
+  if (a->act < SAH_ACT_RELU || a->act > SAH_ACT_TANH) return sah_fail(SAH_EINVAL, "sah_hash_signatures: activation %d", a->act);
+  if (a->code_pitch < a->code_offset + a->L) return sah_fail(SAH_ECAPACITY, "sah_hash_signatures: code_pitch too small");
+
+  sig_params P;
+  P.x = a->x; P.xs_b = a->xs_b; P.xs_h = a->xs_h; P.xs_l = a->xs_l;
+  P.B = a->B; P.Hq = a->Hq; P.group = a->group; P.L = a->L; P.D = a->D;
+  P.n_layers = a->n_layers;
+  for (int i = 0; i < SAH_MAX_MLP_LAYERS; ++i) {
+    P.W[i] = a->W[i]; P.bias[i] = a->bias[i]; P.d_out[i] = a->d_out[i];
+  }
+  P.act = a->act;
+  P.codes = a->codes; P.code_pitch = a->code_pitch; P.code_offset = a->code_offset;
+  dim3 g((a->L + SIG_TL - 1) / SIG_TL, a->B * a->Hq), b(SIG_NT);
+  hipStream_t st = (hipStream_t)a->stream;
+  switch (a->dtype) {
+    case SAH_F32: hipLaunchKernelGGL(k_hash_sig_tile<SAH_F32>, g, b, 0, st, P); break;
+    case SAH_BF16: hipLaunchKernelGGL(k_hash_sig_tile<SAH_BF16>, g, b, 0, st, P); break;
+    case SAH_F16: hipLaunchKernelGGL(k_hash_sig_tile<SAH_F16>, g, b, 0, st, P); break;
+    default: return sah_fail(SAH_EDTYPE, "sah_hash_signatures: dtype %d", a->dtype);
+  }
+  return sah_launch_status("sah_hash_signatures");
+}

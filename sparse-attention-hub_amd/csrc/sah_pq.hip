@@ -1,0 +1,351 @@
+// PQCache kernels: batched Lloyd iteration (assignment + centre update) over
+// the sub-vectors of the key cache, quantisation of newly appended keys, and
+// asymmetric-distance (ADC) scoring through an LDS-resident lookup table.
+//
+// A group g = (b*Hkv + hk)*n_sub + s is one sub-space of one KV head. The
+// assignment kernel keeps the group's centres (n_cent x d_sub fp32, <= 16 KB) in
+// LDS, one thread per key, and accumulates the per-centre sums in LDS before a
+// single flush of global atomics per workgroup, so no (b, n, k, d) tensor ever
+// exists. Blocks are ordered sub-space-fastest so the n_sub workgroups that read
+// different 16 B slices of the same key rows run next to each other and share
+// the rows in L2.
+#include "sah_common.h"
+
+#define PQ_NT 256
+#define PQ_MAX_D 16
+#define PQ_MAX_CENT 256
+#define PQ_TILES 8  // key tiles of PQ_NT per workgroup
+
+struct pq_assign_params {
+  const void* k; int64_t ks_b, ks_h, ks_l;
+  int Hkv, n_sub, d_sub, n_cent;
+  int key_offset, n_keys;
+  const float* centres;
+  uint8_t* codes; int64_t code_pitch, code_offset;
+  float* sums; int* counts;
+  int round_dist;
+  const int* skip_flag;
+};
+
+template <int DT>
+__global__ __launch_bounds__(PQ_NT) void k_pq_assign(pq_assign_params P) {
+  __shared__ float s_c[PQ_MAX_CENT * PQ_MAX_D];
+  __shared__ float s_sum[PQ_MAX_CENT * PQ_MAX_D];
+  __shared__ int s_cnt[PQ_MAX_CENT];
+  if (P.skip_flag && *P.skip_flag) return;
+  const int tid = threadIdx.x;
+  const int s = blockIdx.x % P.n_sub;
+  const int tg = blockIdx.x / P.n_sub;
+  const int bh = blockIdx.y;  // b*Hkv + hk
+  const int hk = bh % P.Hkv;
+  const int b = bh / P.Hkv;
+  const int g = bh * P.n_sub + s;
+  const int d_sub = P.d_sub, n_cent = P.n_cent;
+  const int cd = n_cent * d_sub;
+
+  for (int i = tid; i < cd; i += PQ_NT) {
+    s_c[i] = P.centres[(int64_t)g * cd + i];
+    s_sum[i] = 0.f;
+  }
+  for (int i = tid; i < n_cent; i += PQ_NT) s_cnt[i] = 0;
+  __syncthreads();
+
+  const int64_t kbase = (int64_t)b * P.ks_b + (int64_t)hk * P.ks_h + (int64_t)s * d_sub;
+  for (int t = 0; t < PQ_TILES; ++t) {
+    const int n = (tg * PQ_TILES + t) * PQ_NT + tid;
+    if (n >= P.n_keys) continue;
+    float x[PQ_MAX_D];
+    const int64_t off = kbase + (int64_t)(P.key_offset + n) * P.ks_l;
+#pragma unroll
+    for (int d = 0; d < PQ_MAX_D; ++d) x[d] = (d < d_sub) ? sah_load<DT>(P.k, off + d) : 0.f;
+    int best = 0;
+    float bd = INFINITY;
+    for (int c = 0; c < n_cent; ++c) {
+      const float* cc = s_c + c * d_sub;
+      float dist = 0.f;
+      if (P.round_dist) {
+#pragma unroll
+        for (int d = 0; d < PQ_MAX_D; ++d) {
+          if (d < d_sub) {
+            const float df = sah_round<DT>(x[d] - cc[d]);
+            dist += sah_round<DT>(df * df);
+          }
+        }
+        dist = sah_round<DT>(dist);
+      } else {
+#pragma unroll
+        for (int d = 0; d < PQ_MAX_D; ++d) {
+          if (d < d_sub) {
+            const float df = x[d] - cc[d];
+            dist = fmaf(df, df, dist);
+          }
+        }
+      }
+      if (dist < bd) {
+        bd = dist;
+        best = c;
+      }
+    }
+    P.codes[(((int64_t)bh * P.code_pitch) + P.code_offset + n) * P.n_sub + s] = (uint8_t)best;
+    if (P.sums) {
+#pragma unroll
+      for (int d = 0; d < PQ_MAX_D; ++d)
+        if (d < d_sub) atomicAdd(&s_sum[best * d_sub + d], x[d]);
+      atomicAdd(&s_cnt[best], 1);
+    }
+  }
+  if (!P.sums) return;
+  __syncthreads();
+  for (int c = tid; c < n_cent; c += PQ_NT) {
+    const int cn = s_cnt[c];
+    if (cn) {
+      atomicAdd(&P.counts[(int64_t)g * n_cent + c], cn);
+      for (int d = 0; d < d_sub; ++d) atomicAdd(&P.sums[(int64_t)g * cd + c * d_sub + d], s_sum[c * d_sub + d]);
+    }
+  }
+}
+
+struct pq_update_params {
+  const void* k; int64_t ks_b, ks_h, ks_l;
+  int Hkv, n_sub, d_sub, n_cent, key_offset;
+  float* centres;
+  const float* sums; const int* counts;
+  const int* reseed_idx;
+  float* shift2;
+  float tol;
+  int* state;
+  int n_groups;
+};
+
+template <int DT>
+__global__ __launch_bounds__(PQ_NT) void k_pq_update(pq_update_params P) {
+  __shared__ float s_red[PQ_NT / SAH_WAVE];
+  if (P.state[2]) return;
+  const int tid = threadIdx.x;
+  const int g = blockIdx.x;
+  const int s = g % P.n_sub;
+  const int bh = g / P.n_sub;
+  const int hk = bh % P.Hkv;
+  const int b = bh / P.Hkv;
+  const int d_sub = P.d_sub, n_cent = P.n_cent;
+  float move = 0.f;
+  if (tid < n_cent) {
+    const int c = tid;
+    const int cn = P.counts[(int64_t)g * n_cent + c];
+    float* cc = P.centres + ((int64_t)g * n_cent + c) * d_sub;
+    const float* ss = P.sums + ((int64_t)g * n_cent + c) * d_sub;
+    float acc = 0.f;
+    int64_t roff = 0;
+    if (cn == 0) {
+      const int ridx = P.reseed_idx[(int64_t)g * n_cent + c];
+      roff = (int64_t)b * P.ks_b + (int64_t)hk * P.ks_h + (int64_t)(P.key_offset + ridx) * P.ks_l + (int64_t)s * d_sub;
+    }
+    for (int d = 0; d < d_sub; ++d) {
+      const float nv = (cn > 0) ? ss[d] / (float)cn : sah_load<DT>(P.k, roff + d);
+      const float df = nv - cc[d];
+      acc = fmaf(df, df, acc);
+      cc[d] = nv;
+    }
+    move = sqrtf(acc);
+  }
+  move = sah_wave_sum(move);
+  if ((tid & (SAH_WAVE - 1)) == 0) s_red[tid / SAH_WAVE] = move;
+  __syncthreads();
+  if (tid == 0) {
+    float tot = 0.f;
+    for (int i = 0; i < PQ_NT / SAH_WAVE; ++i) tot += s_red[i];
+    const float sh2 = tot * tot;
+    P.shift2[g] = sh2;
+    if (sh2 < P.tol) atomicAdd(&P.state[0], 1);
+    __threadfence();
+    const int ticket = atomicAdd(&P.state[1], 1);
+    if (ticket == P.n_groups - 1) {
+      // last group of this iteration: publish the verdict and reset the counters
+      const int conv = atomicAdd(&P.state[0], 0);
+      P.state[3] = (conv == P.n_groups) ? 1 : 0;
+      P.state[0] = 0;
+      P.state[1] = 0;
+    }
+  }
+}
+
+// state[3] -> state[2] is promoted by a separate one-thread kernel so that every
+// group of the iteration in flight still sees the old flag.
+__global__ void k_pq_promote(int* state) {
+  if (threadIdx.x == 0 && blockIdx.x == 0 && state[3]) state[2] = 1;
+}
+
+struct pq_adc_params {
+  const void* q; int64_t qs_b, qs_h, qs_l;
+  int Hq, Hkv, Lq, n_sub, d_sub, n_cent;
+  const float* centres;
+  const uint8_t* codes; int64_t code_pitch;
+  int n_cand;
+  void* keys_out; int64_t key_pitch;
+};
+
+#define ADC_TILES 8
+#define ADC_MAX_LUT 4096  // n_sub * n_cent
+
+template <int DT>
+__global__ __launch_bounds__(PQ_NT) void k_pq_adc(pq_adc_params P) {
+  constexpr int NQ = (DT == SAH_F32) ? 2 : 4;
+  typedef typename std::conditional<DT == SAH_F32, float, uint16_t>::type lut_t;
+  typedef typename std::conditional<DT == SAH_F32, uint32_t, uint16_t>::type key_t;
+  __shared__ lut_t s_lut[NQ * ADC_MAX_LUT];
+  const int tid = threadIdx.x;
+  const int bh = blockIdx.y;
+  const int hk = bh % P.Hkv;
+  const int b = bh / P.Hkv;
+  const int G = P.Hq / P.Hkv;
+  const int nvec = G * P.Lq;
+  const int v0 = blockIdx.z * NQ;
+  const int n_sub = P.n_sub, d_sub = P.d_sub, n_cent = P.n_cent;
+  const int lut_n = n_sub * n_cent;
+
+  int row[NQ];
+#pragma unroll
+  for (int i = 0; i < NQ; ++i) {
+    const int v = v0 + i;
+    row[i] = -1;
+    if (v < nvec) row[i] = (b * P.Hq + hk * G + v / P.Lq) * P.Lq + v % P.Lq;
+  }
+  for (int idx = tid; idx < NQ * lut_n; idx += PQ_NT) {
+    const int i = idx / lut_n;
+    const int rem = idx % lut_n;
+    const int s = rem / n_cent, c = rem % n_cent;
+    const int v = v0 + i;
+    float val = 0.f;
+    if (v < nvec) {
+      const int h = hk * G + v / P.Lq, qi = v % P.Lq;
+      const int64_t qo = (int64_t)b * P.qs_b + (int64_t)h * P.qs_h + (int64_t)qi * P.qs_l + (int64_t)s * d_sub;
+      const float* cc = P.centres + (((int64_t)bh * n_sub + s) * n_cent + c) * d_sub;
+      float acc = 0.f;
+      for (int d = 0; d < d_sub; ++d) acc = fmaf(sah_load<DT>(P.q, qo + d), cc[d], acc);
+      val = sah_round<DT>(acc);
+    }
+    if (DT == SAH_F32) s_lut[idx] = (lut_t)val;
+    else if (DT == SAH_BF16) s_lut[idx] = (lut_t)sah_float_to_bf16(val);
+    else s_lut[idx] = (lut_t)sah_float_to_f16(val);
+  }
+  __syncthreads();
+
+  for (int t = 0; t < ADC_TILES; ++t) {
+    const int n = (blockIdx.x * ADC_TILES + t) * PQ_NT + tid;
+    if (n >= P.n_cand) continue;
+    const uint8_t* code = P.codes + ((int64_t)bh * P.code_pitch + n) * n_sub;
+    float acc[NQ];
+#pragma unroll
+    for (int i = 0; i < NQ; ++i) acc[i] = 0.f;
+    for (int s = 0; s < n_sub; ++s) {
+      const int c = code[s];
+#pragma unroll
+      for (int i = 0; i < NQ; ++i) {
+        const lut_t raw = s_lut[i * lut_n + s * n_cent + c];
+        float lv;
+        if (DT == SAH_F32) lv = (float)raw;
+        else if (DT == SAH_BF16) lv = sah_bf16_to_float((uint16_t)raw);
+        else lv = sah_f16_to_float((uint16_t)raw);
+        acc[i] += lv;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < NQ; ++i) {
+      if (row[i] >= 0)
+        ((key_t*)P.keys_out)[(int64_t)row[i] * P.key_pitch + n] = (key_t)sah_sort_key<DT>(sah_round<DT>(acc[i]));
+    }
+  }
+}
+
+static int pq_check_common(const char* what, int B, int Hkv, int n_sub, int d_sub, int n_cent) {
+  if (B <= 0 || Hkv <= 0 || n_sub <= 0) return sah_fail(SAH_EINVAL, "%s: bad B/Hkv/n_sub", what);
+  if (d_sub <= 0 || d_sub > PQ_MAX_D) return sah_fail(SAH_ESHAPE, "%s: d_sub %d not in [1, %d]", what, d_sub, PQ_MAX_D);
+  if (n_cent <= 0 || n_cent > PQ_MAX_CENT) return sah_fail(SAH_ESHAPE, "%s: n_cent %d not in [1, %d]", what, n_cent, PQ_MAX_CENT);
+  if ((int64_t)B * Hkv > 65535) return sah_fail(SAH_ESHAPE, "%s: B*Hkv > 65535", what);
+  return SAH_OK;
+}
+
+extern "C" int sah_pq_kmeans_assign(const sah_pq_assign_args* a) {
+  if (!a) return sah_fail(SAH_ENULL, "sah_pq_kmeans_assign: args is NULL");
+  int rc = pq_check_common("sah_pq_kmeans_assign", a->B, a->Hkv, a->n_sub, a->d_sub, a->n_cent);
+  if (rc) return rc;
+  if (!a->k || !a->centres || !a->codes) return sah_fail(SAH_ENULL, "sah_pq_kmeans_assign: NULL tensor");
+  if ((a->sums == nullptr) != (a->counts == nullptr)) return sah_fail(SAH_EINVAL, "sah_pq_kmeans_assign: sums and counts go together");
+  if (a->n_keys <= 0) return SAH_OK;
+  if (a->key_offset < 0 || a->code_offset < 0 || a->code_pitch < a->code_offset + a->n_keys)
+    return sah_fail(SAH_ECAPACITY, "sah_pq_kmeans_assign: code_pitch %lld < code_offset %lld + n_keys %d",
+                    (long long)a->code_pitch, (long long)a->code_offset, a->n_keys);
+  pq_assign_params P;
+  P.k = a->k; P.ks_b = a->ks_b; P.ks_h = a->ks_h; P.ks_l = a->ks_l;
+  P.Hkv = a->Hkv; P.n_sub = a->n_sub; P.d_sub = a->d_sub; P.n_cent = a->n_cent;
+  P.key_offset = a->key_offset; P.n_keys = a->n_keys;
+  P.centres = a->centres;
+  P.codes = a->codes; P.code_pitch = a->code_pitch; P.code_offset = a->code_offset;
+  P.sums = a->sums; P.counts = a->counts;
+  P.round_dist = a->round_dist;
+  P.skip_flag = a->skip_flag;
+  const int per_wg = PQ_NT * PQ_TILES;
+  dim3 g(((a->n_keys + per_wg - 1) / per_wg) * a->n_sub, a->B * a->Hkv), blk(PQ_NT);
+  hipStream_t st = (hipStream_t)a->stream;
+  switch (a->dtype) {
+    case SAH_F32: hipLaunchKernelGGL(k_pq_assign<SAH_F32>, g, blk, 0, st, P); break;
+    case SAH_BF16: hipLaunchKernelGGL(k_pq_assign<SAH_BF16>, g, blk, 0, st, P); break;
+    case SAH_F16: hipLaunchKernelGGL(k_pq_assign<SAH_F16>, g, blk, 0, st, P); break;
+    default: return sah_fail(SAH_EDTYPE, "sah_pq_kmeans_assign: dtype %d", a->dtype);
+  }
+  return sah_launch_status("sah_pq_kmeans_assign");
+}
+
+extern "C" int sah_pq_kmeans_update(const sah_pq_update_args* a) {
+  if (!a) return sah_fail(SAH_ENULL, "sah_pq_kmeans_update: args is NULL");
+  int rc = pq_check_common("sah_pq_kmeans_update", a->B, a->Hkv, a->n_sub, a->d_sub, a->n_cent);
+  if (rc) return rc;
+  if (!a->k || !a->centres || !a->sums || !a->counts || !a->reseed_idx || !a->shift2 || !a->state)
+    return sah_fail(SAH_ENULL, "sah_pq_kmeans_update: NULL tensor");
+  pq_update_params P;
+  P.k = a->k; P.ks_b = a->ks_b; P.ks_h = a->ks_h; P.ks_l = a->ks_l;
+  P.Hkv = a->Hkv; P.n_sub = a->n_sub; P.d_sub = a->d_sub; P.n_cent = a->n_cent; P.key_offset = a->key_offset;
+  P.centres = a->centres; P.sums = a->sums; P.counts = a->counts; P.reseed_idx = a->reseed_idx;
+  P.shift2 = a->shift2; P.tol = a->tol; P.state = a->state;
+  P.n_groups = a->B * a->Hkv * a->n_sub;
+  dim3 g(P.n_groups), blk(PQ_NT);
+  hipStream_t st = (hipStream_t)a->stream;
+  switch (a->dtype) {
+    case SAH_F32: hipLaunchKernelGGL(k_pq_update<SAH_F32>, g, blk, 0, st, P); break;
+    case SAH_BF16: hipLaunchKernelGGL(k_pq_update<SAH_BF16>, g, blk, 0, st, P); break;
+    case SAH_F16: hipLaunchKernelGGL(k_pq_update<SAH_F16>, g, blk, 0, st, P); break;
+    default: return sah_fail(SAH_EDTYPE, "sah_pq_kmeans_update: dtype %d", a->dtype);
+  }
+  rc = sah_launch_status("sah_pq_kmeans_update");
+  if (rc) return rc;
+  hipLaunchKernelGGL(k_pq_promote, dim3(1), dim3(SAH_WAVE), 0, st, a->state);
+  return sah_launch_status("sah_pq_kmeans_update(promote)");
+}
+
+extern "C" int sah_pq_adc_scores(const sah_pq_adc_args* a) {
+  if (!a) return sah_fail(SAH_ENULL, "sah_pq_adc_scores: args is NULL");
+  int rc = pq_check_common("sah_pq_adc_scores", a->B, a->Hkv, a->n_sub, a->d_sub, a->n_cent);
+  if (rc) return rc;
+  if (!a->q || !a->centres || !a->codes || !a->keys_out) return sah_fail(SAH_ENULL, "sah_pq_adc_scores: NULL tensor");
+  if (a->Hq <= 0 || a->Lq <= 0 || a->Hq % a->Hkv) return sah_fail(SAH_EINVAL, "sah_pq_adc_scores: bad Hq/Lq");
+  if (a->n_sub * a->n_cent > ADC_MAX_LUT) return sah_fail(SAH_ESHAPE, "sah_pq_adc_scores: n_sub*n_cent > %d", ADC_MAX_LUT);
+  if (a->n_cand <= 0) return SAH_OK;
+  if (a->code_pitch < a->n_cand || a->key_pitch < a->n_cand) return sah_fail(SAH_ECAPACITY, "sah_pq_adc_scores: pitch < n_cand");
+  pq_adc_params P;
+  P.q = a->q; P.qs_b = a->qs_b; P.qs_h = a->qs_h; P.qs_l = a->qs_l;
+  P.Hq = a->Hq; P.Hkv = a->Hkv; P.Lq = a->Lq; P.n_sub = a->n_sub; P.d_sub = a->d_sub; P.n_cent = a->n_cent;
+  P.centres = a->centres; P.codes = a->codes; P.code_pitch = a->code_pitch; P.n_cand = a->n_cand;
+  P.keys_out = a->keys_out; P.key_pitch = a->key_pitch;
+  const int nvec = (a->Hq / a->Hkv) * a->Lq;
+  const int nq = a->dtype == SAH_F32 ? 2 : 4;
+  const int per_wg = PQ_NT * ADC_TILES;
+  dim3 g((a->n_cand + per_wg - 1) / per_wg, a->B * a->Hkv, (nvec + nq - 1) / nq), blk(PQ_NT);
+  hipStream_t st = (hipStream_t)a->stream;
+  switch (a->dtype) {
+    case SAH_F32: hipLaunchKernelGGL(k_pq_adc<SAH_F32>, g, blk, 0, st, P); break;
+    case SAH_BF16: hipLaunchKernelGGL(k_pq_adc<SAH_BF16>, g, blk, 0, st, P); break;
+    case SAH_F16: hipLaunchKernelGGL(k_pq_adc<SAH_F16>, g, blk, 0, st, P); break;
+    default: return sah_fail(SAH_EDTYPE, "sah_pq_adc_scores: dtype %d", a->dtype);
+  }
+  return sah_launch_status("sah_pq_adc_scores");
+}

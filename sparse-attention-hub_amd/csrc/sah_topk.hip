@@ -1,0 +1,321 @@
+// Row-wise top-k selection with the canonical tie rule "lowest column first".
+//
+// One workgroup (1024 threads = 16 waves) per mask row. Keys are unsigned and
+// order-preserving (larger = better); already-active columns take a caller
+// chosen key so they rank exactly where the reference's `scores[prev != 0] =
+// min` puts them. The k-th key is found by MSB-first radix select with an LDS
+// histogram per digit; the winners are then written in ascending column order
+// by a wave-ordered compaction (ballot + mbcnt inside a wave, one LDS exchange
+// across the 16 waves), which is what makes ties resolve to the lowest column.
+// Each wave owns 64-column aligned chunks, so the bitmap words it updates are
+// touched by no other wave and need no atomics.
+#include "sah_common.h"
+
+#define SEL_NT 1024
+#define SEL_NW (SEL_NT / SAH_WAVE)
+#define SEL_DIGIT_BITS 13
+#define SEL_BINS (1 << SEL_DIGIT_BITS)
+
+// ---- key sources -----------------------------------------------------------
+struct key_src_mem16 {
+  const uint16_t* keys;  // row base, indexed by candidate
+  __device__ __forceinline__ uint32_t operator()(int cand) const { return keys[cand]; }
+};
+struct key_src_mem32 {
+  const uint32_t* keys;
+  __device__ __forceinline__ uint32_t operator()(int cand) const { return keys[cand]; }
+};
+// signature score of the reference, sum_e q_e k_e with q_e, k_e in {-1, 0, +1}:
+// popc(nz) - 2 popc((q ^ k) & nz), nz = bits where both are non-zero; in [-32, 32]
+__device__ __forceinline__ int sig_score(uint2 q, uint2 k) {
+  const uint32_t nz = q.y & k.y;
+  return __popc(nz) - 2 * __popc((q.x ^ k.x) & nz);
+}
+struct key_src_hamming {
+  const uint2* kcodes;  // code stream base: (positive plane, non-zero plane) per key
+  uint2 qcode;
+  // score + 33 in [1, 65], so every real column outranks the excluded key 0
+  __device__ __forceinline__ uint32_t operator()(int cand) const { return (uint32_t)(sig_score(qcode, kcodes[cand]) + 33); }
+};
+
+struct sel_shared {
+  uint32_t hist[SEL_BINS];
+  int scan[SEL_NW + 1];
+  int wave_gt[SEL_NW];
+  int wave_eq[SEL_NW];
+  int wave_out[SEL_NW];
+  int wave_tie[SEL_NW];
+  uint32_t digit;
+  int need;
+  int total_out;
+};
+
+// KEYBITS: number of significant key bits (7, 16 or 32)
+template <typename SRC, int KEYBITS>
+__device__ __forceinline__ void select_row(sel_shared& S, const sah_rows& R, int r, const SRC& src, int n_cand,
+                                           int col_offset, int k, uint32_t excluded_key) {
+  const int tid = threadIdx.x;
+  const int lane = tid & (SAH_WAVE - 1);
+  const int wave = tid / SAH_WAVE;
+  const uint32_t* bm = R.bitmap + (int64_t)r * R.n_words;
+
+  // 64-column aligned chunks of the candidate range, split contiguously over waves
+  const int c_first = col_offset / SAH_WAVE;
+  const int c_last = (col_offset + n_cand - 1) / SAH_WAVE;
+  const int n_chunks = c_last - c_first + 1;
+  const int cpw = (n_chunks + SEL_NW - 1) / SEL_NW;
+  const int my_c0 = c_first + wave * cpw;
+  int my_c1 = my_c0 + cpw;
+  if (my_c1 > c_last + 1) my_c1 = c_last + 1;
+
+  auto eff_key = [&](int col, bool& valid, bool& excl) -> uint32_t {
+    const int cand = col - col_offset;
+    valid = (cand >= 0 && cand < n_cand);
+    excl = false;
+    if (!valid) return 0u;
+    excl = (bm[col >> 5] >> (col & 31)) & 1u;
+    return excl ? excluded_key : src(cand);
+  };
+
+  if (k > n_cand) k = n_cand;
+  int need = k;
+  uint32_t prefix = 0;
+  int bits_done = 0;
+
+  // ---- radix select of the k-th largest key --------------------------------
+  while (bits_done < KEYBITS) {
+    int wd = KEYBITS - bits_done;
+    if (wd > SEL_DIGIT_BITS) wd = SEL_DIGIT_BITS;
+    const int sh = KEYBITS - bits_done - wd;
+    const int nb = 1 << wd;
+    for (int i = tid; i < nb; i += SEL_NT) S.hist[i] = 0;
+    __syncthreads();
+    for (int c = my_c0; c < my_c1; ++c) {
+      const int col = c * SAH_WAVE + lane;
+      bool valid, excl;
+      const uint32_t key = eff_key(col, valid, excl);
+      if (valid) {
+        const bool match = (bits_done == 0) || ((key >> (sh + wd)) == prefix);
+        if (match) atomicAdd(&S.hist[(key >> sh) & (uint32_t)(nb - 1)], 1u);
+      }
+    }
+    __syncthreads();
+    // descending scan over digits: thread t owns the t-th highest group of bins
+    constexpr int GROUPS = SEL_NT;
+    const int per = (nb + GROUPS - 1) / GROUPS;  // bins per thread (1 or 8)
+    const int hi_bin = nb - 1 - tid * per;       // my highest bin
+    int mine = 0;
+    for (int i = 0; i < per; ++i) {
+      const int bin = hi_bin - i;
+      if (bin >= 0) mine += (int)S.hist[bin];
+    }
+    int total;
+    const int above = sah_block_excl_scan<SEL_NT>(mine, S.scan, &total);
+    if (above < need && need <= above + mine) {
+      int run = above;
+      for (int i = 0; i < per; ++i) {
+        const int bin = hi_bin - i;
+        if (bin < 0) break;
+        const int cbin = (int)S.hist[bin];
+        if (need <= run + cbin) {
+          S.digit = (uint32_t)bin;
+          S.need = need - run;
+          break;
+        }
+        run += cbin;
+      }
+    }
+    __syncthreads();
+    prefix = (prefix << wd) | S.digit;
+    need = S.need;
+    bits_done += wd;
+    __syncthreads();
+  }
+  const uint32_t T = prefix;  // k-th largest key; `need` ties at T are taken, lowest column first
+
+  // ---- per-wave counts, then ordered compaction -------------------------------
+  int n_gt = 0, n_eq = 0;
+  for (int c = my_c0; c < my_c1; ++c) {
+    const int col = c * SAH_WAVE + lane;
+    bool valid, excl;
+    const uint32_t key = eff_key(col, valid, excl);
+    n_gt += __popcll(__ballot(valid && !excl && key > T));
+    n_eq += __popcll(__ballot(valid && key == T));
+  }
+  if (lane == 0) {
+    S.wave_gt[wave] = n_gt;
+    S.wave_eq[wave] = n_eq;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int tie_run = 0, out_run = 0;
+    for (int wv = 0; wv < SEL_NW; ++wv) {
+      S.wave_tie[wv] = tie_run;
+      S.wave_out[wv] = out_run;
+      // ties are consumed in column order; excluded ties use up rank but emit nothing,
+      // so the emitted count of this wave is only known after its walk: recomputed below
+      tie_run += S.wave_eq[wv];
+      out_run += S.wave_gt[wv];
+    }
+  }
+  __syncthreads();
+
+  // The number of *emitted* ties per wave depends on which of its ties are excluded,
+  // so output offsets take a second exchange: each wave counts its emitted ties first.
+  int tie_rank = S.wave_tie[wave];
+  int emit_ties = 0;
+  for (int c = my_c0; c < my_c1; ++c) {
+    const int col = c * SAH_WAVE + lane;
+    bool valid, excl;
+    const uint32_t key = eff_key(col, valid, excl);
+    const bool is_tie = valid && key == T;
+    const uint64_t tm = __ballot(is_tie);
+    const bool take = is_tie && !excl && (tie_rank + sah_lane_prefix(tm) < need);
+    emit_ties += __popcll(__ballot(take));
+    tie_rank += __popcll(tm);
+  }
+  __syncthreads();  // wave_eq is re-used below
+  if (lane == 0) S.wave_eq[wave] = emit_ties;
+  __syncthreads();
+  if (tid == 0) {
+    int out_run = 0;
+    for (int wv = 0; wv < SEL_NW; ++wv) {
+      S.wave_out[wv] = out_run;
+      out_run += S.wave_gt[wv] + S.wave_eq[wv];
+    }
+    S.total_out = out_run;
+  }
+  __syncthreads();
+
+  int cnt0 = R.cnt[r];
+  if (cnt0 > R.cap) cnt0 = R.cap;
+  int* cols = R.cols + (int64_t)r * R.cap;
+  float* w = R.w ? R.w + (int64_t)r * R.cap : nullptr;
+  uint32_t* bmw = R.bitmap + (int64_t)r * R.n_words;
+  int out_pos = cnt0 + S.wave_out[wave];
+  tie_rank = S.wave_tie[wave];
+  for (int c = my_c0; c < my_c1; ++c) {
+    const int col = c * SAH_WAVE + lane;
+    bool valid, excl;
+    const uint32_t key = eff_key(col, valid, excl);
+    const bool is_tie = valid && key == T;
+    const uint64_t tm = __ballot(is_tie);
+    const bool sel = valid && !excl && (key > T || (is_tie && (tie_rank + sah_lane_prefix(tm) < need)));
+    const uint64_t sm = __ballot(sel);
+    if (sel) {
+      const int pos = out_pos + sah_lane_prefix(sm);
+      if (pos < R.cap) {
+        cols[pos] = col;
+        if (w) w[pos] = 1.0f;
+      }
+    }
+    if (sm) {
+      const int w0 = c * 2;
+      if (lane == 0 && (uint32_t)sm) bmw[w0] |= (uint32_t)sm;
+      if (lane == 32 && (uint32_t)(sm >> 32) && w0 + 1 < R.n_words) bmw[w0 + 1] |= (uint32_t)(sm >> 32);
+    }
+    out_pos += __popcll(sm);
+    tie_rank += __popcll(tm);
+  }
+  __syncthreads();  // all reads of the old bitmap/cnt precede the count update
+  if (tid == 0) R.cnt[r] = cnt0 + S.total_out;
+}
+
+template <int KB>
+__global__ __launch_bounds__(SEL_NT) void k_select_topk(sah_rows R, const void* keys, int64_t pitch, int n_cand,
+                                                        int col_offset, int k, uint32_t excluded_key) {
+  __shared__ sel_shared S;
+  const int r = blockIdx.x;
+  if (KB == 16) {
+    key_src_mem16 src{(const uint16_t*)keys + (int64_t)r * pitch};
+    select_row<key_src_mem16, 16>(S, R, r, src, n_cand, col_offset, k, excluded_key);
+  } else {
+    key_src_mem32 src{(const uint32_t*)keys + (int64_t)r * pitch};
+    select_row<key_src_mem32, 32>(S, R, r, src, n_cand, col_offset, k, excluded_key);
+  }
+}
+
+__global__ __launch_bounds__(SEL_NT) void k_hamming_topk(sah_rows R, const uint2* kcodes, int64_t pitch,
+                                                         const uint2* qcodes, int lq, int k) {
+  __shared__ sel_shared S;
+  const int r = blockIdx.x;
+  key_src_hamming src{kcodes + (int64_t)(r / lq) * pitch, qcodes[r]};
+  select_row<key_src_hamming, 7>(S, R, r, src, R.n_keys, 0, k, 0u);
+}
+
+// Signature scores as sortable float keys, for callers that pass an additive
+// attention mask: score = round_to_dtype(float(sig_score) + amask).
+template <int DT>
+__global__ __launch_bounds__(256) void k_hamming_scores(const uint2* kcodes, int64_t code_pitch, const uint2* qcodes,
+                                                        int Hq, int Lq, int n_keys, const void* amask,
+                                                        int64_t ms_b, int64_t ms_h, int64_t ms_l, void* keys_out,
+                                                        int64_t key_pitch) {
+  typedef typename std::conditional<DT == SAH_F32, uint32_t, uint16_t>::type key_t;
+  const int r = blockIdx.y;
+  const int j = blockIdx.x * 256 + threadIdx.x;
+  if (j >= n_keys) return;
+  const int qi = r % Lq;
+  const int h = (r / Lq) % Hq;
+  const int b = r / (Lq * Hq);
+  float s = (float)sig_score(qcodes[r], kcodes[(int64_t)(r / Lq) * code_pitch + j]);
+  if (amask) s = sah_round<DT>(s + sah_load<DT>(amask, (int64_t)b * ms_b + (int64_t)h * ms_h + (int64_t)qi * ms_l + j));
+  ((key_t*)keys_out)[(int64_t)r * key_pitch + j] = (key_t)sah_sort_key<DT>(s);
+}
+
+extern "C" int sah_hamming_scores(const sah_hamming_scores_args* a) {
+  if (!a) return sah_fail(SAH_ENULL, "sah_hamming_scores: args is NULL");
+  if (!a->kcodes || !a->qcodes || !a->keys_out) return sah_fail(SAH_ENULL, "sah_hamming_scores: NULL tensor");
+  if (a->B <= 0 || a->Hq <= 0 || a->Lq <= 0 || a->n_keys <= 0)
+    return sah_fail(SAH_EINVAL, "sah_hamming_scores: bad dimensions");
+  if (a->code_pitch < a->n_keys || a->key_pitch < a->n_keys) return sah_fail(SAH_ECAPACITY, "sah_hamming_scores: pitch < n_keys");
+  const int n_rows = a->B * a->Hq * a->Lq;
+  if (n_rows > 65535) return sah_fail(SAH_ESHAPE, "sah_hamming_scores: more than 65535 rows");
+  dim3 g((a->n_keys + 255) / 256, n_rows), blk(256);
+  hipStream_t st = (hipStream_t)a->stream;
+#define SAH_HS_LAUNCH(DTC)                                                                                          \
+  hipLaunchKernelGGL(k_hamming_scores<DTC>, g, blk, 0, st, (const uint2*)a->kcodes, a->code_pitch,                  \
+                     (const uint2*)a->qcodes, a->Hq, a->Lq, a->n_keys, a->amask, a->ms_b, a->ms_h, a->ms_l,        \
+                     a->keys_out, a->key_pitch)
+  switch (a->dtype) {
+    case SAH_F32: SAH_HS_LAUNCH(SAH_F32); break;
+    case SAH_BF16: SAH_HS_LAUNCH(SAH_BF16); break;
+    case SAH_F16: SAH_HS_LAUNCH(SAH_F16); break;
+    default: return sah_fail(SAH_EDTYPE, "sah_hamming_scores: dtype %d", a->dtype);
+  }
+#undef SAH_HS_LAUNCH
+  return sah_launch_status("sah_hamming_scores");
+}
+
+extern "C" int sah_select_topk(const sah_select_topk_args* a) {
+  if (!a) return sah_fail(SAH_ENULL, "sah_select_topk: args is NULL");
+  int rc = sah_check_rows(a->rows, "sah_select_topk");
+  if (rc) return rc;
+  if (!a->keys) return sah_fail(SAH_ENULL, "sah_select_topk: keys is NULL");
+  if (a->key_bits != 16 && a->key_bits != 32) return sah_fail(SAH_EINVAL, "sah_select_topk: key_bits must be 16 or 32");
+  if (a->n_cand <= 0 || a->col_offset < 0 || (int64_t)a->col_offset + a->n_cand > a->rows.n_keys)
+    return sah_fail(SAH_EINVAL, "sah_select_topk: candidate range [%d, %d) outside [0, %d)", a->col_offset,
+                    a->col_offset + a->n_cand, a->rows.n_keys);
+  if (a->k <= 0) return sah_fail(SAH_EINVAL, "sah_select_topk: k must be > 0");
+  if (a->key_pitch < a->n_cand) return sah_fail(SAH_EINVAL, "sah_select_topk: key_pitch < n_cand");
+  hipStream_t st = (hipStream_t)a->stream;
+  if (a->key_bits == 16)
+    hipLaunchKernelGGL(k_select_topk<16>, dim3(a->rows.n_rows), dim3(SEL_NT), 0, st, a->rows, a->keys, a->key_pitch,
+                       a->n_cand, a->col_offset, a->k, a->excluded_key);
+  else
+    hipLaunchKernelGGL(k_select_topk<32>, dim3(a->rows.n_rows), dim3(SEL_NT), 0, st, a->rows, a->keys, a->key_pitch,
+                       a->n_cand, a->col_offset, a->k, a->excluded_key);
+  return sah_launch_status("sah_select_topk");
+}
+
+extern "C" int sah_hamming_topk(const sah_hamming_topk_args* a) {
+  if (!a) return sah_fail(SAH_ENULL, "sah_hamming_topk: args is NULL");
+  int rc = sah_check_rows(a->rows, "sah_hamming_topk");
+  if (rc) return rc;
+  if (!a->kcodes || !a->qcodes) return sah_fail(SAH_ENULL, "sah_hamming_topk: codes are NULL");
+  if (a->lq <= 0 || a->rows.n_rows % a->lq) return sah_fail(SAH_EINVAL, "sah_hamming_topk: lq must divide n_rows");
+  if (a->k <= 0) return sah_fail(SAH_EINVAL, "sah_hamming_topk: k must be > 0");
+  if (a->code_pitch < a->rows.n_keys) return sah_fail(SAH_EINVAL, "sah_hamming_topk: code_pitch < n_keys");
+  hipLaunchKernelGGL(k_hamming_topk, dim3(a->rows.n_rows), dim3(SEL_NT), 0, (hipStream_t)a->stream, a->rows,
+                     (const uint2*)a->kcodes, a->code_pitch, (const uint2*)a->qcodes, a->lq, a->k);
+  return sah_launch_status("sah_hamming_topk");
+}

@@ -1,0 +1,44 @@
+"""The C-ABI library loads and exports exactly what include/sah.h declares (no compute)."""
+import ctypes
+import os
+import re
+
+from sparse_attention_hub_amd import _native as N
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "sah.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(?:int|int64_t|const char\*)\s+(sah_\w+)\s*\(", text)))
+
+
+def test_library_is_built_and_loads():
+    assert N.library_path().exists(), "build it with python sparse-attention-hub_amd/build.py"
+    lib = N.lib()
+    assert lib.sah_version() == 1
+
+
+def test_every_declared_symbol_is_exported_and_bound():
+    declared = _declared_functions()
+    assert len(declared) >= 15
+    handle = ctypes.CDLL(str(N.library_path()))
+    for name in declared:
+        assert hasattr(handle, name), f"{name} declared in include/sah.h but not exported"
+    assert sorted(N.EXPECTED_SYMBOLS) == declared
+
+
+def test_argument_errors_are_reported_without_a_gpu():
+    # NULL args never launch anything; the error string names the entry point
+    lib = N.lib()
+    assert lib.sah_sparse_attention(None) == -2
+    assert b"sah_sparse_attention" in lib.sah_last_error()
+    assert lib.sah_select_topk(None) == -2
+    assert N.work_floats(256, 2688, 128) == 256 * 11 * 130
+
+
+def test_struct_layouts_match_header_sizes():
+    # sah_rows: 4 pointers + 4 int32
+    assert ctypes.sizeof(N.Rows) == 4 * 8 + 4 * 4
+    assert ctypes.sizeof(N.SinkLocalArgs) == ctypes.sizeof(N.Rows) + 5 * 4 + 4 + 8

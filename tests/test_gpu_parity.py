@@ -1,0 +1,307 @@
+"""GPU parity tests: the HIP path (through the C ABI) against the CPU oracle on the same
+seeded inputs. Bars: index sets bit-exact (ties to the lowest column); attention outputs
+within 1e-5 relative error for fp32 and 2e-2 for bf16."""
+import math
+
+import pytest
+import torch
+
+from _util import make_qkv, rel_err
+from oracle import reference_path as O
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2, torch.float16: 2e-2}
+
+
+def _sa():
+    import sparse_attention_hub_amd.sparse_attention as sa
+
+    return sa
+
+
+def _run_chain(cuda, cfgs, specs, B, Hq, Hkv, Lq, Lk, D, dtype, amask=None, sinks=None, outliers=False, seed=0,
+               meta=None, check_weights=True):
+    sa = _sa()
+    q, k, v = make_qkv(B, Hq, Hkv, Lq, Lk, D, dtype, seed=seed, outliers=outliers)
+    ra = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=cfgs))
+    scaling = D ** -0.5
+    meta = {} if meta is None else meta
+    kw = dict(sparse_meta_data=meta, layer_idx=0)
+    if sinks is not None:
+        kw["s_aux"] = sinks.to(cuda)
+    out, w = ra.custom_attention(None, q.to(cuda), k.to(cuda), v.to(cuda), None if amask is None else amask.to(cuda),
+                                 scaling, 0.0, **kw)
+    torch.cuda.synchronize()
+    oo, ow, om = O.research_attention(specs, q, k, v, amask, scaling, sinks)
+    assert out.shape == oo.shape and out.dtype == dtype
+    err = rel_err(out, oo)
+    assert err < TOL[dtype], f"output rel err {err}"
+    if check_weights:
+        assert w.shape == ow.shape
+        if om.kind == "dense":
+            assert torch.equal(w.cpu() != 0, ow != 0)
+        assert (w.float().cpu() - ow.float()).abs().max().item() < (1e-6 if dtype == torch.float32 else 1e-2)
+    return out, w, om, meta
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("D", [16, 64, 128])
+def test_sink_local_chain(cuda, dtype, D):
+    sa = _sa()
+    _run_chain(cuda, [sa.SinkMaskerConfig(sink_size=4), sa.LocalMaskerConfig(window_size=8)],
+               [("sink", 4), ("local", 8)], 2, 4, 2, 1, 333, D, dtype)
+
+
+def test_sink_local_index_form_is_bit_exact(cuda):
+    sa = _sa()
+    B, Hq, Lq, Lk = 2, 4, 3, 70
+    q, k, v = make_qkv(B, Hq, 2, Lq, Lk, 16, torch.float32)
+    m = sa.Mask.create_empty_mask((B, Hq, Lq, Lk), torch.float32, cuda)
+    for cfg in (sa.SinkMaskerConfig(sink_size=5), sa.LocalMaskerConfig(window_size=9)):
+        m = sa.ResearchMasker.create_masker_from_config(cfg).add_mask(
+            keys=k.to(cuda), queries=q.to(cuda), values=v.to(cuda), attention_mask=None, scaling=1.0, dropout=0.0,
+            sparse_meta_data={}, previous_mask=m)
+    om = O.local(O.sink(O.OMask.empty((B, Hq, Lq, Lk), torch.float32), 5), 9)
+    idx, ptr, data = m.get_index_mask()
+    oidx, optr, odata = om.index_form()
+    assert idx.dtype == torch.int64 and ptr.dtype == torch.int64
+    assert torch.equal(idx.cpu(), oidx) and torch.equal(ptr.cpu(), optr) and torch.equal(data.cpu(), odata)
+    assert torch.equal(m.get_dense_mask().cpu(), om.to_dense())
+
+
+def test_local_merges_into_dense_previous_and_clears_future(cuda):
+    # reference pattern: previous [0,1] + local window 2 on Lq=3, Lk=8 (test_basic_fixed.py:299-312)
+    sa = _sa()
+    prev = torch.zeros(1, 1, 3, 8)
+    prev[..., :2] = 1.0
+    prev[..., 0, 7] = 1.0   # a future column of query 0: must be cleared
+    pm = sa.Mask.create_mask_from_dense_mask((1, 1, 3, 8), prev.to(cuda), torch.float32)
+    q, k, v = make_qkv(1, 1, 1, 3, 8, 16, torch.float32)
+    m = sa.LocalMasker(sa.LocalMaskerConfig(window_size=2)).add_mask(
+        keys=k.to(cuda), queries=q.to(cuda), values=v.to(cuda), attention_mask=None, scaling=1.0, dropout=0.0,
+        sparse_meta_data={}, previous_mask=pm)
+    want = torch.tensor([[1, 1, 0, 0, 1, 1, 0, 0], [1, 1, 0, 0, 0, 1, 1, 0], [1, 1, 0, 0, 0, 0, 1, 1]], dtype=torch.float32)
+    assert torch.equal(m.get_dense_mask()[0, 0].cpu(), want)
+
+
+def test_full_mask_shortcuts(cuda):
+    sa = _sa()
+    q, k, v = make_qkv(1, 2, 1, 1, 8, 16, torch.float32)
+    args = dict(keys=k.to(cuda), queries=q.to(cuda), values=v.to(cuda), attention_mask=None, scaling=1.0, dropout=0.0,
+                sparse_meta_data={})
+    e = sa.Mask.create_empty_mask((1, 2, 1, 8), torch.float32, cuda)
+    assert sa.SinkMasker(sa.SinkMaskerConfig(sink_size=8)).add_mask(previous_mask=e, **args).is_full_mask()
+    assert sa.LocalMasker(sa.LocalMaskerConfig(window_size=7)).add_mask(previous_mask=e, **args).is_full_mask()
+    assert sa.OracleTopK(sa.OracleTopKConfig(heavy_size=8)).add_mask(previous_mask=e, **args).is_full_mask()
+    f = sa.Mask.create_full_mask((1, 2, 1, 8), torch.float32, cuda)
+    assert sa.SinkMasker(sa.SinkMaskerConfig(sink_size=2)).add_mask(previous_mask=f, **args) is f
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_dense_attention_with_sinks_and_additive_mask(cuda, dtype):
+    B, Hq, Hkv, Lq, Lk, D = 2, 4, 2, 2, 700, 64
+    am = torch.zeros(B, 1, Lq, Lk)
+    am[0, :, :, -50:] = torch.finfo(torch.float32).min
+    am = am.to(dtype)
+    _run_chain(cuda, [], [], B, Hq, Hkv, Lq, Lk, D, dtype, amask=am, sinks=torch.tensor([0.1, -0.3, 0.5, 1.0]))
+
+
+@pytest.mark.parametrize("dtype,D,Lk,heavy", [(torch.float32, 32, 1000, 50), (torch.bfloat16, 128, 4096, 0.05),
+                                              (torch.bfloat16, 64, 777, 33), (torch.float32, 128, 5000, 0.02)])
+def test_oracle_topk_chain(cuda, dtype, D, Lk, heavy):
+    sa = _sa()
+    _run_chain(cuda, [sa.SinkMaskerConfig(sink_size=16), sa.LocalMaskerConfig(window_size=32), sa.OracleTopKConfig(heavy_size=heavy)],
+               [("sink", 16), ("local", 32), ("oracle_topk", heavy)], 2, 8, 2, 1, Lk, D, dtype, outliers=True)
+
+
+def test_oracle_topk_many_ties_lowest_index(cuda):
+    # integer-valued keys => heavy ties at the threshold; the selected set must be the lowest columns
+    sa = _sa()
+    g = torch.Generator().manual_seed(0)
+    B, Hq, Hkv, Lk, D = 1, 2, 1, 3000, 16
+    q = torch.zeros(B, Hq, 1, D)
+    q[..., 0] = 1.0
+    k = torch.zeros(B, Hkv, Lk, D)
+    k[..., 0] = torch.randint(-3, 4, (B, Hkv, Lk), generator=g).float()
+    v = torch.randn(B, Hkv, Lk, D, generator=g)
+    for dtype in (torch.float32, torch.bfloat16):
+        ra = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(
+            masker_configs=[sa.SinkMaskerConfig(sink_size=3), sa.OracleTopKConfig(heavy_size=500)]))
+        out, w = ra.custom_attention(None, q.to(dtype).to(cuda), k.to(dtype).to(cuda), v.to(dtype).to(cuda), None, 0.25, 0.0,
+                                     sparse_meta_data={})
+        _, ow, om = O.research_attention([("sink", 3), ("oracle_topk", 500)], q.to(dtype), k.to(dtype), v.to(dtype), None, 0.25)
+        assert torch.equal(w.cpu() != 0, om.to_dense() != 0)
+
+
+def _hat(sa, Hq, D, dtype, hidden=32, bits=32, seed=1):
+    from sparse_attention_hub_amd.sparse_attention.utils.hashattention_utils import random_hat_weights
+
+    return random_hat_weights(1, Hq, D, bits, 3, hidden, dtype=dtype, seed=seed)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("use_amask", [False, True])
+def test_hash_topk_chain(cuda, dtype, use_amask):
+    """Selection + attention are bit-exact / in tolerance *given the signatures*: the oracle scores
+    the kernel's own codes (unpacked to the reference's +-1/0 floats), so MLP rounding noise
+    (tested separately below) cannot move a key across the top-k threshold."""
+    sa = _sa()
+    from sparse_attention_hub_amd.sparse_attention.research_attention.maskers.fixed.implementations.hashattention_top_k import (
+        HashAttentionTopKMasker,
+    )
+
+    B, Hq, Hkv, Lk, D = 2, 8, 2, 1500, 128
+    wts = _hat(sa, Hq, D, dtype, hidden=128)
+    cfg = sa.HashAttentionTopKMaskerConfig(heavy_size=128, hat_bits=32, hat_mlp_layers=3, hat_mlp_hidden_size=128,
+                                           hat_mlp_activation="silu", hat_weights=wts)
+    am = None
+    if use_amask:
+        am = torch.zeros(B, 1, 1, Lk)
+        am[1, :, :, 100:400] = torch.finfo(torch.float32).min
+        am = am.to(dtype)
+    q, k, v = make_qkv(B, Hq, Hkv, 1, Lk, D, dtype)
+    ra = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(
+        masker_configs=[sa.SinkMaskerConfig(sink_size=16), sa.LocalMaskerConfig(window_size=64), cfg]))
+    meta = {}
+    out, w = ra.custom_attention(None, q.to(cuda), k.to(cuda), v.to(cuda), None if am is None else am.to(cuda),
+                                 D ** -0.5, 0.0, sparse_meta_data=meta, layer_idx=0)
+    ksig = meta["key"][0].unpack(torch.float32).cpu()
+    masker = HashAttentionTopKMasker(cfg)
+    qcodes = torch.empty((B * Hq, 2), dtype=torch.int32, device=cuda)
+    masker._hash(q.to(cuda), Hq, Hq, 0, 1, 0, "query", qcodes, 1, 0)
+    qc = qcodes.cpu().to(torch.int64) & 0xFFFFFFFF
+    shifts = torch.arange(32)
+    qsig = ((((qc[:, 0:1] >> shifts) & 1) * 2 - 1) * ((qc[:, 1:2] >> shifts) & 1)).float().view(B, Hq, 1, 32)
+    state = {"key_sig": ksig, "query_sig": qsig}
+    oo, ow, om = O.research_attention([("sink", 16), ("local", 64), ("hash_topk", 128, wts[0], "silu")], q, k, v, am,
+                                      D ** -0.5, state=state)
+    assert torch.equal(w.cpu() != 0, om.to_dense() != 0)            # index sets: bit-exact
+    assert torch.all((om.to_dense() != 0).sum(-1) == 16 + 64 + 128)
+    assert rel_err(out, oo) < TOL[dtype]
+    # and the signatures themselves agree with the float MLP almost everywhere
+    sig = O.hash_signatures(O.repeat_kv(k, Hq // Hkv), wts[0]["key_matrix"], wts[0]["key_bias"], "silu")
+    assert (ksig == sig.float()).float().mean().item() >= 0.9995
+
+
+def test_hash_signatures_bits_and_cache_growth(cuda):
+    sa = _sa()
+    from sparse_attention_hub_amd.sparse_attention.research_attention.maskers.fixed.implementations.hashattention_top_k import (
+        HashAttentionTopKMasker,
+    )
+
+    for dtype in (torch.float32, torch.bfloat16):
+        B, Hq, Hkv, Lk, D = 1, 4, 2, 300, 64
+        wts = _hat(sa, Hq, D, dtype, hidden=48, bits=24)
+        cfg = sa.HashAttentionTopKMaskerConfig(heavy_size=8, hat_bits=24, hat_mlp_layers=3, hat_mlp_hidden_size=48,
+                                               hat_mlp_activation="gelu", hat_weights=wts)
+        masker = HashAttentionTopKMasker(cfg)
+        _, k, _ = make_qkv(B, Hq, Hkv, 1, Lk, D, dtype)
+        meta = {}
+        kc = k.to(cuda)
+        masker._update_key_signatures(kc[:, :, :200].contiguous(), Hq, meta, 0)
+        cache = masker._update_key_signatures(kc, Hq, meta, 0)          # only keys 200.. are hashed now
+        assert cache.shape == (B, Hq, Lk, 24)
+        sig = O.hash_signatures(O.repeat_kv(k, 2), wts[0]["key_matrix"], wts[0]["key_bias"], "gelu")
+        got = cache.unpack(torch.float32).cpu()
+        agree = (got == sig.float()).float().mean().item()
+        # accumulation order differs from torch's: a value within rounding noise of 0 (or, in bf16, of a
+        # rounding boundary of an intermediate activation) may land on the other side
+        assert agree >= 0.9995, agree
+        with pytest.raises(ValueError, match="less than cached"):
+            masker._update_key_signatures(kc[:, :, :100].contiguous(), Hq, meta, 0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_pq_chain_cold_and_warm(cuda, dtype):
+    sa = _sa()
+    from sparse_attention_hub_amd.sparse_attention.research_attention.maskers.fixed.implementations.utils.pq_utils import (
+        gather_sub_vectors, seeded_initial_centres,
+    )
+
+    B, Hq, Hkv, Lk, D = 2, 8, 2, 1200, 64
+    n_sub, bits, off, iters, heavy = 8, 4, 16, 5, 64
+    n_cent = 2 ** bits
+    q, k, v = make_qkv(B, Hq, Hkv, 1, Lk, D, dtype, outliers=True)
+    cfg = sa.PQCacheConfig(heavy_size=heavy, pq_group_factor=n_sub, pq_bits=bits, kmeans_iter=iters, init_offset=off,
+                           metric="euclidean")
+    ra = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(
+        masker_configs=[sa.SinkMaskerConfig(sink_size=off), sa.LocalMaskerConfig(window_size=32), cfg]))
+    meta = {}
+    out, w = ra.custom_attention(None, q.to(cuda), k.to(cuda), v.to(cuda), None, D ** -0.5, 0.0, sparse_meta_data=meta, layer_idx=0)
+    # Lloyd parity from the same start (and the same reseed table)
+    X = O.pq_split(k, off, n_sub)
+    start = seeded_initial_centres(B * Hkv * n_sub, Lk - off, n_cent, 0, torch.device("cpu"))
+    c0 = gather_sub_vectors(k, off, n_sub, start)
+    reseed = torch.randint(0, Lk - off, (iters, B * Hkv * n_sub, n_cent), generator=torch.Generator().manual_seed(1), dtype=torch.int32)
+    codes_o, cent_o = O.kmeans_lloyd(X, c0, iters, reseed_idx=reseed)
+    book = meta["pq_codebook"][0]
+    assert book.shape == (B, Lk - off, Hkv, n_sub)
+    codes = book.to_reference().cpu()
+    codes_o = codes_o.reshape(B, Hkv, n_sub, Lk - off).permute(0, 3, 1, 2)
+    assert (codes == codes_o).float().mean().item() >= 0.999
+    cent = meta["pq_centroids"][0]
+    assert cent.dtype == dtype and cent.shape == (B, Hkv, n_sub, n_cent, D // n_sub)
+    # centres: fp32 sums are accumulated with atomics (order differs); bf16 storage may land one ulp apart
+    rtol = 1e-3 if dtype == torch.float32 else 2 ** -7
+    assert torch.allclose(cent.float().cpu().reshape(-1), cent_o.float().reshape(-1), rtol=rtol, atol=1e-3)
+    # scoring + top-k + attention given the kernel's own codebook
+    oo, ow, om = O.research_attention([("sink", off), ("local", 32), ("pq_topk", heavy, off, cent.cpu(), codes)], q, k, v, None, D ** -0.5)
+    assert rel_err(out, oo) < TOL[dtype]
+    assert torch.equal(w.cpu() != 0, om.to_dense() != 0)
+    # warm step: three appended keys are quantised against the frozen centroids
+    q2, kn, vn = make_qkv(B, Hq, Hkv, 1, 3, D, dtype, seed=5)
+    k2, v2 = torch.cat([k, kn], 2), torch.cat([v, vn], 2)
+    out2, w2 = ra.custom_attention(None, q2.to(cuda), k2.to(cuda), v2.to(cuda), None, D ** -0.5, 0.0, sparse_meta_data=meta, layer_idx=0)
+    codes2 = meta["pq_codebook"][0].to_reference().cpu()
+    assert torch.equal(codes2[:, : Lk - off], codes)
+    assert torch.equal(codes2[:, Lk - off:], O.pq_quantize_new(kn, cent.cpu()))
+    oo2, _, om2 = O.research_attention([("sink", off), ("local", 32), ("pq_topk", heavy, off, cent.cpu(), codes2)], q2, k2, v2, None, D ** -0.5)
+    assert rel_err(out2, oo2) < TOL[dtype]
+    assert torch.equal(w2.cpu() != 0, om2.to_dense() != 0)
+
+
+def test_rows_from_dense_round_trip_with_weights(cuda):
+    sa = _sa()
+    g = torch.Generator().manual_seed(3)
+    dense = (torch.rand(3, 5, 2, 300, generator=g) > 0.8).float() * (torch.rand(3, 5, 2, 300, generator=g) * 0.5 + 0.5)
+    m = sa.Mask.create_mask_from_dense_mask(dense.shape, dense.to(cuda), torch.float32)
+    rows = m.to_rows(0)
+    back = sa.Mask.create_mask_from_rows(dense.shape, rows, torch.float32)
+    assert torch.equal(back.get_dense_mask().cpu(), dense)
+    idx, ptr, data = back.get_index_mask()
+    oidx, optr, odata = O.OMask("dense", tuple(dense.shape), torch.float32, dense).index_form()
+    assert torch.equal(idx.cpu(), oidx) and torch.equal(ptr.cpu(), optr) and torch.equal(data.cpu(), odata)
+
+
+def test_weighted_mask_attention(cuda):
+    # inverse-weight semantics exp/(w + 1e-6) incl. bf16 evaluation of the reciprocal
+    sa = _sa()
+    from sparse_attention_hub_amd.sparse_attention.utils.mask_attention_utils import get_masked_attention_output
+
+    for dtype in (torch.float32, torch.bfloat16):
+        B, Hq, Hkv, Lk, D = 1, 4, 2, 500, 64
+        q, k, v = make_qkv(B, Hq, Hkv, 1, Lk, D, dtype, seed=2)
+        g = torch.Generator().manual_seed(4)
+        dm = ((torch.rand(B, Hq, 1, Lk, generator=g) > 0.7).float() * torch.rand(B, Hq, 1, Lk, generator=g)).to(dtype)
+        dm[..., :4] = 1.0
+        mask = sa.Mask.create_mask_from_dense_mask(dm.shape, dm.to(cuda), dtype)
+        out, w = get_masked_attention_output(None, q.to(cuda), k.to(cuda), v.to(cuda), None, None, D ** -0.5, 0.0, mask,
+                                             return_attention_weights=True)
+        oo, ow = O.masked_attention(q, k, v, None, None, D ** -0.5, O.OMask("dense", tuple(dm.shape), dtype, dm))
+        assert rel_err(out, oo) < TOL[dtype]
+        assert torch.equal(w.cpu() != 0, ow != 0)
+
+
+def test_missing_sparse_meta_data_and_layer_idx_raise(cuda):
+    sa = _sa()
+    q, k, v = make_qkv(1, 2, 1, 1, 64, 16, torch.float32)
+    ra = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=[]))
+    with pytest.raises(ValueError, match="sparse_meta_data must be provided"):
+        ra.custom_attention(None, q.to(cuda), k.to(cuda), v.to(cuda), None, 1.0, 0.0)
+    wts = _hat(sa, 2, 16, torch.float32)
+    cfg = sa.HashAttentionTopKMaskerConfig(heavy_size=4, hat_bits=32, hat_mlp_layers=3, hat_mlp_hidden_size=32,
+                                           hat_mlp_activation="silu", hat_weights=wts)
+    ra = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=[cfg]))
+    with pytest.raises(ValueError, match="layer_idx must be provided"):
+        ra.custom_attention(None, q.to(cuda), k.to(cuda), v.to(cuda), None, 1.0, 0.0, sparse_meta_data={})
