@@ -1,0 +1,239 @@
+#!/usr/bin/env python3
+"""Decode layer-step benchmark of the MI355X ResearchAttention path.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 1|2|3|4]
+
+A step is one `ResearchAttention.custom_attention` call with one query token on a warm
+cache (hash signatures / PQ codes of all earlier keys already built, one new key appended
+per step), on synthetic inputs that are resident in HBM before the timed region. Default
+workload: BASELINE config 3, the one the headline target is quoted on (Sink 128 + Local 512
++ HashAttention top-2048, batch 8, 32 query / 8 KV heads, head_dim 128, 32768 keys, bf16).
+
+Prints ONE JSON line: whole-step microseconds (`value`), the roofline of the dominant kernel
+from HIP-event timings taken inside this run, and the CPU oracle timed on the host cores.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "sparse-attention-hub_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+HBM_PEAK_GBS = 8000.0
+OUTLIER_CHANNELS = (7, 33, 71, 101)
+
+WORKLOADS = {
+    1: dict(name="cfg1 Sink128+Local256 fp32 B1 Lk4096", B=1, Lk=4096, dtype="f32", sink=128, local=256, kind="none", k=0),
+    2: dict(name="cfg2 Sink128+Local512+OracleTopK5% bf16 B4 Lk32768", B=4, Lk=32768, dtype="bf16", sink=128, local=512,
+            kind="oracle", k=1638, outliers=True),
+    3: dict(name="cfg3 Sink128+Local512+HashAttention top-2048 bf16 B8 Lk32768", B=8, Lk=32768, dtype="bf16", sink=128,
+            local=512, kind="hash", k=2048),
+    4: dict(name="cfg4 Sink128+Local256+PQCache top-1024 bf16 B4 Lk32768", B=4, Lk=32768, dtype="bf16", sink=128, local=256,
+            kind="pq", k=1024, outliers=True),
+}
+HQ, HKV, D = 32, 8, 128
+
+
+def algorithmic_bytes(w) -> dict:
+    """Unique bytes that must cross HBM once per warm layer-step (formulas in DESIGN.md):
+    sink/local rows shared by the 4 query heads of a KV group, top-k rows not shared,
+    int32 indices written once and read once, Q and out."""
+    es = 4 if w["dtype"] == "f32" else 2
+    row = D * es
+    B, Lk = w["B"], w["Lk"]
+    R = B * HQ
+    fixed = w["sink"] + w["local"]
+    gather_topk = R * w["k"] * row * 2
+    gather_fixed = B * HKV * fixed * row * 2
+    idx = R * (fixed + w["k"]) * 4 * 2
+    qo = 2 * R * D * es
+    scan = {"none": 0, "oracle": B * HKV * Lk * row, "hash": R * Lk * 8, "pq": B * HKV * (Lk - w["sink"]) * 16}[w["kind"]]
+    attn = gather_topk + gather_fixed + R * (fixed + w["k"]) * 4 + qo
+    return dict(step=gather_topk + gather_fixed + idx + qo + scan, attention_kernel=attn, scan=scan)
+
+
+def build_workload(w, device, total_keys):
+    import torch
+
+    from sparse_attention_hub_amd.sparse_attention import (
+        HashAttentionTopKMaskerConfig, LocalMaskerConfig, OracleTopKConfig, PQCacheConfig, ResearchAttention,
+        ResearchAttentionConfig, SinkMaskerConfig,
+    )
+    from sparse_attention_hub_amd.sparse_attention.utils.hashattention_utils import random_hat_weights
+
+    dtype = torch.float32 if w["dtype"] == "f32" else torch.bfloat16
+    g = torch.Generator().manual_seed(0)
+    B = w["B"]
+    k = torch.randn(B, HKV, total_keys, D, generator=g)
+    v = torch.randn(B, HKV, total_keys, D, generator=g)
+    if w.get("outliers"):
+        for c in OUTLIER_CHANNELS:
+            k[..., c] *= 8.0
+    qs = torch.randn(64, B, HQ, 1, D, generator=g)
+    cfgs = [SinkMaskerConfig(sink_size=w["sink"]), LocalMaskerConfig(window_size=w["local"])]
+    extra = {}
+    if w["kind"] == "oracle":
+        cfgs.append(OracleTopKConfig(heavy_size=w["k"]))
+    elif w["kind"] == "hash":
+        wts = random_hat_weights(1, HQ, D, 32, 3, 128, dtype=dtype, seed=1)
+        extra["hat_weights"] = wts
+        cfgs.append(HashAttentionTopKMaskerConfig(heavy_size=w["k"], hat_bits=32, hat_mlp_layers=3, hat_mlp_hidden_size=128,
+                                                  hat_mlp_activation="silu", hat_weights=wts))
+    elif w["kind"] == "pq":
+        cfgs.append(PQCacheConfig(heavy_size=w["k"], pq_group_factor=16, pq_bits=8, kmeans_iter=10, init_offset=w["sink"],
+                                  metric="euclidean"))
+    ra = ResearchAttention.create_from_config(ResearchAttentionConfig(masker_configs=cfgs))
+    ra.return_attention_weights = False  # HF attention modules drop the dense probabilities in decode
+    return ra, qs.to(dtype).to(device), k.to(dtype).to(device), v.to(dtype).to(device), extra
+
+
+def cpu_baseline(w, extra, ra_meta, k_dev, v_dev, q_dev, n_keys, budget_s=25.0):
+    """The reference algorithm (dense masks, repeat_kv, full-key fp32 softmax) as restated by the
+    oracle, timed on the host cores for ONE batch row and scaled by the batch size (rows are
+    independent); the warm caches are taken from the GPU run so only the layer-step is timed."""
+    import torch
+
+    from oracle import reference_path as O
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    q = q_dev[:1].cpu()
+    k = k_dev[:1, :, :n_keys].cpu()
+    v = v_dev[:1, :, :n_keys].cpu()
+    specs = [("sink", w["sink"]), ("local", w["local"])]
+    state = {}
+    if w["kind"] == "oracle":
+        specs.append(("oracle_topk", w["k"]))
+    elif w["kind"] == "hash":
+        specs.append(("hash_topk", w["k"], extra["hat_weights"][0], "silu"))
+        cache = ra_meta["key"][0]
+        sub = type(cache).__new__(type(cache))            # one batch row, the n_keys - 1 earlier keys
+        sub.bits, sub.n, sub.codes = cache.bits, n_keys - 1, cache.codes[:1]
+        state["key_sig"] = sub.unpack(q.dtype).cpu()
+    elif w["kind"] == "pq":
+        cent = ra_meta["pq_centroids"][0][:1].cpu()
+        book = ra_meta["pq_codebook"][0].to_reference()[:1, : n_keys - w["sink"]].cpu()
+        specs.append(("pq_topk", w["k"], w["sink"], cent, book))
+    times = []
+    t_all = time.perf_counter()
+    for it in range(12):
+        st = dict(state)
+        t0 = time.perf_counter()
+        O.research_attention(specs, q, k, v, None, D ** -0.5, state=st)
+        times.append(time.perf_counter() - t0)
+        if time.perf_counter() - t_all > budget_s and it >= 1:
+            break
+    per_row = sorted(times[1:] or times)[len(times[1:] or times) // 2]
+    return dict(value=per_row * w["B"] * 1e6, unit="us/layer-step", cores=cores, kind="port",
+                sample=f"oracle (torch-CPU restatement of the reference path) on 1 of {w['B']} batch rows, "
+                       f"median of {max(1, len(times) - 1)} warm steps x {w['B']}; torch threads={cores}")
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", type=int, default=3, choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this path runs on ONE GPU (no collectives on the decode path); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from sparse_attention_hub_amd import _native as N
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the MI355X kernels have no CPU fallback", file=sys.stderr)
+        sys.exit(3)
+    N.lib()
+    dev = torch.device("cuda:0")
+    w = WORKLOADS[args.config]
+    steps, warm = args.steps, args.warmup
+    probe = max(20, min(steps, 100))                      # instrumented steps for the per-kernel roofline
+    total_keys = w["Lk"] + probe
+    first = w["Lk"] - (warm + steps)                      # the last timed step runs at exactly Lk keys
+    ra, qs, k, v, extra = build_workload(w, dev, total_keys)
+    meta = {}
+    scaling = D ** -0.5
+
+    def step(i, n_keys):
+        return ra.custom_attention(None, qs[i % qs.shape[0]], k[:, :, :n_keys], v[:, :, :n_keys], None, scaling, 0.0,
+                                   sparse_meta_data=meta, layer_idx=0)
+
+    # cold call: builds all signatures / runs k-means; reported apart
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    step(0, first)
+    torch.cuda.synchronize()
+    cold_ms = (time.perf_counter() - t0) * 1e3
+
+    for i in range(warm):
+        step(i, first + 1 + i)
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()
+    for i in range(steps):
+        step(i, first + warm + 1 + i)
+    ev1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    gpu_ms = ev0.elapsed_time(ev1)
+    ms_per_step = wall_ms / steps
+
+    # per-kernel durations, HIP events on the launch stream, same process, same buffers
+    N.timing_enable(True)
+    for i in range(probe):
+        step(i, w["Lk"] + 1 + i)
+    torch.cuda.synchronize()
+    kt = N.timing_collect()
+    N.timing_enable(False)
+    kernels = {name: dict(launches=c, avg_us=1e3 * ms / c) for name, (c, ms) in kt.items()}
+    ab = algorithmic_bytes(w)
+    dom = "k_sparse_attn"
+    dom_us = kernels[dom]["avg_us"]
+    achieved = ab["attention_kernel"] / (dom_us * 1e-6) / 1e9
+    roofline = dict(bound="hbm", kernel=dom, achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s",
+                    frac=round(achieved / HBM_PEAK_GBS, 4), traffic=None,
+                    algorithmic_bytes_per_launch=ab["attention_kernel"], avg_launch_us=round(dom_us, 2))
+    step_gbs = ab["step"] / (ms_per_step * 1e-3) / 1e9
+
+    out = {
+        "metric": "sparse decode us/layer-step at 32K ctx; achieved HBM GB/s vs peak",
+        "value": round(ms_per_step * 1e3, 2),
+        "unit": "us/layer-step",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": warm,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": w["dtype"],
+        "data": "synthetic",
+        "config": {"workload": w["name"], "q_heads": HQ, "kv_heads": HKV, "head_dim": D, "batch": w["B"], "keys": w["Lk"],
+                   "keys_per_row": w["sink"] + w["local"] + w["k"], "attention_weights_output": False},
+        "gpu_ms_per_step": round(gpu_ms / steps, 5),
+        "step_algorithmic_bytes": ab["step"],
+        "step_achieved_GBps": round(step_gbs, 1),
+        "step_frac_of_hbm_peak": round(step_gbs / HBM_PEAK_GBS, 4),
+        "cold_call_ms": round(cold_ms, 2),
+        "kernels_avg_us": {n: round(d["avg_us"], 2) for n, d in sorted(kernels.items())},
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(w, extra, meta, k, v, qs[0], w["Lk"])
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

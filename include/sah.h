@@ -67,6 +67,15 @@ typedef struct sah_rows {
 int sah_version(void);
 const char* sah_last_error(void);
 
+/* Opt-in per-kernel timing for benchmarks; no counterpart in the reference (its
+ * profile/profile_research_attention.py:273-319 times whole calls from Python).
+ * While enabled every entry point brackets its kernel with a HIP event pair on
+ * the caller's stream. sah_timing_collect waits for the recorded events, sums
+ * the elapsed milliseconds per kernel name into names/counts/total_ms (host
+ * arrays of `max` entries), clears the log and returns the number of names. */
+int sah_timing_enable(int on);
+int sah_timing_collect(const char** names, int* counts, float* total_ms, int max);
+
 /* ---------------------------------------------------------------------------
  * Fused Sink + Local builder. Replaces SinkMasker.get_updated_mask_dense
  * (maskers/fixed/implementations/basic_fixed.py:354-363) and

@@ -47,14 +47,55 @@ __device__ __forceinline__ float att_group_sum(float v) {
   return v;
 }
 
+// raw 8-element row slice as loaded (16 B for 2-byte types, 32 B for fp32)
+template <int DT>
+struct att_raw {
+  uint4 lo;
+  uint4 hi;  // only used for fp32
+};
+
+template <int DT>
+__device__ __forceinline__ void att_load_raw(const char* p, att_raw<DT>& r) {
+  r.lo = *(const uint4*)p;
+  if (DT == SAH_F32) r.hi = *(const uint4*)(p + 16);
+}
+
+template <int DT>
+__device__ __forceinline__ void att_unpack(const att_raw<DT>& r, float (&o)[8]) {
+  const uint32_t w[4] = {r.lo.x, r.lo.y, r.lo.z, r.lo.w};
+  if (DT == SAH_F32) {
+    const uint32_t v[4] = {r.hi.x, r.hi.y, r.hi.z, r.hi.w};
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      o[t] = sah_bits_to_float(w[t]);
+      o[4 + t] = sah_bits_to_float(v[t]);
+    }
+  } else {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      if (DT == SAH_BF16) {
+        o[2 * t] = sah_bits_to_float(w[t] << 16);
+        o[2 * t + 1] = sah_bits_to_float(w[t] & 0xffff0000u);
+      } else {
+        o[2 * t] = sah_f16_to_float((uint16_t)(w[t] & 0xffffu));
+        o[2 * t + 1] = sah_f16_to_float((uint16_t)(w[t] >> 16));
+      }
+    }
+  }
+}
+
+// Each wave keeps its own online-softmax state (m uniform across the wave, l and acc
+// per lane group) and walks its 64-key slices in batches of UB iterations; the K and V
+// rows of a batch are requested together so 2*UB row loads are in flight per lane.
 template <int DT, int D>
 __global__ __launch_bounds__(ATT_NT) void k_sparse_attn(att_params P) {
   constexpr int LPK = D / 8;            // lanes per key
   constexpr int KPI = SAH_WAVE / LPK;   // keys per wave iteration
-  constexpr int IT = SAH_WAVE / KPI;    // iterations per 64-key wave chunk (== LPK)
-  constexpr int UB = (DT == SAH_F32) ? (IT < 4 ? IT : 4) : (IT < 8 ? IT : 8);  // loads in flight per batch
+  constexpr int IT = SAH_WAVE / KPI;    // iterations per 64-key wave slice (== LPK)
+  constexpr int UB = IT < 4 ? IT : 4;   // iterations per batch
+  constexpr int ES = (DT == SAH_F32) ? 4 : 2;
 
-  __shared__ float s_max[ATT_NW];
+  __shared__ float s_m[ATT_NW];
   __shared__ float s_l[ATT_NW];
   __shared__ float s_acc[ATT_NW][D];
 
@@ -88,11 +129,9 @@ __global__ __launch_bounds__(ATT_NT) void k_sparse_attn(att_params P) {
 
   const int* cols = P.dense ? nullptr : P.rows.cols + (int64_t)r * P.rows.cap;
   const float* wts = (!P.dense && P.rows.w) ? P.rows.w + (int64_t)r * P.rows.cap : nullptr;
-  const char* kbase = (const char*)P.k;
-  const char* vbase = (const char*)P.v;
-  constexpr int ES = (DT == SAH_F32) ? 4 : 2;
-  const int64_t koff = ((int64_t)b * P.ks_b + (int64_t)hk * P.ks_h) * ES;
-  const int64_t voff = ((int64_t)b * P.vs_b + (int64_t)hk * P.vs_h) * ES;
+  const char* kbase = (const char*)P.k + ((int64_t)b * P.ks_b + (int64_t)hk * P.ks_h + sub * 8) * ES;
+  const char* vbase = (const char*)P.v + ((int64_t)b * P.vs_b + (int64_t)hk * P.vs_h + sub * 8) * ES;
+  const int64_t krow = P.ks_l * ES, vrow = P.vs_l * ES;
   const int64_t moff = P.amask ? ((int64_t)b * P.ms_b + (int64_t)h * P.ms_h + (int64_t)qi * P.ms_l) : 0;
 
   float qv[8];
@@ -104,9 +143,9 @@ __global__ __launch_bounds__(ATT_NT) void k_sparse_attn(att_params P) {
   float l_run = 0.f;
   float m_run = -INFINITY;
 
-  for (int cbase = begin; cbase < end; cbase += ATT_CHUNK) {
-    // one column (and its inverse weight) per lane: this wave's 64 keys
-    const int my = cbase + wave * SAH_WAVE + lane;
+  for (int cbase = begin + wave * SAH_WAVE; cbase < end; cbase += ATT_CHUNK) {
+    // one column (and its inverse weight) per lane: this wave's next 64 keys
+    const int my = cbase + lane;
     int idx_l = -1;
     float invw_l = P.unit_inv_w;
     if (my < end) {
@@ -115,93 +154,69 @@ __global__ __launch_bounds__(ATT_NT) void k_sparse_attn(att_params P) {
       if (wts) invw_l = sah_round<DT>(1.0f / sah_round<DT>(wts[my] + 1e-6f));
       if (idx_l < 0 || idx_l >= P.Lk) idx_l = -1;
     }
-
-    // ---- phase 1: logits of this wave's keys -----------------------------
-    float z[IT];
 #pragma unroll
     for (int ib = 0; ib < IT; ib += UB) {
-      float kv[UB][8];
+      if (cbase + ib * KPI >= end) break;  // uniform across the wave
+      att_raw<DT> kr[UB], vr[UB];
       int id[UB];
 #pragma unroll
       for (int u = 0; u < UB; ++u) {
         id[u] = __shfl(idx_l, (ib + u) * KPI + grp);
-        if (id[u] >= 0) {
-          sah_load8<DT>(kbase + koff + (int64_t)id[u] * P.ks_l * ES, sub * 8, kv[u]);
-        } else {
-#pragma unroll
-          for (int e = 0; e < 8; ++e) kv[u][e] = 0.f;
-        }
+        const int safe = id[u] >= 0 ? id[u] : 0;  // invalid lanes read row 0 and are masked below
+        att_load_raw<DT>(kbase + (int64_t)safe * krow, kr[u]);
+        att_load_raw<DT>(vbase + (int64_t)safe * vrow, vr[u]);
       }
+      float z[UB];
+      float mb = -INFINITY;
 #pragma unroll
       for (int u = 0; u < UB; ++u) {
+        float kf[8];
+        att_unpack<DT>(kr[u], kf);
         float d = 0.f;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) d = fmaf(qv[e], kv[u][e], d);
+        for (int e = 0; e < 8; ++e) d = fmaf(qv[e], kf[e], d);
         d = att_group_sum<LPK>(d) * P.scaling;
         if (id[u] >= 0) {
           if (P.amask) d += sah_load<DT>(P.amask, moff + id[u]);
         } else {
           d = -INFINITY;
         }
-        z[ib + u] = d;
+        z[u] = d;
+        mb = fmaxf(mb, d);
       }
-    }
-    if (P.logits_out && sub == 0) {
+      if (P.logits_out && sub == 0) {
 #pragma unroll
-      for (int it = 0; it < IT; ++it) {
-        const int pos = cbase + wave * SAH_WAVE + it * KPI + grp;
-        if (pos < end) {
-          const int64_t at = P.dense ? (int64_t)pos : (int64_t)pos;
-          P.logits_out[(int64_t)r * P.logits_pitch + at] = z[it];
+        for (int u = 0; u < UB; ++u) {
+          const int pos = cbase + (ib + u) * KPI + grp;
+          if (pos < end) P.logits_out[(int64_t)r * P.logits_pitch + pos] = z[u];
         }
       }
-    }
-
-    float m_loc = z[0];
+      // batch max over the lane groups of the wave: m stays uniform across the wave
 #pragma unroll
-    for (int it = 1; it < IT; ++it) m_loc = fmaxf(m_loc, z[it]);
-    m_loc = sah_wave_max(m_loc);
-    __syncthreads();  // s_max free (previous chunk's readers are done)
-    if (lane == 0) s_max[wave] = m_loc;
-    __syncthreads();
-    float m_new = m_run;
+      for (int o = LPK; o < SAH_WAVE; o <<= 1) mb = fmaxf(mb, __shfl_xor(mb, o));
+      const float m_new = fmaxf(m_run, mb);
+      if (m_new != -INFINITY) {
+        const float rescale = (m_run == -INFINITY) ? 0.f : att_exp<DT>(m_run - m_new);
 #pragma unroll
-    for (int wv = 0; wv < ATT_NW; ++wv) m_new = fmaxf(m_new, s_max[wv]);
-
-    const float rescale = (m_run == -INFINITY) ? 0.f : att_exp<DT>(m_run - m_new);
+        for (int e = 0; e < 8; ++e) acc[e] *= rescale;
+        l_run *= rescale;
+        m_run = m_new;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] *= rescale;
-    l_run *= rescale;
-    m_run = m_new;
-
-    // ---- phase 2: weighted sum of this wave's value rows -------------------
+        for (int u = 0; u < UB; ++u) {
+          const float iw = __shfl(invw_l, (ib + u) * KPI + grp);
+          float p = 0.f;
+          if (z[u] != -INFINITY) p = att_exp<DT>(z[u] - m_new) * iw;
+          l_run += p;
+          float vf[8];
+          att_unpack<DT>(vr[u], vf);
 #pragma unroll
-    for (int ib = 0; ib < IT; ib += UB) {
-      float vv[UB][8];
-      int id[UB];
-#pragma unroll
-      for (int u = 0; u < UB; ++u) {
-        id[u] = __shfl(idx_l, (ib + u) * KPI + grp);
-        if (id[u] >= 0) {
-          sah_load8<DT>(vbase + voff + (int64_t)id[u] * P.vs_l * ES, sub * 8, vv[u]);
-        } else {
-#pragma unroll
-          for (int e = 0; e < 8; ++e) vv[u][e] = 0.f;
+          for (int e = 0; e < 8; ++e) acc[e] = fmaf(p, vf[e], acc[e]);
         }
-      }
-#pragma unroll
-      for (int u = 0; u < UB; ++u) {
-        const float iw = __shfl(invw_l, (ib + u) * KPI + grp);
-        float p = 0.f;
-        if (id[u] >= 0 && z[ib + u] != -INFINITY) p = att_exp<DT>(z[ib + u] - m_new) * iw;
-        l_run += p;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[e] = fmaf(p, vv[u][e], acc[e]);
       }
     }
   }
 
-  // ---- reduce the KPI lane groups of the wave, then the waves -----------------
+  // ---- reduce the KPI lane groups of the wave, then the waves (rescaled to a common max)
 #pragma unroll
   for (int o = LPK; o < SAH_WAVE; o <<= 1) {
 #pragma unroll
@@ -212,19 +227,28 @@ __global__ __launch_bounds__(ATT_NT) void k_sparse_attn(att_params P) {
 #pragma unroll
     for (int e = 0; e < 8; ++e) s_acc[wave][sub * 8 + e] = acc[e];
   }
-  if (lane == 0) s_l[wave] = l_run;
+  if (lane == 0) {
+    s_l[wave] = l_run;
+    s_m[wave] = m_run;
+  }
   __syncthreads();
+  float M = s_m[0];
+#pragma unroll
+  for (int wv = 1; wv < ATT_NW; ++wv) M = fmaxf(M, s_m[wv]);
+  float sc[ATT_NW];
+#pragma unroll
+  for (int wv = 0; wv < ATT_NW; ++wv) sc[wv] = (s_m[wv] == -INFINITY) ? 0.f : att_exp<DT>(s_m[wv] - M);
   if (tid < D) {
     float a = 0.f;
 #pragma unroll
-    for (int wv = 0; wv < ATT_NW; ++wv) a += s_acc[wv][tid];
+    for (int wv = 0; wv < ATT_NW; ++wv) a = fmaf(s_acc[wv][tid], sc[wv], a);
     wout[2 + tid] = a;
   }
   if (tid == 0) {
     float l = 0.f;
 #pragma unroll
-    for (int wv = 0; wv < ATT_NW; ++wv) l += s_l[wv];
-    wout[0] = m_run;
+    for (int wv = 0; wv < ATT_NW; ++wv) l = fmaf(s_l[wv], sc[wv], l);
+    wout[0] = M;
     wout[1] = l;
   }
 }
@@ -311,9 +335,14 @@ extern "C" int64_t sah_sparse_attention_work_floats(int32_t n_rows, int32_t max_
 template <int DT, int D>
 static int att_launch(const sah_attention_args* a, const att_params& P) {
   hipStream_t st = (hipStream_t)a->stream;
-  hipLaunchKernelGGL((k_sparse_attn<DT, D>), dim3(P.n_split, a->rows.n_rows), dim3(ATT_NT), 0, st, P);
-  int rc = sah_launch_status("sah_sparse_attention");
+  int rc;
+  {
+    sah_timed timed("k_sparse_attn", a->stream);
+    hipLaunchKernelGGL((k_sparse_attn<DT, D>), dim3(P.n_split, a->rows.n_rows), dim3(ATT_NT), 0, st, P);
+    rc = sah_launch_status("sah_sparse_attention");
+  }
   if (rc) return rc;
+  sah_timed timed("k_attn_combine", a->stream);
   hipLaunchKernelGGL((k_attn_combine<DT, D>), dim3(a->rows.n_rows), dim3(D < 64 ? 64 : D), 0, st,
                      (const float*)a->work, P.n_split, a->Hq, a->Lq, a->sinks, a->out, a->stats_out);
   return sah_launch_status("sah_sparse_attention(combine)");
@@ -391,6 +420,7 @@ extern "C" int sah_attention_weights(const sah_attention_weights_args* a) {
   const int64_t pitch = dense ? a->rows.n_keys : a->rows.cap;
   dim3 g((max_cnt + 255) / 256, a->rows.n_rows), b(256);
   hipStream_t st = (hipStream_t)a->stream;
+  sah_timed timed("k_attn_weights", a->stream);
   switch (a->dtype) {
     case SAH_F32: hipLaunchKernelGGL(k_attn_weights<SAH_F32>, g, b, 0, st, a->rows, a->logits, pitch, a->stats, a->unit_inv_w, dense, a->weights); break;
     case SAH_BF16: hipLaunchKernelGGL(k_attn_weights<SAH_BF16>, g, b, 0, st, a->rows, a->logits, pitch, a->stats, a->unit_inv_w, dense, a->weights); break;

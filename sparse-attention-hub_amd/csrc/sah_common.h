@@ -25,6 +25,22 @@ static inline int sah_fail(int code, const char* fmt, ...) {
   return code;
 }
 
+// Opt-in per-kernel timing with HIP events on the launch stream (see sah_timing_* in
+// include/sah.h). A scope brackets one kernel launch; it costs nothing when disabled.
+bool sah_timing_enabled();
+void sah_timing_begin(const char* name, hipStream_t st);
+void sah_timing_end(hipStream_t st);
+struct sah_timed {
+  hipStream_t st;
+  bool on;
+  sah_timed(const char* name, void* stream) : st((hipStream_t)stream), on(sah_timing_enabled()) {
+    if (on) sah_timing_begin(name, st);
+  }
+  ~sah_timed() {
+    if (on) sah_timing_end(st);
+  }
+};
+
 static inline int sah_launch_status(const char* what) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) {

@@ -107,6 +107,138 @@ __global__ __launch_bounds__(SIG_NT) void k_hash_sig_tile(sig_params P) {
   }
 }
 
+// ---------------------------------------------------------------------------
+// Decode path: a handful of vectors per head (one new key, one query). One
+// workgroup per (b, h, group of up to GV vectors); the layer matrix W[h] (d_in x
+// d_out, row-major) is read once with 16-byte loads: thread t owns 8 adjacent
+// output columns (cg = t % CG) of the rows d = rg, rg + RG, ... (rg = t / CG), all
+// of its row loads are in flight together, and the RG partial sums are reduced by
+// wave shuffles and one pass through LDS. Three layers = three memory round trips.
+// Needs every layer width to be a power of two in [8, 256] and D % 8 == 0.
+// ---------------------------------------------------------------------------
+#define GEMV_NT 256
+#define GEMV_NW (GEMV_NT / SAH_WAVE)
+#define GEMV_GV 4
+#define GEMV_MAXROWS 8  // rows per thread: d_in * d_out / 8 / GEMV_NT <= 8 for 256 x 256
+
+template <int DT>
+__global__ __launch_bounds__(GEMV_NT) void k_hash_sig_gemv(sig_params P) {
+  __shared__ float s_x[GEMV_GV][SIG_MAXD];
+  __shared__ float s_part[GEMV_NW][GEMV_GV][SIG_MAXD];
+  const int tid = threadIdx.x;
+  const int lane = tid & (SAH_WAVE - 1);
+  const int wave = tid / SAH_WAVE;
+  const int bh = blockIdx.y;
+  const int h = bh % P.Hq;
+  const int b = bh / P.Hq;
+  const int hx = h / P.group;
+  const int l0 = blockIdx.x * GEMV_GV;
+  int nl = P.L - l0;
+  if (nl > GEMV_GV) nl = GEMV_GV;
+
+  for (int i = tid; i < GEMV_GV * P.D; i += GEMV_NT) {
+    const int t = i / P.D, d = i % P.D;
+    float v = 0.f;
+    if (t < nl) v = sah_load<DT>(P.x, (int64_t)b * P.xs_b + (int64_t)hx * P.xs_h + (int64_t)(l0 + t) * P.xs_l + d);
+    s_x[t][d] = v;
+  }
+  __syncthreads();
+
+  int din = P.D;
+  for (int layer = 0; layer < P.n_layers; ++layer) {
+    const int dout = P.d_out[layer];
+    const bool last = (layer == P.n_layers - 1);
+    const int CG = dout / 8;            // column groups (power of two, <= 32)
+    const int RG = GEMV_NT / CG;        // row groups
+    const int cg = tid % CG, rg = tid / CG;
+    const char* wbase = (const char*)P.W[layer] + ((int64_t)h * din * dout + cg * 8) * (DT == SAH_F32 ? 4 : 2);
+    float acc[GEMV_GV][8];
+#pragma unroll
+    for (int t = 0; t < GEMV_GV; ++t)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[t][e] = 0.f;
+    float wv[GEMV_MAXROWS][8];
+#pragma unroll
+    for (int i = 0; i < GEMV_MAXROWS; ++i) {
+      const int d = rg + i * RG;
+      if (d < din) {
+        sah_load8<DT>(wbase, (int64_t)d * dout, wv[i]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) wv[i][e] = 0.f;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < GEMV_MAXROWS; ++i) {
+      const int d = rg + i * RG;
+      if (d < din) {
+#pragma unroll
+        for (int t = 0; t < GEMV_GV; ++t) {
+          const float xv = s_x[t][d];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[t][e] = fmaf(xv, wv[i][e], acc[t][e]);
+        }
+      }
+    }
+    // lanes of a wave that share cg differ by multiples of CG
+    for (int o = CG; o < SAH_WAVE; o <<= 1) {
+#pragma unroll
+      for (int t = 0; t < GEMV_GV; ++t)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[t][e] += __shfl_xor(acc[t][e], o);
+    }
+    if (lane < CG) {
+#pragma unroll
+      for (int t = 0; t < GEMV_GV; ++t)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s_part[wave][t][cg * 8 + e] = acc[t][e];
+    }
+    __syncthreads();
+    // CG > 64 cannot happen (dout <= 256 => CG <= 32), so every wave holds all column groups
+    for (int i = tid; i < GEMV_GV * dout; i += GEMV_NT) {
+      const int t = i / dout, e = i % dout;
+      float y = 0.f;
+#pragma unroll
+      for (int wv2 = 0; wv2 < GEMV_NW; ++wv2) y += s_part[wv2][t][e];
+      y = sah_round<DT>(y);
+      y = sah_round<DT>(y + sah_load<DT>(P.bias[layer], (int64_t)h * dout + e));
+      if (!last) y = sah_round<DT>(sig_act(P.act, y));
+      s_x[t][e] = y;
+    }
+    __syncthreads();
+    din = dout;
+  }
+
+  if (tid < SAH_WAVE) {
+    const int bits = din;
+    for (int t = 0; t < nl; ++t) {
+      const float y = (tid < bits) ? s_x[t][tid] : 0.f;
+      const uint64_t pos = __ballot(y > 0.f);
+      const uint64_t nz = __ballot(y != 0.f);
+      if (tid == 0) {
+        uint2 c;
+        c.x = (uint32_t)pos;
+        c.y = (uint32_t)nz;
+        ((uint2*)P.codes)[(int64_t)bh * P.code_pitch + P.code_offset + l0 + t] = c;
+      }
+    }
+  }
+}
+
+static bool sig_gemv_ok(const sah_hash_sig_args* a) {
+  if (a->L > 64 || a->D % 8 || a->D > SIG_MAXD) return false;
+  int din = a->D;
+  for (int i = 0; i < a->n_layers; ++i) {
+    const int dout = a->d_out[i];
+    if (dout < 8 || dout > 256 || (dout & (dout - 1))) return false;
+    if ((int64_t)din * dout > (int64_t)8 * GEMV_NT * GEMV_MAXROWS) return false;
+    const int es = a->dtype == SAH_F32 ? 4 : 2;
+    if (((uintptr_t)a->W[i]) % (8 * es)) return false;
+    din = dout;
+  }
+  return true;
+}
+
 extern "C" int sah_hash_signatures(const sah_hash_sig_args* a) {
   if (!a) return sah_fail(SAH_ENULL, "sah_hash_signatures: args is NULL");
   if (!a->x || !a->codes) return sah_fail(SAH_ENULL, "sah_hash_signatures: x / codes is NULL");
@@ -135,8 +267,20 @@ extern "C" int sah_hash_signatures(const sah_hash_sig_args* a) {
   }
   P.act = a->act;
   P.codes = a->codes; P.code_pitch = a->code_pitch; P.code_offset = a->code_offset;
-  dim3 g((a->L + SIG_TL - 1) / SIG_TL, a->B * a->Hq), b(SIG_NT);
   hipStream_t st = (hipStream_t)a->stream;
+  if (sig_gemv_ok(a)) {
+    dim3 gg((a->L + GEMV_GV - 1) / GEMV_GV, a->B * a->Hq), gb(GEMV_NT);
+    sah_timed timed("k_hash_sig_gemv", a->stream);
+    switch (a->dtype) {
+      case SAH_F32: hipLaunchKernelGGL(k_hash_sig_gemv<SAH_F32>, gg, gb, 0, st, P); break;
+      case SAH_BF16: hipLaunchKernelGGL(k_hash_sig_gemv<SAH_BF16>, gg, gb, 0, st, P); break;
+      case SAH_F16: hipLaunchKernelGGL(k_hash_sig_gemv<SAH_F16>, gg, gb, 0, st, P); break;
+      default: return sah_fail(SAH_EDTYPE, "sah_hash_signatures: dtype %d", a->dtype);
+    }
+    return sah_launch_status("sah_hash_signatures");
+  }
+  dim3 g((a->L + SIG_TL - 1) / SIG_TL, a->B * a->Hq), b(SIG_NT);
+  sah_timed timed("k_hash_sig_tile", a->stream);
   switch (a->dtype) {
     case SAH_F32: hipLaunchKernelGGL(k_hash_sig_tile<SAH_F32>, g, b, 0, st, P); break;
     case SAH_BF16: hipLaunchKernelGGL(k_hash_sig_tile<SAH_BF16>, g, b, 0, st, P); break;

@@ -287,6 +287,7 @@ extern "C" int sah_pq_kmeans_assign(const sah_pq_assign_args* a) {
   const int per_wg = PQ_NT * PQ_TILES;
   dim3 g(((a->n_keys + per_wg - 1) / per_wg) * a->n_sub, a->B * a->Hkv), blk(PQ_NT);
   hipStream_t st = (hipStream_t)a->stream;
+  sah_timed timed("k_pq_assign", a->stream);
   switch (a->dtype) {
     case SAH_F32: hipLaunchKernelGGL(k_pq_assign<SAH_F32>, g, blk, 0, st, P); break;
     case SAH_BF16: hipLaunchKernelGGL(k_pq_assign<SAH_BF16>, g, blk, 0, st, P); break;
@@ -310,11 +311,14 @@ extern "C" int sah_pq_kmeans_update(const sah_pq_update_args* a) {
   P.n_groups = a->B * a->Hkv * a->n_sub;
   dim3 g(P.n_groups), blk(PQ_NT);
   hipStream_t st = (hipStream_t)a->stream;
-  switch (a->dtype) {
-    case SAH_F32: hipLaunchKernelGGL(k_pq_update<SAH_F32>, g, blk, 0, st, P); break;
-    case SAH_BF16: hipLaunchKernelGGL(k_pq_update<SAH_BF16>, g, blk, 0, st, P); break;
-    case SAH_F16: hipLaunchKernelGGL(k_pq_update<SAH_F16>, g, blk, 0, st, P); break;
-    default: return sah_fail(SAH_EDTYPE, "sah_pq_kmeans_update: dtype %d", a->dtype);
+  {
+    sah_timed timed("k_pq_update", a->stream);
+    switch (a->dtype) {
+      case SAH_F32: hipLaunchKernelGGL(k_pq_update<SAH_F32>, g, blk, 0, st, P); break;
+      case SAH_BF16: hipLaunchKernelGGL(k_pq_update<SAH_BF16>, g, blk, 0, st, P); break;
+      case SAH_F16: hipLaunchKernelGGL(k_pq_update<SAH_F16>, g, blk, 0, st, P); break;
+      default: return sah_fail(SAH_EDTYPE, "sah_pq_kmeans_update: dtype %d", a->dtype);
+    }
   }
   rc = sah_launch_status("sah_pq_kmeans_update");
   if (rc) return rc;
@@ -341,6 +345,7 @@ extern "C" int sah_pq_adc_scores(const sah_pq_adc_args* a) {
   const int per_wg = PQ_NT * ADC_TILES;
   dim3 g((a->n_cand + per_wg - 1) / per_wg, a->B * a->Hkv, (nvec + nq - 1) / nq), blk(PQ_NT);
   hipStream_t st = (hipStream_t)a->stream;
+  sah_timed timed("k_pq_adc", a->stream);
   switch (a->dtype) {
     case SAH_F32: hipLaunchKernelGGL(k_pq_adc<SAH_F32>, g, blk, 0, st, P); break;
     case SAH_BF16: hipLaunchKernelGGL(k_pq_adc<SAH_BF16>, g, blk, 0, st, P); break;

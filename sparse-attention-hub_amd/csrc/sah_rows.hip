@@ -6,6 +6,78 @@
 static thread_local char g_err[512];
 char* sah_err_buf() { return g_err; }
 
+// ---------------------------------------------------------------------------
+// opt-in kernel timing
+// ---------------------------------------------------------------------------
+#include <mutex>
+#include <string>
+#include <vector>
+namespace {
+struct timing_rec {
+  const char* name;
+  hipEvent_t a, b;
+};
+std::mutex g_tmu;
+bool g_timing = false;
+std::vector<timing_rec> g_recs;
+std::vector<std::pair<hipEvent_t, hipEvent_t>> g_pool;
+}  // namespace
+
+bool sah_timing_enabled() { return g_timing; }
+
+void sah_timing_begin(const char* name, hipStream_t st) {
+  std::lock_guard<std::mutex> lk(g_tmu);
+  timing_rec r;
+  r.name = name;
+  if (!g_pool.empty()) {
+    r.a = g_pool.back().first;
+    r.b = g_pool.back().second;
+    g_pool.pop_back();
+  } else {
+    if (hipEventCreate(&r.a) != hipSuccess || hipEventCreate(&r.b) != hipSuccess) return;
+  }
+  (void)hipEventRecord(r.a, st);
+  g_recs.push_back(r);
+}
+
+void sah_timing_end(hipStream_t st) {
+  std::lock_guard<std::mutex> lk(g_tmu);
+  if (!g_recs.empty()) (void)hipEventRecord(g_recs.back().b, st);
+}
+
+extern "C" int sah_timing_enable(int on) {
+  std::lock_guard<std::mutex> lk(g_tmu);
+  g_timing = on != 0;
+  return SAH_OK;
+}
+
+// Waits for the recorded events, adds up the time per kernel name and clears the log.
+// names: out array of `max` pointers to static strings; returns the number of distinct kernels.
+extern "C" int sah_timing_collect(const char** names, int* counts, float* total_ms, int max) {
+  std::lock_guard<std::mutex> lk(g_tmu);
+  int n = 0;
+  for (auto& r : g_recs) {
+    float ms = 0.f;
+    if (hipEventSynchronize(r.b) == hipSuccess && hipEventElapsedTime(&ms, r.a, r.b) == hipSuccess) {
+      int i = 0;
+      for (; i < n; ++i)
+        if (names[i] == r.name) break;
+      if (i == n) {
+        if (n >= max) continue;
+        names[n] = r.name;
+        counts[n] = 0;
+        total_ms[n] = 0.f;
+        ++n;
+      }
+      counts[i] += 1;
+      total_ms[i] += ms;
+    }
+    g_pool.push_back({r.a, r.b});
+  }
+  g_recs.clear();
+  return n;
+}
+
 extern "C" int sah_version(void) { return SAH_VERSION; }
 extern "C" const char* sah_last_error(void) { return g_err; }
 
@@ -147,6 +219,7 @@ extern "C" int sah_sink_local_indices(const sah_sink_local_args* a) {
       return sah_fail(SAH_ECAPACITY, "sah_sink_local_indices: cap %d < sink+window %lld", a->rows.cap,
                       (long long)worst);
   }
+  sah_timed timed("k_sink_local", a->stream);
   hipLaunchKernelGGL(k_sink_local, dim3(a->rows.n_rows), dim3(ROWS_NT), 0, (hipStream_t)a->stream, a->rows,
                      a->lq, a->sink, a->window, a->fresh, a->clear_future);
   return sah_launch_status("sah_sink_local_indices");
@@ -231,6 +304,7 @@ extern "C" int sah_rows_from_dense(const sah_dense_rows_args* a) {
     return sah_fail(SAH_ESHAPE, "sah_rows_from_dense: n_keys %d exceeds %d", a->rows.n_keys, ROWS_MAX_WORDS * 32);
   dim3 g(a->rows.n_rows), b(ROWS_NT);
   hipStream_t st = (hipStream_t)a->stream;
+  sah_timed timed("k_rows_from_dense", a->stream);
   switch (a->dtype) {
     case SAH_F32: hipLaunchKernelGGL(k_rows_from_dense<SAH_F32>, g, b, 0, st, a->rows, (const void*)a->dense); break;
     case SAH_BF16: hipLaunchKernelGGL(k_rows_from_dense<SAH_BF16>, g, b, 0, st, a->rows, (const void*)a->dense); break;
@@ -247,6 +321,7 @@ extern "C" int sah_rows_to_dense(const sah_dense_rows_args* a) {
   if (!a->dense) return sah_fail(SAH_ENULL, "sah_rows_to_dense: dense is NULL");
   dim3 g(a->rows.n_rows), b(ROWS_NT);
   hipStream_t st = (hipStream_t)a->stream;
+  sah_timed timed("k_rows_to_dense", a->stream);
   switch (a->dtype) {
     case SAH_F32: hipLaunchKernelGGL(k_rows_to_dense<SAH_F32>, g, b, 0, st, a->rows, a->dense); break;
     case SAH_BF16: hipLaunchKernelGGL(k_rows_to_dense<SAH_BF16>, g, b, 0, st, a->rows, a->dense); break;

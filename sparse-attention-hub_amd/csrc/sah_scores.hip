@@ -120,6 +120,7 @@ static int qk_launch(const sah_qk_scores_args* a, const qk_params& P) {
   const int G = a->Hq / a->Hkv;
   const int nvec = G * a->Lq;
   dim3 g((a->Lk + SC_TILE * SC_ITERS - 1) / (SC_TILE * SC_ITERS), a->B * a->Hkv, (nvec + SC_NQ - 1) / SC_NQ);
+  sah_timed timed("k_qk_scores", a->stream);
   hipLaunchKernelGGL((k_qk_scores<DT, D>), g, dim3(SC_NT), 0, (hipStream_t)a->stream, P);
   return sah_launch_status("sah_qk_scores");
 }

@@ -39,7 +39,6 @@ struct key_src_hamming {
 };
 
 struct sel_shared {
-  uint32_t hist[SEL_BINS];
   int scan[SEL_NW + 1];
   int wave_gt[SEL_NW];
   int wave_eq[SEL_NW];
@@ -50,14 +49,28 @@ struct sel_shared {
   int total_out;
 };
 
-// KEYBITS: number of significant key bits (7, 16 or 32)
-template <typename SRC, int KEYBITS>
-__device__ __forceinline__ void select_row(sel_shared& S, const sah_rows& R, int r, const SRC& src, int n_cand,
-                                           int col_offset, int k, uint32_t excluded_key) {
+#define SEL_LOAD_BATCH 8  // 64-column chunks requested together in the staging pass
+
+// Dynamic LDS layout of one row: [histogram 4*nbins][bitmap row 4*n_words][staged keys].
+// The bitmap row and (when they fit) the effective keys of all candidates are staged once,
+// with SEL_LOAD_BATCH chunks of loads in flight per wave, so that the digit passes and the
+// two compaction passes run out of LDS instead of re-reading global memory.
+struct sel_layout {
+  int hist_bins;      // bins of the widest digit
+  int stage_keys;     // 1: effective keys are staged in LDS
+};
+
+// KEYBITS: number of significant key bits (7, 16 or 32); STG: LDS type of a staged key
+template <typename SRC, int KEYBITS, typename STG>
+__device__ __forceinline__ void select_row(sel_shared& S, unsigned char* dyn, sel_layout L, const sah_rows& R, int r,
+                                           const SRC& src, int n_cand, int col_offset, int k, uint32_t excluded_key) {
   const int tid = threadIdx.x;
   const int lane = tid & (SAH_WAVE - 1);
   const int wave = tid / SAH_WAVE;
-  const uint32_t* bm = R.bitmap + (int64_t)r * R.n_words;
+  uint32_t* hist = (uint32_t*)dyn;
+  uint32_t* s_bm = hist + L.hist_bins;
+  STG* staged = (STG*)(s_bm + R.n_words);
+  uint32_t* bm = R.bitmap + (int64_t)r * R.n_words;
 
   // 64-column aligned chunks of the candidate range, split contiguously over waves
   const int c_first = col_offset / SAH_WAVE;
@@ -67,14 +80,28 @@ __device__ __forceinline__ void select_row(sel_shared& S, const sah_rows& R, int
   const int my_c0 = c_first + wave * cpw;
   int my_c1 = my_c0 + cpw;
   if (my_c1 > c_last + 1) my_c1 = c_last + 1;
+  const int col_base = c_first * SAH_WAVE;  // staged[] is indexed by col - col_base
 
-  auto eff_key = [&](int col, bool& valid, bool& excl) -> uint32_t {
+  for (int i = tid; i < R.n_words; i += SEL_NT) s_bm[i] = bm[i];
+  __syncthreads();
+
+  // effective key of a column: straight from global memory (branch-free, clamped addresses)
+  auto eff_key_global = [&](int col, bool& valid, bool& excl) -> uint32_t {
     const int cand = col - col_offset;
     valid = (cand >= 0 && cand < n_cand);
-    excl = false;
-    if (!valid) return 0u;
-    excl = (bm[col >> 5] >> (col & 31)) & 1u;
-    return excl ? excluded_key : src(cand);
+    const int cc = valid ? cand : 0;
+    const int cl = valid ? col : col_offset;
+    const uint32_t key = src(cc);
+    excl = valid && ((s_bm[cl >> 5] >> (cl & 31)) & 1u);
+    return valid ? (excl ? excluded_key : key) : 0u;
+  };
+  auto eff_key = [&](int col, bool& valid, bool& excl) -> uint32_t {
+    if (!L.stage_keys) return eff_key_global(col, valid, excl);
+    const int cand = col - col_offset;
+    valid = (cand >= 0 && cand < n_cand);
+    const int cl = valid ? col : col_offset;
+    excl = valid && ((s_bm[cl >> 5] >> (cl & 31)) & 1u);
+    return valid ? (uint32_t)staged[cl - col_base] : 0u;
   };
 
   if (k > n_cand) k = n_cand;
@@ -88,26 +115,45 @@ __device__ __forceinline__ void select_row(sel_shared& S, const sah_rows& R, int
     if (wd > SEL_DIGIT_BITS) wd = SEL_DIGIT_BITS;
     const int sh = KEYBITS - bits_done - wd;
     const int nb = 1 << wd;
-    for (int i = tid; i < nb; i += SEL_NT) S.hist[i] = 0;
+    for (int i = tid; i < nb; i += SEL_NT) hist[i] = 0;
     __syncthreads();
-    for (int c = my_c0; c < my_c1; ++c) {
-      const int col = c * SAH_WAVE + lane;
-      bool valid, excl;
-      const uint32_t key = eff_key(col, valid, excl);
-      if (valid) {
-        const bool match = (bits_done == 0) || ((key >> (sh + wd)) == prefix);
-        if (match) atomicAdd(&S.hist[(key >> sh) & (uint32_t)(nb - 1)], 1u);
+    if (bits_done == 0) {
+      // first pass: batched global loads, stage the keys, histogram of the top digit
+      for (int c0 = my_c0; c0 < my_c1; c0 += SEL_LOAD_BATCH) {
+        uint32_t key[SEL_LOAD_BATCH];
+        bool valid[SEL_LOAD_BATCH];
+#pragma unroll
+        for (int u = 0; u < SEL_LOAD_BATCH; ++u) {
+          bool excl;
+          const int col = (c0 + u) * SAH_WAVE + lane;
+          key[u] = eff_key_global(col, valid[u], excl);
+          valid[u] = valid[u] && (c0 + u < my_c1);
+        }
+#pragma unroll
+        for (int u = 0; u < SEL_LOAD_BATCH; ++u) {
+          if (valid[u]) {
+            const int col = (c0 + u) * SAH_WAVE + lane;
+            if (L.stage_keys) staged[col - col_base] = (STG)key[u];
+            atomicAdd(&hist[(key[u] >> sh) & (uint32_t)(nb - 1)], 1u);
+          }
+        }
+      }
+    } else {
+      for (int c = my_c0; c < my_c1; ++c) {
+        const int col = c * SAH_WAVE + lane;
+        bool valid, excl;
+        const uint32_t key = eff_key(col, valid, excl);
+        if (valid && ((key >> (sh + wd)) == prefix)) atomicAdd(&hist[(key >> sh) & (uint32_t)(nb - 1)], 1u);
       }
     }
     __syncthreads();
     // descending scan over digits: thread t owns the t-th highest group of bins
-    constexpr int GROUPS = SEL_NT;
-    const int per = (nb + GROUPS - 1) / GROUPS;  // bins per thread (1 or 8)
+    const int per = (nb + SEL_NT - 1) / SEL_NT;  // bins per thread (1 or 8)
     const int hi_bin = nb - 1 - tid * per;       // my highest bin
     int mine = 0;
     for (int i = 0; i < per; ++i) {
       const int bin = hi_bin - i;
-      if (bin >= 0) mine += (int)S.hist[bin];
+      if (bin >= 0) mine += (int)hist[bin];
     }
     int total;
     const int above = sah_block_excl_scan<SEL_NT>(mine, S.scan, &total);
@@ -116,7 +162,7 @@ __device__ __forceinline__ void select_row(sel_shared& S, const sah_rows& R, int
       for (int i = 0; i < per; ++i) {
         const int bin = hi_bin - i;
         if (bin < 0) break;
-        const int cbin = (int)S.hist[bin];
+        const int cbin = (int)hist[bin];
         if (need <= run + cbin) {
           S.digit = (uint32_t)bin;
           S.need = need - run;
@@ -133,7 +179,9 @@ __device__ __forceinline__ void select_row(sel_shared& S, const sah_rows& R, int
   }
   const uint32_t T = prefix;  // k-th largest key; `need` ties at T are taken, lowest column first
 
-  // ---- per-wave counts, then ordered compaction -------------------------------
+  // ---- per-wave counts: keys above T that will be emitted, ties, emitted ties ----
+  // Ties are consumed in column order; an already-active tie uses up rank but emits nothing,
+  // so a wave first learns how many ties precede it, then counts the ties it will emit.
   int n_gt = 0, n_eq = 0;
   for (int c = my_c0; c < my_c1; ++c) {
     const int col = c * SAH_WAVE + lane;
@@ -148,31 +196,26 @@ __device__ __forceinline__ void select_row(sel_shared& S, const sah_rows& R, int
   }
   __syncthreads();
   if (tid == 0) {
-    int tie_run = 0, out_run = 0;
+    int tie_run = 0;
     for (int wv = 0; wv < SEL_NW; ++wv) {
       S.wave_tie[wv] = tie_run;
-      S.wave_out[wv] = out_run;
-      // ties are consumed in column order; excluded ties use up rank but emit nothing,
-      // so the emitted count of this wave is only known after its walk: recomputed below
       tie_run += S.wave_eq[wv];
-      out_run += S.wave_gt[wv];
     }
   }
   __syncthreads();
-
-  // The number of *emitted* ties per wave depends on which of its ties are excluded,
-  // so output offsets take a second exchange: each wave counts its emitted ties first.
   int tie_rank = S.wave_tie[wave];
   int emit_ties = 0;
-  for (int c = my_c0; c < my_c1; ++c) {
-    const int col = c * SAH_WAVE + lane;
-    bool valid, excl;
-    const uint32_t key = eff_key(col, valid, excl);
-    const bool is_tie = valid && key == T;
-    const uint64_t tm = __ballot(is_tie);
-    const bool take = is_tie && !excl && (tie_rank + sah_lane_prefix(tm) < need);
-    emit_ties += __popcll(__ballot(take));
-    tie_rank += __popcll(tm);
+  if (tie_rank < need && n_eq > 0) {
+    for (int c = my_c0; c < my_c1; ++c) {
+      const int col = c * SAH_WAVE + lane;
+      bool valid, excl;
+      const uint32_t key = eff_key(col, valid, excl);
+      const bool is_tie = valid && key == T;
+      const uint64_t tm = __ballot(is_tie);
+      const bool take = is_tie && !excl && (tie_rank + sah_lane_prefix(tm) < need);
+      emit_ties += __popcll(__ballot(take));
+      tie_rank += __popcll(tm);
+    }
   }
   __syncthreads();  // wave_eq is re-used below
   if (lane == 0) S.wave_eq[wave] = emit_ties;
@@ -187,11 +230,11 @@ __device__ __forceinline__ void select_row(sel_shared& S, const sah_rows& R, int
   }
   __syncthreads();
 
+  // ---- ordered compaction ----------------------------------------------------
   int cnt0 = R.cnt[r];
   if (cnt0 > R.cap) cnt0 = R.cap;
   int* cols = R.cols + (int64_t)r * R.cap;
   float* w = R.w ? R.w + (int64_t)r * R.cap : nullptr;
-  uint32_t* bmw = R.bitmap + (int64_t)r * R.n_words;
   int out_pos = cnt0 + S.wave_out[wave];
   tie_rank = S.wave_tie[wave];
   for (int c = my_c0; c < my_c1; ++c) {
@@ -210,37 +253,61 @@ __device__ __forceinline__ void select_row(sel_shared& S, const sah_rows& R, int
       }
     }
     if (sm) {
+      // this wave owns words 2c and 2c+1 of the row: plain read-modify-write
       const int w0 = c * 2;
-      if (lane == 0 && (uint32_t)sm) bmw[w0] |= (uint32_t)sm;
-      if (lane == 32 && (uint32_t)(sm >> 32) && w0 + 1 < R.n_words) bmw[w0 + 1] |= (uint32_t)(sm >> 32);
+      if (lane == 0 && (uint32_t)sm) bm[w0] = s_bm[w0] | (uint32_t)sm;
+      if (lane == 32 && (uint32_t)(sm >> 32) && w0 + 1 < R.n_words) bm[w0 + 1] = s_bm[w0 + 1] | (uint32_t)(sm >> 32);
     }
     out_pos += __popcll(sm);
     tie_rank += __popcll(tm);
   }
-  __syncthreads();  // all reads of the old bitmap/cnt precede the count update
   if (tid == 0) R.cnt[r] = cnt0 + S.total_out;
 }
 
+// dynamic LDS bytes and staging decision for one launch
+static size_t sel_plan(int key_bits, int stage_bytes, int n_words, int n_cand, int col_offset, sel_layout* L) {
+  const int wd = key_bits < SEL_DIGIT_BITS ? key_bits : SEL_DIGIT_BITS;
+  L->hist_bins = 1 << wd;
+  size_t fixed = (size_t)L->hist_bins * 4 + (size_t)n_words * 4;
+  const int c_first = col_offset / SAH_WAVE;
+  const int c_last = (col_offset + n_cand - 1) / SAH_WAVE;
+  size_t stage = (size_t)(c_last - c_first + 1) * SAH_WAVE * stage_bytes;
+  const size_t budget = 150 * 1024;  // of the 160 KB LDS of a CU, minus the static part
+  L->stage_keys = (fixed + stage <= budget) ? 1 : 0;
+  return fixed + (L->stage_keys ? stage : 0);
+}
+
 template <int KB>
-__global__ __launch_bounds__(SEL_NT) void k_select_topk(sah_rows R, const void* keys, int64_t pitch, int n_cand,
-                                                        int col_offset, int k, uint32_t excluded_key) {
+__global__ __launch_bounds__(SEL_NT) void k_select_topk(sah_rows R, sel_layout L, const void* keys, int64_t pitch,
+                                                        int n_cand, int col_offset, int k, uint32_t excluded_key) {
   __shared__ sel_shared S;
+  HIP_DYNAMIC_SHARED(unsigned char, sel_dyn)
   const int r = blockIdx.x;
   if (KB == 16) {
     key_src_mem16 src{(const uint16_t*)keys + (int64_t)r * pitch};
-    select_row<key_src_mem16, 16>(S, R, r, src, n_cand, col_offset, k, excluded_key);
+    select_row<key_src_mem16, 16, uint16_t>(S, sel_dyn, L, R, r, src, n_cand, col_offset, k, excluded_key);
   } else {
     key_src_mem32 src{(const uint32_t*)keys + (int64_t)r * pitch};
-    select_row<key_src_mem32, 32>(S, R, r, src, n_cand, col_offset, k, excluded_key);
+    select_row<key_src_mem32, 32, uint32_t>(S, sel_dyn, L, R, r, src, n_cand, col_offset, k, excluded_key);
   }
 }
 
-__global__ __launch_bounds__(SEL_NT) void k_hamming_topk(sah_rows R, const uint2* kcodes, int64_t pitch,
+__global__ __launch_bounds__(SEL_NT) void k_hamming_topk(sah_rows R, sel_layout L, const uint2* kcodes, int64_t pitch,
                                                          const uint2* qcodes, int lq, int k) {
   __shared__ sel_shared S;
+  HIP_DYNAMIC_SHARED(unsigned char, sel_dyn)
   const int r = blockIdx.x;
   key_src_hamming src{kcodes + (int64_t)(r / lq) * pitch, qcodes[r]};
-  select_row<key_src_hamming, 7>(S, R, r, src, R.n_keys, 0, k, 0u);
+  select_row<key_src_hamming, 7, uint8_t>(S, sel_dyn, L, R, r, src, R.n_keys, 0, k, 0u);
+}
+
+// kernels may use up to 160 KB of LDS; HIP needs to be told once per kernel
+template <typename K>
+static int sel_allow_lds(K kernel, size_t bytes, const char* what) {
+  if (bytes <= 48 * 1024) return SAH_OK;
+  hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 1024);
+  if (e != hipSuccess) return sah_fail((int)e, "%s: cannot raise the dynamic LDS limit: %s", what, hipGetErrorString(e));
+  return SAH_OK;
 }
 
 // Signature scores as sortable float keys, for callers that pass an additive
@@ -272,6 +339,7 @@ extern "C" int sah_hamming_scores(const sah_hamming_scores_args* a) {
   if (n_rows > 65535) return sah_fail(SAH_ESHAPE, "sah_hamming_scores: more than 65535 rows");
   dim3 g((a->n_keys + 255) / 256, n_rows), blk(256);
   hipStream_t st = (hipStream_t)a->stream;
+  sah_timed timed("k_hamming_scores", a->stream);
 #define SAH_HS_LAUNCH(DTC)                                                                                          \
   hipLaunchKernelGGL(k_hamming_scores<DTC>, g, blk, 0, st, (const uint2*)a->kcodes, a->code_pitch,                  \
                      (const uint2*)a->qcodes, a->Hq, a->Lq, a->n_keys, a->amask, a->ms_b, a->ms_h, a->ms_l,        \
@@ -298,12 +366,19 @@ extern "C" int sah_select_topk(const sah_select_topk_args* a) {
   if (a->k <= 0) return sah_fail(SAH_EINVAL, "sah_select_topk: k must be > 0");
   if (a->key_pitch < a->n_cand) return sah_fail(SAH_EINVAL, "sah_select_topk: key_pitch < n_cand");
   hipStream_t st = (hipStream_t)a->stream;
+  sel_layout L;
+  const size_t lds = sel_plan(a->key_bits, a->key_bits / 8, a->rows.n_words, a->n_cand, a->col_offset, &L);
+  if (lds > 159 * 1024) return sah_fail(SAH_ESHAPE, "sah_select_topk: %d keys need %zu bytes of LDS", a->rows.n_keys, lds);
+  rc = a->key_bits == 16 ? sel_allow_lds(k_select_topk<16>, lds, "sah_select_topk")
+                         : sel_allow_lds(k_select_topk<32>, lds, "sah_select_topk");
+  if (rc) return rc;
+  sah_timed timed("k_select_topk", a->stream);
   if (a->key_bits == 16)
-    hipLaunchKernelGGL(k_select_topk<16>, dim3(a->rows.n_rows), dim3(SEL_NT), 0, st, a->rows, a->keys, a->key_pitch,
-                       a->n_cand, a->col_offset, a->k, a->excluded_key);
+    hipLaunchKernelGGL(k_select_topk<16>, dim3(a->rows.n_rows), dim3(SEL_NT), lds, st, a->rows, L, a->keys,
+                       a->key_pitch, a->n_cand, a->col_offset, a->k, a->excluded_key);
   else
-    hipLaunchKernelGGL(k_select_topk<32>, dim3(a->rows.n_rows), dim3(SEL_NT), 0, st, a->rows, a->keys, a->key_pitch,
-                       a->n_cand, a->col_offset, a->k, a->excluded_key);
+    hipLaunchKernelGGL(k_select_topk<32>, dim3(a->rows.n_rows), dim3(SEL_NT), lds, st, a->rows, L, a->keys,
+                       a->key_pitch, a->n_cand, a->col_offset, a->k, a->excluded_key);
   return sah_launch_status("sah_select_topk");
 }
 
@@ -315,7 +390,13 @@ extern "C" int sah_hamming_topk(const sah_hamming_topk_args* a) {
   if (a->lq <= 0 || a->rows.n_rows % a->lq) return sah_fail(SAH_EINVAL, "sah_hamming_topk: lq must divide n_rows");
   if (a->k <= 0) return sah_fail(SAH_EINVAL, "sah_hamming_topk: k must be > 0");
   if (a->code_pitch < a->rows.n_keys) return sah_fail(SAH_EINVAL, "sah_hamming_topk: code_pitch < n_keys");
-  hipLaunchKernelGGL(k_hamming_topk, dim3(a->rows.n_rows), dim3(SEL_NT), 0, (hipStream_t)a->stream, a->rows,
+  sel_layout L;
+  const size_t lds = sel_plan(7, 1, a->rows.n_words, a->rows.n_keys, 0, &L);
+  if (lds > 159 * 1024) return sah_fail(SAH_ESHAPE, "sah_hamming_topk: %d keys need %zu bytes of LDS", a->rows.n_keys, lds);
+  rc = sel_allow_lds(k_hamming_topk, lds, "sah_hamming_topk");
+  if (rc) return rc;
+  sah_timed timed("k_hamming_topk", a->stream);
+  hipLaunchKernelGGL(k_hamming_topk, dim3(a->rows.n_rows), dim3(SEL_NT), lds, (hipStream_t)a->stream, a->rows, L,
                      (const uint2*)a->kcodes, a->code_pitch, (const uint2*)a->qcodes, a->lq, a->k);
   return sah_launch_status("sah_hamming_topk");
 }

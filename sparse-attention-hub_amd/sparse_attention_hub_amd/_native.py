@@ -26,6 +26,8 @@ _DTYPE_CODE = {torch.float32: SAH_F32, torch.bfloat16: SAH_BF16, torch.float16: 
 EXPECTED_SYMBOLS = (
     "sah_version",
     "sah_last_error",
+    "sah_timing_enable",
+    "sah_timing_collect",
     "sah_sink_local_indices",
     "sah_rows_from_dense",
     "sah_rows_to_dense",
@@ -298,7 +300,8 @@ def lib() -> C.CDLL:
     handle.sah_sparse_attention_work_floats.restype = C.c_int64
     handle.sah_sparse_attention_work_floats.argtypes = [C.c_int32, C.c_int32, C.c_int32]
     for name in EXPECTED_SYMBOLS:
-        if name in ("sah_version", "sah_last_error", "sah_sparse_attention_work_floats"):
+        if name in ("sah_version", "sah_last_error", "sah_sparse_attention_work_floats",
+                    "sah_timing_enable", "sah_timing_collect"):
             continue
         fn = getattr(handle, name)
         fn.restype = C.c_int
@@ -316,6 +319,22 @@ def call(name: str, args: C.Structure) -> None:
         if rc in (-1, -3, -4, -5):
             raise ValueError(f"{name}: {msg} (code {rc})")
         raise NativeLibraryError(f"{name}: {msg} (code {rc})")
+
+
+def timing_enable(on: bool) -> None:
+    """Switch the library's per-kernel HIP-event timing on or off (benchmarks only)."""
+    lib().sah_timing_enable(1 if on else 0)
+
+
+def timing_collect(max_names: int = 64):
+    """{kernel name: (launch count, total milliseconds)} since the last collect; waits for the events."""
+    handle = lib()
+    names = (C.c_char_p * max_names)()
+    counts = (C.c_int * max_names)()
+    total = (C.c_float * max_names)()
+    handle.sah_timing_collect.restype = C.c_int
+    n = handle.sah_timing_collect(names, counts, total, max_names)
+    return {names[i].decode(): (int(counts[i]), float(total[i])) for i in range(n)}
 
 
 def work_floats(n_rows: int, max_cnt: int, head_dim: int) -> int:
