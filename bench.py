@@ -185,6 +185,7 @@ def main() -> None:
     for i in range(steps):
         step(i, first + warm + 1 + i)
     ev1.record()
+    host_ms = (time.perf_counter() - t0) * 1e3          # launch loop only: host cost when the GPU keeps up
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
     gpu_ms = ev0.elapsed_time(ev1)
@@ -223,6 +224,7 @@ def main() -> None:
         "config": {"workload": w["name"], "q_heads": HQ, "kv_heads": HKV, "head_dim": D, "batch": w["B"], "keys": w["Lk"],
                    "keys_per_row": w["sink"] + w["local"] + w["k"], "attention_weights_output": False},
         "gpu_ms_per_step": round(gpu_ms / steps, 5),
+        "host_launch_ms_per_step": round(host_ms / steps, 5),
         "step_algorithmic_bytes": ab["step"],
         "step_achieved_GBps": round(step_gbs, 1),
         "step_frac_of_hbm_peak": round(step_gbs / HBM_PEAK_GBS, 4),

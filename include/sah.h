@@ -152,6 +152,9 @@ typedef struct sah_hash_sig_args {
   void* stream;
 } sah_hash_sig_args;
 int sah_hash_signatures(const sah_hash_sig_args* a);
+/* Two independent jobs (a decode step hashes its new keys and its queries) in one
+ * launch when both are small; same results as two sah_hash_signatures calls. */
+int sah_hash_signatures_pair(const sah_hash_sig_args* a, const sah_hash_sig_args* b);
 
 /* ---------------------------------------------------------------------------
  * Signature top-k. Replaces the score half of

@@ -253,23 +253,42 @@ __global__ __launch_bounds__(ATT_NT) void k_sparse_attn(att_params P) {
   }
 }
 
-// merge the splits of one row: out = sum_s acc_s e^(m_s-M) / sum_s l_s e^(m_s-M)
+// merge the splits of one row: out = sum_s acc_s e^(m_s-M) / sum_s l_s e^(m_s-M).
+// The (m, l) pairs go through LDS and each thread's partial values are requested together,
+// so the kernel costs about two memory round trips whatever the number of splits.
+#define ATT_MAX_SPLIT 64
 template <int DT, int D>
 __global__ __launch_bounds__(D < 64 ? 64 : D) void k_attn_combine(const float* work, int n_split, int Hq, int Lq,
                                                                   const float* sinks, void* out, float* stats) {
+  __shared__ float s_m[ATT_MAX_SPLIT];
+  __shared__ float s_l[ATT_MAX_SPLIT];
   const int r = blockIdx.x;
   const int d = threadIdx.x;
   const float* w = work + (int64_t)r * n_split * (D + 2);
-  float M = -INFINITY;
-  for (int s = 0; s < n_split; ++s) M = fmaxf(M, w[(int64_t)s * (D + 2)]);
-  float L = 0.f, a = 0.f;
-  for (int s = 0; s < n_split; ++s) {
-    const float* ws = w + (int64_t)s * (D + 2);
-    const float ms = ws[0];
-    if (ms == -INFINITY) continue;
-    const float sc = att_exp<DT>(ms - M);
-    L = fmaf(ws[1], sc, L);
-    if (d < D) a = fmaf(ws[2 + d], sc, a);
+  if (d < n_split) {
+    s_m[d] = w[(int64_t)d * (D + 2)];
+    s_l[d] = w[(int64_t)d * (D + 2) + 1];
+  }
+  float part[ATT_MAX_SPLIT / 4];
+  float a = 0.f;
+  float M = -INFINITY, L = 0.f;
+  for (int s0 = 0; s0 < n_split; s0 += ATT_MAX_SPLIT / 4) {
+#pragma unroll
+    for (int u = 0; u < ATT_MAX_SPLIT / 4; ++u) {
+      const int sidx = s0 + u;
+      part[u] = (sidx < n_split && d < D) ? w[(int64_t)sidx * (D + 2) + 2 + d] : 0.f;
+    }
+    if (s0 == 0) {
+      __syncthreads();
+      for (int sidx = 0; sidx < n_split; ++sidx) M = fmaxf(M, s_m[sidx]);
+      for (int sidx = 0; sidx < n_split; ++sidx)
+        if (s_m[sidx] != -INFINITY) L = fmaf(s_l[sidx], att_exp<DT>(s_m[sidx] - M), L);
+    }
+#pragma unroll
+    for (int u = 0; u < ATT_MAX_SPLIT / 4; ++u) {
+      const int sidx = s0 + u;
+      if (sidx < n_split && s_m[sidx] != -INFINITY) a = fmaf(part[u], att_exp<DT>(s_m[sidx] - M), a);
+    }
   }
   const int qi = r % Lq;
   const int h = (r / Lq) % Hq;

@@ -142,6 +142,20 @@ __device__ __forceinline__ uint32_t sah_sort_key(float score) {
   }
 }
 
+// Pins a loaded value at this point of the program: the load that produced it must have
+// been issued (and is waited for) here, so the compiler can neither sink it into a later
+// branch nor serialise a batch of independent loads one wait at a time.
+__device__ __forceinline__ void sah_keep(uint32_t& v) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("" : "+v"(v));
+#endif
+}
+__device__ __forceinline__ void sah_keep(float& v) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("" : "+v"(v));
+#endif
+}
+
 // ---------------------------------------------------------------------------
 // device side: cross-lane helpers
 // ---------------------------------------------------------------------------

@@ -119,12 +119,43 @@ __global__ __launch_bounds__(SIG_NT) void k_hash_sig_tile(sig_params P) {
 #define GEMV_NT 256
 #define GEMV_NW (GEMV_NT / SAH_WAVE)
 #define GEMV_GV 4
-#define GEMV_MAXROWS 8  // rows per thread: d_in * d_out / 8 / GEMV_NT <= 8 for 256 x 256
+
+
+struct sig_pair {
+  sig_params p[2];
+};
+
+// acc[t][e] += sum over this thread's NR rows of x[t][d] * W[d][8 columns]; the NR row
+// loads (16 or 32 bytes each) are all in flight before the first multiply
+template <int DT, int NR>
+__device__ __forceinline__ void gemv_rows(const char* wbase, int dout, int rg, int RG, const float (*s_x)[SIG_MAXD],
+                                          float (&acc)[GEMV_GV][8]) {
+  float wv[NR][8];
+#pragma unroll
+  for (int i = 0; i < NR; ++i) sah_load8<DT>(wbase, (int64_t)(rg + i * RG) * dout, wv[i]);
+#pragma unroll
+  for (int i = 0; i < NR; ++i)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) sah_keep(wv[i][e]);
+#pragma unroll
+  for (int i = 0; i < NR; ++i) {
+    const int d = rg + i * RG;
+#pragma unroll
+    for (int t = 0; t < GEMV_GV; ++t) {
+      const float xv = s_x[t][d];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[t][e] = fmaf(xv, wv[i][e], acc[t][e]);
+    }
+  }
+}
 
 template <int DT>
-__global__ __launch_bounds__(GEMV_NT) void k_hash_sig_gemv(sig_params P) {
+__global__ __launch_bounds__(GEMV_NT) void k_hash_sig_gemv(sig_pair PP) {
+  const sig_params& P = PP.p[blockIdx.z];
+  if ((int)blockIdx.x * GEMV_GV >= P.L) return;  // the two jobs may differ in vector count
   __shared__ float s_x[GEMV_GV][SIG_MAXD];
   __shared__ float s_part[GEMV_NW][GEMV_GV][SIG_MAXD];
+  __shared__ float s_bias[SIG_MAXD];
   const int tid = threadIdx.x;
   const int lane = tid & (SAH_WAVE - 1);
   const int wave = tid / SAH_WAVE;
@@ -157,28 +188,15 @@ __global__ __launch_bounds__(GEMV_NT) void k_hash_sig_gemv(sig_params P) {
     for (int t = 0; t < GEMV_GV; ++t)
 #pragma unroll
       for (int e = 0; e < 8; ++e) acc[t][e] = 0.f;
-    float wv[GEMV_MAXROWS][8];
-#pragma unroll
-    for (int i = 0; i < GEMV_MAXROWS; ++i) {
-      const int d = rg + i * RG;
-      if (d < din) {
-        sah_load8<DT>(wbase, (int64_t)d * dout, wv[i]);
-      } else {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) wv[i][e] = 0.f;
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < GEMV_MAXROWS; ++i) {
-      const int d = rg + i * RG;
-      if (d < din) {
-#pragma unroll
-        for (int t = 0; t < GEMV_GV; ++t) {
-          const float xv = s_x[t][d];
-#pragma unroll
-          for (int e = 0; e < 8; ++e) acc[t][e] = fmaf(xv, wv[i][e], acc[t][e]);
-        }
-      }
+    // the bias is requested with the weights so its latency hides behind theirs
+    float bias_v = 0.f;
+    if (tid < dout) bias_v = sah_load<DT>(P.bias[layer], (int64_t)h * dout + tid);
+    const int nrow = din / RG;  // rows per thread: 1, 2, 4 or 8 (checked on the host)
+    switch (nrow) {
+      case 1: gemv_rows<DT, 1>(wbase, dout, rg, RG, s_x, acc); break;
+      case 2: gemv_rows<DT, 2>(wbase, dout, rg, RG, s_x, acc); break;
+      case 4: gemv_rows<DT, 4>(wbase, dout, rg, RG, s_x, acc); break;
+      default: gemv_rows<DT, 8>(wbase, dout, rg, RG, s_x, acc); break;
     }
     // lanes of a wave that share cg differ by multiples of CG
     for (int o = CG; o < SAH_WAVE; o <<= 1) {
@@ -193,6 +211,7 @@ __global__ __launch_bounds__(GEMV_NT) void k_hash_sig_gemv(sig_params P) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) s_part[wave][t][cg * 8 + e] = acc[t][e];
     }
+    if (tid < dout) s_bias[tid] = bias_v;
     __syncthreads();
     // CG > 64 cannot happen (dout <= 256 => CG <= 32), so every wave holds all column groups
     for (int i = tid; i < GEMV_GV * dout; i += GEMV_NT) {
@@ -201,7 +220,7 @@ __global__ __launch_bounds__(GEMV_NT) void k_hash_sig_gemv(sig_params P) {
 #pragma unroll
       for (int wv2 = 0; wv2 < GEMV_NW; ++wv2) y += s_part[wv2][t][e];
       y = sah_round<DT>(y);
-      y = sah_round<DT>(y + sah_load<DT>(P.bias[layer], (int64_t)h * dout + e));
+      y = sah_round<DT>(y + s_bias[e]);
       if (!last) y = sah_round<DT>(sig_act(P.act, y));
       s_x[t][e] = y;
     }
@@ -231,7 +250,10 @@ static bool sig_gemv_ok(const sah_hash_sig_args* a) {
   for (int i = 0; i < a->n_layers; ++i) {
     const int dout = a->d_out[i];
     if (dout < 8 || dout > 256 || (dout & (dout - 1))) return false;
-    if ((int64_t)din * dout > (int64_t)8 * GEMV_NT * GEMV_MAXROWS) return false;
+    const int rows_per_thread = (int)((int64_t)din * dout / (8 * GEMV_NT));
+    if ((int64_t)din * dout % (8 * GEMV_NT) || (rows_per_thread != 1 && rows_per_thread != 2 && rows_per_thread != 4 &&
+                                                 rows_per_thread != 8))
+      return false;
     const int es = a->dtype == SAH_F32 ? 4 : 2;
     if (((uintptr_t)a->W[i]) % (8 * es)) return false;
     din = dout;
@@ -239,12 +261,11 @@ static bool sig_gemv_ok(const sah_hash_sig_args* a) {
   return true;
 }
 
-extern "C" int sah_hash_signatures(const sah_hash_sig_args* a) {
+static int sig_validate(const sah_hash_sig_args* a) {
   if (!a) return sah_fail(SAH_ENULL, "sah_hash_signatures: args is NULL");
   if (!a->x || !a->codes) return sah_fail(SAH_ENULL, "sah_hash_signatures: x / codes is NULL");
   if (a->B <= 0 || a->Hq <= 0 || a->group <= 0 || a->D <= 0 || a->Hq % a->group)
     return sah_fail(SAH_EINVAL, "sah_hash_signatures: bad B/Hq/group/D");
-  if (a->L <= 0) return SAH_OK;  // nothing to hash
   if (a->n_layers < 1 || a->n_layers > SAH_MAX_MLP_LAYERS)
     return sah_fail(SAH_ESHAPE, "sah_hash_signatures: n_layers %d not in [1, %d]", a->n_layers, SAH_MAX_MLP_LAYERS);
   if (a->D > SIG_MAXD) return sah_fail(SAH_ESHAPE, "sah_hash_signatures: D %d > %d", a->D, SIG_MAXD);
@@ -254,11 +275,15 @@ extern "C" int sah_hash_signatures(const sah_hash_sig_args* a) {
       return sah_fail(SAH_ESHAPE, "sah_hash_signatures: layer %d width %d not in [1, %d]", i, a->d_out[i], SIG_MAXD);
   }
   if (a->d_out[a->n_layers - 1] > 32)
-    return sah_fail(SAH_ESHAPE, "sah_hash_signatures: %d signature bits do not fit one uint32 code", a->d_out[a->n_layers - 1]);
+    return sah_fail(SAH_ESHAPE, "sah_hash_signatures: %d signature bits do not fit one 32-bit plane", a->d_out[a->n_layers - 1]);
   if (a->act < SAH_ACT_RELU || a->act > SAH_ACT_TANH) return sah_fail(SAH_EINVAL, "sah_hash_signatures: activation %d", a->act);
-  if (a->code_pitch < a->code_offset + a->L) return sah_fail(SAH_ECAPACITY, "sah_hash_signatures: code_pitch too small");
+  if (a->L > 0 && a->code_pitch < a->code_offset + a->L) return sah_fail(SAH_ECAPACITY, "sah_hash_signatures: code_pitch too small");
+  if ((int64_t)a->B * a->Hq > 65535) return sah_fail(SAH_ESHAPE, "sah_hash_signatures: B*Hq > 65535");
+  if (a->dtype != SAH_F32 && a->dtype != SAH_BF16 && a->dtype != SAH_F16) return sah_fail(SAH_EDTYPE, "sah_hash_signatures: dtype %d", a->dtype);
+  return SAH_OK;
+}
 
-  sig_params P;
+static void sig_fill(const sah_hash_sig_args* a, sig_params& P) {
   P.x = a->x; P.xs_b = a->xs_b; P.xs_h = a->xs_h; P.xs_l = a->xs_l;
   P.B = a->B; P.Hq = a->Hq; P.group = a->group; P.L = a->L; P.D = a->D;
   P.n_layers = a->n_layers;
@@ -267,25 +292,57 @@ extern "C" int sah_hash_signatures(const sah_hash_sig_args* a) {
   }
   P.act = a->act;
   P.codes = a->codes; P.code_pitch = a->code_pitch; P.code_offset = a->code_offset;
+}
+
+static int sig_launch_gemv(const sah_hash_sig_args* a, const sah_hash_sig_args* b2) {
+  sig_pair PP;
+  sig_fill(a, PP.p[0]);
+  sig_fill(b2 ? b2 : a, PP.p[1]);
+  const int maxL = (b2 && b2->L > a->L) ? b2->L : a->L;
+  dim3 gg((maxL + GEMV_GV - 1) / GEMV_GV, a->B * a->Hq, b2 ? 2 : 1), gb(GEMV_NT);
   hipStream_t st = (hipStream_t)a->stream;
-  if (sig_gemv_ok(a)) {
-    dim3 gg((a->L + GEMV_GV - 1) / GEMV_GV, a->B * a->Hq), gb(GEMV_NT);
-    sah_timed timed("k_hash_sig_gemv", a->stream);
-    switch (a->dtype) {
-      case SAH_F32: hipLaunchKernelGGL(k_hash_sig_gemv<SAH_F32>, gg, gb, 0, st, P); break;
-      case SAH_BF16: hipLaunchKernelGGL(k_hash_sig_gemv<SAH_BF16>, gg, gb, 0, st, P); break;
-      case SAH_F16: hipLaunchKernelGGL(k_hash_sig_gemv<SAH_F16>, gg, gb, 0, st, P); break;
-      default: return sah_fail(SAH_EDTYPE, "sah_hash_signatures: dtype %d", a->dtype);
-    }
-    return sah_launch_status("sah_hash_signatures");
+  sah_timed timed("k_hash_sig_gemv", a->stream);
+  switch (a->dtype) {
+    case SAH_F32: hipLaunchKernelGGL(k_hash_sig_gemv<SAH_F32>, gg, gb, 0, st, PP); break;
+    case SAH_BF16: hipLaunchKernelGGL(k_hash_sig_gemv<SAH_BF16>, gg, gb, 0, st, PP); break;
+    default: hipLaunchKernelGGL(k_hash_sig_gemv<SAH_F16>, gg, gb, 0, st, PP); break;
   }
+  return sah_launch_status("sah_hash_signatures");
+}
+
+static int sig_launch_one(const sah_hash_sig_args* a) {
+  if (a->L <= 0) return SAH_OK;  // nothing to hash
+  if (sig_gemv_ok(a)) return sig_launch_gemv(a, nullptr);
+  sig_params P;
+  sig_fill(a, P);
   dim3 g((a->L + SIG_TL - 1) / SIG_TL, a->B * a->Hq), b(SIG_NT);
+  hipStream_t st = (hipStream_t)a->stream;
   sah_timed timed("k_hash_sig_tile", a->stream);
   switch (a->dtype) {
     case SAH_F32: hipLaunchKernelGGL(k_hash_sig_tile<SAH_F32>, g, b, 0, st, P); break;
     case SAH_BF16: hipLaunchKernelGGL(k_hash_sig_tile<SAH_BF16>, g, b, 0, st, P); break;
-    case SAH_F16: hipLaunchKernelGGL(k_hash_sig_tile<SAH_F16>, g, b, 0, st, P); break;
-    default: return sah_fail(SAH_EDTYPE, "sah_hash_signatures: dtype %d", a->dtype);
+    default: hipLaunchKernelGGL(k_hash_sig_tile<SAH_F16>, g, b, 0, st, P); break;
   }
   return sah_launch_status("sah_hash_signatures");
+}
+
+extern "C" int sah_hash_signatures(const sah_hash_sig_args* a) {
+  int rc = sig_validate(a);
+  if (rc) return rc;
+  return sig_launch_one(a);
+}
+
+// Two independent signature jobs (typically: the new keys of a decode step and its
+// queries) in one launch when both are small; otherwise one launch each.
+extern "C" int sah_hash_signatures_pair(const sah_hash_sig_args* a, const sah_hash_sig_args* b) {
+  int rc = sig_validate(a);
+  if (rc) return rc;
+  rc = sig_validate(b);
+  if (rc) return rc;
+  if (a->L > 0 && b->L > 0 && sig_gemv_ok(a) && sig_gemv_ok(b) && a->dtype == b->dtype && a->stream == b->stream &&
+      (int64_t)a->B * a->Hq == (int64_t)b->B * b->Hq)
+    return sig_launch_gemv(a, b);
+  rc = sig_launch_one(a);
+  if (rc) return rc;
+  return sig_launch_one(b);
 }

@@ -17,13 +17,20 @@
 #define SEL_BINS (1 << SEL_DIGIT_BITS)
 
 // ---- key sources -----------------------------------------------------------
+// A source splits "fetch" (one global load, issued in batches) from "key" (ALU only).
 struct key_src_mem16 {
+  typedef uint32_t raw_t;
   const uint16_t* keys;  // row base, indexed by candidate
-  __device__ __forceinline__ uint32_t operator()(int cand) const { return keys[cand]; }
+  __device__ __forceinline__ raw_t fetch(int cand) const { return keys[cand]; }
+  __device__ __forceinline__ uint32_t key(raw_t r) const { return r; }
+  __device__ __forceinline__ static void keep(raw_t& r) { sah_keep(r); }
 };
 struct key_src_mem32 {
+  typedef uint32_t raw_t;
   const uint32_t* keys;
-  __device__ __forceinline__ uint32_t operator()(int cand) const { return keys[cand]; }
+  __device__ __forceinline__ raw_t fetch(int cand) const { return keys[cand]; }
+  __device__ __forceinline__ uint32_t key(raw_t r) const { return r; }
+  __device__ __forceinline__ static void keep(raw_t& r) { sah_keep(r); }
 };
 // signature score of the reference, sum_e q_e k_e with q_e, k_e in {-1, 0, +1}:
 // popc(nz) - 2 popc((q ^ k) & nz), nz = bits where both are non-zero; in [-32, 32]
@@ -32,10 +39,16 @@ __device__ __forceinline__ int sig_score(uint2 q, uint2 k) {
   return __popc(nz) - 2 * __popc((q.x ^ k.x) & nz);
 }
 struct key_src_hamming {
+  typedef uint2 raw_t;
   const uint2* kcodes;  // code stream base: (positive plane, non-zero plane) per key
   uint2 qcode;
+  __device__ __forceinline__ raw_t fetch(int cand) const { return kcodes[cand]; }
   // score + 33 in [1, 65], so every real column outranks the excluded key 0
-  __device__ __forceinline__ uint32_t operator()(int cand) const { return (uint32_t)(sig_score(qcode, kcodes[cand]) + 33); }
+  __device__ __forceinline__ uint32_t key(raw_t r) const { return (uint32_t)(sig_score(qcode, r) + 33); }
+  __device__ __forceinline__ static void keep(raw_t& r) {
+    sah_keep(r.x);
+    sah_keep(r.y);
+  }
 };
 
 struct sel_shared {
@@ -49,7 +62,7 @@ struct sel_shared {
   int total_out;
 };
 
-#define SEL_LOAD_BATCH 8  // 64-column chunks requested together in the staging pass
+#define SEL_LOAD_BATCH 16  // 64-column chunks requested together in the staging pass
 
 // Dynamic LDS layout of one row: [histogram 4*nbins][bitmap row 4*n_words][staged keys].
 // The bitmap row and (when they fit) the effective keys of all candidates are staged once,
@@ -59,6 +72,18 @@ struct sel_layout {
   int hist_bins;      // bins of the widest digit
   int stage_keys;     // 1: effective keys are staged in LDS
 };
+
+// sum of one int per thread over the block; every thread gets the total
+__device__ __forceinline__ int sel_block_sum(int v, int* scratch) {
+  v = sah_wave_sum_i(v);
+  __syncthreads();
+  if ((threadIdx.x & (SAH_WAVE - 1)) == 0) scratch[threadIdx.x / SAH_WAVE] = v;
+  __syncthreads();
+  int t = 0;
+#pragma unroll
+  for (int i = 0; i < SEL_NW; ++i) t += scratch[i];
+  return t;
+}
 
 // KEYBITS: number of significant key bits (7, 16 or 32); STG: LDS type of a staged key
 template <typename SRC, int KEYBITS, typename STG>
@@ -82,18 +107,40 @@ __device__ __forceinline__ void select_row(sel_shared& S, unsigned char* dyn, se
   if (my_c1 > c_last + 1) my_c1 = c_last + 1;
   const int col_base = c_first * SAH_WAVE;  // staged[] is indexed by col - col_base
 
+  // read before any barrier: thread 0 overwrites the count at the very end
+  int cnt0 = R.cnt[r];
+  if (cnt0 > R.cap) cnt0 = R.cap;
   for (int i = tid; i < R.n_words; i += SEL_NT) s_bm[i] = bm[i];
   __syncthreads();
 
-  // effective key of a column: straight from global memory (branch-free, clamped addresses)
+  // effective key of a column: straight from global memory (clamped address)
   auto eff_key_global = [&](int col, bool& valid, bool& excl) -> uint32_t {
     const int cand = col - col_offset;
     valid = (cand >= 0 && cand < n_cand);
     const int cc = valid ? cand : 0;
     const int cl = valid ? col : col_offset;
-    const uint32_t key = src(cc);
+    const uint32_t key = src.key(src.fetch(cc));
     excl = valid && ((s_bm[cl >> 5] >> (cl & 31)) & 1u);
     return valid ? (excl ? excluded_key : key) : 0u;
+  };
+  // one batch of SEL_LOAD_BATCH chunks: every global load is issued before the first use
+  auto load_batch = [&](int c0, uint32_t (&key)[SEL_LOAD_BATCH], bool (&valid)[SEL_LOAD_BATCH]) {
+    typename SRC::raw_t raw[SEL_LOAD_BATCH];
+#pragma unroll
+    for (int u = 0; u < SEL_LOAD_BATCH; ++u) {
+      const int cand = (c0 + u) * SAH_WAVE + lane - col_offset;
+      valid[u] = (c0 + u < my_c1) && cand >= 0 && cand < n_cand;
+      raw[u] = src.fetch(valid[u] ? cand : 0);
+    }
+#pragma unroll
+    for (int u = 0; u < SEL_LOAD_BATCH; ++u) SRC::keep(raw[u]);
+#pragma unroll
+    for (int u = 0; u < SEL_LOAD_BATCH; ++u) {
+      const int col = (c0 + u) * SAH_WAVE + lane;
+      const int cl = valid[u] ? col : col_offset;
+      const bool excl = (s_bm[cl >> 5] >> (cl & 31)) & 1u;
+      key[u] = valid[u] ? (excl ? excluded_key : src.key(raw[u])) : 0u;
+    }
   };
   auto eff_key = [&](int col, bool& valid, bool& excl) -> uint32_t {
     if (!L.stage_keys) return eff_key_global(col, valid, excl);
@@ -109,6 +156,38 @@ __device__ __forceinline__ void select_row(sel_shared& S, unsigned char* dyn, se
   uint32_t prefix = 0;
   int bits_done = 0;
 
+  if (KEYBITS == 7 && L.stage_keys) {
+    // ---- byte keys staged in LDS: bisection on the threshold, no atomics ------
+    // (a 65-value histogram would serialise on a handful of LDS addresses)
+    const int n_bytes = n_chunks * SAH_WAVE;
+    for (int c0 = my_c0; c0 < my_c1; c0 += SEL_LOAD_BATCH) {
+      uint32_t key[SEL_LOAD_BATCH];
+      bool valid[SEL_LOAD_BATCH];
+      load_batch(c0, key, valid);
+#pragma unroll
+      for (int u = 0; u < SEL_LOAD_BATCH; ++u)
+        if (c0 + u < my_c1) staged[(c0 + u) * SAH_WAVE + lane - col_base] = (STG)key[u];  // 0 outside the range
+    }
+    __syncthreads();
+    const uint32_t* words = (const uint32_t*)staged;
+    const int n_w = n_bytes / 4;
+    auto count_ge = [&](uint32_t t) -> int {
+      // bytes are < 128: (b | 0x80) - t keeps bit 7 exactly when b >= t, without borrows
+      int c = 0;
+      const uint32_t tt = t * 0x01010101u;
+      for (int i = tid; i < n_w; i += SEL_NT) c += __popc(((words[i] | 0x80808080u) - tt) & 0x80808080u);
+      return sel_block_sum(c, S.scan);
+    };
+    uint32_t T7 = 0;
+    for (int bit = 6; bit >= 0; --bit) {
+      const uint32_t cand = T7 | (1u << bit);
+      if (count_ge(cand) >= k) T7 = cand;
+    }
+    const int above = (T7 >= 127u) ? 0 : count_ge(T7 + 1);
+    prefix = T7;
+    need = k - above;
+    bits_done = KEYBITS;
+  }
   // ---- radix select of the k-th largest key --------------------------------
   while (bits_done < KEYBITS) {
     int wd = KEYBITS - bits_done;
@@ -122,13 +201,7 @@ __device__ __forceinline__ void select_row(sel_shared& S, unsigned char* dyn, se
       for (int c0 = my_c0; c0 < my_c1; c0 += SEL_LOAD_BATCH) {
         uint32_t key[SEL_LOAD_BATCH];
         bool valid[SEL_LOAD_BATCH];
-#pragma unroll
-        for (int u = 0; u < SEL_LOAD_BATCH; ++u) {
-          bool excl;
-          const int col = (c0 + u) * SAH_WAVE + lane;
-          key[u] = eff_key_global(col, valid[u], excl);
-          valid[u] = valid[u] && (c0 + u < my_c1);
-        }
+        load_batch(c0, key, valid);
 #pragma unroll
         for (int u = 0; u < SEL_LOAD_BATCH; ++u) {
           if (valid[u]) {
@@ -231,8 +304,6 @@ __device__ __forceinline__ void select_row(sel_shared& S, unsigned char* dyn, se
   __syncthreads();
 
   // ---- ordered compaction ----------------------------------------------------
-  int cnt0 = R.cnt[r];
-  if (cnt0 > R.cap) cnt0 = R.cap;
   int* cols = R.cols + (int64_t)r * R.cap;
   float* w = R.w ? R.w + (int64_t)r * R.cap : nullptr;
   int out_pos = cnt0 + S.wave_out[wave];
@@ -299,6 +370,213 @@ __global__ __launch_bounds__(SEL_NT) void k_hamming_topk(sah_rows R, sel_layout 
   const int r = blockIdx.x;
   key_src_hamming src{kcodes + (int64_t)(r / lq) * pitch, qcodes[r]};
   select_row<key_src_hamming, 7, uint8_t>(S, sel_dyn, L, R, r, src, R.n_keys, 0, k, 0u);
+}
+
+// ---------------------------------------------------------------------------
+// Signature top-k, SWAR form. Scores fit a byte (score + 33 in [1, 65], 0 = column already
+// active or out of range), so a lane handles 4 consecutive columns as one 32-bit word:
+//   P0  each lane loads its 4 codes (32 B, whole wave: 2 KB contiguous), scores them, zeroes
+//       the already-active ones with a nibble of the bitmap row and parks the word in LDS;
+//   P1  bisection on the threshold T with byte-parallel compares (no atomics);
+//   P2  per-wave counts of "above T" and "equal T";
+//   P3  ordered write: wave scan of per-lane counts, up to 4 columns per lane, ties taken
+//       lowest column first until `need` are used; new bits are OR-ed into the LDS copy of
+//       the bitmap row, which is written back once at the end.
+// Active columns hold byte 0 and T >= 1 whenever k inactive columns exist, so P2/P3 never
+// look at the bitmap again.
+// ---------------------------------------------------------------------------
+#define HSW_NT 1024
+#define HSW_NW (HSW_NT / SAH_WAVE)
+#define HSW_BATCH 4  // 256-column chunks requested together in P0
+
+// per byte b < 128 of w: 0x80 if b >= t (t in [0, 128]) else 0
+__device__ __forceinline__ uint32_t swar_ge(uint32_t w, uint32_t t) {
+  return ((w | 0x80808080u) - t * 0x01010101u) & 0x80808080u;
+}
+
+__global__ __launch_bounds__(HSW_NT) void k_hamming_topk_swar(sah_rows R, const uint2* kcodes, int64_t pitch,
+                                                              const uint2* qcodes, int lq, int k) {
+  __shared__ int s_red[HSW_NW];
+  __shared__ int s_gt[HSW_NW];
+  __shared__ int s_eq[HSW_NW];
+  HIP_DYNAMIC_SHARED(unsigned char, hsw_dyn)
+  const int r = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int lane = tid & (SAH_WAVE - 1);
+  const int wave = tid / SAH_WAVE;
+  const int n = R.n_keys;
+  const int n_ch = (n + 255) / 256;            // chunks of 256 columns = 64 words
+  const int cpw = (n_ch + HSW_NW - 1) / HSW_NW;
+  const int my_c0 = wave * cpw;
+  int my_c1 = my_c0 + cpw;
+  if (my_c1 > n_ch) my_c1 = n_ch;
+  uint32_t* s_bm = (uint32_t*)hsw_dyn;                       // n_words (+ padding to a chunk)
+  uint32_t* s_key = s_bm + n_ch * 8;                         // n_ch * 64 words
+  uint32_t* bm = R.bitmap + (int64_t)r * R.n_words;
+  const uint2* kc = kcodes + (int64_t)(r / lq) * pitch;
+  const uint2 q = qcodes[r];
+  int cnt0 = R.cnt[r];
+  if (cnt0 > R.cap) cnt0 = R.cap;
+  if (k > n) k = n;
+
+  for (int i = tid; i < n_ch * 8; i += HSW_NT) s_bm[i] = i < R.n_words ? bm[i] : 0u;
+  __syncthreads();
+
+  // ---- P0: score and stage --------------------------------------------------
+  for (int c0 = my_c0; c0 < my_c1; c0 += HSW_BATCH) {
+    uint4 ra[HSW_BATCH], rb[HSW_BATCH];
+#pragma unroll
+    for (int u = 0; u < HSW_BATCH; ++u) {
+      const int j0 = ((c0 + u) * SAH_WAVE + lane) * 4;
+      // clamp to the last full group of 4 codes: out-of-range lanes re-read valid memory
+      int jl = j0;
+      if (jl + 4 > n) jl = n >= 4 ? ((n - 4) & ~1) : 0;
+      const uint4* p = (const uint4*)(kc + jl);
+      ra[u] = p[0];
+      rb[u] = p[1];
+    }
+#pragma unroll
+    for (int u = 0; u < HSW_BATCH; ++u) {
+      sah_keep(ra[u].x); sah_keep(ra[u].y); sah_keep(ra[u].z); sah_keep(ra[u].w);
+      sah_keep(rb[u].x); sah_keep(rb[u].y); sah_keep(rb[u].z); sah_keep(rb[u].w);
+    }
+#pragma unroll
+    for (int u = 0; u < HSW_BATCH; ++u) {
+      if (c0 + u >= my_c1) break;
+      const int wi = (c0 + u) * SAH_WAVE + lane;
+      const int j0 = wi * 4;
+      uint32_t word;
+      if (j0 + 4 <= n) {
+        const uint32_t s0 = (uint32_t)(sig_score(q, make_uint2(ra[u].x, ra[u].y)) + 33);
+        const uint32_t s1 = (uint32_t)(sig_score(q, make_uint2(ra[u].z, ra[u].w)) + 33);
+        const uint32_t s2 = (uint32_t)(sig_score(q, make_uint2(rb[u].x, rb[u].y)) + 33);
+        const uint32_t s3 = (uint32_t)(sig_score(q, make_uint2(rb[u].z, rb[u].w)) + 33);
+        word = s0 | (s1 << 8) | (s2 << 16) | (s3 << 24);
+      } else {
+        word = 0;  // ragged tail: the few columns of the last, partial group
+        for (int t = 0; t < 4; ++t)
+          if (j0 + t < n) word |= (uint32_t)(sig_score(q, kc[j0 + t]) + 33) << (8 * t);
+      }
+      // zero the bytes of already-active columns: nibble -> byte mask
+      const uint32_t nib = (s_bm[j0 >> 5] >> (j0 & 31)) & 0xFu;
+      const uint32_t act = ((nib * 0x00204081u) & 0x01010101u) * 0xFFu;
+      s_key[wi] = word & ~act;
+    }
+  }
+  __syncthreads();
+
+  // ---- P1: largest T with count(key >= T) >= k --------------------------------
+  const int n_w = n_ch * SAH_WAVE;
+  auto count_ge = [&](uint32_t t) -> int {
+    int c = 0;
+    for (int i = tid; i < n_w; i += HSW_NT) c += __popc(swar_ge(s_key[i], t));
+    c = sah_wave_sum_i(c);
+    __syncthreads();
+    if (lane == 0) s_red[wave] = c;
+    __syncthreads();
+    int tot = 0;
+#pragma unroll
+    for (int i = 0; i < HSW_NW; ++i) tot += s_red[i];
+    return tot;
+  };
+  uint32_t T = 0;
+  for (int bit = 6; bit >= 0; --bit) {
+    const uint32_t cand = T | (1u << bit);
+    if (count_ge(cand) >= k) T = cand;
+  }
+  const int above = count_ge(T + 1);
+  // T == 0: fewer than k inactive columns exist; take them all, byte-0 "ties" emit nothing
+  const int need = (T == 0) ? 0 : k - above;
+
+  // ---- P2: per-wave counts ---------------------------------------------------------
+  int n_gt = 0, n_eq = 0;
+  for (int c = my_c0; c < my_c1; ++c) {
+    const uint32_t w = s_key[c * SAH_WAVE + lane];
+    const uint32_t g = swar_ge(w, T + 1);
+    n_gt += __popc(g);
+    n_eq += __popc(swar_ge(w, T) & ~g);
+  }
+  n_gt = sah_wave_sum_i(n_gt);
+  n_eq = sah_wave_sum_i(n_eq);
+  if (lane == 0) {
+    s_gt[wave] = n_gt;
+    s_eq[wave] = n_eq;
+  }
+  __syncthreads();
+  int tie_base = 0, out_base = 0, total_out = 0;
+  {
+    int tie_run = 0, out_run = 0;
+#pragma unroll
+    for (int wv = 0; wv < HSW_NW; ++wv) {
+      if (wv == wave) {
+        tie_base = tie_run;
+        out_base = out_run;
+      }
+      int take = need - tie_run;
+      if (take < 0) take = 0;
+      if (take > s_eq[wv]) take = s_eq[wv];
+      out_run += s_gt[wv] + take;
+      tie_run += s_eq[wv];
+    }
+    total_out = out_run;
+  }
+
+  // ---- P3: ordered write --------------------------------------------------------------
+  int* cols = R.cols + (int64_t)r * R.cap;
+  float* wts = R.w ? R.w + (int64_t)r * R.cap : nullptr;
+  const bool ties_all = (tie_base + n_eq <= need);   // every tie of this wave is taken
+  const bool ties_none = (tie_base >= need);         // none is
+  int out_pos = cnt0 + out_base;
+  int tie_run = tie_base;
+  for (int c = my_c0; c < my_c1; ++c) {
+    const int wi = c * SAH_WAVE + lane;
+    const uint32_t w = s_key[wi];
+    const uint32_t g = swar_ge(w, T + 1) >> 7;            // bits 0, 8, 16, 24
+    uint32_t e = (swar_ge(w, T) >> 7) & ~g;
+    if (ties_none) {
+      e = 0;
+    } else if (!ties_all) {
+      const int ne = __popc(e);
+      const int before = sah_wave_incl_scan(ne) - ne;     // ties in lower lanes of this chunk
+      int allowed = need - (tie_run + before);
+      if (allowed < ne) {                                  // keep only the lowest `allowed` ties
+        uint32_t kept = 0;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const uint32_t bit = e & (1u << (8 * t));
+          if (bit && allowed > 0) {
+            kept |= bit;
+            --allowed;
+          }
+        }
+        e = kept;
+      }
+      tie_run += sah_wave_sum_i(ne);
+    }
+    const uint32_t sel = g | e;
+    const int ns = __popc(sel);
+    const int incl = sah_wave_incl_scan(ns);
+    int pos = out_pos + incl - ns;
+    if (sel) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        if (sel & (1u << (8 * t))) {
+          if (pos < R.cap) {
+            cols[pos] = wi * 4 + t;
+            if (wts) wts[pos] = 1.0f;
+          }
+          ++pos;
+        }
+      }
+      const uint32_t nib = ((sel * 0x00204081u) >> 21) & 0xFu;
+      const int j0 = wi * 4;
+      atomicOr(&s_bm[j0 >> 5], nib << (j0 & 31));
+    }
+    out_pos += __shfl(incl, SAH_WAVE - 1);
+  }
+  __syncthreads();
+  for (int i = tid; i < R.n_words; i += HSW_NT) bm[i] = s_bm[i];
+  if (tid == 0) R.cnt[r] = cnt0 + total_out;
 }
 
 // kernels may use up to 160 KB of LDS; HIP needs to be told once per kernel
@@ -390,6 +668,19 @@ extern "C" int sah_hamming_topk(const sah_hamming_topk_args* a) {
   if (a->lq <= 0 || a->rows.n_rows % a->lq) return sah_fail(SAH_EINVAL, "sah_hamming_topk: lq must divide n_rows");
   if (a->k <= 0) return sah_fail(SAH_EINVAL, "sah_hamming_topk: k must be > 0");
   if (a->code_pitch < a->rows.n_keys) return sah_fail(SAH_EINVAL, "sah_hamming_topk: code_pitch < n_keys");
+  {
+    // SWAR kernel: bitmap row + one byte per column in LDS; needs 16-byte aligned code streams
+    const int n_ch = (a->rows.n_keys + 255) / 256;
+    const size_t lds = (size_t)n_ch * 8 * 4 + (size_t)n_ch * 64 * 4;
+    if (lds <= 150 * 1024 && a->code_pitch % 2 == 0 && ((uintptr_t)a->kcodes % 16) == 0 && a->rows.n_keys >= 4) {
+      rc = sel_allow_lds(k_hamming_topk_swar, lds, "sah_hamming_topk");
+      if (rc) return rc;
+      sah_timed timed("k_hamming_topk", a->stream);
+      hipLaunchKernelGGL(k_hamming_topk_swar, dim3(a->rows.n_rows), dim3(HSW_NT), lds, (hipStream_t)a->stream, a->rows,
+                         (const uint2*)a->kcodes, a->code_pitch, (const uint2*)a->qcodes, a->lq, a->k);
+      return sah_launch_status("sah_hamming_topk");
+    }
+  }
   sel_layout L;
   const size_t lds = sel_plan(7, 1, a->rows.n_words, a->rows.n_keys, 0, &L);
   if (lds > 159 * 1024) return sah_fail(SAH_ESHAPE, "sah_hamming_topk: %d keys need %zu bytes of LDS", a->rows.n_keys, lds);

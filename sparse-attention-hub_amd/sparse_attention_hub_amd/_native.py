@@ -32,6 +32,7 @@ EXPECTED_SYMBOLS = (
     "sah_rows_from_dense",
     "sah_rows_to_dense",
     "sah_hash_signatures",
+    "sah_hash_signatures_pair",
     "sah_hamming_topk",
     "sah_hamming_scores",
     "sah_qk_scores",
@@ -303,6 +304,10 @@ def lib() -> C.CDLL:
         if name in ("sah_version", "sah_last_error", "sah_sparse_attention_work_floats",
                     "sah_timing_enable", "sah_timing_collect"):
             continue
+        if name == "sah_hash_signatures_pair":
+            getattr(handle, name).restype = C.c_int
+            getattr(handle, name).argtypes = [C.c_void_p, C.c_void_p]
+            continue
         fn = getattr(handle, name)
         fn.restype = C.c_int
         fn.argtypes = [C.c_void_p]
@@ -314,6 +319,17 @@ def call(name: str, args: C.Structure) -> None:
     """Invoke an `int sah_*(const args*)` entry point and raise on a non-zero code."""
     handle = lib()
     rc = getattr(handle, name)(C.addressof(args))
+    if rc != 0:
+        msg = handle.sah_last_error().decode("utf-8", "replace")
+        if rc in (-1, -3, -4, -5):
+            raise ValueError(f"{name}: {msg} (code {rc})")
+        raise NativeLibraryError(f"{name}: {msg} (code {rc})")
+
+
+def call2(name: str, a: C.Structure, b: C.Structure) -> None:
+    """Invoke an `int sah_*(const args*, const args*)` entry point and raise on a non-zero code."""
+    handle = lib()
+    rc = getattr(handle, name)(C.addressof(a), C.addressof(b))
     if rc != 0:
         msg = handle.sah_last_error().decode("utf-8", "replace")
         if rc in (-1, -3, -4, -5):

@@ -19,6 +19,7 @@ from ..utils.mask import Mask
 from ..utils.mask_attention_utils import get_masked_attention_output
 from ..utils.native_rows import NativeRows
 from .maskers.base import MaskerConfig, ResearchMasker
+from .maskers.fixed.implementations.basic_fixed import LocalMasker, SinkMasker, fused_sink_local
 from .maskers.sampling.base import SamplingMasker
 
 
@@ -80,7 +81,14 @@ class ResearchAttention(SparseAttention):
                 rows = NativeRows(mask_shape[0] * mask_shape[1] * mask_shape[2], mask_shape[3], planned, queries.device)
                 mask = _EmptyRowsMask(mask_shape, rows, queries.dtype)
 
-        for masker in self.maskers:
+        maskers = self.maskers
+        if (len(maskers) >= 2 and type(maskers[0]) is SinkMasker and type(maskers[1]) is LocalMasker
+                and not mask.is_full_mask()):
+            # Sink directly followed by Local on a still-empty mask: one fused launch writes both ranges
+            mask = fused_sink_local(maskers[0], maskers[1], keys, queries, mask)
+            maskers = maskers[2:]
+
+        for masker in maskers:
             mask = masker.add_mask(
                 keys=keys,
                 queries=queries,

@@ -29,7 +29,7 @@ def _launch_sink_local(rows, lq: int, sink: int, window: int, clear_future: bool
     N.call("sah_sink_local_indices", args)
     added = min(sink, rows.n_keys) + window
     # exact when the rows were empty and the two ranges cannot overlap for any query row
-    exact = fresh and (window == 0 or sink == 0 or rows.n_keys - lq - window + 1 >= sink) and not (clear_future and lq > 1)
+    exact = fresh and (window == 0 or sink == 0 or rows.n_keys - lq - window + 1 >= sink) and lq == 1
     rows.note_added(added, exact=exact)
 
 
@@ -145,3 +145,23 @@ class SinkMasker(FixedMasker):
         if not isinstance(config, SinkMaskerConfig):
             raise ValueError(f"Invalid config type: {type(config)}")
         return cls(config)
+
+
+def fused_sink_local(sink_masker: SinkMasker, local_masker: LocalMasker, keys: torch.Tensor, queries: torch.Tensor,
+                     previous_mask: Mask) -> Mask:
+    """SinkMasker.add_mask followed by LocalMasker.add_mask on an empty previous mask, as one
+    `sah_sink_local_indices` launch. Same results as the two calls, including the full-mask
+    short-circuits of either masker."""
+    if not previous_mask.is_empty_mask():
+        raise ValueError("fused_sink_local needs an empty previous mask")
+    dims = sink_masker._extract_tensor_dimensions(keys, queries)
+    sink = sink_masker._calculate_effective_sink_size(dims.seq_len_keys)
+    window = local_masker._calculate_effective_window_size(dims.seq_len_keys)
+    if sink_masker._should_use_full_attention(dims, sink) or local_masker._should_use_full_attention(dims, window):
+        return sink_masker._create_full_mask(dims, previous_mask.dtype, previous_mask.device)
+    N.require_device(keys, "keys")
+    rows = previous_mask.to_rows(extra=max(0, sink) + window)
+    if not rows.fresh:
+        raise ValueError("fused_sink_local needs uninitialised rows")
+    _launch_sink_local(rows, dims.seq_len_queries, max(0, sink), window, clear_future=True)
+    return Mask.create_mask_from_rows(sink_masker._mask_shape(dims), rows, previous_mask.dtype)

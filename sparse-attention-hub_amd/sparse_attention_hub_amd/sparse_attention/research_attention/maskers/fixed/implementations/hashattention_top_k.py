@@ -143,11 +143,9 @@ class HashAttentionTopKMasker(TopKMasker):
         self._prepared[key] = (mats, biases)
         return mats, biases
 
-    def _hash(self, x: torch.Tensor, x_heads: int, n_heads: int, first: int, count: int, layer_idx: int,
-              kind: str, codes: torch.Tensor, code_pitch: int, code_offset: int) -> None:
-        """Signatures of x[:, :, first:first+count, :] into codes[..., code_offset:]."""
-        if count <= 0:
-            return
+    def _hash_args(self, x: torch.Tensor, x_heads: int, n_heads: int, first: int, count: int, layer_idx: int,
+                   kind: str, codes: torch.Tensor, code_pitch: int, code_offset: int) -> "N.HashSigArgs":
+        """Argument block for the signatures of x[:, :, first:first+count, :] into codes[..., code_offset:]."""
         mats, biases = self._weights_for(layer_idx, kind, x.device, x.dtype)
         if mats[0].shape[0] != n_heads or mats[0].shape[1] != x.shape[-1]:
             raise ValueError(
@@ -166,10 +164,21 @@ class HashAttentionTopKMasker(TopKMasker):
             len(mats), W, Bv, dout, N.SAH_ACT[self.hat_mlp_activation],
             codes.data_ptr(), code_pitch, code_offset, N.stream_ptr(x.device),
         )
-        N.call("sah_hash_signatures", args)
+        args._keepalive = (W, Bv, dout)
+        return args
 
-    def _update_key_signatures(self, keys: torch.Tensor, n_heads: int, sparse_meta_data, layer_idx: int) -> PackedSignatureCache:
-        """Hash only the keys beyond the cached count and append them (reference :255-341)."""
+    def _hash(self, x: torch.Tensor, x_heads: int, n_heads: int, first: int, count: int, layer_idx: int,
+              kind: str, codes: torch.Tensor, code_pitch: int, code_offset: int) -> None:
+        """Signatures of x[:, :, first:first+count, :] into codes[..., code_offset:]."""
+        if count <= 0:
+            return
+        N.call("sah_hash_signatures",
+               self._hash_args(x, x_heads, n_heads, first, count, layer_idx, kind, codes, code_pitch, code_offset))
+
+    def _update_key_signatures(self, keys: torch.Tensor, n_heads: int, sparse_meta_data, layer_idx: int,
+                               pair_with=None) -> PackedSignatureCache:
+        """Hash only the keys beyond the cached count and append them (reference :255-341).
+        pair_with=(queries, qcodes): also hash the queries, in the same launch when both jobs are small."""
         cache_map = sparse_meta_data.setdefault("key", {})
         cache = cache_map.get(layer_idx)
         B, Hkv, Lk = keys.shape[0], keys.shape[1], keys.shape[2]
@@ -178,10 +187,22 @@ class HashAttentionTopKMasker(TopKMasker):
             cache_map[layer_idx] = cache
         if Lk < cache.n:
             raise ValueError(f"Current number of keys ({Lk}) is less than cached number of keys ({cache.n})")
+        qargs = None
+        if pair_with is not None:
+            q, qcodes = pair_with
+            qargs = self._hash_args(q, n_heads, n_heads, 0, q.shape[2], layer_idx, "query", qcodes, q.shape[2], 0)
         if Lk > cache.n:
             cache.reserve(Lk)
-            self._hash(keys, Hkv, n_heads, cache.n, Lk - cache.n, layer_idx, "key", cache.codes, cache.capacity, cache.n)
+            kargs = self._hash_args(keys, Hkv, n_heads, cache.n, Lk - cache.n, layer_idx, "key", cache.codes,
+                                    cache.capacity, cache.n)
+            if qargs is not None:
+                N.call2("sah_hash_signatures_pair", kargs, qargs)
+                qargs = None
+            else:
+                N.call("sah_hash_signatures", kargs)
             cache.n = Lk
+        if qargs is not None:
+            N.call("sah_hash_signatures", qargs)
         return cache
 
     # ------------------------------------------------------------------- main
@@ -204,9 +225,8 @@ class HashAttentionTopKMasker(TopKMasker):
         q = _inner_contiguous(queries)
         k = _inner_contiguous(keys)
 
-        cache = self._update_key_signatures(k, Hq, sparse_meta_data, layer_idx)
         qcodes = torch.empty((B * Hq * Lq, 2), dtype=torch.int32, device=q.device)
-        self._hash(q, Hq, Hq, 0, Lq, layer_idx, "query", qcodes, Lq, 0)
+        cache = self._update_key_signatures(k, Hq, sparse_meta_data, layer_idx, pair_with=(q, qcodes))
 
         rows = previous_mask.to_rows(extra=k_eff)
         rows.zero_if_fresh()
