@@ -375,6 +375,30 @@ typedef struct sah_attention_weights_args {
 } sah_attention_weights_args;
 int sah_attention_weights(const sah_attention_weights_args* a);
 
+/* ---------------------------------------------------------------------------
+ * One decode layer-step as a single call: runs, in this order and on the stream
+ * each block names, every stage whose pointer is not NULL -
+ *   sink_local -> (sig_a, sig_b as sah_hash_signatures_pair) -> hamming
+ *   -> qk -> pq_assign -> pq_adc -> select -> attention.
+ * The blocks are the argument structures of the entry points above, unchanged;
+ * a caller keeps them alive between steps and only patches the fields that move
+ * (tensor pointers, key count). Replaces the per-masker Python dispatch of
+ * ResearchAttention.custom_attention (research_attention/base.py:108-148) on the
+ * decode path; stops at the first stage that fails and returns its code.
+ * ------------------------------------------------------------------------- */
+typedef struct sah_chain_args {
+  const sah_sink_local_args* sink_local;
+  const sah_hash_sig_args* sig_a;
+  const sah_hash_sig_args* sig_b;
+  const sah_hamming_topk_args* hamming;
+  const sah_qk_scores_args* qk;
+  const sah_pq_assign_args* pq_assign;
+  const sah_pq_adc_args* pq_adc;
+  const sah_select_topk_args* select;
+  const sah_attention_args* attention;
+} sah_chain_args;
+int sah_run_chain(const sah_chain_args* a);
+
 #ifdef __cplusplus
 }
 #endif

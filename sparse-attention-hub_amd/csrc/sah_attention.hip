@@ -448,3 +448,23 @@ extern "C" int sah_attention_weights(const sah_attention_weights_args* a) {
   }
   return sah_launch_status("sah_attention_weights");
 }
+
+extern "C" int sah_run_chain(const sah_chain_args* a) {
+  if (!a) return sah_fail(SAH_ENULL, "sah_run_chain: args is NULL");
+  int rc = SAH_OK;
+  if (a->sink_local && (rc = sah_sink_local_indices(a->sink_local))) return rc;
+  if (a->sig_a && a->sig_b) {
+    if ((rc = sah_hash_signatures_pair(a->sig_a, a->sig_b))) return rc;
+  } else if (a->sig_a) {
+    if ((rc = sah_hash_signatures(a->sig_a))) return rc;
+  } else if (a->sig_b) {
+    if ((rc = sah_hash_signatures(a->sig_b))) return rc;
+  }
+  if (a->hamming && (rc = sah_hamming_topk(a->hamming))) return rc;
+  if (a->qk && (rc = sah_qk_scores(a->qk))) return rc;
+  if (a->pq_assign && (rc = sah_pq_kmeans_assign(a->pq_assign))) return rc;
+  if (a->pq_adc && (rc = sah_pq_adc_scores(a->pq_adc))) return rc;
+  if (a->select && (rc = sah_select_topk(a->select))) return rc;
+  if (a->attention && (rc = sah_sparse_attention(a->attention))) return rc;
+  return SAH_OK;
+}

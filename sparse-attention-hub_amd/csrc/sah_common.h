@@ -191,26 +191,31 @@ __device__ __forceinline__ float sah_wave_max(float v) {
   return v;
 }
 
-__device__ __forceinline__ int sah_wave_sum_i(int v) {
-#pragma unroll
-  for (int o = 1; o < SAH_WAVE; o <<= 1) v += __shfl_xor(v, o);
+template <int CTRL, int ROW_MASK, bool BOUND>
+__device__ __forceinline__ int sah_dpp_i(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, CTRL, ROW_MASK, 0xF, BOUND);
+}
+
+// inclusive scan of one int per lane across the wave, all in DPP (no LDS traffic):
+// Hillis-Steele inside each row of 16 lanes, then the row totals are carried across rows
+__device__ __forceinline__ int sah_wave_incl_scan(int v) {
+  v += sah_dpp_i<0x111, 0xF, true>(v);   // row_shr:1, lanes without a source add 0
+  v += sah_dpp_i<0x112, 0xF, true>(v);   // row_shr:2
+  v += sah_dpp_i<0x114, 0xF, true>(v);   // row_shr:4
+  v += sah_dpp_i<0x118, 0xF, true>(v);   // row_shr:8
+  v += sah_dpp_i<0x142, 0xA, false>(v);  // row_bcast:15 into rows 1 and 3
+  v += sah_dpp_i<0x143, 0xC, false>(v);  // row_bcast:31 into rows 2 and 3
   return v;
+}
+
+// sum over the wave; every lane gets it
+__device__ __forceinline__ int sah_wave_sum_i(int v) {
+  return __builtin_amdgcn_readlane(sah_wave_incl_scan(v), SAH_WAVE - 1);
 }
 
 // number of set bits of `m` at lane positions below the calling lane
 __device__ __forceinline__ int sah_lane_prefix(uint64_t m) {
   return __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0));
-}
-
-// inclusive scan of one int per lane across the wave
-__device__ __forceinline__ int sah_wave_incl_scan(int v) {
-  const int lane = threadIdx.x & (SAH_WAVE - 1);
-#pragma unroll
-  for (int o = 1; o < SAH_WAVE; o <<= 1) {
-    int t = __shfl_up(v, o);
-    if (lane >= o) v += t;
-  }
-  return v;
 }
 
 // Exclusive scan of one int per thread across a block of NT threads

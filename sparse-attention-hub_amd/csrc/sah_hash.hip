@@ -34,6 +34,39 @@ __device__ __forceinline__ float sig_act(int act, float v) {
   }
 }
 
+// 8 weights of one row as loaded: 16 B for 2-byte types, 32 B for fp32
+template <int DT>
+struct att_raw_w {
+  uint4 lo;
+  uint4 hi;
+  __device__ __forceinline__ void load(const char* p) {
+    lo = *(const uint4*)p;
+    if (DT == SAH_F32) hi = *(const uint4*)(p + 16);
+  }
+  __device__ __forceinline__ void unpack(float (&o)[8]) const {
+    const uint32_t w[4] = {lo.x, lo.y, lo.z, lo.w};
+    if (DT == SAH_F32) {
+      const uint32_t v[4] = {hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        o[t] = sah_bits_to_float(w[t]);
+        o[4 + t] = sah_bits_to_float(v[t]);
+      }
+    } else {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        if (DT == SAH_BF16) {
+          o[2 * t] = sah_bits_to_float(w[t] << 16);
+          o[2 * t + 1] = sah_bits_to_float(w[t] & 0xffff0000u);
+        } else {
+          o[2 * t] = sah_f16_to_float((uint16_t)(w[t] & 0xffffu));
+          o[2 * t + 1] = sah_f16_to_float((uint16_t)(w[t] >> 16));
+        }
+      }
+    }
+  }
+};
+
 template <int DT>
 __global__ __launch_bounds__(SIG_NT) void k_hash_sig_tile(sig_params P) {
   __shared__ float s_a[SIG_TL][SIG_MAXD];
@@ -113,7 +146,8 @@ __global__ __launch_bounds__(SIG_NT) void k_hash_sig_tile(sig_params P) {
 // d_out, row-major) is read once with 16-byte loads: thread t owns 8 adjacent
 // output columns (cg = t % CG) of the rows d = rg, rg + RG, ... (rg = t / CG), all
 // of its row loads are in flight together, and the RG partial sums are reduced by
-// wave shuffles and one pass through LDS. Three layers = three memory round trips.
+// wave shuffles and one pass through LDS. With 2-byte weights every layer is requested
+// up-front (the weights do not depend on the activations): one memory round trip in all.
 // Needs every layer width to be a power of two in [8, 256] and D % 8 == 0.
 // ---------------------------------------------------------------------------
 #define GEMV_NT 256
@@ -125,37 +159,37 @@ struct sig_pair {
   sig_params p[2];
 };
 
-// acc[t][e] += sum over this thread's NR rows of x[t][d] * W[d][8 columns]; the NR row
-// loads (16 or 32 bytes each) are all in flight before the first multiply
-template <int DT, int NR>
-__device__ __forceinline__ void gemv_rows(const char* wbase, int dout, int rg, int RG, const float (*s_x)[SIG_MAXD],
-                                          float (&acc)[GEMV_GV][8]) {
-  float wv[NR][8];
+#define GEMV_ROWS 8  // row slots per thread and layer (d_in * d_out / 8 / GEMV_NT <= 8)
+
+// One layer: acc[t][e] = sum over this thread's row slots of x[t][d] * W[d][8 columns].
+// Slots beyond the thread's real row count hold a clamped (valid) row and get weight 0.
+template <int DT, int GV>
+__device__ __forceinline__ void gemv_layer_fma(const att_raw_w<DT> (&raw)[GEMV_ROWS], int nrow, int rg, int RG,
+                                               const float (*s_x)[SIG_MAXD], float (&acc)[GV][8]) {
 #pragma unroll
-  for (int i = 0; i < NR; ++i) sah_load8<DT>(wbase, (int64_t)(rg + i * RG) * dout, wv[i]);
+  for (int i = 0; i < GEMV_ROWS; ++i) {
+    float wv[8];
+    raw[i].unpack(wv);
+    const int d = rg + (i < nrow ? i : 0) * RG;
 #pragma unroll
-  for (int i = 0; i < NR; ++i)
+    for (int t = 0; t < GV; ++t) {
+      const float xv = (i < nrow) ? s_x[t][d] : 0.f;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) sah_keep(wv[i][e]);
-#pragma unroll
-  for (int i = 0; i < NR; ++i) {
-    const int d = rg + i * RG;
-#pragma unroll
-    for (int t = 0; t < GEMV_GV; ++t) {
-      const float xv = s_x[t][d];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) acc[t][e] = fmaf(xv, wv[i][e], acc[t][e]);
+      for (int e = 0; e < 8; ++e) acc[t][e] = fmaf(xv, wv[e], acc[t][e]);
     }
   }
 }
 
-template <int DT>
+template <int DT, int GV>
 __global__ __launch_bounds__(GEMV_NT) void k_hash_sig_gemv(sig_pair PP) {
   const sig_params& P = PP.p[blockIdx.z];
-  if ((int)blockIdx.x * GEMV_GV >= P.L) return;  // the two jobs may differ in vector count
-  __shared__ float s_x[GEMV_GV][SIG_MAXD];
-  __shared__ float s_part[GEMV_NW][GEMV_GV][SIG_MAXD];
-  __shared__ float s_bias[SIG_MAXD];
+  if ((int)blockIdx.x * GV >= P.L) return;  // the two jobs may differ in vector count
+  __shared__ float s_x[GV][SIG_MAXD];
+  __shared__ float s_part[GEMV_NW][GV][SIG_MAXD];
+  __shared__ float s_bias[SAH_MAX_MLP_LAYERS][SIG_MAXD];
+  constexpr int ES = (DT == SAH_F32) ? 4 : 2;
+  // fp32 weights are 32 B per row slot: prefetching every layer would not fit the registers
+  constexpr int PF = (DT == SAH_F32) ? 1 : SAH_MAX_MLP_LAYERS;
   const int tid = threadIdx.x;
   const int lane = tid & (SAH_WAVE - 1);
   const int wave = tid / SAH_WAVE;
@@ -163,11 +197,38 @@ __global__ __launch_bounds__(GEMV_NT) void k_hash_sig_gemv(sig_pair PP) {
   const int h = bh % P.Hq;
   const int b = bh / P.Hq;
   const int hx = h / P.group;
-  const int l0 = blockIdx.x * GEMV_GV;
+  const int l0 = blockIdx.x * GV;
   int nl = P.L - l0;
-  if (nl > GEMV_GV) nl = GEMV_GV;
+  if (nl > GV) nl = GV;
 
-  for (int i = tid; i < GEMV_GV * P.D; i += GEMV_NT) {
+  // The weights do not depend on the activations: request every layer's rows (and biases)
+  // now, so the three layers cost one memory round trip instead of three.
+  att_raw_w<DT> raw[PF][GEMV_ROWS];
+  auto fetch_layer = [&](int layer, int din, att_raw_w<DT> (&dst)[GEMV_ROWS]) {
+    const int dout = P.d_out[layer];
+    const int CG = dout / 8, RG = GEMV_NT / CG;
+    const int cg = tid % CG, rg = tid / CG;
+    const int nrow = din / RG;
+    const char* wbase = (const char*)P.W[layer] + ((int64_t)h * din * dout + cg * 8) * ES;
+#pragma unroll
+    for (int i = 0; i < GEMV_ROWS; ++i) {
+      const int d = rg + (i < nrow ? i : 0) * RG;
+      dst[i].load(wbase + (int64_t)d * dout * ES);
+    }
+    if (tid < dout) s_bias[layer][tid] = sah_load<DT>(P.bias[layer], (int64_t)h * dout + tid);
+  };
+  if (PF > 1) {
+    int din0 = P.D;
+#pragma unroll
+    for (int layer = 0; layer < PF; ++layer) {
+      if (layer < P.n_layers) {
+        fetch_layer(layer, din0, raw[layer]);
+        din0 = P.d_out[layer];
+      }
+    }
+  }
+
+  for (int i = tid; i < GV * P.D; i += GEMV_NT) {
     const int t = i / P.D, d = i % P.D;
     float v = 0.f;
     if (t < nl) v = sah_load<DT>(P.x, (int64_t)b * P.xs_b + (int64_t)hx * P.xs_h + (int64_t)(l0 + t) * P.xs_l + d);
@@ -176,51 +237,48 @@ __global__ __launch_bounds__(GEMV_NT) void k_hash_sig_gemv(sig_pair PP) {
   __syncthreads();
 
   int din = P.D;
-  for (int layer = 0; layer < P.n_layers; ++layer) {
+#pragma unroll
+  for (int layer = 0; layer < SAH_MAX_MLP_LAYERS; ++layer) {
+    if (layer >= P.n_layers) break;
     const int dout = P.d_out[layer];
     const bool last = (layer == P.n_layers - 1);
     const int CG = dout / 8;            // column groups (power of two, <= 32)
     const int RG = GEMV_NT / CG;        // row groups
     const int cg = tid % CG, rg = tid / CG;
-    const char* wbase = (const char*)P.W[layer] + ((int64_t)h * din * dout + cg * 8) * (DT == SAH_F32 ? 4 : 2);
-    float acc[GEMV_GV][8];
+    const int nrow = din / RG;          // real rows of this thread: 1, 2, 4 or 8
+    float acc[GV][8];
 #pragma unroll
-    for (int t = 0; t < GEMV_GV; ++t)
+    for (int t = 0; t < GV; ++t)
 #pragma unroll
       for (int e = 0; e < 8; ++e) acc[t][e] = 0.f;
-    // the bias is requested with the weights so its latency hides behind theirs
-    float bias_v = 0.f;
-    if (tid < dout) bias_v = sah_load<DT>(P.bias[layer], (int64_t)h * dout + tid);
-    const int nrow = din / RG;  // rows per thread: 1, 2, 4 or 8 (checked on the host)
-    switch (nrow) {
-      case 1: gemv_rows<DT, 1>(wbase, dout, rg, RG, s_x, acc); break;
-      case 2: gemv_rows<DT, 2>(wbase, dout, rg, RG, s_x, acc); break;
-      case 4: gemv_rows<DT, 4>(wbase, dout, rg, RG, s_x, acc); break;
-      default: gemv_rows<DT, 8>(wbase, dout, rg, RG, s_x, acc); break;
+    if (PF > 1) {
+      gemv_layer_fma<DT, GV>(raw[layer < PF ? layer : 0], nrow, rg, RG, s_x, acc);
+    } else {
+      fetch_layer(layer, din, raw[0]);
+      gemv_layer_fma<DT, GV>(raw[0], nrow, rg, RG, s_x, acc);
     }
     // lanes of a wave that share cg differ by multiples of CG
     for (int o = CG; o < SAH_WAVE; o <<= 1) {
 #pragma unroll
-      for (int t = 0; t < GEMV_GV; ++t)
+      for (int t = 0; t < GV; ++t)
 #pragma unroll
         for (int e = 0; e < 8; ++e) acc[t][e] += __shfl_xor(acc[t][e], o);
     }
     if (lane < CG) {
 #pragma unroll
-      for (int t = 0; t < GEMV_GV; ++t)
+      for (int t = 0; t < GV; ++t)
 #pragma unroll
         for (int e = 0; e < 8; ++e) s_part[wave][t][cg * 8 + e] = acc[t][e];
     }
-    if (tid < dout) s_bias[tid] = bias_v;
     __syncthreads();
-    // CG > 64 cannot happen (dout <= 256 => CG <= 32), so every wave holds all column groups
-    for (int i = tid; i < GEMV_GV * dout; i += GEMV_NT) {
+    // dout <= 256 => CG <= 32 < 64, so every wave holds all column groups
+    for (int i = tid; i < GV * dout; i += GEMV_NT) {
       const int t = i / dout, e = i % dout;
       float y = 0.f;
 #pragma unroll
       for (int wv2 = 0; wv2 < GEMV_NW; ++wv2) y += s_part[wv2][t][e];
       y = sah_round<DT>(y);
-      y = sah_round<DT>(y + s_bias[e]);
+      y = sah_round<DT>(y + s_bias[layer][e]);
       if (!last) y = sah_round<DT>(sig_act(P.act, y));
       s_x[t][e] = y;
     }
@@ -299,13 +357,23 @@ static int sig_launch_gemv(const sah_hash_sig_args* a, const sah_hash_sig_args* 
   sig_fill(a, PP.p[0]);
   sig_fill(b2 ? b2 : a, PP.p[1]);
   const int maxL = (b2 && b2->L > a->L) ? b2->L : a->L;
-  dim3 gg((maxL + GEMV_GV - 1) / GEMV_GV, a->B * a->Hq, b2 ? 2 : 1), gb(GEMV_NT);
   hipStream_t st = (hipStream_t)a->stream;
   sah_timed timed("k_hash_sig_gemv", a->stream);
-  switch (a->dtype) {
-    case SAH_F32: hipLaunchKernelGGL(k_hash_sig_gemv<SAH_F32>, gg, gb, 0, st, PP); break;
-    case SAH_BF16: hipLaunchKernelGGL(k_hash_sig_gemv<SAH_BF16>, gg, gb, 0, st, PP); break;
-    default: hipLaunchKernelGGL(k_hash_sig_gemv<SAH_F16>, gg, gb, 0, st, PP); break;
+  dim3 gb(GEMV_NT);
+  if (maxL == 1) {  // decode: one vector per head and job
+    dim3 gg(1, a->B * a->Hq, b2 ? 2 : 1);
+    switch (a->dtype) {
+      case SAH_F32: hipLaunchKernelGGL((k_hash_sig_gemv<SAH_F32, 1>), gg, gb, 0, st, PP); break;
+      case SAH_BF16: hipLaunchKernelGGL((k_hash_sig_gemv<SAH_BF16, 1>), gg, gb, 0, st, PP); break;
+      default: hipLaunchKernelGGL((k_hash_sig_gemv<SAH_F16, 1>), gg, gb, 0, st, PP); break;
+    }
+  } else {
+    dim3 gg((maxL + GEMV_GV - 1) / GEMV_GV, a->B * a->Hq, b2 ? 2 : 1);
+    switch (a->dtype) {
+      case SAH_F32: hipLaunchKernelGGL((k_hash_sig_gemv<SAH_F32, GEMV_GV>), gg, gb, 0, st, PP); break;
+      case SAH_BF16: hipLaunchKernelGGL((k_hash_sig_gemv<SAH_BF16, GEMV_GV>), gg, gb, 0, st, PP); break;
+      default: hipLaunchKernelGGL((k_hash_sig_gemv<SAH_F16, GEMV_GV>), gg, gb, 0, st, PP); break;
+    }
   }
   return sah_launch_status("sah_hash_signatures");
 }

@@ -43,6 +43,7 @@ EXPECTED_SYMBOLS = (
     "sah_sparse_attention_work_floats",
     "sah_sparse_attention",
     "sah_attention_weights",
+    "sah_run_chain",
 )
 
 
@@ -251,6 +252,20 @@ class AttentionArgs(C.Structure):
         ("logits_out", C.c_void_p),
         ("stats_out", C.c_void_p),
         ("stream", C.c_void_p),
+    ]
+
+
+class ChainArgs(C.Structure):
+    _fields_ = [
+        ("sink_local", C.c_void_p),
+        ("sig_a", C.c_void_p),
+        ("sig_b", C.c_void_p),
+        ("hamming", C.c_void_p),
+        ("qk", C.c_void_p),
+        ("pq_assign", C.c_void_p),
+        ("pq_adc", C.c_void_p),
+        ("select", C.c_void_p),
+        ("attention", C.c_void_p),
     ]
 
 

@@ -14,10 +14,12 @@ from typing import Any, Dict, List, Optional, Tuple
 import torch
 from torch import nn
 
+from ... import _native
 from ..base import SparseAttention, SparseAttentionConfig
 from ..utils.mask import Mask
 from ..utils.mask_attention_utils import get_masked_attention_output
 from ..utils.native_rows import NativeRows
+from .decode_plan import DecodePlan, plan_kind
 from .maskers.base import MaskerConfig, ResearchMasker
 from .maskers.fixed.implementations.basic_fixed import LocalMasker, SinkMasker, fused_sink_local
 from .maskers.sampling.base import SamplingMasker
@@ -44,6 +46,8 @@ class ResearchAttention(SparseAttention):
                 "Only one sampling masker supported for efficiency; consider implementing all sampling logic in one masker"
             )
         self.maskers = maskers
+        self._plan_kind = plan_kind(maskers)
+        self._plans: Dict[Any, DecodePlan] = {}
 
     def _planned_capacity(self, dims) -> Optional[int]:
         """Entries per row the whole chain can add, if every masker can tell without the device."""
@@ -70,6 +74,19 @@ class ResearchAttention(SparseAttention):
         if "sparse_meta_data" not in kwargs:
             raise ValueError("sparse_meta_data must be provided in kwargs while calling custom_attention()")
         sparse_meta_data: Dict[Any, Any] = kwargs.pop("sparse_meta_data")
+
+        if (not self.return_attention_weights and attention_mask is None and self._plan_kind is not None
+                and not isinstance(kwargs.get("s_aux"), torch.Tensor) and queries.dim() == 4
+                and (queries.is_cuda or not _native.REQUIRE_DEVICE_TENSORS)
+                and not (dropout > 0.0 and module is not None and getattr(module, "training", False))):
+            # decode fast path: the whole chain as one native call over cached argument blocks
+            key = (queries.device, queries.dtype, tuple(queries.shape), keys.shape[1])
+            plan = self._plans.get(key)
+            if plan is None:
+                plan = self._plans[key] = DecodePlan(self.maskers, self._plan_kind, queries, keys)
+            out = plan.run(queries, keys, values, scaling, sparse_meta_data, kwargs.get("layer_idx"))
+            if out is not None:
+                return out, None
 
         mask_shape = (queries.shape[0], queries.shape[1], queries.shape[2], keys.shape[2])
         mask = Mask.create_empty_mask(mask_shape, dtype=queries.dtype, device=queries.device)

@@ -1,0 +1,251 @@
+"""Cached launch plan for the common decode chains.
+
+`ResearchAttention.custom_attention` (reference: research_attention/base.py:63-170) walks
+its maskers in Python and then calls the masked attention. For the chains every decode
+benchmark of this path uses —
+
+    Sink, Local [, HashAttentionTopK | OracleTopK | PQCache]      (no additive mask, no sink
+                                                                    logits, weights not requested)
+
+— the same kernels can be driven from argument blocks that are built once and patched per
+step (tensor pointers, key count), then handed to `sah_run_chain` in ONE native call. The
+results are those of the masker-by-masker path (same kernels, same order); what goes away
+is the per-step Python: Mask objects, row-buffer allocation, five ctypes dispatches.
+
+Anything the plan does not cover (first call of a layer that has to hash every key or run
+k-means, a full-mask short-circuit, an additive attention mask, ...) returns None and the
+caller takes the general path.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Any, Dict, Optional, Tuple
+
+import torch
+
+from ... import _native as N
+from ..utils.mask_attention_utils import _workspace, unit_inverse_weight
+from .maskers.fixed.base import sortable_key_of
+from .maskers.fixed.implementations.basic_fixed import LocalMasker, SinkMasker
+from .maskers.fixed.implementations.hashattention_top_k import HashAttentionTopKMasker, PackedSignatureCache
+from .maskers.fixed.implementations.oracle_top_k import OracleTopK
+from .maskers.fixed.implementations.pq_top_k import PQCache, PQCodebook
+
+_MAX_NEW_KEYS = 64  # more than this many unseen keys => not a decode step, take the general path
+
+
+def plan_kind(maskers) -> Optional[str]:
+    """'fixed' | 'hash' | 'oracle' | 'pq' if the masker list is a chain the plan covers."""
+    if len(maskers) < 2 or type(maskers[0]) is not SinkMasker or type(maskers[1]) is not LocalMasker:
+        return None
+    if len(maskers) == 2:
+        return "fixed"
+    if len(maskers) == 3:
+        t = type(maskers[2])
+        if t is HashAttentionTopKMasker:
+            return "hash"
+        if t is OracleTopK:
+            return "oracle"
+        if t is PQCache:
+            return "pq"
+    return None
+
+
+class _LayerBlocks:
+    """Per-layer argument blocks (signature weights differ per layer)."""
+
+    __slots__ = ("sig_a", "sig_b", "weights_key")
+
+    def __init__(self):
+        self.sig_a = None
+        self.sig_b = None
+        self.weights_key = None
+
+
+class DecodePlan:
+    def __init__(self, maskers, kind: str, q: torch.Tensor, k: torch.Tensor):
+        self.kind = kind
+        self.sink_masker, self.local_masker = maskers[0], maskers[1]
+        self.top = maskers[2] if len(maskers) == 3 else None
+        self.device = q.device
+        self.dtype = q.dtype
+        self.dt = N.dtype_code(q.dtype)
+        self.B, self.Hq, self.Lq, self.D = q.shape
+        self.Hkv = k.shape[1]
+        self.n_rows = self.B * self.Hq * self.Lq
+        self.es = q.element_size()
+        self.key_bits = 32 if q.dtype == torch.float32 else 16
+        self.cap = 0
+        self.words_alloc = 0
+        self.cols = self.cnt = self.bitmap = None
+        self.qcodes = None
+        self.keybuf = None
+        self.keybuf_pitch = 0
+        self.layers: Dict[int, _LayerBlocks] = {}
+        self.sink_local = N.SinkLocalArgs()
+        self.hamming = N.HammingTopkArgs()
+        self.qk = N.QkScoresArgs()
+        self.pq_assign = N.PqAssignArgs()
+        self.pq_adc = N.PqAdcArgs()
+        self.select = N.SelectTopkArgs()
+        self.att = N.AttentionArgs()
+        self.chain = N.ChainArgs()
+        self.unit = unit_inverse_weight(q.dtype)
+        self._excluded_min = sortable_key_of(torch.finfo(q.dtype).min, q.dtype)
+
+    def signature(self, q: torch.Tensor, k: torch.Tensor) -> Tuple:
+        return (q.device, q.dtype, tuple(q.shape), k.shape[1])
+
+    # ------------------------------------------------------------------ buffers
+    def _ensure_rows(self, cap: int, n_keys: int) -> None:
+        words = (n_keys + 31) // 32
+        if cap > self.cap or self.cols is None:
+            self.cap = cap + 64
+            self.cols = torch.empty((self.n_rows, self.cap), dtype=torch.int32, device=self.device)
+            self.cnt = torch.empty((self.n_rows,), dtype=torch.int32, device=self.device)
+        if words > self.words_alloc or self.bitmap is None:
+            self.words_alloc = words + 256
+            self.bitmap = torch.empty((self.n_rows * self.words_alloc,), dtype=torch.int32, device=self.device)
+
+    def _rows_struct(self, n_keys: int) -> N.Rows:
+        return N.Rows(self.cols.data_ptr(), self.cnt.data_ptr(), None, self.bitmap.data_ptr(), self.n_rows, self.cap,
+                      n_keys, (n_keys + 31) // 32)
+
+    def _ensure_keybuf(self, n_cols: int) -> None:
+        if self.keybuf is None or n_cols > self.keybuf_pitch:
+            self.keybuf_pitch = (n_cols + 4096 + 63) // 64 * 64
+            kdt = torch.int32 if self.dtype == torch.float32 else torch.int16
+            self.keybuf = torch.empty((self.n_rows, self.keybuf_pitch), dtype=kdt, device=self.device)
+
+    # --------------------------------------------------------------------- run
+    def run(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scaling: float,
+            sparse_meta_data: Dict[Any, Any], layer_idx: Optional[int]) -> Optional[torch.Tensor]:
+        """One layer-step; returns the attention output (B, Lq, Hq, D) or None if not applicable."""
+        Lk = k.shape[2]
+        Lq = self.Lq
+        sink = self.sink_masker._calculate_effective_sink_size(Lk)
+        window = self.local_masker._calculate_effective_window_size(Lk)
+        if sink <= 0 or window <= 0 or Lk <= sink or Lk <= window + Lq:
+            return None
+        k_eff = 0
+        top = self.top
+        if top is not None:
+            if layer_idx is None and self.kind in ("hash", "pq"):
+                return None  # the general path raises the reference's ValueError
+            k_eff = top._calculate_effective_size(top.heavy_size, Lk)
+            if k_eff <= 0 or Lk <= k_eff:
+                return None
+        if q.stride(3) != 1 or k.stride(3) != 1 or v.stride(3) != 1 or v.shape[2] != Lk:
+            return None
+        stream = N.stream_ptr(self.device)
+        cap = sink + window + k_eff
+        self._ensure_rows(cap, Lk)
+        rows = self._rows_struct(Lk)
+        chain = self.chain
+        es = self.es
+
+        sl = self.sink_local
+        sl.rows, sl.lq, sl.sink, sl.window, sl.fresh, sl.clear_future, sl.stream = rows, Lq, sink, window, 1, 1, stream
+        chain.sink_local = C.addressof(sl)
+        chain.sig_a = chain.sig_b = chain.hamming = chain.qk = chain.pq_assign = chain.pq_adc = chain.select = None
+
+        if self.kind == "hash":
+            cache = sparse_meta_data.get("key", {}).get(layer_idx)
+            if not isinstance(cache, PackedSignatureCache) or Lk < cache.n or Lk - cache.n > _MAX_NEW_KEYS:
+                return None
+            if cache.codes.shape[0] != self.B or cache.codes.shape[1] != self.Hq:
+                return None
+            blocks = self.layers.get(layer_idx)
+            wkey = (id(top.hat_weights), layer_idx)
+            if blocks is None or blocks.weights_key != wkey:
+                blocks = _LayerBlocks()
+                blocks.weights_key = wkey
+                blocks.sig_a = top._hash_args(k, self.Hkv, self.Hq, 0, 1, layer_idx, "key", cache.codes, cache.capacity, 0)
+                if self.qcodes is None:
+                    self.qcodes = torch.empty((self.n_rows, 2), dtype=torch.int32, device=self.device)
+                blocks.sig_b = top._hash_args(q, self.Hq, self.Hq, 0, Lq, layer_idx, "query", self.qcodes, Lq, 0)
+                self.layers[layer_idx] = blocks
+            n_new = Lk - cache.n
+            cache.reserve(Lk)
+            if n_new > 0:
+                a = blocks.sig_a
+                a.x = k.data_ptr() + cache.n * k.stride(2) * es
+                a.xs_b, a.xs_h, a.xs_l = k.stride(0), k.stride(1), k.stride(2)
+                a.L = n_new
+                a.codes, a.code_pitch, a.code_offset, a.stream = cache.codes.data_ptr(), cache.capacity, cache.n, stream
+                chain.sig_a = C.addressof(a)
+            bq = blocks.sig_b
+            bq.x = q.data_ptr()
+            bq.xs_b, bq.xs_h, bq.xs_l, bq.stream = q.stride(0), q.stride(1), q.stride(2), stream
+            chain.sig_b = C.addressof(bq)
+            hm = self.hamming
+            hm.rows, hm.kcodes, hm.code_pitch = rows, cache.codes.data_ptr(), cache.capacity
+            hm.qcodes, hm.lq, hm.k, hm.stream = self.qcodes.data_ptr(), Lq, k_eff, stream
+            chain.hamming = C.addressof(hm)
+            cache.n = Lk
+        elif self.kind == "oracle":
+            self._ensure_keybuf(Lk)
+            qa = self.qk
+            qa.q, qa.qs_b, qa.qs_h, qa.qs_l = q.data_ptr(), q.stride(0), q.stride(1), q.stride(2)
+            qa.k, qa.ks_b, qa.ks_h, qa.ks_l = k.data_ptr(), k.stride(0), k.stride(1), k.stride(2)
+            qa.amask = None
+            qa.dtype, qa.B, qa.Hq, qa.Hkv, qa.Lq, qa.Lk, qa.D = self.dt, self.B, self.Hq, self.Hkv, Lq, Lk, self.D
+            qa.keys_out, qa.key_pitch, qa.stream = self.keybuf.data_ptr(), self.keybuf_pitch, stream
+            chain.qk = C.addressof(qa)
+            se = self.select
+            se.rows, se.keys, se.key_pitch, se.key_bits = rows, self.keybuf.data_ptr(), self.keybuf_pitch, self.key_bits
+            se.n_cand, se.col_offset, se.k, se.excluded_key, se.stream = Lk, 0, k_eff, self._excluded_min, stream
+            chain.select = C.addressof(se)
+        elif self.kind == "pq":
+            off = top.init_offset
+            if Lk <= k_eff + off + Lq + 2 ** top.pq_bits:
+                return None
+            book = sparse_meta_data.get("pq_codebook", {}).get(layer_idx)
+            cf32 = sparse_meta_data.get("pq_centroids_f32", {}).get(layer_idx)
+            if not isinstance(book, PQCodebook) or cf32 is None:
+                return None
+            current = Lk - off
+            if current < book.n or current - book.n > _MAX_NEW_KEYS or book.codes.shape[0] != self.B:
+                return None
+            n_sub, d_sub, n_cent = top._geometry(k)
+            book.reserve(current)
+            if current > book.n:
+                pa = self.pq_assign
+                pa.k, pa.ks_b, pa.ks_h, pa.ks_l = k.data_ptr(), k.stride(0), k.stride(1), k.stride(2)
+                pa.dtype, pa.B, pa.Hkv, pa.n_sub, pa.d_sub, pa.n_cent = self.dt, self.B, self.Hkv, n_sub, d_sub, n_cent
+                pa.key_offset, pa.n_keys = off + book.n, current - book.n
+                pa.centres, pa.codes, pa.code_pitch, pa.code_offset = cf32.data_ptr(), book.codes.data_ptr(), book.capacity, book.n
+                pa.sums = pa.counts = pa.skip_flag = None
+                pa.round_dist, pa.stream = 1, stream
+                chain.pq_assign = C.addressof(pa)
+                book.n = current
+            self._ensure_keybuf(current)
+            ad = self.pq_adc
+            ad.q, ad.qs_b, ad.qs_h, ad.qs_l = q.data_ptr(), q.stride(0), q.stride(1), q.stride(2)
+            ad.dtype, ad.B, ad.Hq, ad.Hkv, ad.Lq = self.dt, self.B, self.Hq, self.Hkv, Lq
+            ad.n_sub, ad.d_sub, ad.n_cent = n_sub, d_sub, n_cent
+            ad.centres, ad.codes, ad.code_pitch, ad.n_cand = cf32.data_ptr(), book.codes.data_ptr(), book.capacity, current
+            ad.keys_out, ad.key_pitch, ad.stream = self.keybuf.data_ptr(), self.keybuf_pitch, stream
+            chain.pq_adc = C.addressof(ad)
+            se = self.select
+            se.rows, se.keys, se.key_pitch, se.key_bits = rows, self.keybuf.data_ptr(), self.keybuf_pitch, self.key_bits
+            se.n_cand, se.col_offset, se.k, se.excluded_key, se.stream = current, off, k_eff, self._excluded_min, stream
+            chain.select = C.addressof(se)
+
+        out = torch.empty((self.B, Lq, self.Hq, self.D), dtype=self.dtype, device=self.device)
+        work = _workspace(self.device, N.work_floats(self.n_rows, cap, self.D))
+        at = self.att
+        at.rows = rows
+        at.q, at.qs_b, at.qs_h, at.qs_l = q.data_ptr(), q.stride(0), q.stride(1), q.stride(2)
+        at.k, at.ks_b, at.ks_h, at.ks_l = k.data_ptr(), k.stride(0), k.stride(1), k.stride(2)
+        at.v, at.vs_b, at.vs_h, at.vs_l = v.data_ptr(), v.stride(0), v.stride(1), v.stride(2)
+        at.amask = None
+        at.sinks = None
+        at.dtype, at.B, at.Hq, at.Hkv, at.Lq, at.Lk, at.D = self.dt, self.B, self.Hq, self.Hkv, Lq, Lk, self.D
+        at.scaling, at.unit_inv_w, at.dense, at.max_cnt = float(scaling), self.unit, 0, cap
+        at.out, at.work, at.work_floats = out.data_ptr(), work.data_ptr(), work.numel()
+        at.logits_out = at.stats_out = None
+        at.stream = stream
+        chain.attention = C.addressof(at)
+        N.call("sah_run_chain", chain)
+        return out

@@ -305,3 +305,38 @@ def test_missing_sparse_meta_data_and_layer_idx_raise(cuda):
     ra = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=[cfg]))
     with pytest.raises(ValueError, match="layer_idx must be provided"):
         ra.custom_attention(None, q.to(cuda), k.to(cuda), v.to(cuda), None, 1.0, 0.0, sparse_meta_data={})
+
+
+@pytest.mark.parametrize("kind", ["fixed", "hash", "oracle", "pq"])
+def test_decode_plan_matches_masker_by_masker_path(cuda, kind):
+    """The one-call decode plan (weights not requested) gives bit-identical outputs to the general
+    masker-by-masker path over several appended-key steps, and really is the path taken."""
+    sa = _sa()
+    dtype = torch.bfloat16
+    B, Hq, Hkv, Lk, D = 2, 8, 2, 2000, 128
+    q, k, v = make_qkv(B, Hq, Hkv, 1, Lk + 4, D, dtype, outliers=True)
+    cfgs = [sa.SinkMaskerConfig(sink_size=16), sa.LocalMaskerConfig(window_size=64)]
+    if kind == "hash":
+        cfgs.append(sa.HashAttentionTopKMaskerConfig(heavy_size=100, hat_bits=32, hat_mlp_layers=3, hat_mlp_hidden_size=128,
+                                                     hat_mlp_activation="silu", hat_weights=_hat(sa, Hq, D, dtype, hidden=128)))
+    elif kind == "oracle":
+        cfgs.append(sa.OracleTopKConfig(heavy_size=0.05))
+    elif kind == "pq":
+        cfgs.append(sa.PQCacheConfig(heavy_size=64, pq_group_factor=16, pq_bits=6, kmeans_iter=4, init_offset=16, metric="euclidean"))
+    fast = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=cfgs))
+    fast.return_attention_weights = False
+    ref = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=cfgs))
+    m1, m2 = {}, {}
+    kc, vc = k.to(cuda), v.to(cuda)
+    calls = []
+    orig = type(fast._plans).get
+
+    for step in range(4):
+        n = Lk + step
+        qq = make_qkv(B, Hq, Hkv, 1, 1, D, dtype, seed=50 + step)[0].to(cuda)
+        o1, w1 = fast.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m1, layer_idx=0)
+        o2, w2 = ref.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m2, layer_idx=0)
+        assert w1 is None and w2 is not None
+        assert torch.equal(o1, o2), f"step {step}"
+    plan = next(iter(fast._plans.values()))
+    assert plan.att.out is not None and plan.att.Lk == Lk + 3     # the last step went through the plan
