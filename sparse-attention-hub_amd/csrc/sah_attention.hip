@@ -14,6 +14,7 @@
 #define ATT_NT 256
 #define ATT_NW (ATT_NT / SAH_WAVE)
 #define ATT_CHUNK (ATT_NT)  // keys per workgroup iteration: 64 per wave
+#define ATT_XCDS 8           // accelerator complex dies of an MI355X, one L2 each
 
 struct att_params {
   sah_rows rows;
@@ -88,7 +89,7 @@ __device__ __forceinline__ void att_unpack(const att_raw<DT>& r, float (&o)[8]) 
 // per lane group) and walks its 64-key slices in batches of UB iterations; the K and V
 // rows of a batch are requested together so 2*UB row loads are in flight per lane.
 template <int DT, int D>
-__global__ __launch_bounds__(ATT_NT) void k_sparse_attn(att_params P) {
+__global__ __launch_bounds__(ATT_NT, 5) void k_sparse_attn(att_params P) {
   constexpr int LPK = D / 8;            // lanes per key
   constexpr int KPI = SAH_WAVE / LPK;   // keys per wave iteration
   constexpr int IT = SAH_WAVE / KPI;    // iterations per 64-key wave slice (== LPK)
@@ -99,18 +100,28 @@ __global__ __launch_bounds__(ATT_NT) void k_sparse_attn(att_params P) {
   __shared__ float s_l[ATT_NW];
   __shared__ float s_acc[ATT_NW][D];
 
-  const int split = blockIdx.x;
-  const int r = blockIdx.y;
+  // Workgroup -> work mapping. The hardware deals consecutive workgroup ids round-robin to the 8
+  // XCDs, each with its own L2. A tile is (GQA group, split); tile t runs on XCD t % 8 and the G
+  // query heads of the group take adjacent slots of that XCD, so the K/V rows they have in common
+  // (all sink/local rows, every row in dense mode) are fetched from HBM once and shared in L2,
+  // while every XCD gets the same number of tiles.
+  const int G = P.Hq / P.Hkv;
+  const int slot = blockIdx.x / ATT_XCDS;
+  const int tile = (slot / G) * ATT_XCDS + (int)(blockIdx.x % ATT_XCDS);
+  const int n_groups = P.rows.n_rows / G;
+  if (tile >= n_groups * P.n_split) return;  // padding to a multiple of 8 tiles
+  const int split = tile % P.n_split;
+  const int gidx = tile / P.n_split;          // (b * Hkv + hk) * Lq + qi
+  const int qi = gidx % P.Lq;
+  const int hk = (gidx / P.Lq) % P.Hkv;
+  const int b = gidx / (P.Lq * P.Hkv);
+  const int h = hk * G + slot % G;
+  const int r = (b * P.Hq + h) * P.Lq + qi;
   const int tid = threadIdx.x;
   const int lane = tid & (SAH_WAVE - 1);
   const int wave = tid / SAH_WAVE;
   const int sub = lane % LPK;   // which 8-element slice of the row
   const int grp = lane / LPK;   // which key of the iteration
-
-  const int qi = r % P.Lq;
-  const int h = (r / P.Lq) % P.Hq;
-  const int b = r / (P.Lq * P.Hq);
-  const int hk = h / (P.Hq / P.Hkv);
 
   int cnt = P.dense ? P.Lk : P.rows.cnt[r];
   if (!P.dense && cnt > P.rows.cap) cnt = P.rows.cap;
@@ -357,7 +368,10 @@ static int att_launch(const sah_attention_args* a, const att_params& P) {
   int rc;
   {
     sah_timed timed("k_sparse_attn", a->stream);
-    hipLaunchKernelGGL((k_sparse_attn<DT, D>), dim3(P.n_split, a->rows.n_rows), dim3(ATT_NT), 0, st, P);
+    const int G = a->Hq / a->Hkv;
+    const int n_tiles = (a->rows.n_rows / G) * P.n_split;
+    const int n_wg = (n_tiles + ATT_XCDS - 1) / ATT_XCDS * ATT_XCDS * G;
+    hipLaunchKernelGGL((k_sparse_attn<DT, D>), dim3(n_wg), dim3(ATT_NT), 0, st, P);
     rc = sah_launch_status("sah_sparse_attention");
   }
   if (rc) return rc;
