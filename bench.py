@@ -36,11 +36,14 @@ WORKLOADS = {
             local=512, kind="hash", k=2048),
     4: dict(name="cfg4 Sink128+Local256+PQCache top-1024 bf16 B4 Lk32768", B=4, Lk=32768, dtype="bf16", sink=128, local=256,
             kind="pq", k=1024, outliers=True),
+    5: dict(name="cfg5 Sink128+Local1024+OracleTopK2%+AdaptiveSampling(1%, eps=delta=0.05) bf16 B16 Lk131072", B=16,
+            Lk=131072, dtype="bf16", sink=128, local=1024, kind="oracle", k=2621, outliers=True,
+            adaptive=dict(rate=0.01, epsilon=0.05, delta=0.05)),
 }
 HQ, HKV, D = 32, 8, 128
 
 
-def algorithmic_bytes(w) -> dict:
+def algorithmic_bytes(w, sampled_per_row: float = 0.0) -> dict:
     """Unique bytes that must cross HBM once per warm layer-step (formulas in DESIGN.md):
     sink/local rows shared by the 4 query heads of a KV group, top-k rows not shared,
     int32 indices written once and read once, Q and out."""
@@ -49,14 +52,15 @@ def algorithmic_bytes(w) -> dict:
     B, Lk = w["B"], w["Lk"]
     R = B * HQ
     fixed = w["sink"] + w["local"]
-    gather_topk = R * w["k"] * row * 2
+    # `sampled_per_row`: mean number of columns the adaptive sampler added to a row (data dependent, measured)
+    gather_topk = int(R * (w["k"] + sampled_per_row) * row * 2)
     gather_fixed = B * HKV * fixed * row * 2
-    idx = R * (fixed + w["k"]) * 4 * 2
+    idx = int(R * (fixed + w["k"] + 2 * sampled_per_row) * 4 * 2)   # sampled entries carry a 4-byte weight too
     qo = 2 * R * D * es
     # one 4-byte signature per (query head, key): the packed code proper; the non-zero plane the kernels also
     # read (another 4 bytes) is implementation traffic, not algorithmic
     scan = {"none": 0, "oracle": B * HKV * Lk * row, "hash": R * Lk * 4, "pq": B * HKV * (Lk - w["sink"]) * 16}[w["kind"]]
-    attn = gather_topk + gather_fixed + R * (fixed + w["k"]) * 4 + qo
+    attn = gather_topk + gather_fixed + int(R * (fixed + w["k"] + 2 * sampled_per_row) * 4) + qo
     return dict(step=gather_topk + gather_fixed + idx + qo + scan, attention_kernel=attn, scan=scan)
 
 
@@ -76,7 +80,7 @@ def build_workload(w, device, total_keys):
     import torch
 
     from sparse_attention_hub_amd.sparse_attention import (
-        HashAttentionTopKMaskerConfig, LocalMaskerConfig, OracleTopKConfig, PQCacheConfig, ResearchAttention,
+        AdaptiveSamplingMaskerConfig, HashAttentionTopKMaskerConfig, LocalMaskerConfig, OracleTopKConfig, PQCacheConfig, ResearchAttention,
         ResearchAttentionConfig, SinkMaskerConfig,
     )
     from sparse_attention_hub_amd.sparse_attention.utils.hashattention_utils import random_hat_weights
@@ -102,7 +106,13 @@ def build_workload(w, device, total_keys):
     elif w["kind"] == "pq":
         cfgs.append(PQCacheConfig(heavy_size=w["k"], pq_group_factor=16, pq_bits=8, kmeans_iter=10, init_offset=w["sink"],
                                   metric="euclidean"))
+    if w.get("adaptive"):
+        a = w["adaptive"]
+        cfgs.append(AdaptiveSamplingMaskerConfig(base_rate_sampling=a["rate"], epsilon=a["epsilon"], delta=a["delta"],
+                                                 init_offset=w["sink"], local_offset=w["local"]))
     ra = ResearchAttention.create_from_config(ResearchAttentionConfig(masker_configs=cfgs))
+    if w.get("adaptive"):
+        ra.maskers[-1].seed = 0
     ra.return_attention_weights = False  # HF attention modules drop the dense probabilities in decode
     return ra, qs.to(dtype).to(device), k.to(dtype).to(device), v.to(dtype).to(device), extra
 
@@ -134,6 +144,9 @@ def cpu_baseline(w, extra, ra_meta, k_dev, v_dev, q_dev, n_keys, budget_s=25.0):
         cent = ra_meta["pq_centroids"][0][:1].cpu()
         book = ra_meta["pq_codebook"][0].to_reference()[:1, : n_keys - w["sink"]].cpu()
         specs.append(("pq_topk", w["k"], w["sink"], cent, book))
+    if w.get("adaptive"):
+        a = w["adaptive"]
+        specs.append(("adaptive", a["rate"], a["epsilon"], a["delta"], w["sink"], w["local"], 0, 0))
     times = []
     t_all = time.perf_counter()
     for it in range(12):
@@ -226,7 +239,11 @@ def main() -> None:
     kt = N.timing_collect()
     N.timing_enable(False)
     kernels = {name: dict(launches=c, avg_us=1e3 * ms / c) for name, (c, ms) in kt.items()}
-    ab = algorithmic_bytes(w)
+    sampled = 0.0
+    if w.get("adaptive"):
+        # mean entries per row after the last step, minus what the fixed maskers put there
+        sampled = float(ra.maskers[-1].last_rows.cnt.float().mean().item()) - (w["sink"] + w["local"] + w["k"])
+    ab = algorithmic_bytes(w, sampled)
     dom = "k_sparse_attn"
     dom_us = kernels[dom]["avg_us"]
     achieved = ab["attention_kernel"] / (dom_us * 1e-6) / 1e9
@@ -249,7 +266,7 @@ def main() -> None:
         "dtype": w["dtype"],
         "data": "synthetic",
         "config": {"workload": w["name"], "q_heads": HQ, "kv_heads": HKV, "head_dim": D, "batch": w["B"], "keys": w["Lk"],
-                   "keys_per_row": w["sink"] + w["local"] + w["k"], "attention_weights_output": False},
+                   "keys_per_row": round(w["sink"] + w["local"] + w["k"] + sampled, 1), "attention_weights_output": False},
         "gpu_ms_per_step": round(gpu_ms / steps, 5),
         "host_launch_ms_per_step": round(host_ms / steps, 5),
         "step_algorithmic_bytes": ab["step"],

@@ -376,6 +376,80 @@ typedef struct sah_attention_weights_args {
 int sah_attention_weights(const sah_attention_weights_args* a);
 
 /* ---------------------------------------------------------------------------
+ * Adaptive sampling (vAttention). Replaces the tensor work of
+ * AdaptiveSamplingMasker.add_mask
+ * (maskers/sampling/implementations/adaptive_sampling.py:183-302, 365-407) and
+ * create_sampling_mask_with_per_head_budget (utils/mask_attention_utils.py:105-184).
+ *
+ * Both calls read the row's order-preserving score keys as written by
+ * sah_qk_scores WITHOUT an additive mask (key of round_to_dtype(q.k), 16-bit for
+ * bf16/f16, 32-bit for fp32); the numerators are recomputed from them as the
+ * reference's torch ops round them in `dtype`:
+ *     z[j] = round(round(s[j] * scaling) + amask[j]),  e[j] = round(exp(round(z[j] - max_j z[j]))).
+ *
+ * Random draws: Philox4x32-10 with key (seed lo, seed hi) and counter
+ * (i / 4, row, offset lo, offset hi); draw i of a row is output word i % 4 and
+ * maps to the column start + ((u * range) >> 32): uniform on [start, start+range),
+ * with replacement, like torch.randint in the reference.
+ *
+ * sah_adaptive_budget, per row r:
+ *   static_den = round(sum over the row's entries of round(e[col] * inv(w)))   (:370)
+ *                with inv(w) = round(1 / round(w + 1e-6)); prev_empty != 0: plain
+ *                sum of e over all keys (utils/mask_attention_utils.py:97-99);
+ *   n_base draws; sigma = max(round(unbiased std of e over the draws), 1e-8)     (:251-264)
+ *   sampled_den = round(sum over DISTINCT drawn columns of
+ *                 round(e * inv(round(n_base / range))))                         (:266-278, :389)
+ *   budget = clamp(trunc(clamp(round(round(round(ppf*sigma)*range /
+ *            max(round(eps*(static_den+sampled_den)), 1e-8))^2), 1, range)), n_base, range)
+ *                                                                           (:282-302, :394)
+ *   prob   = round(budget / range)                                               (:397)
+ * budget[r] int32, prob[r] float. stats (optional, [n_rows,4]) receives
+ * static_den, sigma, the denominator estimate and max z for inspection.
+ *
+ * sah_adaptive_sample, per row r: budget[r] draws (use another `offset` than
+ * the budget call); the distinct drawn columns are merged into the row as the
+ * reference's dense merge does (utils/mask.py:875-877): a column already in the
+ * row gets min(1, round(w + prob)), a new one is appended (ascending column
+ * order) with weight prob; bitmap and cnt are updated. rows.w is required;
+ * w_fresh != 0 says it holds garbage and every existing entry weighs 1.0.
+ * Capacity: the row may grow by up to `range` entries; entries beyond rows.cap
+ * are dropped, so size cap >= min(n_keys, cnt + range).
+ * The sampling range is limited to what one workgroup's LDS bitmap holds
+ * (1,179,648 columns).
+ * ------------------------------------------------------------------------- */
+typedef struct sah_adaptive_budget_args {
+  sah_rows rows;
+  const void* keys;       /* [n_rows, key_pitch] uint16 (bf16/f16) or uint32 (fp32) */
+  int64_t key_pitch;
+  const void* amask;      /* additive mask in `dtype`, or NULL */
+  int64_t ms_b, ms_h, ms_l;
+  int32_t dtype;
+  int32_t Hq, Lq;         /* row r = (b * Hq + h) * Lq + q, for the amask strides */
+  float scaling;
+  int32_t start, range, n_base;
+  float eps, delta_ppf;   /* delta_ppf = Phi^-1(1 - delta) */
+  uint64_t seed, offset;
+  int32_t prev_empty;
+  int32_t* budget;        /* [n_rows] out */
+  float* prob;            /* [n_rows] out */
+  float* stats;           /* [n_rows, 4] out, or NULL */
+  void* stream;
+} sah_adaptive_budget_args;
+int sah_adaptive_budget(const sah_adaptive_budget_args* a);
+
+typedef struct sah_adaptive_sample_args {
+  sah_rows rows;
+  const int32_t* budget;  /* [n_rows] */
+  const float* prob;      /* [n_rows] */
+  int32_t dtype;          /* mask dtype: rounding of w + prob */
+  int32_t start, range;
+  uint64_t seed, offset;
+  int32_t w_fresh;
+  void* stream;
+} sah_adaptive_sample_args;
+int sah_adaptive_sample(const sah_adaptive_sample_args* a);
+
+/* ---------------------------------------------------------------------------
  * One decode layer-step as a single call: runs, in this order and on the stream
  * each block names, every stage whose pointer is not NULL -
  *   sink_local -> (sig_a, sig_b as sah_hash_signatures_pair) -> hamming

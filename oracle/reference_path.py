@@ -22,7 +22,9 @@ and HF eager attention equality are taken from the reference's own unit tests.
 Parity unpinned (no reference vector exists, checked against closed forms and
 brute force only): the float values of the signature MLP (`hash_signatures`), the
 k-means trajectory beyond one Lloyd step from given centres (`kmeans_lloyd`), the
-adaptive-sampling index streams (`adaptive_*` take the draws as inputs), and the
+adaptive-sampling index streams (torch.randint in the reference; `adaptive_budget` and
+`adaptive_merge` take the draws as inputs, `adaptive_sampling` draws them with Philox4x32-10,
+itself pinned by the published known-answer vectors), and the
 full masker-chain -> output composition (`research_attention`).
 """
 from __future__ import annotations
@@ -361,6 +363,12 @@ def adaptive_base_count(rate: Size, sampling_range: int) -> int:
     return max(2, rate) if isinstance(rate, int) else max(2, int(rate * sampling_range))
 
 
+def adaptive_budget_formula(std: torch.Tensor, est_den: torch.Tensor, n: int, epsilon: float, ppf: float) -> torch.Tensor:
+    """_compute_adaptive_budget — adaptive_sampling.py:282-302 (int64, before the base-count clamp)."""
+    err = torch.clamp(epsilon * est_den, min=1e-8)
+    return torch.clamp((ppf * std * n / err) ** 2, min=1.0, max=float(n)).long()
+
+
 def adaptive_budget(prev: OMask, expw: torch.Tensor, base_idx: torch.Tensor, start: int, end: int,
                     epsilon: float, delta: float) -> Tuple[torch.Tensor, torch.Tensor]:
     """(budget int64 (B,H,Lq,1), probability in the mask dtype) from given base draws
@@ -378,8 +386,7 @@ def adaptive_budget(prev: OMask, expw: torch.Tensor, base_idx: torch.Tensor, sta
     base_dense.scatter_(-1, base_idx, torch.full_like(base_idx, nb / n, dtype=expw.dtype).to(prev.dtype))
     sampled_den = apply_inv_mask_dense(expw, base_dense).sum(dim=-1, keepdim=True)
     est = static_den + sampled_den
-    err = torch.clamp(epsilon * est, min=1e-8)
-    budget = torch.clamp((ppf * std * n / err) ** 2, min=1.0, max=float(n)).long()
+    budget = adaptive_budget_formula(std, est, n, epsilon, ppf)
     budget = torch.clamp(budget, min=nb, max=n)
     return budget, (budget / n).to(prev.dtype)
 
@@ -398,6 +405,82 @@ def adaptive_merge(prev: OMask, draws: List[torch.Tensor], prob: torch.Tensor) -
     if prev.kind == "empty":
         return OMask("dense", prev.shape, prev.dtype, samp)
     return OMask("dense", prev.shape, prev.dtype, merge_dense(prev.to_dense(), samp))
+
+
+# Counter-based random numbers for the sampling masker. The reference draws with
+# torch.randint from torch's global generator (adaptive_sampling.py:251-256,
+# utils/mask_attention_utils.py:152-158); its streams are generator- and
+# device-specific, so only their distribution (uniform on [start, end), with
+# replacement) is part of the contract. The kernels use Philox4x32-10 (Salmon, Moraes,
+# Dror, Shaw: "Parallel random numbers: as easy as 1, 2, 3", SC'11); this is the same
+# published algorithm in numpy, pinned in the tests by the paper's known-answer vectors.
+_PHILOX_M0 = 0xD2511F53
+_PHILOX_M1 = 0xCD9E8D57
+_PHILOX_W0 = 0x9E3779B9
+_PHILOX_W1 = 0xBB67AE85
+
+
+def philox4x32_10(counter, key):
+    """counter: (..., 4) uint32, key: (2,) uint32 -> (..., 4) uint32."""
+    import numpy as np
+
+    c = np.asarray(counter, dtype=np.uint64) & 0xFFFFFFFF
+    c0, c1, c2, c3 = (c[..., i].copy() for i in range(4))
+    k0, k1 = int(key[0]) & 0xFFFFFFFF, int(key[1]) & 0xFFFFFFFF
+    for _ in range(10):
+        p0 = c0 * _PHILOX_M0
+        p1 = c2 * _PHILOX_M1
+        n0 = (p1 >> 32) ^ c1 ^ k0
+        n2 = (p0 >> 32) ^ c3 ^ k1
+        c0, c1, c2, c3 = n0, p1 & 0xFFFFFFFF, n2, p0 & 0xFFFFFFFF
+        k0 = (k0 + _PHILOX_W0) & 0xFFFFFFFF
+        k1 = (k1 + _PHILOX_W1) & 0xFFFFFFFF
+    return np.stack([c0, c1, c2, c3], axis=-1).astype(np.uint32)
+
+
+def philox_columns(seed: int, offset: int, row: int, n: int, start: int, rng: int) -> torch.Tensor:
+    """Draws 0..n-1 of mask row `row`: draw i is word i % 4 of the block with counter
+    (i // 4, row, offset lo, offset hi) under key (seed lo, seed hi), mapped to the column
+    start + ((u * range) >> 32)."""
+    import numpy as np
+
+    n_blocks = (n + 3) // 4
+    ctr = np.zeros((n_blocks, 4), dtype=np.uint64)
+    ctr[:, 0] = np.arange(n_blocks, dtype=np.uint64)
+    ctr[:, 1] = row
+    ctr[:, 2] = offset & 0xFFFFFFFF
+    ctr[:, 3] = (offset >> 32) & 0xFFFFFFFF
+    u = philox4x32_10(ctr, (seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF)).reshape(-1)[:n].astype(np.uint64)
+    cols = start + ((u * np.uint64(rng)) >> np.uint64(32)).astype(np.int64)
+    return torch.from_numpy(cols)
+
+
+def adaptive_sampling(prev: OMask, q, k, attention_mask, scaling: float, rate: Size, epsilon: float, delta: float,
+                      init_offset: Size, local_offset: Size, seed: int, offset: int,
+                      budget_override: Optional[torch.Tensor] = None):
+    """AdaptiveSamplingMasker.add_mask — adaptive_sampling.py:304-407, with the draws of
+    call `offset` taken from Philox (base sample: offset, budgeted sample: offset + 1).
+    `budget_override` (int64, one per row) replaces the computed budget, so that the merge
+    can be checked bit-exactly for a budget obtained elsewhere. Returns (mask, budget, prob)."""
+    if prev.kind == "full":
+        return prev, None, None
+    if rate == 0:
+        return prev, None, None
+    B, H, Lq, Lk = prev.shape
+    start, end, n = adaptive_sampling_range(Lk, init_offset, local_offset)
+    if n < 2:
+        return OMask.full(prev.shape, prev.dtype), None, None
+    expw = adaptive_exp_scores(q, k, scaling, attention_mask)
+    nb = adaptive_base_count(rate, n)
+    R = B * H * Lq
+    base = torch.stack([philox_columns(seed, offset, r, nb, start, n) for r in range(R)]).view(B, H, Lq, nb)
+    budget, prob = adaptive_budget(prev, expw, base, start, end, epsilon, delta)
+    if budget_override is not None:
+        budget = budget_override.view(B, H, Lq, 1).to(torch.int64)
+        prob = (budget / n).to(prev.dtype)
+    flat = budget.reshape(-1)
+    draws = [philox_columns(seed, offset + 1, r, int(flat[r]), start, n) for r in range(R)]
+    return adaptive_merge(prev, draws, prob), budget, prob
 
 
 # ----------------------------------------------------------------------- attention
@@ -435,7 +518,8 @@ def research_attention(masker_specs: Sequence[Tuple], q, k, v, attention_mask, s
                        sinks: Optional[torch.Tensor] = None, state: Optional[dict] = None):
     """ResearchAttention.custom_attention — research_attention/base.py:63-170.
     masker_specs: ("sink", size) | ("local", size) | ("oracle_topk", heavy) |
-    ("hash_topk", heavy, weights, activation) | ("pq_topk", heavy, init_offset, centroids, codebook).
+    ("hash_topk", heavy, weights, activation) | ("pq_topk", heavy, init_offset, centroids, codebook) |
+    ("adaptive", rate, epsilon, delta, init_offset, local_offset, seed, offset).
     Returns (out, weights, final OMask)."""
     shape = (q.shape[0], q.shape[1], q.shape[2], k.shape[2])
     m = OMask.empty(shape, q.dtype)
@@ -461,6 +545,11 @@ def research_attention(masker_specs: Sequence[Tuple], q, k, v, attention_mask, s
                     m = OMask.full(shape, q.dtype)
                 else:
                     m = pq_topk(m, pq_scores(q, k.shape[1], cent, book), heavy, off)
+        elif kind == "adaptive":
+            # ("adaptive", rate, epsilon, delta, init_offset, local_offset, seed, offset)
+            m, budget, _ = adaptive_sampling(m, q, k, attention_mask, scaling, spec[1], spec[2], spec[3], spec[4],
+                                             spec[5], spec[6], spec[7], state.get("budget"))
+            state["budget_oracle"] = budget
         else:
             raise ValueError(kind)
     out, w = masked_attention(q, k, v, attention_mask, sinks, scaling, m)

@@ -1,0 +1,409 @@
+// Adaptive sampling (vAttention): per mask row, a budget from a base sample of the
+// softmax numerators, then that many uniform draws merged into the row with their
+// sampling probability as weight.
+//
+// Both kernels run one workgroup per mask row. The numerators e[j] are never
+// stored: they are a pure function of the row's order-preserving score keys (the
+// output of the QK scoring pass, 2 or 4 bytes per key), which stay L2-resident
+// while a row is worked on. Random numbers come from Philox4x32-10 with the
+// counter (block of 4 draws, row, call offset), so a row's draws do not depend
+// on the launch geometry and a CPU restatement can reproduce them bit for bit.
+#include "sah_common.h"
+
+#define AD_NT 1024
+#define AD_NW (AD_NT / SAH_WAVE)
+#define AD_MAX_LDS_WORDS 36864  // 144 KB bitmap: sampling range up to ~1.17 M keys
+
+// ---------------------------------------------------------------------------
+// Philox4x32-10 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3")
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ uint32_t ad_mulhi(uint32_t a, uint32_t b) { return (uint32_t)(((uint64_t)a * b) >> 32); }
+
+__device__ __forceinline__ void ad_philox(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1,
+                                          uint32_t (&out)[4]) {
+#pragma unroll
+  for (int round = 0; round < 10; ++round) {
+    const uint32_t hi0 = ad_mulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
+    const uint32_t hi1 = ad_mulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+    const uint32_t n0 = hi1 ^ c1 ^ k0, n2 = hi0 ^ c3 ^ k1;
+    c0 = n0; c1 = lo1; c2 = n2; c3 = lo0;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+// uniform column of [start, start + range) from one 32-bit draw
+__device__ __forceinline__ int ad_column(uint32_t u, int start, int range) { return start + (int)ad_mulhi(u, (uint32_t)range); }
+
+// ---------------------------------------------------------------------------
+// score keys -> numerators, rounded where the reference's torch ops round
+// ---------------------------------------------------------------------------
+template <int DT>
+__device__ __forceinline__ float ad_key_score(uint32_t k) {
+  if (DT == SAH_F32) return sah_bits_to_float((k & 0x80000000u) ? (k ^ 0x80000000u) : ~k);
+  const uint32_t u = (k & 0x8000u) ? (k & 0x7fffu) : ((~k) & 0xffffu);
+  return DT == SAH_BF16 ? sah_bf16_to_float((uint16_t)u) : sah_f16_to_float((uint16_t)u);
+}
+
+template <int DT>
+struct ad_row {
+  typedef typename std::conditional<DT == SAH_F32, uint32_t, uint16_t>::type key_t;
+  const key_t* keys;
+  const void* amask;  // additive mask row or NULL
+  int64_t moff;
+  float scaling;
+  float zmax;
+  __device__ __forceinline__ float z(int j) const {
+    float s = sah_round<DT>(ad_key_score<DT>(keys[j]) * scaling);
+    if (amask) s = sah_round<DT>(s + sah_load<DT>(amask, moff + j));
+    return s;
+  }
+  __device__ __forceinline__ float e(int j) const { return sah_round<DT>(expf(sah_round<DT>(z(j) - zmax))); }
+};
+
+__device__ __forceinline__ float ad_block_sum(float v, float* s_red) {
+  v = sah_wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & (SAH_WAVE - 1)) == 0) s_red[threadIdx.x / SAH_WAVE] = v;
+  __syncthreads();
+  float t = 0.f;
+#pragma unroll
+  for (int i = 0; i < AD_NW; ++i) t += s_red[i];
+  return t;
+}
+
+__device__ __forceinline__ float ad_block_max(float v, float* s_red) {
+  v = sah_wave_max(v);
+  __syncthreads();
+  if ((threadIdx.x & (SAH_WAVE - 1)) == 0) s_red[threadIdx.x / SAH_WAVE] = v;
+  __syncthreads();
+  float t = s_red[0];
+#pragma unroll
+  for (int i = 1; i < AD_NW; ++i) t = fmaxf(t, s_red[i]);
+  return t;
+}
+
+struct ad_budget_params {
+  sah_rows rows;
+  const void* keys; int64_t key_pitch;
+  const void* amask; int64_t ms_b, ms_h, ms_l;
+  int Hq, Lq;
+  float scaling;
+  int start, range, n_base;
+  float eps, ppf;
+  uint32_t k0, k1, o0, o1;
+  int prev_empty;
+  int* budget;
+  float* prob;
+  float* stats;
+};
+
+template <int DT>
+__global__ __launch_bounds__(AD_NT) void k_adaptive_budget(ad_budget_params P) {
+  HIP_DYNAMIC_SHARED(uint32_t, s_bits)  // one bit per column of the sampling range (word aligned)
+  __shared__ float s_red[AD_NW];
+  const int tid = threadIdx.x;
+  const int r = blockIdx.x;
+  const int Lk = P.rows.n_keys;
+  const int end = P.start + P.range;
+  const int w0 = P.start >> 5;
+  const int nw = ((end + 31) >> 5) - w0;
+
+  ad_row<DT> row;
+  row.keys = (const typename ad_row<DT>::key_t*)P.keys + (int64_t)r * P.key_pitch;
+  row.amask = P.amask;
+  row.moff = 0;
+  if (P.amask) {
+    const int qi = r % P.Lq, h = (r / P.Lq) % P.Hq, b = r / (P.Lq * P.Hq);
+    row.moff = (int64_t)b * P.ms_b + (int64_t)h * P.ms_h + (int64_t)qi * P.ms_l;
+  }
+  row.scaling = P.scaling;
+  row.zmax = 0.f;
+
+  for (int i = tid; i < nw; i += AD_NT) s_bits[i] = 0u;
+
+  // ---- row maximum of z over ALL keys (adaptive_sampling.py:195-196)
+  float zm = -INFINITY;
+  for (int j = tid; j < Lk; j += AD_NT) zm = fmaxf(zm, row.z(j));
+  row.zmax = ad_block_max(zm, s_red);
+
+  // ---- static denominator: numerators of the active entries times their inverse weight
+  float part = 0.f;
+  if (P.prev_empty) {
+    for (int j = tid; j < Lk; j += AD_NT) part += row.e(j);
+  } else {
+    int cnt = P.rows.cnt[r];
+    if (cnt > P.rows.cap) cnt = P.rows.cap;
+    const int* cols = P.rows.cols + (int64_t)r * P.rows.cap;
+    const float* w = P.rows.w ? P.rows.w + (int64_t)r * P.rows.cap : nullptr;
+    for (int i = tid; i < cnt; i += AD_NT) {
+      const int c = cols[i];
+      if (c < 0 || c >= Lk) continue;
+      float iw = sah_round<DT>(1.0f / sah_round<DT>(1.0f + 1e-6f));
+      if (w) iw = sah_round<DT>(1.0f / sah_round<DT>(w[i] + 1e-6f));
+      part += sah_round<DT>(row.e(c) * iw);
+    }
+  }
+  const float static_den = sah_round<DT>(ad_block_sum(part, s_red));
+
+  // ---- base sample: mean, unbiased std, and the set of distinct columns
+  const int n_calls = (P.n_base + 3) >> 2;
+  part = 0.f;
+  for (int c = tid; c < n_calls; c += AD_NT) {
+    uint32_t u[4];
+    ad_philox((uint32_t)c, (uint32_t)r, P.o0, P.o1, P.k0, P.k1, u);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      if (4 * c + t < P.n_base) {
+        const int j = ad_column(u[t], P.start, P.range);
+        part += row.e(j);
+        atomicOr(&s_bits[(j >> 5) - w0], 1u << (j & 31));
+      }
+    }
+  }
+  const float mean = ad_block_sum(part, s_red) / (float)P.n_base;
+  part = 0.f;
+  for (int c = tid; c < n_calls; c += AD_NT) {
+    uint32_t u[4];
+    ad_philox((uint32_t)c, (uint32_t)r, P.o0, P.o1, P.k0, P.k1, u);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      if (4 * c + t < P.n_base) {
+        const float d = row.e(ad_column(u[t], P.start, P.range)) - mean;
+        part = fmaf(d, d, part);
+      }
+    }
+  }
+  const float var = ad_block_sum(part, s_red) / (float)(P.n_base - 1);
+  float sigma = sah_round<DT>(sqrtf(var));
+  sigma = fmaxf(sigma, sah_round<DT>(1e-8f));
+
+  // ---- denominator estimate from the distinct base columns, each weighted 1/(nb/n + 1e-6)
+  const float wb = sah_round<DT>((float)((double)P.n_base / (double)P.range));
+  const float inv_b = sah_round<DT>(1.0f / sah_round<DT>(wb + 1e-6f));
+  part = 0.f;
+  for (int wi = tid; wi < nw; wi += AD_NT) {
+    uint32_t m = s_bits[wi];
+    while (m) {
+      const int bit = __builtin_ctz(m);
+      m &= m - 1;
+      part += sah_round<DT>(row.e(((w0 + wi) << 5) + bit) * inv_b);
+    }
+  }
+  const float sampled_den = sah_round<DT>(ad_block_sum(part, s_red));
+
+  if (tid == 0) {
+    // adaptive_sampling.py:282-302 and :394-397, every intermediate rounded to the tensor dtype
+    const float est = sah_round<DT>(static_den + sampled_den);
+    const float err = fmaxf(sah_round<DT>(P.eps * est), sah_round<DT>(1e-8f));
+    const float num = sah_round<DT>(sah_round<DT>(P.ppf * sigma) * (float)P.range);
+    const float ratio = sah_round<DT>(num / err);
+    float sq = sah_round<DT>(ratio * ratio);
+    const float hi = sah_round<DT>((float)P.range);
+    if (!(sq >= 1.0f)) sq = 1.0f;  // also catches NaN the way clamp(min=) orders its compares
+    if (sq > hi) sq = hi;
+    long long b = (long long)sq;
+    if (b < P.n_base) b = P.n_base;
+    if (b > P.range) b = P.range;
+    P.budget[r] = (int)b;
+    P.prob[r] = sah_round<DT>((float)b / (float)P.range);
+    if (P.stats) {
+      float* s = P.stats + (int64_t)r * 4;
+      s[0] = static_den;
+      s[1] = sigma;
+      s[2] = est;
+      s[3] = row.zmax;
+    }
+  }
+}
+
+struct ad_sample_params {
+  sah_rows rows;
+  const int* budget;
+  const float* prob;
+  int start, range;
+  uint32_t k0, k1, o0, o1;
+  int w_fresh;
+};
+
+template <int DT>
+__global__ __launch_bounds__(AD_NT) void k_adaptive_sample(ad_sample_params P) {
+  HIP_DYNAMIC_SHARED(uint32_t, s_bits)
+  __shared__ int s_scan[AD_NW + 1];
+  const int tid = threadIdx.x;
+  const int r = blockIdx.x;
+  const int end = P.start + P.range;
+  const int w0 = P.start >> 5;
+  const int nw = ((end + 31) >> 5) - w0;
+  const int cap = P.rows.cap;
+
+  int cnt0 = P.rows.cnt[r];  // read before any barrier: thread 0 rewrites it at the end
+  if (cnt0 > cap) cnt0 = cap;
+  int budget = P.budget[r];
+  if (budget > P.range) budget = P.range;
+  const float p = P.prob[r];
+
+  for (int i = tid; i < nw; i += AD_NT) s_bits[i] = 0u;
+  __syncthreads();
+
+  const int n_calls = (budget + 3) >> 2;
+  for (int c = tid; c < n_calls; c += AD_NT) {
+    uint32_t u[4];
+    ad_philox((uint32_t)c, (uint32_t)r, P.o0, P.o1, P.k0, P.k1, u);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      if (4 * c + t < budget) {
+        const int j = ad_column(u[t], P.start, P.range);
+        atomicOr(&s_bits[(j >> 5) - w0], 1u << (j & 31));
+      }
+    }
+  }
+  __syncthreads();
+
+  int* cols = P.rows.cols + (int64_t)r * cap;
+  float* w = P.rows.w + (int64_t)r * cap;
+  uint32_t* gbits = P.rows.bitmap + (int64_t)r * P.rows.n_words;
+
+  // entries already in the row: clamp(w + p, 0, 1) when drawn (utils/mask.py:875-877)
+  for (int i = tid; i < cnt0; i += AD_NT) {
+    const int c = cols[i];
+    float wv = P.w_fresh ? 1.0f : w[i];
+    bool changed = P.w_fresh != 0;
+    if (c >= P.start && c < end && ((s_bits[(c >> 5) - w0] >> (c & 31)) & 1u)) {
+      wv = fminf(1.0f, sah_round<DT>(wv + p));
+      changed = true;
+    }
+    if (changed) w[i] = wv;
+  }
+
+  // new columns, ascending: every thread owns a contiguous run of bitmap words
+  const int wpt = (nw + AD_NT - 1) / AD_NT;
+  const int wa = tid * wpt;
+  int wb = wa + wpt;
+  if (wb > nw) wb = nw;
+  int mine = 0;
+  for (int wi = wa; wi < wb; ++wi) mine += __builtin_popcount(s_bits[wi] & ~gbits[w0 + wi]);
+  int total = 0;
+  int pos = cnt0 + sah_block_excl_scan<AD_NT>(mine, s_scan, &total);
+  for (int wi = wa; wi < wb; ++wi) {
+    const uint32_t drawn = s_bits[wi];
+    if (!drawn) continue;
+    const uint32_t old = gbits[w0 + wi];
+    uint32_t fresh = drawn & ~old;
+    if (fresh) gbits[w0 + wi] = old | drawn;
+    while (fresh) {
+      const int bit = __builtin_ctz(fresh);
+      fresh &= fresh - 1;
+      if (pos < cap) {
+        cols[pos] = ((w0 + wi) << 5) + bit;
+        w[pos] = p;
+      }
+      ++pos;
+    }
+  }
+  if (tid == 0) {
+    int c = cnt0 + total;
+    P.rows.cnt[r] = c < cap ? c : cap;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// host
+// ---------------------------------------------------------------------------
+static int ad_lds_words(int start, int range) { return ((start + range + 31) >> 5) - (start >> 5); }
+
+template <typename K>
+static int ad_allow_lds(K kernel, int bytes, bool* done, const char* what) {
+  if (*done) return SAH_OK;
+  hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, AD_MAX_LDS_WORDS * 4);
+  if (e != hipSuccess) return sah_fail((int)e, "%s: cannot raise the LDS limit: %s", what, hipGetErrorString(e));
+  *done = true;
+  return SAH_OK;
+}
+
+static int ad_check_range(const sah_rows& rows, int start, int range, const char* what) {
+  if (start < 0 || range < 2 || (int64_t)start + range > rows.n_keys)
+    return sah_fail(SAH_EINVAL, "%s: sampling range [%d, %d) must hold >= 2 columns inside [0, %d)", what, start,
+                    start + range, rows.n_keys);
+  if (ad_lds_words(start, range) > AD_MAX_LDS_WORDS)
+    return sah_fail(SAH_ESHAPE, "%s: sampling range %d exceeds the %d columns one workgroup's LDS bitmap holds", what,
+                    range, AD_MAX_LDS_WORDS * 32);
+  return SAH_OK;
+}
+
+template <int DT>
+static int ad_budget_launch(const sah_adaptive_budget_args* a, const ad_budget_params& P) {
+  static bool allowed = false;
+  int rc = ad_allow_lds(k_adaptive_budget<DT>, 0, &allowed, "sah_adaptive_budget");
+  if (rc) return rc;
+  const size_t lds = (size_t)ad_lds_words(a->start, a->range) * 4;
+  sah_timed timed("k_adaptive_budget", a->stream);
+  hipLaunchKernelGGL(k_adaptive_budget<DT>, dim3(a->rows.n_rows), dim3(AD_NT), lds, (hipStream_t)a->stream, P);
+  return sah_launch_status("sah_adaptive_budget");
+}
+
+extern "C" int sah_adaptive_budget(const sah_adaptive_budget_args* a) {
+  if (!a) return sah_fail(SAH_ENULL, "sah_adaptive_budget: args is NULL");
+  int rc = sah_check_rows(a->rows, "sah_adaptive_budget", !a->prev_empty);
+  if (rc) return rc;
+  if (!a->keys || !a->budget || !a->prob) return sah_fail(SAH_ENULL, "sah_adaptive_budget: NULL keys / budget / prob");
+  if (a->key_pitch < a->rows.n_keys) return sah_fail(SAH_EINVAL, "sah_adaptive_budget: key_pitch < n_keys");
+  if (a->Hq <= 0 || a->Lq <= 0 || a->rows.n_rows % (a->Hq * a->Lq))
+    return sah_fail(SAH_EINVAL, "sah_adaptive_budget: n_rows is not a multiple of Hq * Lq");
+  rc = ad_check_range(a->rows, a->start, a->range, "sah_adaptive_budget");
+  if (rc) return rc;
+  if (a->n_base < 2) return sah_fail(SAH_EINVAL, "sah_adaptive_budget: n_base must be >= 2");
+  ad_budget_params P;
+  P.rows = a->rows;
+  P.keys = a->keys; P.key_pitch = a->key_pitch;
+  P.amask = a->amask; P.ms_b = a->ms_b; P.ms_h = a->ms_h; P.ms_l = a->ms_l;
+  P.Hq = a->Hq; P.Lq = a->Lq;
+  P.scaling = a->scaling;
+  P.start = a->start; P.range = a->range; P.n_base = a->n_base;
+  P.eps = a->eps; P.ppf = a->delta_ppf;
+  P.k0 = (uint32_t)a->seed; P.k1 = (uint32_t)(a->seed >> 32);
+  P.o0 = (uint32_t)a->offset; P.o1 = (uint32_t)(a->offset >> 32);
+  P.prev_empty = a->prev_empty;
+  P.budget = a->budget; P.prob = a->prob; P.stats = a->stats;
+  switch (a->dtype) {
+    case SAH_F32: return ad_budget_launch<SAH_F32>(a, P);
+    case SAH_BF16: return ad_budget_launch<SAH_BF16>(a, P);
+    case SAH_F16: return ad_budget_launch<SAH_F16>(a, P);
+    default: return sah_fail(SAH_EDTYPE, "sah_adaptive_budget: dtype %d", a->dtype);
+  }
+}
+
+template <int DT>
+static int ad_sample_launch(const sah_adaptive_sample_args* a, const ad_sample_params& P) {
+  static bool allowed = false;
+  int rc = ad_allow_lds(k_adaptive_sample<DT>, 0, &allowed, "sah_adaptive_sample");
+  if (rc) return rc;
+  const size_t lds = (size_t)ad_lds_words(a->start, a->range) * 4;
+  sah_timed timed("k_adaptive_sample", a->stream);
+  hipLaunchKernelGGL(k_adaptive_sample<DT>, dim3(a->rows.n_rows), dim3(AD_NT), lds, (hipStream_t)a->stream, P);
+  return sah_launch_status("sah_adaptive_sample");
+}
+
+extern "C" int sah_adaptive_sample(const sah_adaptive_sample_args* a) {
+  if (!a) return sah_fail(SAH_ENULL, "sah_adaptive_sample: args is NULL");
+  int rc = sah_check_rows(a->rows, "sah_adaptive_sample");
+  if (rc) return rc;
+  if (!a->rows.w) return sah_fail(SAH_ENULL, "sah_adaptive_sample: rows.w is NULL (sampled entries carry weights)");
+  if (!a->budget || !a->prob) return sah_fail(SAH_ENULL, "sah_adaptive_sample: NULL budget / prob");
+  rc = ad_check_range(a->rows, a->start, a->range, "sah_adaptive_sample");
+  if (rc) return rc;
+  ad_sample_params P;
+  P.rows = a->rows;
+  P.budget = a->budget; P.prob = a->prob;
+  P.start = a->start; P.range = a->range;
+  P.k0 = (uint32_t)a->seed; P.k1 = (uint32_t)(a->seed >> 32);
+  P.o0 = (uint32_t)a->offset; P.o1 = (uint32_t)(a->offset >> 32);
+  P.w_fresh = a->w_fresh;
+  switch (a->dtype) {
+    case SAH_F32: return ad_sample_launch<SAH_F32>(a, P);
+    case SAH_BF16: return ad_sample_launch<SAH_BF16>(a, P);
+    case SAH_F16: return ad_sample_launch<SAH_F16>(a, P);
+    default: return sah_fail(SAH_EDTYPE, "sah_adaptive_sample: dtype %d", a->dtype);
+  }
+}

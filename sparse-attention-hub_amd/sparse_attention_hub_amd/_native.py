@@ -40,6 +40,8 @@ EXPECTED_SYMBOLS = (
     "sah_pq_kmeans_assign",
     "sah_pq_kmeans_update",
     "sah_pq_adc_scores",
+    "sah_adaptive_budget",
+    "sah_adaptive_sample",
     "sah_sparse_attention_work_floats",
     "sah_sparse_attention",
     "sah_attention_weights",
@@ -206,18 +208,18 @@ class PqAdcArgs(C.Structure):
 class AdaptiveBudgetArgs(C.Structure):
     _fields_ = [
         ("rows", Rows),
-        ("q", C.c_void_p), ("qs_b", C.c_int64), ("qs_h", C.c_int64), ("qs_l", C.c_int64),
-        ("k", C.c_void_p), ("ks_b", C.c_int64), ("ks_h", C.c_int64), ("ks_l", C.c_int64),
+        ("keys", C.c_void_p), ("key_pitch", C.c_int64),
         ("amask", C.c_void_p), ("ms_b", C.c_int64), ("ms_h", C.c_int64), ("ms_l", C.c_int64),
         ("dtype", C.c_int32),
-        ("B", C.c_int32), ("Hq", C.c_int32), ("Hkv", C.c_int32), ("Lq", C.c_int32), ("Lk", C.c_int32), ("D", C.c_int32),
+        ("Hq", C.c_int32), ("Lq", C.c_int32),
         ("scaling", C.c_float),
         ("start", C.c_int32), ("range", C.c_int32), ("n_base", C.c_int32),
         ("eps", C.c_float), ("delta_ppf", C.c_float),
-        ("seed", C.c_uint64),
-        ("empty_is_dense", C.c_int32),
-        ("e_work", C.c_void_p),
+        ("seed", C.c_uint64), ("offset", C.c_uint64),
+        ("prev_empty", C.c_int32),
         ("budget", C.c_void_p),
+        ("prob", C.c_void_p),
+        ("stats", C.c_void_p),
         ("stream", C.c_void_p),
     ]
 
@@ -226,9 +228,11 @@ class AdaptiveSampleArgs(C.Structure):
     _fields_ = [
         ("rows", Rows),
         ("budget", C.c_void_p),
+        ("prob", C.c_void_p),
         ("dtype", C.c_int32),
         ("start", C.c_int32), ("range", C.c_int32),
-        ("seed", C.c_uint64),
+        ("seed", C.c_uint64), ("offset", C.c_uint64),
+        ("w_fresh", C.c_int32),
         ("stream", C.c_void_p),
     ]
 

@@ -7,7 +7,9 @@ from .research_attention.maskers.fixed import (
     LocalMasker, LocalMaskerConfig, OracleTopK, OracleTopKConfig, PQCache, PQCacheConfig, SinkMasker,
     SinkMaskerConfig, TopKMasker, TopKMaskerConfig,
 )
-from .research_attention.maskers.sampling import SamplingMasker, SamplingMaskerConfig
+from .research_attention.maskers.sampling import (
+    AdaptiveSamplingMasker, AdaptiveSamplingMaskerConfig, SamplingMasker, SamplingMaskerConfig,
+)
 from .utils.mask import Mask
 
 __all__ = [
@@ -16,5 +18,6 @@ __all__ = [
     "FixedMasker", "FixedMaskerConfig", "TopKMasker", "TopKMaskerConfig",
     "CausalMasker", "LocalMasker", "LocalMaskerConfig", "SinkMasker", "SinkMaskerConfig",
     "OracleTopK", "OracleTopKConfig", "HashAttentionTopKMasker", "HashAttentionTopKMaskerConfig",
-    "PQCache", "PQCacheConfig", "SamplingMasker", "SamplingMaskerConfig", "Mask",
+    "PQCache", "PQCacheConfig", "SamplingMasker", "SamplingMaskerConfig",
+    "AdaptiveSamplingMasker", "AdaptiveSamplingMaskerConfig", "Mask",
 ]

@@ -105,6 +105,8 @@ class ResearchAttention(SparseAttention):
             mask = fused_sink_local(maskers[0], maskers[1], keys, queries, mask)
             maskers = maskers[2:]
 
+        # per-call scratch the maskers may share (e.g. the QK score keys of one scoring pass)
+        call_scratch: Dict[str, Any] = {}
         for masker in maskers:
             mask = masker.add_mask(
                 keys=keys,
@@ -115,6 +117,7 @@ class ResearchAttention(SparseAttention):
                 dropout=dropout,
                 sparse_meta_data=sparse_meta_data,
                 previous_mask=mask,
+                _call_scratch=call_scratch,
                 **kwargs,
             )
 

@@ -5,6 +5,8 @@ from .fixed import (  # noqa: F401  (importing registers the maskers)
     LocalMasker, LocalMaskerConfig, OracleTopK, OracleTopKConfig, PQCache, PQCacheConfig, SinkMasker,
     SinkMaskerConfig, TopKMasker, TopKMaskerConfig,
 )
-from .sampling import SamplingMasker, SamplingMaskerConfig  # noqa: F401
+from .sampling import (  # noqa: F401
+    AdaptiveSamplingMasker, AdaptiveSamplingMaskerConfig, SamplingMasker, SamplingMaskerConfig,
+)
 
 __all__ = ["AttentionTensorDimensions", "MaskerConfig", "MaskerRegistry", "ResearchMasker"]

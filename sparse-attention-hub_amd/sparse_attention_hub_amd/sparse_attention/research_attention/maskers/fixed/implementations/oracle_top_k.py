@@ -91,6 +91,9 @@ class OracleTopK(TopKMasker):
             keybuf.data_ptr(), keybuf.stride(0), N.stream_ptr(q.device),
         )
         N.call("sah_qk_scores", args)
+        shared = kwargs.get("_call_scratch")
+        if am_ptr is None and isinstance(shared, dict):
+            shared["qk_score_keys"] = keybuf  # later maskers of this call can skip their own scoring pass
         # active columns rank where `scores[prev != 0] = finfo(mask dtype).min` puts them
         excluded = sortable_key_of(torch.finfo(previous_mask.dtype).min, q.dtype)
         self._select_into_rows(rows, keybuf, 32 if q.dtype == torch.float32 else 16, Lk, 0, k_eff, excluded)

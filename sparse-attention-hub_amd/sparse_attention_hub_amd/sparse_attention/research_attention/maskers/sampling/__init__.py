@@ -1,4 +1,5 @@
 """Sampling maskers."""
 from .base import SamplingMasker, SamplingMaskerConfig
+from .implementations import AdaptiveSamplingMasker, AdaptiveSamplingMaskerConfig
 
-__all__ = ["SamplingMasker", "SamplingMaskerConfig"]
+__all__ = ["SamplingMasker", "SamplingMaskerConfig", "AdaptiveSamplingMasker", "AdaptiveSamplingMaskerConfig"]

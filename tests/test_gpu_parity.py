@@ -340,3 +340,164 @@ def test_decode_plan_matches_masker_by_masker_path(cuda, kind):
         assert torch.equal(o1, o2), f"step {step}"
     plan = next(iter(fast._plans.values()))
     assert plan.att.out is not None and plan.att.Lk == Lk + 3     # the last step went through the plan
+
+
+# ------------------------------------------------------------------------ adaptive sampling
+def _adaptive_case(cuda, pre_cfgs, pre_specs, rate, eps, delta, io, lo, B, Hq, Hkv, Lq, Lk, D, dtype, amask=None,
+                   seed=1234, outliers=False):
+    sa = _sa()
+    q, k, v = make_qkv(B, Hq, Hkv, Lq, Lk, D, dtype, seed=5, outliers=outliers)
+    acfg = sa.AdaptiveSamplingMaskerConfig(base_rate_sampling=rate, epsilon=eps, delta=delta, init_offset=io,
+                                           local_offset=lo)
+    ra = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=pre_cfgs + [acfg]))
+    masker = ra.maskers[-1]
+    masker.seed = seed
+    scaling = D ** -0.5
+    out, w = ra.custom_attention(None, q.to(cuda), k.to(cuda), v.to(cuda), None if amask is None else amask.to(cuda),
+                                 scaling, 0.0, sparse_meta_data={}, layer_idx=0)
+    torch.cuda.synchronize()
+    specs = pre_specs + [("adaptive", rate, eps, delta, io, lo, seed, 0)]
+    # 1) the budget: float arithmetic in the tensor dtype, compared with the oracle's
+    st = {}
+    O.research_attention(specs, q, k, v, amask, scaling, None, st)
+    b_oracle = st["budget_oracle"].reshape(-1)
+    b_kernel = masker.last_budget.cpu().long()
+    return q, k, v, out, w, specs, scaling, b_kernel, b_oracle
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("chain", ["alone", "sink_local", "oracle", "amask", "lq2"])
+def test_adaptive_sampling_chain(cuda, dtype, chain):
+    """Budgets agree with the oracle (they are floats truncated to integers: a last-place difference in a sum
+    may move one by a unit of its precision); given the kernel's budgets, the sampled index sets are bit-exact
+    and outputs are within tolerance."""
+    sa = _sa()
+    pre_cfgs, pre_specs, amask = [], [], None
+    B, Hq, Hkv, Lq, Lk, D = 2, 4, 2, 1, 1500, 32
+    io, lo = 0, 0
+    if chain != "alone":
+        pre_cfgs = [sa.SinkMaskerConfig(sink_size=16), sa.LocalMaskerConfig(window_size=32)]
+        pre_specs = [("sink", 16), ("local", 32)]
+        io, lo = 16, 32
+    if chain == "oracle":
+        pre_cfgs.append(sa.OracleTopKConfig(heavy_size=0.02))
+        pre_specs.append(("oracle_topk", 0.02))
+    if chain == "amask":
+        amask = torch.zeros(B, 1, Lq, Lk)
+        amask[..., 900:1000] = -1e4
+        amask = amask.to(dtype)
+    if chain == "lq2":
+        Lq, io, lo = 2, 0.01, 0.02
+    q, k, v, out, w, specs, scaling, b_kernel, b_oracle = _adaptive_case(
+        cuda, pre_cfgs, pre_specs, 0.02, 0.1, 0.1, io, lo, B, Hq, Hkv, Lq, Lk, D, dtype, amask)
+    n = O.adaptive_sampling_range(Lk, io, lo)[2]
+    nb = O.adaptive_base_count(0.02, n)
+    assert int(b_kernel.min()) >= nb and int(b_kernel.max()) <= n
+    assert int(b_kernel.max()) > nb  # the case exercises the formula, not only its lower clamp
+    unit = (2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -20)
+    close = (b_kernel - b_oracle).abs().double() <= 1 + 2 * unit * b_oracle.double()
+    assert bool(close.all()), (b_kernel.tolist(), b_oracle.tolist())
+    assert float((b_kernel == b_oracle).double().mean()) >= 0.75
+    # 2) index sets and outputs for the kernel's own budgets
+    oo, ow, om = O.research_attention(specs, q, k, v, amask, scaling, None, {"budget": b_kernel})
+    assert torch.equal(w.cpu() != 0, ow != 0)
+    assert rel_err(out, oo) < TOL[dtype]
+    assert (w.float().cpu() - ow.float()).abs().max().item() < (1e-6 if dtype == torch.float32 else 1e-2)
+
+
+def test_adaptive_sampling_mask_weights_and_reproducibility(cuda):
+    """The dense form of the final mask equals the oracle's (weights included), torch.manual_seed reseeds the
+    sampler, and consecutive calls draw fresh samples."""
+    sa = _sa()
+    B, Hq, Hkv, Lq, Lk, D = 1, 4, 2, 1, 800, 16
+    q, k, v = make_qkv(B, Hq, Hkv, Lq, Lk, D, torch.float32, seed=9)
+    cfg = sa.AdaptiveSamplingMaskerConfig(base_rate_sampling=0.05, epsilon=0.2, delta=0.2, init_offset=8, local_offset=8)
+    masks = []
+    for rep in range(3):
+        if rep < 2:
+            torch.manual_seed(77)
+        m = sa.AdaptiveSamplingMasker(cfg)
+        prev = sa.Mask.create_empty_mask((B, Hq, Lq, Lk), torch.float32, cuda)
+        prev = sa.SinkMasker(sa.SinkMaskerConfig(sink_size=8)).add_mask(k.to(cuda), q.to(cuda), v.to(cuda), None, 0.25, 0.0, {}, prev)
+        first = m.add_mask(k.to(cuda), q.to(cuda), v.to(cuda), None, 0.25, 0.0, {}, prev).get_dense_mask().cpu()
+        masks.append(first)
+        if rep == 0:
+            om, budget, prob = O.adaptive_sampling(O.sink(O.OMask.empty((B, Hq, Lq, Lk), torch.float32), 8), q, k, None,
+                                                   0.25, 0.05, 0.2, 0.2, 8, 8, seed=77, offset=0,
+                                                   budget_override=m.last_budget.cpu().long())
+            assert torch.equal(first, om.to_dense())
+            again = m.add_mask(k.to(cuda), q.to(cuda), v.to(cuda), None, 0.25, 0.0, {},
+                               sa.Mask.create_empty_mask((B, Hq, Lq, Lk), torch.float32, cuda)).get_dense_mask().cpu()
+            assert not torch.equal(again != 0, first != 0)
+    assert torch.equal(masks[0], masks[1])
+    assert not torch.equal(masks[0], masks[2]) or torch.initial_seed() == 77
+
+
+def test_adaptive_sampling_denominator_guarantee_at_scale(cuda):
+    """Size-independent property on a long context: the importance-weighted sum over the sampled mask estimates the
+    full softmax denominator within epsilon for at least (1 - delta) of the rows (with slack for the normal
+    approximation), and the rows' entries are distinct and inside the key range."""
+    sa = _sa()
+    B, Hq, Hkv, Lq, Lk, D = 2, 32, 8, 1, 32768, 128
+    eps, delta = 0.1, 0.1
+    q, k, v = make_qkv(B, Hq, Hkv, Lq, Lk, D, torch.bfloat16, seed=21, outliers=False, device=cuda)
+    q = q * 0.5
+    cfgs = [sa.SinkMaskerConfig(sink_size=128), sa.LocalMaskerConfig(window_size=512),
+            sa.OracleTopKConfig(heavy_size=0.02),
+            sa.AdaptiveSamplingMaskerConfig(base_rate_sampling=0.01, epsilon=eps, delta=delta, init_offset=128,
+                                            local_offset=512)]
+    ra = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=cfgs))
+    mask = sa.Mask.create_empty_mask((B, Hq, Lq, Lk), torch.bfloat16, cuda)
+    scaling = D ** -0.5
+    scratch = {}
+    for m in ra.maskers:
+        mask = m.add_mask(k, q, v, None, scaling, 0.0, {}, mask, layer_idx=0, _call_scratch=scratch)
+    rows = mask.rows
+    torch.cuda.synchronize()
+    cnt = rows.cnt.long().cpu()
+    budget = ra.maskers[-1].last_budget.long().cpu()
+    n = Lk - 128 - 512
+    fixed = 128 + 512 + int(0.02 * Lk)
+    assert int(budget.min()) >= int(0.01 * n) and int(budget.max()) <= n
+    assert bool((cnt <= fixed + budget).all()) and bool((cnt > fixed).all())
+    # weighted estimate of the denominator against the exact one, in fp64 on the device
+    kk = k.double().repeat_interleave(Hq // Hkv, dim=1)
+    z = torch.matmul(q.double(), kk.transpose(-1, -2)) * scaling
+    e = torch.exp(z - z.amax(dim=-1, keepdim=True)).reshape(B * Hq, Lk)
+    true_den = e.sum(dim=-1)
+    cols = rows.cols.long()
+    pos = torch.arange(rows.cap, device=cuda).unsqueeze(0)
+    valid = pos < rows.cnt.long().unsqueeze(1)
+    wts = rows.w.double()
+    est = (torch.where(valid, torch.gather(e, 1, cols.clamp(0, Lk - 1)) / wts.clamp_min(1e-9), torch.zeros_like(wts))).sum(dim=-1)
+    rel = ((est - true_den).abs() / true_den).cpu()
+    assert float((rel <= eps).double().mean()) >= 1.0 - delta - 0.08, float((rel <= eps).double().mean())
+    # entries are distinct and in range
+    big = torch.where(valid, cols, torch.full_like(cols, Lk + 1) + pos)
+    srt = torch.sort(big, dim=1).values
+    assert bool((srt[:, 1:] != srt[:, :-1]).all())
+    assert bool(((cols >= 0) & (cols < Lk) | ~valid).all())
+
+
+def test_adaptive_sampling_abi_rejects_bad_arguments(cuda):
+    from sparse_attention_hub_amd import _native as N
+    from sparse_attention_hub_amd.sparse_attention.utils.native_rows import NativeRows
+
+    rows = NativeRows(4, 100, 100, cuda)
+    rows.zero_if_fresh()
+    keys = torch.zeros((4, 128), dtype=torch.int16, device=cuda)
+    budget = torch.zeros(4, dtype=torch.int32, device=cuda)
+    prob = torch.zeros(4, dtype=torch.float32, device=cuda)
+
+    def budget_args(start, rng, nb):
+        return N.AdaptiveBudgetArgs(rows.as_struct(), keys.data_ptr(), 128, None, 0, 0, 0, N.dtype_code(torch.bfloat16),
+                                    4, 1, 1.0, start, rng, nb, 0.1, 1.0, 1, 0, 0, budget.data_ptr(), prob.data_ptr(),
+                                    None, N.stream_ptr(cuda))
+
+    for bad in (budget_args(0, 1, 2), budget_args(50, 60, 2), budget_args(0, 100, 1)):
+        with pytest.raises(ValueError):
+            N.call("sah_adaptive_budget", bad)
+    sample = N.AdaptiveSampleArgs(rows.as_struct(), budget.data_ptr(), prob.data_ptr(), N.dtype_code(torch.bfloat16),
+                                  0, 100, 1, 1, 1, N.stream_ptr(cuda))
+    with pytest.raises(N.NativeLibraryError, match="rows.w is NULL"):
+        N.call("sah_adaptive_sample", sample)
