@@ -169,6 +169,8 @@ def main() -> None:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", type=int, default=3, choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--batch", type=int, default=0, help="study only: override the workload's batch size")
+    ap.add_argument("--keys", type=int, default=0, help="study only: override the workload's key count")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="short run for `rocprofv3 --pmc`: a few layer-steps plus three 256 MiB copy kernels of known size")
     args = ap.parse_args()
@@ -185,7 +187,11 @@ def main() -> None:
         sys.exit(3)
     N.lib()
     dev = torch.device("cuda:0")
-    w = WORKLOADS[args.config]
+    w = dict(WORKLOADS[args.config])
+    if args.batch or args.keys:
+        w["B"] = args.batch or w["B"]
+        w["Lk"] = args.keys or w["Lk"]
+        w["name"] += f" [size override: B={w['B']} Lk={w['Lk']}]"
     steps, warm = args.steps, args.warmup
     probe = max(20, min(steps, 100))                      # instrumented steps for the per-kernel roofline
     total_keys = w["Lk"] + probe

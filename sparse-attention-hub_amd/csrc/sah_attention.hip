@@ -15,6 +15,7 @@
 #define ATT_NW (ATT_NT / SAH_WAVE)
 #define ATT_CHUNK (ATT_NT)  // keys per workgroup iteration: 64 per wave
 #define ATT_XCDS 8           // accelerator complex dies of an MI355X, one L2 each
+#define ATT_MAX_SPLIT 64
 
 struct att_params {
   sah_rows rows;
@@ -25,7 +26,6 @@ struct att_params {
   int Hq, Hkv, Lq, Lk;
   float scaling, unit_inv_w;
   int dense;
-  int kps;      // keys per split (multiple of ATT_CHUNK)
   int n_split;
   float* work;
   float* logits_out;
@@ -125,8 +125,12 @@ __global__ __launch_bounds__(ATT_NT, 5) void k_sparse_attn(att_params P) {
 
   int cnt = P.dense ? P.Lk : P.rows.cnt[r];
   if (!P.dense && cnt > P.rows.cap) cnt = P.rows.cap;
-  const int begin = split * P.kps;
-  int end = begin + P.kps;
+  // the row's own entry count decides its slices, so rows of very different lengths all spread over the
+  // splits evenly; the host picks n_split from an upper bound only
+  const int row_chunks = (cnt + ATT_CHUNK - 1) / ATT_CHUNK;
+  const int kps = ((row_chunks + P.n_split - 1) / P.n_split) * ATT_CHUNK;
+  const int begin = split * kps;
+  int end = begin + kps;
   if (end > cnt) end = cnt;
 
   float* wout = P.work + ((int64_t)r * P.n_split + split) * (D + 2);
@@ -267,7 +271,6 @@ __global__ __launch_bounds__(ATT_NT, 5) void k_sparse_attn(att_params P) {
 // merge the splits of one row: out = sum_s acc_s e^(m_s-M) / sum_s l_s e^(m_s-M).
 // The (m, l) pairs go through LDS and each thread's partial values are requested together,
 // so the kernel costs about two memory round trips whatever the number of splits.
-#define ATT_MAX_SPLIT 64
 template <int DT, int D>
 __global__ __launch_bounds__(D < 64 ? 64 : D) void k_attn_combine(const float* work, int n_split, int Hq, int Lq,
                                                                   const float* sinks, void* out, float* stats) {
@@ -341,24 +344,23 @@ __global__ __launch_bounds__(256) void k_attn_weights(sah_rows R, const float* l
   sah_store<DT>(weights, (int64_t)r * R.n_keys + c, p);
 }
 
-static int att_pick_split(int n_rows, int max_cnt, int* kps_out) {
-  // enough workgroups to cover 256 CUs several times, at least one chunk each
+// Splits per row, from an upper bound of the row lengths: enough workgroups to cover 256 CUs several times,
+// at least one chunk and at most 16 chunks of keys each (the kernel divides every row's own length by it).
+static int att_pick_split(int n_rows, int max_cnt) {
   int chunks = (max_cnt + ATT_CHUNK - 1) / ATT_CHUNK;
   if (chunks < 1) chunks = 1;
   int want = (4096 + n_rows - 1) / n_rows;  // target ~4096 workgroups
-  if (want < 1) want = 1;
+  const int for_length = (chunks + 15) / 16;
+  if (want < for_length) want = for_length;
   int n_split = chunks < want ? chunks : want;
-  if (n_split > 64) n_split = 64;
-  int cps = (chunks + n_split - 1) / n_split;  // chunks per split
-  n_split = (chunks + cps - 1) / cps;
-  *kps_out = cps * ATT_CHUNK;
-  return n_split;
+  if (n_split > ATT_MAX_SPLIT) n_split = ATT_MAX_SPLIT;
+  const int cps = (chunks + n_split - 1) / n_split;  // chunks per split
+  return (chunks + cps - 1) / cps;
 }
 
 extern "C" int64_t sah_sparse_attention_work_floats(int32_t n_rows, int32_t max_cnt, int32_t D) {
   if (n_rows <= 0 || max_cnt < 0 || D <= 0) return 0;
-  int kps;
-  int n_split = att_pick_split(n_rows, max_cnt, &kps);
+  int n_split = att_pick_split(n_rows, max_cnt);
   return (int64_t)n_rows * n_split * (D + 2);
 }
 
@@ -424,7 +426,7 @@ extern "C" int sah_sparse_attention(const sah_attention_args* a) {
   P.Hq = a->Hq; P.Hkv = a->Hkv; P.Lq = a->Lq; P.Lk = a->Lk;
   P.scaling = a->scaling; P.unit_inv_w = a->unit_inv_w;
   P.dense = a->dense ? 1 : 0;
-  P.n_split = att_pick_split(a->rows.n_rows, max_cnt, &P.kps);
+  P.n_split = att_pick_split(a->rows.n_rows, max_cnt);
   P.work = a->work;
   P.logits_out = a->logits_out;
   P.logits_pitch = a->dense ? a->Lk : a->rows.cap;

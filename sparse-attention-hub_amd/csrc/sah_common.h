@@ -142,6 +142,28 @@ __device__ __forceinline__ uint32_t sah_sort_key(float score) {
   }
 }
 
+// c + a.lo * b.lo + a.hi * b.hi for two packed 16-bit pairs of storage type DT (bf16 or f16),
+// products and sum in fp32: one instruction on the device
+template <int DT>
+__device__ __forceinline__ float sah_dot2(uint32_t a, uint32_t b, float c) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  if (DT == SAH_BF16) {
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf2, a), __builtin_bit_cast(bf2, b), c, false);
+  } else {
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, a), __builtin_bit_cast(h2, b), c, false);
+  }
+#else
+  if (DT == SAH_BF16) {
+    return c + sah_bits_to_float(a << 16) * sah_bits_to_float(b << 16) +
+           sah_bits_to_float(a & 0xffff0000u) * sah_bits_to_float(b & 0xffff0000u);
+  }
+  return c + sah_f16_to_float((uint16_t)(a & 0xffffu)) * sah_f16_to_float((uint16_t)(b & 0xffffu)) +
+         sah_f16_to_float((uint16_t)(a >> 16)) * sah_f16_to_float((uint16_t)(b >> 16));
+#endif
+}
+
 // Pins a loaded value at this point of the program: the load that produced it must have
 // been issued (and is waited for) here, so the compiler can neither sink it into a later
 // branch nor serialise a batch of independent loads one wait at a time.

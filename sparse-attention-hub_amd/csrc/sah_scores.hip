@@ -32,12 +32,82 @@ __device__ __forceinline__ float sc_group_sum(float v) {
   return v;
 }
 
+// One key row slice as loaded: 8 elements of a lane, not yet widened.
+template <int DT>
+struct sc_raw {
+  uint4 a;
+};
+template <>
+struct sc_raw<SAH_F32> {
+  float4 a, b;
+};
+
+template <int DT>
+__device__ __forceinline__ void sc_load(const char* p, sc_raw<DT>& r) {
+  if constexpr (DT == SAH_F32) {
+    r.a = ((const float4*)p)[0];
+    r.b = ((const float4*)p)[1];
+  } else {
+    r.a = *(const uint4*)p;
+  }
+}
+
+template <int DT>
+__device__ __forceinline__ void sc_keep(sc_raw<DT>& r) {
+  if constexpr (DT == SAH_F32) {
+    sah_keep(r.a.x); sah_keep(r.a.y); sah_keep(r.a.z); sah_keep(r.a.w);
+    sah_keep(r.b.x); sah_keep(r.b.y); sah_keep(r.b.z); sah_keep(r.b.w);
+  } else {
+    sah_keep(r.a.x); sah_keep(r.a.y); sah_keep(r.a.z); sah_keep(r.a.w);
+  }
+}
+
+// partial dot product of the lane's 8 elements
+template <int DT>
+__device__ __forceinline__ float sc_dot(const sc_raw<DT>& q, const sc_raw<DT>& k) {
+  if constexpr (DT == SAH_F32) {
+    float d = q.a.x * k.a.x;
+    d = fmaf(q.a.y, k.a.y, d); d = fmaf(q.a.z, k.a.z, d); d = fmaf(q.a.w, k.a.w, d);
+    d = fmaf(q.b.x, k.b.x, d); d = fmaf(q.b.y, k.b.y, d); d = fmaf(q.b.z, k.b.z, d); d = fmaf(q.b.w, k.b.w, d);
+    return d;
+  } else {
+    float d = sah_dot2<DT>(q.a.x, k.a.x, 0.f);
+    d = sah_dot2<DT>(q.a.y, k.a.y, d);
+    d = sah_dot2<DT>(q.a.z, k.a.z, d);
+    return sah_dot2<DT>(q.a.w, k.a.w, d);
+  }
+}
+
+// Sums four per-lane partials (one per query vector) over the LPK lanes of a key, leaving in lane `sub` the
+// total of query 2*(sub&1) + ((sub>>1)&1): each exchange step halves what a lane still carries, so the four
+// reductions cost 3 adds inside the quad instead of 8, plus one add per doubling of the group beyond 4 lanes.
+template <int LPK>
+__device__ __forceinline__ float sc_reduce4(float d0, float d1, float d2, float d3, int sub) {
+  static_assert(LPK >= 4, "needs at least a quad per key");
+  const bool odd = sub & 1;
+  float x0 = odd ? d2 : d0, x1 = odd ? d3 : d1;
+  const float y0 = odd ? d0 : d2, y1 = odd ? d1 : d3;
+  x0 += sah_dpp<0xB1>(y0);  // lane ^ 1
+  x1 += sah_dpp<0xB1>(y1);
+  const bool up = sub & 2;
+  float z = up ? x1 : x0;
+  const float t = up ? x0 : x1;
+  z += sah_dpp<0x4E>(t);    // lane ^ 2
+  if (LPK == 8) z += __shfl_xor(z, 4);
+  if (LPK == 16) {
+    z += sah_dpp<0x124>(z);  // row_ror:4  (rotations keep the position inside the quad)
+    z += sah_dpp<0x128>(z);  // row_ror:8
+  }
+  return z;
+}
+
 template <int DT, int D>
 __global__ __launch_bounds__(SC_NT) void k_qk_scores(qk_params P) {
   constexpr int LPK = D / 8;
   constexpr int KPI = SAH_WAVE / LPK;
   constexpr int IT = SAH_WAVE / KPI;
   constexpr int ES = (DT == SAH_F32) ? 4 : 2;
+  constexpr bool FAST4 = LPK >= 4;  // transposing reduction of all four query vectors at once
   typedef typename std::conditional<DT == SAH_F32, uint32_t, uint16_t>::type key_t;
   __shared__ key_t s_out[SC_NQ][SC_TILE];
 
@@ -53,54 +123,72 @@ __global__ __launch_bounds__(SC_NT) void k_qk_scores(qk_params P) {
   const int v0 = blockIdx.z * SC_NQ;  // first query vector (of G*Lq) handled here
   const int nvec = G * P.Lq;
 
-  float qv[SC_NQ][8];
+  sc_raw<DT> qv[SC_NQ];
   int row[SC_NQ];
   int64_t moff[SC_NQ];
 #pragma unroll
   for (int i = 0; i < SC_NQ; ++i) {
-    const int v = v0 + i;
+    int v = v0 + i;
     row[i] = -1;
     moff[i] = 0;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) qv[i][e] = 0.f;
-    if (v < nvec) {
-      const int h = hk * G + v / P.Lq;
-      const int qi = v % P.Lq;
+    const bool live = v < nvec;
+    if (!live) v = nvec - 1;  // computed and dropped
+    const int h = hk * G + v / P.Lq;
+    const int qi = v % P.Lq;
+    sc_load<DT>((const char*)P.q + ((int64_t)b * P.qs_b + (int64_t)h * P.qs_h + (int64_t)qi * P.qs_l + sub * 8) * ES, qv[i]);
+    if (live) {
       row[i] = (b * P.Hq + h) * P.Lq + qi;
-      sah_load8<DT>(P.q, (int64_t)b * P.qs_b + (int64_t)h * P.qs_h + (int64_t)qi * P.qs_l + sub * 8, qv[i]);
       if (P.amask) moff[i] = (int64_t)b * P.ms_b + (int64_t)h * P.ms_h + (int64_t)qi * P.ms_l;
     }
   }
-  const char* kbase = (const char*)P.k + ((int64_t)b * P.ks_b + (int64_t)hk * P.ks_h) * ES;
+  const char* kbase = (const char*)P.k + ((int64_t)b * P.ks_b + (int64_t)hk * P.ks_h + sub * 8) * ES;
+  const int64_t krow = P.ks_l * ES;
+  // which of the four totals this lane ends up with after sc_reduce4
+  const int mine = FAST4 ? (2 * (sub & 1) + ((sub >> 1) & 1)) : 0;
 
   for (int iter = 0; iter < SC_ITERS; ++iter) {
     const int j0 = (blockIdx.x * SC_ITERS + iter) * SC_TILE;
     if (j0 >= P.Lk) break;  // uniform across the workgroup
-    float kv[IT][8];
+    // every load of the tile is requested before the first use; rows past the end re-read the last row
+    sc_raw<DT> kv[IT];
 #pragma unroll
     for (int it = 0; it < IT; ++it) {
-      const int j = j0 + wave * SAH_WAVE + it * KPI + grp;
-      if (j < P.Lk) {
-        sah_load8<DT>(kbase + (int64_t)j * P.ks_l * ES, sub * 8, kv[it]);
-      } else {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) kv[it][e] = 0.f;
-      }
+      int j = j0 + wave * SAH_WAVE + it * KPI + grp;
+      if (j > P.Lk - 1) j = P.Lk - 1;
+      sc_load<DT>(kbase + (int64_t)j * krow, kv[it]);
     }
+#pragma unroll
+    for (int it = 0; it < IT; ++it) sc_keep<DT>(kv[it]);
 #pragma unroll
     for (int it = 0; it < IT; ++it) {
       const int jl = wave * SAH_WAVE + it * KPI + grp;  // key within the tile
       const int j = j0 + jl;
+      if constexpr (FAST4) {
+        const float d = sc_reduce4<LPK>(sc_dot<DT>(qv[0], kv[it]), sc_dot<DT>(qv[1], kv[it]), sc_dot<DT>(qv[2], kv[it]),
+                                        sc_dot<DT>(qv[3], kv[it]), sub);
+        int rr = row[0];
+        int64_t mo = moff[0];
 #pragma unroll
-      for (int i = 0; i < SC_NQ; ++i) {
-        float d = 0.f;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) d = fmaf(qv[i][e], kv[it][e], d);
-        d = sc_group_sum<LPK>(d);
-        if (sub == (i % LPK) && j < P.Lk && row[i] >= 0) {
+        for (int i = 1; i < SC_NQ; ++i) {
+          if (mine == i) {
+            rr = row[i];
+            mo = moff[i];
+          }
+        }
+        if (sub < 4 && j < P.Lk && rr >= 0) {
           float s = sah_round<DT>(d);
-          if (P.amask) s = sah_round<DT>(s + sah_load<DT>(P.amask, moff[i] + j));
-          s_out[i][jl] = (key_t)sah_sort_key<DT>(s);
+          if (P.amask) s = sah_round<DT>(s + sah_load<DT>(P.amask, mo + j));
+          s_out[mine][jl] = (key_t)sah_sort_key<DT>(s);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < SC_NQ; ++i) {
+          const float d = sc_group_sum<LPK>(sc_dot<DT>(qv[i], kv[it]));
+          if (sub == (i % LPK) && j < P.Lk && row[i] >= 0) {
+            float s = sah_round<DT>(d);
+            if (P.amask) s = sah_round<DT>(s + sah_load<DT>(P.amask, moff[i] + j));
+            s_out[i][jl] = (key_t)sah_sort_key<DT>(s);
+          }
         }
       }
     }
