@@ -450,10 +450,39 @@ typedef struct sah_adaptive_sample_args {
 int sah_adaptive_sample(const sah_adaptive_sample_args* a);
 
 /* ---------------------------------------------------------------------------
+ * One decode step of a Sink + Local + HashAttentionTopK chain on rows that are
+ * still empty, one query per row (Lq = 1, n_rows = B * Hq): the work of
+ * sah_sink_local_indices (fresh = 1), sah_hash_signatures_pair(key_sig, query_sig)
+ * and sah_hamming_topk, in this order, with the same results. Replaces, for a
+ * decode call, SinkMasker / LocalMasker.add_mask (basic_fixed.py:354-363, :48-67),
+ * HashAttentionTopKMasker._update_key_signatures and the query half of
+ * _get_signatures (hashattention_top_k.py:203-305) and the score + top-k + merge
+ * of :365-370 / fixed/base.py:74-85.
+ * rows.cnt / rows.bitmap need no initialisation. query_sig: L = 1, codes =
+ * [n_rows] query codes (written). key_sig: NULL or L = 0 when no key is new,
+ * else the job that appends the newest key's code to the cache. kcodes /
+ * code_pitch: the key-code stream of row r starts at kcodes + r * code_pitch
+ * codes. When shapes allow (16-byte aligned code streams, layer widths powers of
+ * two with d_in * d_out a multiple of 4096, the new key inside the local window)
+ * everything runs in one kernel, otherwise as the three launches above.
+ * ------------------------------------------------------------------------- */
+typedef struct sah_hash_decode_args {
+  sah_rows rows;
+  int32_t sink, window;
+  const sah_hash_sig_args* query_sig;   /* host pointer */
+  const sah_hash_sig_args* key_sig;     /* host pointer or NULL */
+  const uint32_t* kcodes;
+  int64_t code_pitch;
+  int32_t k;
+  void* stream;
+} sah_hash_decode_args;
+int sah_hash_decode_topk(const sah_hash_decode_args* a);
+
+/* ---------------------------------------------------------------------------
  * One decode layer-step as a single call: runs, in this order and on the stream
  * each block names, every stage whose pointer is not NULL -
  *   sink_local -> (sig_a, sig_b as sah_hash_signatures_pair) -> hamming
- *   -> qk -> pq_assign -> pq_adc -> select -> attention.
+ *   -> hash_decode -> qk -> pq_assign -> pq_adc -> select -> attention.
  * The blocks are the argument structures of the entry points above, unchanged;
  * a caller keeps them alive between steps and only patches the fields that move
  * (tensor pointers, key count). Replaces the per-masker Python dispatch of
@@ -465,6 +494,7 @@ typedef struct sah_chain_args {
   const sah_hash_sig_args* sig_a;
   const sah_hash_sig_args* sig_b;
   const sah_hamming_topk_args* hamming;
+  const sah_hash_decode_args* hash_decode;
   const sah_qk_scores_args* qk;
   const sah_pq_assign_args* pq_assign;
   const sah_pq_adc_args* pq_adc;

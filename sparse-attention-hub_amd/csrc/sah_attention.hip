@@ -477,6 +477,7 @@ extern "C" int sah_run_chain(const sah_chain_args* a) {
     if ((rc = sah_hash_signatures(a->sig_b))) return rc;
   }
   if (a->hamming && (rc = sah_hamming_topk(a->hamming))) return rc;
+  if (a->hash_decode && (rc = sah_hash_decode_topk(a->hash_decode))) return rc;
   if (a->qk && (rc = sah_qk_scores(a->qk))) return rc;
   if (a->pq_assign && (rc = sah_pq_kmeans_assign(a->pq_assign))) return rc;
   if (a->pq_adc && (rc = sah_pq_adc_scores(a->pq_adc))) return rc;

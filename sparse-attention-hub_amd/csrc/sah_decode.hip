@@ -1,0 +1,173 @@
+// One decode step of a Sink + Local + HashAttentionTopK chain in a single kernel.
+//
+// One workgroup (1024 threads) per mask row (b, h), one query position. The row is built from
+// scratch in LDS and registers:
+//   1. sink and local columns in closed form: list entries written, bitmap row built in LDS
+//      (never read from memory);
+//   2. the two signature MLPs of the step, side by side: threads 0-511 hash the query of head h,
+//      threads 512-1023 the newest key (its code goes to the signature cache; the column itself
+//      lies inside the local window, so this step's selection never looks at it);
+//   3. signature top-k of the not-yet-active columns (the SWAR selection), appended to the row.
+// Against three separate launches this saves two kernel boundaries, the bitmap round trip through
+// memory and the query-code round trip.
+#include "sah_common.h"
+#include "sah_hsw.h"
+#include "sah_sig.h"
+
+// Threads per MLP job and weight-row slots per thread: the same geometry as the stand-alone signature
+// kernel, so that both sum in the same order and produce the same bits.
+#define HDEC_GROUP 512
+#define HDEC_ROWS 4
+
+typedef sig_gemv_lds<1, HDEC_GROUP> hdec_sig_lds;
+
+struct hdec_params {
+  sah_rows R;
+  sig_params job[2];  // 0: query, 1: newest key
+  int has_key;
+  const uint2* kcodes;
+  int64_t pitch;
+  int k;
+  int sink, window;
+};
+
+template <int DT>
+__global__ __launch_bounds__(HSW_NT) void k_hash_decode(hdec_params P) {
+  __shared__ hsw_lds S;
+  HIP_DYNAMIC_SHARED(unsigned char, hdec_dyn)
+  const sah_rows& R = P.R;
+  const int r = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int n = R.n_keys;
+  const int n_ch = (n + 255) / 256;
+  uint32_t* s_bm = (uint32_t*)hdec_dyn;
+  uint32_t* s_key = s_bm + n_ch * 8;
+  // the MLP scratch shares the space of the staged scores: the MLPs are over before staging starts
+  hdec_sig_lds* s_sig = (hdec_sig_lds*)s_key;
+
+  // ---- 1. sink + local, one query at position n - 1 (basic_fixed.py:354-363, :48-67)
+  const int s_hi = P.sink < n ? P.sink : n;
+  int lo = 0, hi = 0;
+  if (P.window > 0) {
+    lo = n - P.window;
+    hi = n;
+    if (lo < 0) lo = 0;
+  }
+  const int lo2 = lo > s_hi ? lo : s_hi;
+  const int n_local = hi > lo2 ? hi - lo2 : 0;
+  const int fixed = s_hi + n_local;
+  int* cols = R.cols + (int64_t)r * R.cap;
+  for (int i = tid; i < fixed && i < R.cap; i += HSW_NT) {
+    cols[i] = i < s_hi ? i : lo2 + (i - s_hi);
+    if (R.w) R.w[(int64_t)r * R.cap + i] = 1.0f;
+  }
+  for (int wi = tid; wi < n_ch * 8; wi += HSW_NT)
+    s_bm[wi] = wi < R.n_words ? (sah_range_bits(wi, 0, s_hi) | sah_range_bits(wi, lo, hi)) : 0u;
+
+  // ---- 2. signatures of the query and of the newest key
+  // uniform across the wave, and known to be: the job's parameters are then fetched by scalar loads
+  const int job = __builtin_amdgcn_readfirstlane(tid / HDEC_GROUP);
+  const bool active = job == 0 || P.has_key;
+  const int Hq = P.job[0].Hq;
+  // 2-byte weights: all layers requested up-front; fp32 rows are twice as wide, one layer at a time
+  constexpr int PF = (DT == SAH_F32) ? 1 : SAH_MAX_MLP_LAYERS;
+  sig_gemv_block<DT, 1, HDEC_GROUP, HDEC_ROWS, PF>(P.job[job], active, tid % HDEC_GROUP, r / Hq, r % Hq, 0, 1,
+                                                    P.job[0].n_layers, s_sig[job]);
+  const uint2 q = s_sig[0].code[0];
+  __syncthreads();  // every thread holds q (and the bitmap is complete) before the scores overwrite the scratch
+
+  // ---- 3. top-k over the remaining columns
+  hsw_select_row(R, r, P.kcodes + (int64_t)r * P.pitch, q, P.k, fixed < R.cap ? fixed : R.cap, s_bm, s_key, S);
+}
+
+static size_t hdec_lds_bytes(int n_keys) {
+  const int n_ch = (n_keys + 255) / 256;
+  const size_t bm = (size_t)n_ch * 8 * 4, key = (size_t)n_ch * 64 * 4, sig = 2 * sizeof(hdec_sig_lds);
+  return bm + (key > sig ? key : sig);
+}
+
+template <int DT>
+static int hdec_launch(const sah_hash_decode_args* a, const hdec_params& P, size_t lds) {
+  static bool raised = false;
+  if (!raised) {
+    hipError_t e = hipFuncSetAttribute((const void*)k_hash_decode<DT>, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+    if (e != hipSuccess) return sah_fail((int)e, "sah_hash_decode_topk: cannot raise the LDS limit: %s", hipGetErrorString(e));
+    raised = true;
+  }
+  sah_timed timed("k_hash_decode", a->stream);
+  hipLaunchKernelGGL(k_hash_decode<DT>, dim3(a->rows.n_rows), dim3(HSW_NT), lds, (hipStream_t)a->stream, P);
+  return sah_launch_status("sah_hash_decode_topk");
+}
+
+// can the single-kernel form run this step?
+static bool hdec_fusable(const sah_hash_decode_args* a) {
+  const sah_hash_sig_args* q = a->query_sig;
+  const sah_hash_sig_args* kk = a->key_sig;
+  const int n = a->rows.n_keys;
+  if (q->L != 1 || (int64_t)q->B * q->Hq != a->rows.n_rows) return false;
+  if (!sig_gemv_ok(q, HDEC_GROUP, HDEC_ROWS)) return false;
+  if (kk && kk->L > 0) {
+    if (kk->L != 1 || kk->B != q->B || kk->Hq != q->Hq || kk->n_layers != q->n_layers || kk->dtype != q->dtype) return false;
+    if (!sig_gemv_ok(kk, HDEC_GROUP, HDEC_ROWS)) return false;
+    // the new code is written while the row's codes are scanned: its column must be one the scan ignores
+    if ((const uint32_t*)kk->codes == a->kcodes && kk->code_offset < n - a->window) return false;
+  }
+  if (hdec_lds_bytes(n) > 150 * 1024) return false;
+  if (a->code_pitch % 2 || ((uintptr_t)a->kcodes % 16) || n < 4) return false;
+  return true;
+}
+
+extern "C" int sah_hash_decode_topk(const sah_hash_decode_args* a) {
+  if (!a) return sah_fail(SAH_ENULL, "sah_hash_decode_topk: args is NULL");
+  int rc = sah_check_rows(a->rows, "sah_hash_decode_topk");
+  if (rc) return rc;
+  if (!a->query_sig || !a->kcodes) return sah_fail(SAH_ENULL, "sah_hash_decode_topk: query_sig / kcodes is NULL");
+  if (!a->query_sig->codes) return sah_fail(SAH_ENULL, "sah_hash_decode_topk: query_sig.codes is NULL");
+  if (a->sink < 0 || a->window < 0 || a->k < 0) return sah_fail(SAH_EINVAL, "sah_hash_decode_topk: negative sink / window / k");
+  if (a->code_pitch < a->rows.n_keys) return sah_fail(SAH_EINVAL, "sah_hash_decode_topk: code_pitch < n_keys");
+  rc = sig_validate(a->query_sig);
+  if (rc) return rc;
+  const bool has_key = a->key_sig && a->key_sig->L > 0;
+  if (has_key) {
+    rc = sig_validate(a->key_sig);
+    if (rc) return rc;
+  }
+  if (a->query_sig->L != 1 || (int64_t)a->query_sig->B * a->query_sig->Hq != a->rows.n_rows)
+    return sah_fail(SAH_ESHAPE, "sah_hash_decode_topk: needs one query per row (Lq = 1, n_rows = B * Hq)");
+  int64_t worst = (int64_t)a->sink + a->window + a->k;
+  if (worst > a->rows.n_keys) worst = a->rows.n_keys;
+  if (worst > a->rows.cap)
+    return sah_fail(SAH_ECAPACITY, "sah_hash_decode_topk: cap %d < sink + window + k = %lld", a->rows.cap, (long long)worst);
+
+  if (!hdec_fusable(a)) {
+    // same step as three launches
+    sah_sink_local_args sl;
+    sl.rows = a->rows; sl.lq = 1; sl.sink = a->sink; sl.window = a->window; sl.fresh = 1; sl.clear_future = 0;
+    sl.stream = a->stream;
+    rc = sah_sink_local_indices(&sl);
+    if (rc) return rc;
+    rc = has_key ? sah_hash_signatures_pair(a->key_sig, a->query_sig) : sah_hash_signatures(a->query_sig);
+    if (rc) return rc;
+    sah_hamming_topk_args ht;
+    ht.rows = a->rows; ht.kcodes = a->kcodes; ht.code_pitch = a->code_pitch; ht.qcodes = a->query_sig->codes;
+    ht.lq = 1; ht.k = a->k; ht.stream = a->stream;
+    return sah_hamming_topk(&ht);
+  }
+
+  hdec_params P;
+  P.R = a->rows;
+  sig_fill(a->query_sig, P.job[0]);
+  sig_fill(has_key ? a->key_sig : a->query_sig, P.job[1]);
+  P.has_key = has_key ? 1 : 0;
+  P.kcodes = (const uint2*)a->kcodes;
+  P.pitch = a->code_pitch;
+  P.k = a->k;
+  P.sink = a->sink;
+  P.window = a->window;
+  const size_t lds = hdec_lds_bytes(a->rows.n_keys);
+  switch (a->query_sig->dtype) {
+    case SAH_F32: return hdec_launch<SAH_F32>(a, P, lds);
+    case SAH_BF16: return hdec_launch<SAH_BF16>(a, P, lds);
+    default: return hdec_launch<SAH_F16>(a, P, lds);
+  }
+}

@@ -1,0 +1,268 @@
+// Signature (Hamming) top-k of one mask row, SWAR form: shared by the stand-alone kernel and the
+// fused decode kernel.
+#pragma once
+#include "sah_common.h"
+
+// signature score of the reference, sum_e q_e k_e with q_e, k_e in {-1, 0, +1}:
+// popc(nz) - 2 popc((q ^ k) & nz), nz = bits where both are non-zero; in [-32, 32]
+__device__ __forceinline__ int sig_score(uint2 q, uint2 k) {
+  const uint32_t nz = q.y & k.y;
+  return __popc(nz) - 2 * __popc((q.x ^ k.x) & nz);
+}
+
+// ---------------------------------------------------------------------------
+// Signature top-k, SWAR form. Scores fit a byte (score + 33 in [1, 65], 0 = column already
+// active or out of range), so a lane handles 4 consecutive columns as one 32-bit word:
+//   P0  each lane loads its 4 codes (32 B, whole wave: 2 KB contiguous), scores them, zeroes
+//       the already-active ones with a nibble of the bitmap row and parks the word in LDS;
+//   P1  the threshold T: P0 has already counted the columns at or above 8 coarse thresholds, one more
+//       pass over the staged bytes counts 7 fine ones inside the bracket (byte-parallel compares, no atomics);
+//   P2  per-wave counts of "above T" and "equal T";
+//   P3  ordered write: wave scan of per-lane counts, up to 4 columns per lane, ties taken
+//       lowest column first until `need` are used; new bits are OR-ed into the LDS copy of
+//       the bitmap row, which is written back once at the end.
+// Active columns hold byte 0 and T >= 1 whenever k inactive columns exist, so P2/P3 never
+// look at the bitmap again.
+// ---------------------------------------------------------------------------
+#define HSW_NT 1024
+#define HSW_NW (HSW_NT / SAH_WAVE)
+#define HSW_BATCH 2  // 256-column chunks per register buffer in P0 (two buffers in flight)
+
+// per byte b < 128 of w: 0x80 if b >= t (t in [0, 128]) else 0
+__device__ __forceinline__ uint32_t swar_ge(uint32_t w, uint32_t t) {
+  return ((w | 0x80808080u) - t * 0x01010101u) & 0x80808080u;
+}
+
+#define HSW_PROBES 8  // coarse thresholds 8, 16, ... 64 counted while the scores are staged
+
+struct hsw_lds {
+  int gt[HSW_NW];
+  int eq[HSW_NW];
+  int probe[HSW_NW][HSW_PROBES];
+  int fine[HSW_NW][HSW_PROBES];
+};
+
+// LDS words the row needs: bitmap (padded to whole chunks) and one byte per column
+__host__ __device__ inline size_t hsw_lds_bytes(int n_keys) {
+  const int n_ch = (n_keys + 255) / 256;
+  return (size_t)n_ch * 8 * 4 + (size_t)n_ch * 64 * 4;
+}
+
+// Top-k of row r over the not-yet-active columns. On entry `s_bm` (n_ch * 8 words of dynamic LDS, zero
+// padded) holds the row's bitmap and every thread of the workgroup has passed a barrier after it was
+// written; cnt0 entries of R.cols are already in place. On exit the selected columns are appended, the
+// bitmap row (LDS copy and global) and cnt are updated.
+__device__ __forceinline__ void hsw_select_row(const sah_rows& R, int r, const uint2* kc, const uint2 q, int k, int cnt0,
+                                               uint32_t* s_bm, uint32_t* s_key, hsw_lds& S) {
+  int* s_gt = S.gt;
+  int* s_eq = S.eq;
+  const int tid = threadIdx.x;
+  const int lane = tid & (SAH_WAVE - 1);
+  const int wave = tid / SAH_WAVE;
+  const int n = R.n_keys;
+  const int n_ch = (n + 255) / 256;            // chunks of 256 columns = 64 words
+  const int cpw = (n_ch + HSW_NW - 1) / HSW_NW;
+  const int my_c0 = wave * cpw;
+  int my_c1 = my_c0 + cpw;
+  if (my_c1 > n_ch) my_c1 = n_ch;
+  uint32_t* bm = R.bitmap + (int64_t)r * R.n_words;
+  if (k > n) k = n;
+
+  // ---- P0: score and stage --------------------------------------------------
+  // While the codes stream in the ALUs are idle: count, on the side, the columns at or above each of
+  // HSW_PROBES coarse thresholds, so that P1 only has to resolve the last 3 bits of the threshold.
+  int pc[HSW_PROBES];
+#pragma unroll
+  for (int i = 0; i < HSW_PROBES; ++i) pc[i] = 0;
+  // Two register buffers of HSW_BATCH chunks each: the next batch is requested before the current one is
+  // scored, so the memory pipe stays busy while the ALUs work.
+  auto request = [&](uint4 (&ra)[HSW_BATCH], uint4 (&rb)[HSW_BATCH], int c0) {
+#pragma unroll
+    for (int u = 0; u < HSW_BATCH; ++u) {
+      const int j0 = ((c0 + u) * SAH_WAVE + lane) * 4;
+      // clamp to the last full group of 4 codes: out-of-range lanes re-read valid memory
+      int jl = j0;
+      if (jl + 4 > n) jl = n >= 4 ? ((n - 4) & ~1) : 0;
+      const uint4* p = (const uint4*)(kc + jl);
+      ra[u] = p[0];
+      rb[u] = p[1];
+    }
+  };
+  auto score = [&](uint4 (&ra)[HSW_BATCH], uint4 (&rb)[HSW_BATCH], int c0) {
+#pragma unroll
+    for (int u = 0; u < HSW_BATCH; ++u) {
+      sah_keep(ra[u].x); sah_keep(ra[u].y); sah_keep(ra[u].z); sah_keep(ra[u].w);
+      sah_keep(rb[u].x); sah_keep(rb[u].y); sah_keep(rb[u].z); sah_keep(rb[u].w);
+    }
+#pragma unroll
+    for (int u = 0; u < HSW_BATCH; ++u) {
+      if (c0 + u >= my_c1) break;
+      const int wi = (c0 + u) * SAH_WAVE + lane;
+      const int j0 = wi * 4;
+      uint32_t word;
+      if (j0 + 4 <= n) {
+        const uint32_t s0 = (uint32_t)(sig_score(q, make_uint2(ra[u].x, ra[u].y)) + 33);
+        const uint32_t s1 = (uint32_t)(sig_score(q, make_uint2(ra[u].z, ra[u].w)) + 33);
+        const uint32_t s2 = (uint32_t)(sig_score(q, make_uint2(rb[u].x, rb[u].y)) + 33);
+        const uint32_t s3 = (uint32_t)(sig_score(q, make_uint2(rb[u].z, rb[u].w)) + 33);
+        word = s0 | (s1 << 8) | (s2 << 16) | (s3 << 24);
+      } else {
+        word = 0;  // ragged tail: the few columns of the last, partial group
+        for (int t = 0; t < 4; ++t)
+          if (j0 + t < n) word |= (uint32_t)(sig_score(q, kc[j0 + t]) + 33) << (8 * t);
+      }
+      // zero the bytes of already-active columns: nibble -> byte mask
+      const uint32_t nib = (s_bm[j0 >> 5] >> (j0 & 31)) & 0xFu;
+      const uint32_t act = ((nib * 0x00204081u) & 0x01010101u) * 0xFFu;
+      const uint32_t kw = word & ~act;
+      s_key[wi] = kw;
+      const uint32_t x = kw | 0x80808080u;
+#pragma unroll
+      for (int i = 0; i < HSW_PROBES; ++i) pc[i] += __popc((x - (uint32_t)(8 * (i + 1)) * 0x01010101u) & 0x80808080u);
+    }
+  };
+  {
+    uint4 a0[HSW_BATCH], a1[HSW_BATCH], b0[HSW_BATCH], b1[HSW_BATCH];
+    if (my_c0 < my_c1) request(a0, a1, my_c0);
+    for (int c0 = my_c0; c0 < my_c1; c0 += 2 * HSW_BATCH) {
+      const bool more_b = c0 + HSW_BATCH < my_c1;          // uniform across the wave
+      if (more_b) request(b0, b1, c0 + HSW_BATCH);
+      score(a0, a1, c0);
+      if (c0 + 2 * HSW_BATCH < my_c1) request(a0, a1, c0 + 2 * HSW_BATCH);
+      if (more_b) score(b0, b1, c0 + HSW_BATCH);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < HSW_PROBES; ++i) {
+    const int t = sah_wave_sum_i(pc[i]);
+    if (lane == 0) S.probe[wave][i] = t;
+  }
+  __syncthreads();
+
+  // ---- P1: largest T with count(key >= T) >= k --------------------------------
+  // counts fall as the threshold rises, so the thresholds that still reach k form a prefix
+  const int n_w = n_ch * SAH_WAVE;
+  int tot = 0;
+  if (lane < HSW_PROBES) {
+#pragma unroll
+    for (int wv = 0; wv < HSW_NW; ++wv) tot += S.probe[wv][lane];
+  }
+  const int n_pass = __popcll(__ballot(lane < HSW_PROBES && tot >= k));
+  const uint32_t base = 8u * (uint32_t)n_pass;                         // T is in [base, base + 8)
+  const int next_probe = n_pass < HSW_PROBES ? __shfl(tot, n_pass) : 0;  // count(key >= base + 8)
+  int fc[7];
+#pragma unroll
+  for (int j = 0; j < 7; ++j) fc[j] = 0;
+  for (int i = tid; i < n_w; i += HSW_NT) {
+    const uint32_t x = s_key[i] | 0x80808080u;
+#pragma unroll
+    for (int j = 0; j < 7; ++j) fc[j] += __popc((x - (base + 1u + j) * 0x01010101u) & 0x80808080u);
+  }
+#pragma unroll
+  for (int j = 0; j < 7; ++j) {
+    const int t = sah_wave_sum_i(fc[j]);
+    if (lane == 0) S.fine[wave][j] = t;
+  }
+  __syncthreads();
+  int ftot = 0;
+  if (lane < 7) {
+#pragma unroll
+    for (int wv = 0; wv < HSW_NW; ++wv) ftot += S.fine[wv][lane];
+  }
+  const int n_fine = __popcll(__ballot(lane < 7 && ftot >= k));
+  const uint32_t T = base + (uint32_t)n_fine;
+  const int above = n_fine < 7 ? __shfl(ftot, n_fine) : next_probe;      // count(key >= T + 1)
+  // T == 0: fewer than k inactive columns exist; take them all, byte-0 "ties" emit nothing
+  const int need = (T == 0) ? 0 : k - above;
+
+  // ---- P2: per-wave counts ---------------------------------------------------------
+  int n_gt = 0, n_eq = 0;
+  for (int c = my_c0; c < my_c1; ++c) {
+    const uint32_t w = s_key[c * SAH_WAVE + lane];
+    const uint32_t g = swar_ge(w, T + 1);
+    n_gt += __popc(g);
+    n_eq += __popc(swar_ge(w, T) & ~g);
+  }
+  n_gt = sah_wave_sum_i(n_gt);
+  n_eq = sah_wave_sum_i(n_eq);
+  if (lane == 0) {
+    s_gt[wave] = n_gt;
+    s_eq[wave] = n_eq;
+  }
+  __syncthreads();
+  int tie_base = 0, out_base = 0, total_out = 0;
+  {
+    int tie_run = 0, out_run = 0;
+#pragma unroll
+    for (int wv = 0; wv < HSW_NW; ++wv) {
+      if (wv == wave) {
+        tie_base = tie_run;
+        out_base = out_run;
+      }
+      int take = need - tie_run;
+      if (take < 0) take = 0;
+      if (take > s_eq[wv]) take = s_eq[wv];
+      out_run += s_gt[wv] + take;
+      tie_run += s_eq[wv];
+    }
+    total_out = out_run;
+  }
+
+  // ---- P3: ordered write --------------------------------------------------------------
+  int* cols = R.cols + (int64_t)r * R.cap;
+  float* wts = R.w ? R.w + (int64_t)r * R.cap : nullptr;
+  const bool ties_all = (tie_base + n_eq <= need);   // every tie of this wave is taken
+  const bool ties_none = (tie_base >= need);         // none is
+  int out_pos = cnt0 + out_base;
+  int tie_run = tie_base;
+  for (int c = my_c0; c < my_c1; ++c) {
+    const int wi = c * SAH_WAVE + lane;
+    const uint32_t w = s_key[wi];
+    const uint32_t g = swar_ge(w, T + 1) >> 7;            // bits 0, 8, 16, 24
+    uint32_t e = (swar_ge(w, T) >> 7) & ~g;
+    if (ties_none) {
+      e = 0;
+    } else if (!ties_all) {
+      const int ne = __popc(e);
+      const int before = sah_wave_incl_scan(ne) - ne;     // ties in lower lanes of this chunk
+      int allowed = need - (tie_run + before);
+      if (allowed < ne) {                                  // keep only the lowest `allowed` ties
+        uint32_t kept = 0;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const uint32_t bit = e & (1u << (8 * t));
+          if (bit && allowed > 0) {
+            kept |= bit;
+            --allowed;
+          }
+        }
+        e = kept;
+      }
+      tie_run += sah_wave_sum_i(ne);
+    }
+    const uint32_t sel = g | e;
+    const int ns = __popc(sel);
+    const int incl = sah_wave_incl_scan(ns);
+    int pos = out_pos + incl - ns;
+    if (sel) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        if (sel & (1u << (8 * t))) {
+          if (pos < R.cap) {
+            cols[pos] = wi * 4 + t;
+            if (wts) wts[pos] = 1.0f;
+          }
+          ++pos;
+        }
+      }
+      const uint32_t nib = ((sel * 0x00204081u) >> 21) & 0xFu;
+      const int j0 = wi * 4;
+      atomicOr(&s_bm[j0 >> 5], nib << (j0 & 31));
+    }
+    out_pos += __shfl(incl, SAH_WAVE - 1);
+  }
+  __syncthreads();
+  for (int i = tid; i < R.n_words; i += HSW_NT) bm[i] = s_bm[i];
+  if (tid == 0) R.cnt[r] = cnt0 + total_out;
+}
+

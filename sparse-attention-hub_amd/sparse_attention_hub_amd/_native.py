@@ -35,6 +35,7 @@ EXPECTED_SYMBOLS = (
     "sah_hash_signatures_pair",
     "sah_hamming_topk",
     "sah_hamming_scores",
+    "sah_hash_decode_topk",
     "sah_qk_scores",
     "sah_select_topk",
     "sah_pq_kmeans_assign",
@@ -259,12 +260,26 @@ class AttentionArgs(C.Structure):
     ]
 
 
+class HashDecodeArgs(C.Structure):
+    _fields_ = [
+        ("rows", Rows),
+        ("sink", C.c_int32), ("window", C.c_int32),
+        ("query_sig", C.c_void_p),
+        ("key_sig", C.c_void_p),
+        ("kcodes", C.c_void_p),
+        ("code_pitch", C.c_int64),
+        ("k", C.c_int32),
+        ("stream", C.c_void_p),
+    ]
+
+
 class ChainArgs(C.Structure):
     _fields_ = [
         ("sink_local", C.c_void_p),
         ("sig_a", C.c_void_p),
         ("sig_b", C.c_void_p),
         ("hamming", C.c_void_p),
+        ("hash_decode", C.c_void_p),
         ("qk", C.c_void_p),
         ("pq_assign", C.c_void_p),
         ("pq_adc", C.c_void_p),

@@ -84,6 +84,7 @@ class DecodePlan:
         self.layers: Dict[int, _LayerBlocks] = {}
         self.sink_local = N.SinkLocalArgs()
         self.hamming = N.HammingTopkArgs()
+        self.hash_decode = N.HashDecodeArgs()
         self.qk = N.QkScoresArgs()
         self.pq_assign = N.PqAssignArgs()
         self.pq_adc = N.PqAdcArgs()
@@ -148,6 +149,7 @@ class DecodePlan:
         sl.rows, sl.lq, sl.sink, sl.window, sl.fresh, sl.clear_future, sl.stream = rows, Lq, sink, window, 1, 1, stream
         chain.sink_local = C.addressof(sl)
         chain.sig_a = chain.sig_b = chain.hamming = chain.qk = chain.pq_assign = chain.pq_adc = chain.select = None
+        chain.hash_decode = None
 
         if self.kind == "hash":
             cache = sparse_meta_data.get("key", {}).get(layer_idx)
@@ -178,10 +180,19 @@ class DecodePlan:
             bq.x = q.data_ptr()
             bq.xs_b, bq.xs_h, bq.xs_l, bq.stream = q.stride(0), q.stride(1), q.stride(2), stream
             chain.sig_b = C.addressof(bq)
-            hm = self.hamming
-            hm.rows, hm.kcodes, hm.code_pitch = rows, cache.codes.data_ptr(), cache.capacity
-            hm.qcodes, hm.lq, hm.k, hm.stream = self.qcodes.data_ptr(), Lq, k_eff, stream
-            chain.hamming = C.addressof(hm)
+            if Lq == 1 and n_new <= 1:
+                # the whole mask-building half of the step as one entry point (one kernel when shapes allow)
+                hd = self.hash_decode
+                hd.rows, hd.sink, hd.window = rows, sink, window
+                hd.query_sig, hd.key_sig = chain.sig_b, chain.sig_a
+                hd.kcodes, hd.code_pitch, hd.k, hd.stream = cache.codes.data_ptr(), cache.capacity, k_eff, stream
+                chain.hash_decode = C.addressof(hd)
+                chain.sink_local = chain.sig_a = chain.sig_b = None
+            else:
+                hm = self.hamming
+                hm.rows, hm.kcodes, hm.code_pitch = rows, cache.codes.data_ptr(), cache.capacity
+                hm.qcodes, hm.lq, hm.k, hm.stream = self.qcodes.data_ptr(), Lq, k_eff, stream
+                chain.hamming = C.addressof(hm)
             cache.n = Lk
         elif self.kind == "oracle":
             self._ensure_keybuf(Lk)

@@ -54,6 +54,7 @@ class PackedSignatureCache:
     def __init__(self, batch: int, heads: int, bits: int, capacity: int, device: torch.device):
         self.bits = bits
         self.n = 0
+        capacity = (capacity + 63) // 64 * 64  # rows of codes stay 16-byte aligned for the vector loads
         self.codes = torch.empty((batch, heads, capacity, 2), dtype=torch.int32, device=device)
 
     @property
@@ -67,7 +68,7 @@ class PackedSignatureCache:
     def reserve(self, n_total: int) -> None:
         if n_total <= self.capacity:
             return
-        new_cap = max(n_total + 4096, 2 * self.capacity)
+        new_cap = (max(n_total + 4096, 2 * self.capacity) + 63) // 64 * 64
         grown = torch.empty((self.codes.shape[0], self.codes.shape[1], new_cap, 2), dtype=torch.int32, device=self.codes.device)
         if self.n:
             grown[:, :, : self.n] = self.codes[:, :, : self.n]

@@ -342,6 +342,49 @@ def test_decode_plan_matches_masker_by_masker_path(cuda, kind):
     assert plan.att.out is not None and plan.att.Lk == Lk + 3     # the last step went through the plan
 
 
+
+@pytest.mark.parametrize("dtype,Lk", [(torch.bfloat16, 32768), (torch.float16, 5000), (torch.float32, 3001)])
+def test_fused_hash_decode_kernel_matches_separate_launches(cuda, dtype, Lk):
+    """Sink + Local + HashAttention decode steps through the single fused kernel (sink/local rows, both signature
+    MLPs, signature top-k) against the masker-by-masker path: same outputs, same signature cache, bit for bit,
+    at the headline shape (32 query heads, 8 KV heads, 32768 keys, top-2048) and at ragged sizes."""
+    from sparse_attention_hub_amd import _native as N
+
+    sa = _sa()
+    B, Hq, Hkv, D = 2, 32, 8, 128
+    heavy = 2048 if Lk > 8192 else 300
+    q, k, v = make_qkv(B, Hq, Hkv, 1, Lk + 3, D, dtype, seed=3)
+    cfgs = [sa.SinkMaskerConfig(sink_size=128), sa.LocalMaskerConfig(window_size=512),
+            sa.HashAttentionTopKMaskerConfig(heavy_size=heavy, hat_bits=32, hat_mlp_layers=3, hat_mlp_hidden_size=128,
+                                             hat_mlp_activation="silu", hat_weights=_hat(sa, Hq, D, dtype, hidden=128))]
+    fast = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=cfgs))
+    fast.return_attention_weights = False
+    ref = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=cfgs))
+    m1, m2 = {}, {}
+    kc, vc = k.to(cuda), v.to(cuda)
+    for step in range(3):
+        n = Lk + step
+        qq = make_qkv(B, Hq, Hkv, 1, 1, D, dtype, seed=70 + step)[0].to(cuda)
+        if step == 2:
+            N.timing_enable(True)
+        o1, _ = fast.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m1, layer_idx=0)
+        if step == 2:
+            torch.cuda.synchronize()
+            names = set(N.timing_collect())
+            N.timing_enable(False)
+            assert "k_hash_decode" in names and "k_hamming_topk" not in names and "k_sink_local" not in names, names
+        o2, _ = ref.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m2, layer_idx=0)
+        assert torch.equal(o1, o2), f"step {step}"
+        assert torch.equal(m1["key"][0].codes[:, :, :n], m2["key"][0].codes[:, :, :n]), f"cache, step {step}"
+    # the rows the fused kernel built: sink + local + top-k entries, all distinct
+    plan = next(iter(fast._plans.values()))
+    cnt = plan.cnt.cpu()
+    assert bool((cnt == 128 + 512 + heavy).all())
+    cols = plan.cols[:, : 128 + 512 + heavy].long()
+    srt = torch.sort(cols, dim=1).values
+    assert bool((srt[:, 1:] != srt[:, :-1]).all()) and int(cols.min()) == 0 and int(cols.max()) == Lk + 2 - 1
+
+
 # ------------------------------------------------------------------------ adaptive sampling
 def _adaptive_case(cuda, pre_cfgs, pre_specs, rate, eps, delta, io, lo, B, Hq, Hkv, Lq, Lk, D, dtype, amask=None,
                    seed=1234, outliers=False):
