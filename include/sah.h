@@ -332,7 +332,8 @@ int sah_pq_adc_scores(const sah_pq_adc_args* a);
  * (contiguous (B, Lq, Hq, D)). With dense != 0 the rows are ignored and every
  * column j < Lk is used with weight 1 (the reference's treatment of an empty
  * or full Mask, utils/mask.py:733-735).
- * work: fp32 scratch of sah_sparse_attention_work_floats(...) floats.
+ * work: fp32 scratch of sah_sparse_attention_work_floats(...) floats (0 when whole
+ * rows are handled by one workgroup each; work may then be NULL).
  * logits_out (optional, fp32 [n_rows, cap]) receives z[j] per entry and
  * stats_out (optional, fp32 [n_rows, 2]) the final (m, den) so that the dense
  * attention-weight tensor can be produced by sah_attention_weights.
@@ -465,6 +466,8 @@ int sah_adaptive_sample(const sah_adaptive_sample_args* a);
  * codes. When shapes allow (16-byte aligned code streams, layer widths powers of
  * two with d_in * d_out a multiple of 4096, the new key inside the local window)
  * everything runs in one kernel, otherwise as the three launches above.
+ * A caller that consumes only the column lists (the attention kernel does) may
+ * set skip_bitmap and save the write-back of the bitmap rows.
  * ------------------------------------------------------------------------- */
 typedef struct sah_hash_decode_args {
   sah_rows rows;
@@ -474,6 +477,7 @@ typedef struct sah_hash_decode_args {
   const uint32_t* kcodes;
   int64_t code_pitch;
   int32_t k;
+  int32_t skip_bitmap;                  /* != 0: rows.bitmap may be left stale (cols and cnt are complete) */
   void* stream;
 } sah_hash_decode_args;
 int sah_hash_decode_topk(const sah_hash_decode_args* a);

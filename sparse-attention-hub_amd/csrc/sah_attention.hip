@@ -13,6 +13,7 @@
 
 #define ATT_NT 256
 #define ATT_NW (ATT_NT / SAH_WAVE)
+#define ATT_ROW_NT 1024  // threads of the whole-row form
 #define ATT_CHUNK (ATT_NT)  // keys per workgroup iteration: 64 per wave
 #define ATT_XCDS 8           // accelerator complex dies of an MI355X, one L2 each
 #define ATT_MAX_SPLIT 64
@@ -27,6 +28,9 @@ struct att_params {
   float scaling, unit_inv_w;
   int dense;
   int n_split;
+  const float* sinks;
+  void* out;
+  float* stats;
   float* work;
   float* logits_out;
   int64_t logits_pitch;
@@ -88,195 +92,13 @@ __device__ __forceinline__ void att_unpack(const att_raw<DT>& r, float (&o)[8]) 
 // Each wave keeps its own online-softmax state (m uniform across the wave, l and acc
 // per lane group) and walks its 64-key slices in batches of UB iterations; the K and V
 // rows of a batch are requested together so 2*UB row loads are in flight per lane.
-template <int DT, int D>
-__global__ __launch_bounds__(ATT_NT, 5) void k_sparse_attn(att_params P) {
-  constexpr int LPK = D / 8;            // lanes per key
-  constexpr int KPI = SAH_WAVE / LPK;   // keys per wave iteration
-  constexpr int IT = SAH_WAVE / KPI;    // iterations per 64-key wave slice (== LPK)
-  constexpr int UB = IT < 4 ? IT : 4;   // iterations per batch
-  constexpr int ES = (DT == SAH_F32) ? 4 : 2;
-
-  __shared__ float s_m[ATT_NW];
-  __shared__ float s_l[ATT_NW];
-  __shared__ float s_acc[ATT_NW][D];
-
-  // Workgroup -> work mapping. The hardware deals consecutive workgroup ids round-robin to the 8
-  // XCDs, each with its own L2. A tile is (GQA group, split); tile t runs on XCD t % 8 and the G
-  // query heads of the group take adjacent slots of that XCD, so the K/V rows they have in common
-  // (all sink/local rows, every row in dense mode) are fetched from HBM once and shared in L2,
-  // while every XCD gets the same number of tiles.
-  const int G = P.Hq / P.Hkv;
-  const int slot = blockIdx.x / ATT_XCDS;
-  const int tile = (slot / G) * ATT_XCDS + (int)(blockIdx.x % ATT_XCDS);
-  const int n_groups = P.rows.n_rows / G;
-  if (tile >= n_groups * P.n_split) return;  // padding to a multiple of 8 tiles
-  const int split = tile % P.n_split;
-  const int gidx = tile / P.n_split;          // (b * Hkv + hk) * Lq + qi
-  const int qi = gidx % P.Lq;
-  const int hk = (gidx / P.Lq) % P.Hkv;
-  const int b = gidx / (P.Lq * P.Hkv);
-  const int h = hk * G + slot % G;
-  const int r = (b * P.Hq + h) * P.Lq + qi;
-  const int tid = threadIdx.x;
-  const int lane = tid & (SAH_WAVE - 1);
-  const int wave = tid / SAH_WAVE;
-  const int sub = lane % LPK;   // which 8-element slice of the row
-  const int grp = lane / LPK;   // which key of the iteration
-
-  int cnt = P.dense ? P.Lk : P.rows.cnt[r];
-  if (!P.dense && cnt > P.rows.cap) cnt = P.rows.cap;
-  // the row's own entry count decides its slices, so rows of very different lengths all spread over the
-  // splits evenly; the host picks n_split from an upper bound only
-  const int row_chunks = (cnt + ATT_CHUNK - 1) / ATT_CHUNK;
-  const int kps = ((row_chunks + P.n_split - 1) / P.n_split) * ATT_CHUNK;
-  const int begin = split * kps;
-  int end = begin + kps;
-  if (end > cnt) end = cnt;
-
-  float* wout = P.work + ((int64_t)r * P.n_split + split) * (D + 2);
-  if (begin >= end) {
-    if (tid == 0) {
-      wout[0] = -INFINITY;
-      wout[1] = 0.f;
-    }
-    return;
-  }
-
-  const int* cols = P.dense ? nullptr : P.rows.cols + (int64_t)r * P.rows.cap;
-  const float* wts = (!P.dense && P.rows.w) ? P.rows.w + (int64_t)r * P.rows.cap : nullptr;
-  const char* kbase = (const char*)P.k + ((int64_t)b * P.ks_b + (int64_t)hk * P.ks_h + sub * 8) * ES;
-  const char* vbase = (const char*)P.v + ((int64_t)b * P.vs_b + (int64_t)hk * P.vs_h + sub * 8) * ES;
-  const int64_t krow = P.ks_l * ES, vrow = P.vs_l * ES;
-  const int64_t moff = P.amask ? ((int64_t)b * P.ms_b + (int64_t)h * P.ms_h + (int64_t)qi * P.ms_l) : 0;
-
-  float qv[8];
-  sah_load8<DT>(P.q, (int64_t)b * P.qs_b + (int64_t)h * P.qs_h + (int64_t)qi * P.qs_l + sub * 8, qv);
-
-  float acc[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-  float l_run = 0.f;
-  float m_run = -INFINITY;
-
-  for (int cbase = begin + wave * SAH_WAVE; cbase < end; cbase += ATT_CHUNK) {
-    // one column (and its inverse weight) per lane: this wave's next 64 keys
-    const int my = cbase + lane;
-    int idx_l = -1;
-    float invw_l = P.unit_inv_w;
-    if (my < end) {
-      idx_l = P.dense ? my : cols[my];
-      // the reference evaluates 1/(w + 1e-6) in the mask dtype (utils/mask.py:737-740)
-      if (wts) invw_l = sah_round<DT>(1.0f / sah_round<DT>(wts[my] + 1e-6f));
-      if (idx_l < 0 || idx_l >= P.Lk) idx_l = -1;
-    }
-#pragma unroll
-    for (int ib = 0; ib < IT; ib += UB) {
-      if (cbase + ib * KPI >= end) break;  // uniform across the wave
-      att_raw<DT> kr[UB], vr[UB];
-      int id[UB];
-#pragma unroll
-      for (int u = 0; u < UB; ++u) {
-        id[u] = __shfl(idx_l, (ib + u) * KPI + grp);
-        const int safe = id[u] >= 0 ? id[u] : 0;  // invalid lanes read row 0 and are masked below
-        att_load_raw<DT>(kbase + (int64_t)safe * krow, kr[u]);
-        att_load_raw<DT>(vbase + (int64_t)safe * vrow, vr[u]);
-      }
-      float z[UB];
-      float mb = -INFINITY;
-#pragma unroll
-      for (int u = 0; u < UB; ++u) {
-        float kf[8];
-        att_unpack<DT>(kr[u], kf);
-        float d = 0.f;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) d = fmaf(qv[e], kf[e], d);
-        d = att_group_sum<LPK>(d) * P.scaling;
-        if (id[u] >= 0) {
-          if (P.amask) d += sah_load<DT>(P.amask, moff + id[u]);
-        } else {
-          d = -INFINITY;
-        }
-        z[u] = d;
-        mb = fmaxf(mb, d);
-      }
-      if (P.logits_out && sub == 0) {
-#pragma unroll
-        for (int u = 0; u < UB; ++u) {
-          const int pos = cbase + (ib + u) * KPI + grp;
-          if (pos < end) P.logits_out[(int64_t)r * P.logits_pitch + pos] = z[u];
-        }
-      }
-      // batch max over the lane groups of the wave: m stays uniform across the wave
-#pragma unroll
-      for (int o = LPK; o < SAH_WAVE; o <<= 1) mb = fmaxf(mb, __shfl_xor(mb, o));
-      const float m_new = fmaxf(m_run, mb);
-      if (m_new != -INFINITY) {
-        const float rescale = (m_run == -INFINITY) ? 0.f : att_exp<DT>(m_run - m_new);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[e] *= rescale;
-        l_run *= rescale;
-        m_run = m_new;
-#pragma unroll
-        for (int u = 0; u < UB; ++u) {
-          const float iw = __shfl(invw_l, (ib + u) * KPI + grp);
-          float p = 0.f;
-          if (z[u] != -INFINITY) p = att_exp<DT>(z[u] - m_new) * iw;
-          l_run += p;
-          float vf[8];
-          att_unpack<DT>(vr[u], vf);
-#pragma unroll
-          for (int e = 0; e < 8; ++e) acc[e] = fmaf(p, vf[e], acc[e]);
-        }
-      }
-    }
-  }
-
-  // ---- reduce the KPI lane groups of the wave, then the waves (rescaled to a common max)
-#pragma unroll
-  for (int o = LPK; o < SAH_WAVE; o <<= 1) {
-#pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] += __shfl_xor(acc[e], o);
-    l_run += __shfl_xor(l_run, o);
-  }
-  if (lane < LPK) {
-#pragma unroll
-    for (int e = 0; e < 8; ++e) s_acc[wave][sub * 8 + e] = acc[e];
-  }
-  if (lane == 0) {
-    s_l[wave] = l_run;
-    s_m[wave] = m_run;
-  }
-  __syncthreads();
-  float M = s_m[0];
-#pragma unroll
-  for (int wv = 1; wv < ATT_NW; ++wv) M = fmaxf(M, s_m[wv]);
-  float sc[ATT_NW];
-#pragma unroll
-  for (int wv = 0; wv < ATT_NW; ++wv) sc[wv] = (s_m[wv] == -INFINITY) ? 0.f : att_exp<DT>(s_m[wv] - M);
-  if (tid < D) {
-    float a = 0.f;
-#pragma unroll
-    for (int wv = 0; wv < ATT_NW; ++wv) a = fmaf(s_acc[wv][tid], sc[wv], a);
-    wout[2 + tid] = a;
-  }
-  if (tid == 0) {
-    float l = 0.f;
-#pragma unroll
-    for (int wv = 0; wv < ATT_NW; ++wv) l = fmaf(s_l[wv], sc[wv], l);
-    wout[0] = M;
-    wout[1] = l;
-  }
-}
-
 // merge the splits of one row: out = sum_s acc_s e^(m_s-M) / sum_s l_s e^(m_s-M).
 // The (m, l) pairs go through LDS and each thread's partial values are requested together,
-// so the kernel costs about two memory round trips whatever the number of splits.
+// so the merge costs about two memory round trips whatever the number of splits. Every thread of the
+// workgroup calls it (one barrier inside); thread d < D produces output element d.
 template <int DT, int D>
-__global__ __launch_bounds__(D < 64 ? 64 : D) void k_attn_combine(const float* work, int n_split, int Hq, int Lq,
-                                                                  const float* sinks, void* out, float* stats) {
-  __shared__ float s_m[ATT_MAX_SPLIT];
-  __shared__ float s_l[ATT_MAX_SPLIT];
-  const int r = blockIdx.x;
+__device__ __forceinline__ void att_combine_row(const float* work, int n_split, int r, int Hq, int Lq, const float* sinks,
+                                                void* out, float* stats, float* s_m, float* s_l) {
   const int d = threadIdx.x;
   const float* w = work + (int64_t)r * n_split * (D + 2);
   if (d < n_split) {
@@ -322,6 +144,226 @@ __global__ __launch_bounds__(D < 64 ? 64 : D) void k_attn_combine(const float* w
   }
 }
 
+// ROW = false: a workgroup of 4 waves handles one (row, split) tile and leaves (m, l, acc) in the workspace
+//   for the merge kernel - the form for few or very uneven rows.
+// ROW = true: a workgroup of 16 waves handles a whole row, every wave an equal share of the row's entries,
+//   and merges the 16 partial results itself: no workspace, no second kernel, every CU gets the same
+//   amount of work when there are at least as many rows as CUs.
+template <int DT, int D, bool ROW>
+__global__ __launch_bounds__(ROW ? ATT_ROW_NT : ATT_NT, ROW ? 1 : 5) void k_sparse_attn(att_params P) {
+  constexpr int NW = (ROW ? ATT_ROW_NT : ATT_NT) / SAH_WAVE;
+  constexpr int LPK = D / 8;            // lanes per key
+  constexpr int KPI = SAH_WAVE / LPK;   // keys per wave iteration
+  constexpr int IT = SAH_WAVE / KPI;    // iterations per 64-key wave slice (== LPK)
+  constexpr int UB = IT < 4 ? IT : 4;   // iterations per batch
+  constexpr int ES = (DT == SAH_F32) ? 4 : 2;
+
+  __shared__ float s_m[NW];
+  __shared__ float s_l[NW];
+  __shared__ float s_acc[NW][D];
+
+  // Workgroup -> work mapping. The hardware deals consecutive workgroup ids round-robin to the 8
+  // XCDs, each with its own L2. A tile is (GQA group, split); tile t runs on XCD t % 8 and the G
+  // query heads of the group take adjacent slots of that XCD, so the K/V rows they have in common
+  // (all sink/local rows, every row in dense mode) are fetched from HBM once and shared in L2,
+  // while every XCD gets the same number of tiles.
+  const int G = P.Hq / P.Hkv;
+  const int slot = blockIdx.x / ATT_XCDS;
+  const int tile = (slot / G) * ATT_XCDS + (int)(blockIdx.x % ATT_XCDS);
+  const int n_groups = P.rows.n_rows / G;
+  const int n_split = ROW ? 1 : P.n_split;
+  if (tile >= n_groups * n_split) return;  // padding to a multiple of 8 tiles
+  const int split = tile % n_split;
+  const int gidx = tile / n_split;            // (b * Hkv + hk) * Lq + qi
+  const int qi = gidx % P.Lq;
+  const int hk = (gidx / P.Lq) % P.Hkv;
+  const int b = gidx / (P.Lq * P.Hkv);
+  const int h = hk * G + slot % G;
+  const int r = (b * P.Hq + h) * P.Lq + qi;
+  const int tid = threadIdx.x;
+  const int lane = tid & (SAH_WAVE - 1);
+  const int wave = tid / SAH_WAVE;
+  const int sub = lane % LPK;   // which 8-element slice of the row
+  const int grp = lane / LPK;   // which key of the iteration
+
+  int cnt = P.dense ? P.Lk : P.rows.cnt[r];
+  if (!P.dense && cnt > P.rows.cap) cnt = P.rows.cap;
+  // the row's own entry count decides the slices, so rows of very different lengths all spread evenly;
+  // the host picks n_split from an upper bound only
+  int first, bound, stride;  // this wave's slices start at first, first + stride, ... and stop at bound
+  float* wout = nullptr;
+  if constexpr (ROW) {
+    const int per = (((cnt + NW - 1) / NW) + KPI - 1) / KPI * KPI;  // entries per wave
+    first = wave * per;
+    bound = first + per < cnt ? first + per : cnt;
+    stride = SAH_WAVE;
+  } else {
+    const int row_chunks = (cnt + ATT_CHUNK - 1) / ATT_CHUNK;
+    const int kps = ((row_chunks + n_split - 1) / n_split) * ATT_CHUNK;
+    const int begin = split * kps;
+    bound = begin + kps < cnt ? begin + kps : cnt;
+    first = begin + wave * SAH_WAVE;
+    stride = ATT_CHUNK;
+    wout = P.work + ((int64_t)r * n_split + split) * (D + 2);
+    if (begin >= bound) {
+      if (tid == 0) {
+        wout[0] = -INFINITY;
+        wout[1] = 0.f;
+      }
+      return;
+    }
+  }
+
+  const int* cols = P.dense ? nullptr : P.rows.cols + (int64_t)r * P.rows.cap;
+  const float* wts = (!P.dense && P.rows.w) ? P.rows.w + (int64_t)r * P.rows.cap : nullptr;
+  const char* kbase = (const char*)P.k + ((int64_t)b * P.ks_b + (int64_t)hk * P.ks_h + sub * 8) * ES;
+  const char* vbase = (const char*)P.v + ((int64_t)b * P.vs_b + (int64_t)hk * P.vs_h + sub * 8) * ES;
+  const int64_t krow = P.ks_l * ES, vrow = P.vs_l * ES;
+  const int64_t moff = P.amask ? ((int64_t)b * P.ms_b + (int64_t)h * P.ms_h + (int64_t)qi * P.ms_l) : 0;
+
+  float qv[8];
+  sah_load8<DT>(P.q, (int64_t)b * P.qs_b + (int64_t)h * P.qs_h + (int64_t)qi * P.qs_l + sub * 8, qv);
+
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  float l_run = 0.f;
+  float m_run = -INFINITY;
+
+  for (int cbase = first; cbase < bound; cbase += stride) {
+    // one column (and its inverse weight) per lane: this wave's next 64 keys
+    const int my = cbase + lane;
+    int idx_l = -1;
+    float invw_l = P.unit_inv_w;
+    if (my < bound) {
+      idx_l = P.dense ? my : cols[my];
+      // the reference evaluates 1/(w + 1e-6) in the mask dtype (utils/mask.py:737-740)
+      if (wts) invw_l = sah_round<DT>(1.0f / sah_round<DT>(wts[my] + 1e-6f));
+      if (idx_l < 0 || idx_l >= P.Lk) idx_l = -1;
+    }
+#pragma unroll
+    for (int ib = 0; ib < IT; ib += UB) {
+      if (cbase + ib * KPI >= bound) break;  // uniform across the wave
+      att_raw<DT> kr[UB], vr[UB];
+      int id[UB];
+#pragma unroll
+      for (int u = 0; u < UB; ++u) {
+        id[u] = __shfl(idx_l, (ib + u) * KPI + grp);
+        const int safe = id[u] >= 0 ? id[u] : 0;  // invalid lanes read row 0 and are masked below
+        att_load_raw<DT>(kbase + (int64_t)safe * krow, kr[u]);
+        att_load_raw<DT>(vbase + (int64_t)safe * vrow, vr[u]);
+      }
+      float z[UB];
+      float mb = -INFINITY;
+#pragma unroll
+      for (int u = 0; u < UB; ++u) {
+        float kf[8];
+        att_unpack<DT>(kr[u], kf);
+        float d = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) d = fmaf(qv[e], kf[e], d);
+        d = att_group_sum<LPK>(d) * P.scaling;
+        if (id[u] >= 0) {
+          if (P.amask) d += sah_load<DT>(P.amask, moff + id[u]);
+        } else {
+          d = -INFINITY;
+        }
+        z[u] = d;
+        mb = fmaxf(mb, d);
+      }
+      if (P.logits_out && sub == 0) {
+#pragma unroll
+        for (int u = 0; u < UB; ++u) {
+          const int pos = cbase + (ib + u) * KPI + grp;
+          if (pos < bound) P.logits_out[(int64_t)r * P.logits_pitch + pos] = z[u];
+        }
+      }
+      // batch max over the lane groups of the wave: m stays uniform across the wave
+#pragma unroll
+      for (int o = LPK; o < SAH_WAVE; o <<= 1) mb = fmaxf(mb, __shfl_xor(mb, o));
+      const float m_new = fmaxf(m_run, mb);
+      if (m_new != -INFINITY) {
+        const float rescale = (m_run == -INFINITY) ? 0.f : att_exp<DT>(m_run - m_new);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] *= rescale;
+        l_run *= rescale;
+        m_run = m_new;
+#pragma unroll
+        for (int u = 0; u < UB; ++u) {
+          const float iw = __shfl(invw_l, (ib + u) * KPI + grp);
+          float p = 0.f;
+          if (z[u] != -INFINITY) p = att_exp<DT>(z[u] - m_new) * iw;
+          l_run += p;
+          float vf[8];
+          att_unpack<DT>(vr[u], vf);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[e] = fmaf(p, vf[e], acc[e]);
+        }
+      }
+    }
+  }
+
+  // ---- reduce the KPI lane groups of the wave, then the waves (rescaled to a common max)
+#pragma unroll
+  for (int o = LPK; o < SAH_WAVE; o <<= 1) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] += __shfl_xor(acc[e], o);
+    l_run += __shfl_xor(l_run, o);
+  }
+  if (lane < LPK) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s_acc[wave][sub * 8 + e] = acc[e];
+  }
+  if (lane == 0) {
+    s_l[wave] = l_run;
+    s_m[wave] = m_run;
+  }
+  __syncthreads();
+  float M = s_m[0];
+#pragma unroll
+  for (int wv = 1; wv < NW; ++wv) M = fmaxf(M, s_m[wv]);
+  float sc[NW];
+#pragma unroll
+  for (int wv = 0; wv < NW; ++wv) sc[wv] = (s_m[wv] == -INFINITY) ? 0.f : att_exp<DT>(s_m[wv] - M);
+  float a = 0.f, l = 0.f;
+  if (tid < D) {
+#pragma unroll
+    for (int wv = 0; wv < NW; ++wv) a = fmaf(s_acc[wv][tid], sc[wv], a);
+  }
+#pragma unroll
+  for (int wv = 0; wv < NW; ++wv) l = fmaf(s_l[wv], sc[wv], l);
+  if constexpr (ROW) {
+    // the row is complete: normalise (with the optional sink logit, mask_attention_utils.py:357-402) and store
+    float Mf = M, den = l;
+    if (P.sinks) {
+      const float sk = P.sinks[h];
+      Mf = fmaxf(M, sk);
+      const float rs = (M == -INFINITY) ? 0.f : att_exp<DT>(M - Mf);
+      a *= rs;
+      den = l * rs + att_exp<DT>(sk - Mf);
+    }
+    if (tid < D) sah_store<DT>(P.out, (((int64_t)b * P.Lq + qi) * P.Hq + h) * D + tid, a / den);
+    if (P.stats && tid == 0) {
+      P.stats[2 * (int64_t)r] = Mf;
+      P.stats[2 * (int64_t)r + 1] = den;
+    }
+  } else {
+    if (tid < D) wout[2 + tid] = a;
+    if (tid == 0) {
+      wout[0] = M;
+      wout[1] = l;
+    }
+  }
+}
+
+template <int DT, int D>
+__global__ __launch_bounds__(D < 64 ? 64 : D) void k_attn_combine(const float* work, int n_split, int Hq, int Lq,
+                                                                  const float* sinks, void* out, float* stats) {
+  __shared__ float s_m[ATT_MAX_SPLIT];
+  __shared__ float s_l[ATT_MAX_SPLIT];
+  att_combine_row<DT, D>(work, n_split, blockIdx.x, Hq, Lq, sinks, out, stats, s_m, s_l);
+}
+
 template <int DT>
 __global__ __launch_bounds__(256) void k_attn_weights(sah_rows R, const float* logits, int64_t pitch,
                                                       const float* stats, float unit_inv_w, int dense, void* weights) {
@@ -344,6 +386,12 @@ __global__ __launch_bounds__(256) void k_attn_weights(sah_rows R, const float* l
   sah_store<DT>(weights, (int64_t)r * R.n_keys + c, p);
 }
 
+// Whole-row form when every CU can be given rows of its own (or the rows are so short that splitting them
+// only adds a second launch), and rows are not long enough for their spread in length to matter.
+static bool att_use_row_form(int n_rows, int max_cnt) {
+  return max_cnt <= 8192 && (n_rows >= 192 || max_cnt <= 1024);
+}
+
 // Splits per row, from an upper bound of the row lengths: enough workgroups to cover 256 CUs several times,
 // at least one chunk and at most 16 chunks of keys each (the kernel divides every row's own length by it).
 static int att_pick_split(int n_rows, int max_cnt) {
@@ -360,6 +408,7 @@ static int att_pick_split(int n_rows, int max_cnt) {
 
 extern "C" int64_t sah_sparse_attention_work_floats(int32_t n_rows, int32_t max_cnt, int32_t D) {
   if (n_rows <= 0 || max_cnt < 0 || D <= 0) return 0;
+  if (att_use_row_form(n_rows, max_cnt)) return 0;
   int n_split = att_pick_split(n_rows, max_cnt);
   return (int64_t)n_rows * n_split * (D + 2);
 }
@@ -367,13 +416,20 @@ extern "C" int64_t sah_sparse_attention_work_floats(int32_t n_rows, int32_t max_
 template <int DT, int D>
 static int att_launch(const sah_attention_args* a, const att_params& P) {
   hipStream_t st = (hipStream_t)a->stream;
+  const int G = a->Hq / a->Hkv;
+  if (P.n_split == 0) {  // whole-row form
+    sah_timed timed("k_sparse_attn", a->stream);
+    const int n_tiles = a->rows.n_rows / G;
+    const int n_wg = (n_tiles + ATT_XCDS - 1) / ATT_XCDS * ATT_XCDS * G;
+    hipLaunchKernelGGL((k_sparse_attn<DT, D, true>), dim3(n_wg), dim3(ATT_ROW_NT), 0, st, P);
+    return sah_launch_status("sah_sparse_attention");
+  }
   int rc;
   {
     sah_timed timed("k_sparse_attn", a->stream);
-    const int G = a->Hq / a->Hkv;
     const int n_tiles = (a->rows.n_rows / G) * P.n_split;
     const int n_wg = (n_tiles + ATT_XCDS - 1) / ATT_XCDS * ATT_XCDS * G;
-    hipLaunchKernelGGL((k_sparse_attn<DT, D>), dim3(n_wg), dim3(ATT_NT), 0, st, P);
+    hipLaunchKernelGGL((k_sparse_attn<DT, D, false>), dim3(n_wg), dim3(ATT_NT), 0, st, P);
     rc = sah_launch_status("sah_sparse_attention");
   }
   if (rc) return rc;
@@ -396,7 +452,7 @@ static int att_dispatch_d(const sah_attention_args* a, const att_params& P) {
 
 extern "C" int sah_sparse_attention(const sah_attention_args* a) {
   if (!a) return sah_fail(SAH_ENULL, "sah_sparse_attention: args is NULL");
-  if (!a->q || !a->k || !a->v || !a->out || !a->work) return sah_fail(SAH_ENULL, "sah_sparse_attention: NULL tensor");
+  if (!a->q || !a->k || !a->v || !a->out) return sah_fail(SAH_ENULL, "sah_sparse_attention: NULL tensor");
   if (a->B <= 0 || a->Hq <= 0 || a->Hkv <= 0 || a->Lq <= 0 || a->Lk <= 0)
     return sah_fail(SAH_EINVAL, "sah_sparse_attention: non-positive dimension");
   if (a->Hq % a->Hkv) return sah_fail(SAH_EINVAL, "sah_sparse_attention: Hq %% Hkv != 0");
@@ -426,8 +482,9 @@ extern "C" int sah_sparse_attention(const sah_attention_args* a) {
   P.Hq = a->Hq; P.Hkv = a->Hkv; P.Lq = a->Lq; P.Lk = a->Lk;
   P.scaling = a->scaling; P.unit_inv_w = a->unit_inv_w;
   P.dense = a->dense ? 1 : 0;
-  P.n_split = att_pick_split(a->rows.n_rows, max_cnt);
+  P.n_split = att_use_row_form(a->rows.n_rows, max_cnt) ? 0 : att_pick_split(a->rows.n_rows, max_cnt);  // 0: whole rows
   P.work = a->work;
+  P.sinks = a->sinks; P.out = a->out; P.stats = a->stats_out;
   P.logits_out = a->logits_out;
   P.logits_pitch = a->dense ? a->Lk : a->rows.cap;
   const int64_t need = (int64_t)a->rows.n_rows * P.n_split * (a->D + 2);

@@ -29,6 +29,7 @@ struct hdec_params {
   int64_t pitch;
   int k;
   int sink, window;
+  int update_bitmap;
 };
 
 template <int DT>
@@ -77,7 +78,7 @@ __global__ __launch_bounds__(HSW_NT) void k_hash_decode(hdec_params P) {
   __syncthreads();  // every thread holds q (and the bitmap is complete) before the scores overwrite the scratch
 
   // ---- 3. top-k over the remaining columns
-  hsw_select_row(R, r, P.kcodes + (int64_t)r * P.pitch, q, P.k, fixed < R.cap ? fixed : R.cap, s_bm, s_key, S);
+  hsw_select_row(R, r, P.kcodes + (int64_t)r * P.pitch, q, P.k, fixed < R.cap ? fixed : R.cap, s_bm, s_key, S, P.update_bitmap != 0);
 }
 
 static size_t hdec_lds_bytes(int n_keys) {
@@ -164,6 +165,7 @@ extern "C" int sah_hash_decode_topk(const sah_hash_decode_args* a) {
   P.k = a->k;
   P.sink = a->sink;
   P.window = a->window;
+  P.update_bitmap = a->skip_bitmap ? 0 : 1;
   const size_t lds = hdec_lds_bytes(a->rows.n_keys);
   switch (a->query_sig->dtype) {
     case SAH_F32: return hdec_launch<SAH_F32>(a, P, lds);

@@ -18,9 +18,10 @@ __device__ __forceinline__ int sig_score(uint2 q, uint2 k) {
 //   P1  the threshold T: P0 has already counted the columns at or above 8 coarse thresholds, one more
 //       pass over the staged bytes counts 7 fine ones inside the bracket (byte-parallel compares, no atomics);
 //   P2  per-wave counts of "above T" and "equal T";
-//   P3  ordered write: wave scan of per-lane counts, up to 4 columns per lane, ties taken
-//       lowest column first until `need` are used; new bits are OR-ed into the LDS copy of
-//       the bitmap row, which is written back once at the end.
+//   P3  write: one wave scan of per-lane totals, every lane appends the columns of its chunks; ties are
+//       taken lowest column first until `need` are used (the one wave where the budget runs out walks
+//       its chunks in column order); new bits are OR-ed into the LDS copy of the bitmap row, which is
+//       written back once at the end.
 // Active columns hold byte 0 and T >= 1 whenever k inactive columns exist, so P2/P3 never
 // look at the bitmap again.
 // ---------------------------------------------------------------------------
@@ -50,10 +51,10 @@ __host__ __device__ inline size_t hsw_lds_bytes(int n_keys) {
 
 // Top-k of row r over the not-yet-active columns. On entry `s_bm` (n_ch * 8 words of dynamic LDS, zero
 // padded) holds the row's bitmap and every thread of the workgroup has passed a barrier after it was
-// written; cnt0 entries of R.cols are already in place. On exit the selected columns are appended, the
-// bitmap row (LDS copy and global) and cnt are updated.
+// written; cnt0 entries of R.cols are already in place. On exit the selected columns are appended (in no
+// particular order) and cnt is updated; with update_bitmap also the bitmap row (LDS copy and global).
 __device__ __forceinline__ void hsw_select_row(const sah_rows& R, int r, const uint2* kc, const uint2 q, int k, int cnt0,
-                                               uint32_t* s_bm, uint32_t* s_key, hsw_lds& S) {
+                                               uint32_t* s_bm, uint32_t* s_key, hsw_lds& S, bool update_bitmap = true) {
   int* s_gt = S.gt;
   int* s_eq = S.eq;
   const int tid = threadIdx.x;
@@ -175,16 +176,16 @@ __device__ __forceinline__ void hsw_select_row(const sah_rows& R, int r, const u
   // T == 0: fewer than k inactive columns exist; take them all, byte-0 "ties" emit nothing
   const int need = (T == 0) ? 0 : k - above;
 
-  // ---- P2: per-wave counts ---------------------------------------------------------
-  int n_gt = 0, n_eq = 0;
+  // ---- P2: per-lane and per-wave counts ---------------------------------------------
+  int lane_gt = 0, lane_eq = 0;
   for (int c = my_c0; c < my_c1; ++c) {
     const uint32_t w = s_key[c * SAH_WAVE + lane];
     const uint32_t g = swar_ge(w, T + 1);
-    n_gt += __popc(g);
-    n_eq += __popc(swar_ge(w, T) & ~g);
+    lane_gt += __popc(g);
+    lane_eq += __popc(swar_ge(w, T) & ~g);
   }
-  n_gt = sah_wave_sum_i(n_gt);
-  n_eq = sah_wave_sum_i(n_eq);
+  const int n_gt = sah_wave_sum_i(lane_gt);
+  const int n_eq = sah_wave_sum_i(lane_eq);
   if (lane == 0) {
     s_gt[wave] = n_gt;
     s_eq[wave] = n_eq;
@@ -208,21 +209,51 @@ __device__ __forceinline__ void hsw_select_row(const sah_rows& R, int r, const u
     total_out = out_run;
   }
 
-  // ---- P3: ordered write --------------------------------------------------------------
+  // ---- P3: write ----------------------------------------------------------------------
+  // The list of a row is unordered, so a wave whose ties are all taken or all dropped needs one scan: every
+  // lane writes the columns of all its chunks as one run. Only the wave in which the tie budget runs out
+  // has to walk its chunks in column order to keep the lowest ties.
   int* cols = R.cols + (int64_t)r * R.cap;
   float* wts = R.w ? R.w + (int64_t)r * R.cap : nullptr;
   const bool ties_all = (tie_base + n_eq <= need);   // every tie of this wave is taken
   const bool ties_none = (tie_base >= need);         // none is
-  int out_pos = cnt0 + out_base;
-  int tie_run = tie_base;
-  for (int c = my_c0; c < my_c1; ++c) {
-    const int wi = c * SAH_WAVE + lane;
-    const uint32_t w = s_key[wi];
-    const uint32_t g = swar_ge(w, T + 1) >> 7;            // bits 0, 8, 16, 24
-    uint32_t e = (swar_ge(w, T) >> 7) & ~g;
-    if (ties_none) {
-      e = 0;
-    } else if (!ties_all) {
+  auto emit = [&](uint32_t sel, int wi, int pos) {    // sel: bits 0, 8, 16, 24 = columns 4 * wi + 0..3
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      if (sel & (1u << (8 * t))) {
+        const int at = pos + __popc(sel & ((1u << (8 * t)) - 1u));
+        if (at < R.cap) {
+          cols[at] = wi * 4 + t;
+          if (wts) wts[at] = 1.0f;
+        }
+      }
+    }
+    if (update_bitmap) {
+      const uint32_t nib = ((sel * 0x00204081u) >> 21) & 0xFu;
+      const int j0 = wi * 4;
+      atomicOr(&s_bm[j0 >> 5], nib << (j0 & 31));
+    }
+  };
+  if (ties_all || ties_none) {
+    const int mine = lane_gt + (ties_none ? 0 : lane_eq);
+    int pos = cnt0 + out_base + sah_wave_incl_scan(mine) - mine;
+    for (int c = my_c0; c < my_c1; ++c) {
+      const int wi = c * SAH_WAVE + lane;
+      const uint32_t w = s_key[wi];
+      const uint32_t sel = swar_ge(w, ties_none ? T + 1 : T) >> 7;
+      if (sel) {
+        emit(sel, wi, pos);
+        pos += __popc(sel);
+      }
+    }
+  } else {
+    int out_pos = cnt0 + out_base;
+    int tie_run = tie_base;
+    for (int c = my_c0; c < my_c1; ++c) {
+      const int wi = c * SAH_WAVE + lane;
+      const uint32_t w = s_key[wi];
+      const uint32_t g = swar_ge(w, T + 1) >> 7;
+      uint32_t e = (swar_ge(w, T) >> 7) & ~g;
       const int ne = __popc(e);
       const int before = sah_wave_incl_scan(ne) - ne;     // ties in lower lanes of this chunk
       int allowed = need - (tie_run + before);
@@ -239,30 +270,16 @@ __device__ __forceinline__ void hsw_select_row(const sah_rows& R, int r, const u
         e = kept;
       }
       tie_run += sah_wave_sum_i(ne);
+      const uint32_t sel = g | e;
+      const int ns = __popc(sel);
+      const int incl = sah_wave_incl_scan(ns);
+      if (sel) emit(sel, wi, out_pos + incl - ns);
+      out_pos += __shfl(incl, SAH_WAVE - 1);
     }
-    const uint32_t sel = g | e;
-    const int ns = __popc(sel);
-    const int incl = sah_wave_incl_scan(ns);
-    int pos = out_pos + incl - ns;
-    if (sel) {
-#pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        if (sel & (1u << (8 * t))) {
-          if (pos < R.cap) {
-            cols[pos] = wi * 4 + t;
-            if (wts) wts[pos] = 1.0f;
-          }
-          ++pos;
-        }
-      }
-      const uint32_t nib = ((sel * 0x00204081u) >> 21) & 0xFu;
-      const int j0 = wi * 4;
-      atomicOr(&s_bm[j0 >> 5], nib << (j0 & 31));
-    }
-    out_pos += __shfl(incl, SAH_WAVE - 1);
   }
+  if (tid == 0) R.cnt[r] = cnt0 + total_out;
+  if (!update_bitmap) return;
   __syncthreads();
   for (int i = tid; i < R.n_words; i += HSW_NT) bm[i] = s_bm[i];
-  if (tid == 0) R.cnt[r] = cnt0 + total_out;
 }
 

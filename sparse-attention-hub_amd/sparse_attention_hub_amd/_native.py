@@ -269,6 +269,7 @@ class HashDecodeArgs(C.Structure):
         ("kcodes", C.c_void_p),
         ("code_pitch", C.c_int64),
         ("k", C.c_int32),
+        ("skip_bitmap", C.c_int32),
         ("stream", C.c_void_p),
     ]
 

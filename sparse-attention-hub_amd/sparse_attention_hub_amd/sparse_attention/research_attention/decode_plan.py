@@ -186,6 +186,7 @@ class DecodePlan:
                 hd.rows, hd.sink, hd.window = rows, sink, window
                 hd.query_sig, hd.key_sig = chain.sig_b, chain.sig_a
                 hd.kcodes, hd.code_pitch, hd.k, hd.stream = cache.codes.data_ptr(), cache.capacity, k_eff, stream
+                hd.skip_bitmap = 1  # only the attention kernel reads these rows, and it reads the column lists
                 chain.hash_decode = C.addressof(hd)
                 chain.sink_local = chain.sig_a = chain.sig_b = None
             else:
