@@ -72,13 +72,16 @@ __global__ __launch_bounds__(HSW_NT) void k_hash_decode(hdec_params P) {
   const int Hq = P.job[0].Hq;
   // 2-byte weights: all layers requested up-front; fp32 rows are twice as wide, one layer at a time
   constexpr int PF = (DT == SAH_F32) ? 1 : SAH_MAX_MLP_LAYERS;
+  // the first half of the row's codes is requested behind the MLP's own loads and arrives while it computes
+  hsw_bufs buf;
+  const uint2* kc = P.kcodes + (int64_t)r * P.pitch;
   sig_gemv_block<DT, 1, HDEC_GROUP, HDEC_ROWS, PF>(P.job[job], active, tid % HDEC_GROUP, r / Hq, r % Hq, 0, 1,
-                                                    P.job[0].n_layers, s_sig[job]);
+                                                    P.job[0].n_layers, s_sig[job], [&]() { hsw_prefetch(kc, n, buf); });
   const uint2 q = s_sig[0].code[0];
   __syncthreads();  // every thread holds q (and the bitmap is complete) before the scores overwrite the scratch
 
   // ---- 3. top-k over the remaining columns
-  hsw_select_row(R, r, P.kcodes + (int64_t)r * P.pitch, q, P.k, fixed < R.cap ? fixed : R.cap, s_bm, s_key, S, P.update_bitmap != 0);
+  hsw_select_row(R, r, kc, q, P.k, fixed < R.cap ? fixed : R.cap, s_bm, s_key, S, buf, true, P.update_bitmap != 0);
 }
 
 static size_t hdec_lds_bytes(int n_keys) {

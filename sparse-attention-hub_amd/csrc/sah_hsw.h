@@ -49,12 +49,51 @@ __host__ __device__ inline size_t hsw_lds_bytes(int n_keys) {
   return (size_t)n_ch * 8 * 4 + (size_t)n_ch * 64 * 4;
 }
 
+// Register buffers of the staging pass: two batches of HSW_BATCH chunks (4 codes = 32 B per lane and chunk).
+struct hsw_bufs {
+  uint4 a0[HSW_BATCH], a1[HSW_BATCH], b0[HSW_BATCH], b1[HSW_BATCH];
+};
+
+// wave `wave` stages the chunks [c0, c1) of a row of n columns
+__device__ __forceinline__ void hsw_wave_chunks(int n, int wave, int& c0, int& c1) {
+  const int n_ch = (n + 255) / 256;
+  const int cpw = (n_ch + HSW_NW - 1) / HSW_NW;
+  c0 = wave * cpw;
+  c1 = c0 + cpw;
+  if (c1 > n_ch) c1 = n_ch;
+}
+
+__device__ __forceinline__ void hsw_request(const uint2* kc, int n, int lane, uint4 (&ra)[HSW_BATCH], uint4 (&rb)[HSW_BATCH],
+                                            int c0) {
+#pragma unroll
+  for (int u = 0; u < HSW_BATCH; ++u) {
+    const int j0 = ((c0 + u) * SAH_WAVE + lane) * 4;
+    // clamp to the last full group of 4 codes: out-of-range lanes re-read valid memory
+    int jl = j0;
+    if (jl + 4 > n) jl = n >= 4 ? ((n - 4) & ~1) : 0;
+    const uint4* p = (const uint4*)(kc + jl);
+    ra[u] = p[0];
+    rb[u] = p[1];
+  }
+}
+
+// Requests the first two batches of the calling wave ahead of hsw_select_row(..., prefetched = true): the codes
+// do not depend on the query, so a caller that still has to compute the query code can have them on their way.
+__device__ __forceinline__ void hsw_prefetch(const uint2* kc, int n, hsw_bufs& buf) {
+  const int lane = threadIdx.x & (SAH_WAVE - 1);
+  int c0, c1;
+  hsw_wave_chunks(n, threadIdx.x / SAH_WAVE, c0, c1);
+  if (c0 < c1) hsw_request(kc, n, lane, buf.a0, buf.a1, c0);
+  if (c0 + HSW_BATCH < c1) hsw_request(kc, n, lane, buf.b0, buf.b1, c0 + HSW_BATCH);
+}
+
 // Top-k of row r over the not-yet-active columns. On entry `s_bm` (n_ch * 8 words of dynamic LDS, zero
 // padded) holds the row's bitmap and every thread of the workgroup has passed a barrier after it was
 // written; cnt0 entries of R.cols are already in place. On exit the selected columns are appended (in no
 // particular order) and cnt is updated; with update_bitmap also the bitmap row (LDS copy and global).
 __device__ __forceinline__ void hsw_select_row(const sah_rows& R, int r, const uint2* kc, const uint2 q, int k, int cnt0,
-                                               uint32_t* s_bm, uint32_t* s_key, hsw_lds& S, bool update_bitmap = true) {
+                                               uint32_t* s_bm, uint32_t* s_key, hsw_lds& S, hsw_bufs& buf,
+                                               bool prefetched = false, bool update_bitmap = true) {
   int* s_gt = S.gt;
   int* s_eq = S.eq;
   const int tid = threadIdx.x;
@@ -62,10 +101,8 @@ __device__ __forceinline__ void hsw_select_row(const sah_rows& R, int r, const u
   const int wave = tid / SAH_WAVE;
   const int n = R.n_keys;
   const int n_ch = (n + 255) / 256;            // chunks of 256 columns = 64 words
-  const int cpw = (n_ch + HSW_NW - 1) / HSW_NW;
-  const int my_c0 = wave * cpw;
-  int my_c1 = my_c0 + cpw;
-  if (my_c1 > n_ch) my_c1 = n_ch;
+  int my_c0, my_c1;
+  hsw_wave_chunks(n, wave, my_c0, my_c1);
   uint32_t* bm = R.bitmap + (int64_t)r * R.n_words;
   if (k > n) k = n;
 
@@ -77,18 +114,6 @@ __device__ __forceinline__ void hsw_select_row(const sah_rows& R, int r, const u
   for (int i = 0; i < HSW_PROBES; ++i) pc[i] = 0;
   // Two register buffers of HSW_BATCH chunks each: the next batch is requested before the current one is
   // scored, so the memory pipe stays busy while the ALUs work.
-  auto request = [&](uint4 (&ra)[HSW_BATCH], uint4 (&rb)[HSW_BATCH], int c0) {
-#pragma unroll
-    for (int u = 0; u < HSW_BATCH; ++u) {
-      const int j0 = ((c0 + u) * SAH_WAVE + lane) * 4;
-      // clamp to the last full group of 4 codes: out-of-range lanes re-read valid memory
-      int jl = j0;
-      if (jl + 4 > n) jl = n >= 4 ? ((n - 4) & ~1) : 0;
-      const uint4* p = (const uint4*)(kc + jl);
-      ra[u] = p[0];
-      rb[u] = p[1];
-    }
-  };
   auto score = [&](uint4 (&ra)[HSW_BATCH], uint4 (&rb)[HSW_BATCH], int c0) {
 #pragma unroll
     for (int u = 0; u < HSW_BATCH; ++u) {
@@ -122,16 +147,13 @@ __device__ __forceinline__ void hsw_select_row(const sah_rows& R, int r, const u
       for (int i = 0; i < HSW_PROBES; ++i) pc[i] += __popc((x - (uint32_t)(8 * (i + 1)) * 0x01010101u) & 0x80808080u);
     }
   };
-  {
-    uint4 a0[HSW_BATCH], a1[HSW_BATCH], b0[HSW_BATCH], b1[HSW_BATCH];
-    if (my_c0 < my_c1) request(a0, a1, my_c0);
-    for (int c0 = my_c0; c0 < my_c1; c0 += 2 * HSW_BATCH) {
-      const bool more_b = c0 + HSW_BATCH < my_c1;          // uniform across the wave
-      if (more_b) request(b0, b1, c0 + HSW_BATCH);
-      score(a0, a1, c0);
-      if (c0 + 2 * HSW_BATCH < my_c1) request(a0, a1, c0 + 2 * HSW_BATCH);
-      if (more_b) score(b0, b1, c0 + HSW_BATCH);
-    }
+  if (!prefetched && my_c0 < my_c1) hsw_request(kc, n, lane, buf.a0, buf.a1, my_c0);
+  for (int c0 = my_c0; c0 < my_c1; c0 += 2 * HSW_BATCH) {
+    const bool more_b = c0 + HSW_BATCH < my_c1;          // uniform across the wave
+    if (more_b && !(prefetched && c0 == my_c0)) hsw_request(kc, n, lane, buf.b0, buf.b1, c0 + HSW_BATCH);
+    score(buf.a0, buf.a1, c0);
+    if (c0 + 2 * HSW_BATCH < my_c1) hsw_request(kc, n, lane, buf.a0, buf.a1, c0 + 2 * HSW_BATCH);
+    if (more_b) score(buf.b0, buf.b1, c0 + HSW_BATCH);
   }
 #pragma unroll
   for (int i = 0; i < HSW_PROBES; ++i) {

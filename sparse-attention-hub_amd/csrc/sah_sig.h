@@ -101,9 +101,15 @@ __device__ __forceinline__ void gemv_layer_fma(const att_raw_w<DT> (&raw)[ROWS],
 // it contains workgroup barriers (2 + 2 * n_layers of them): threads outside any group pass active = false
 // and only take the barriers. The packed codes land in S.code[t] (valid on return)
 // and, when P.codes is not NULL, in the code stream.
-template <int DT, int GV, int NT, int ROWS, int PF>
+struct sig_no_hook {
+  __device__ __forceinline__ void operator()() const {}
+};
+
+// `after_requests` runs once every load of the MLP has been requested and before the first result is waited
+// for: the place for a caller to put loads of its own on their way without delaying the MLP's.
+template <int DT, int GV, int NT, int ROWS, int PF, typename Hook = sig_no_hook>
 __device__ __forceinline__ void sig_gemv_block(const sig_params& P, bool active, int tid, int b, int h, int l0, int nl,
-                                               int n_layers, sig_gemv_lds<GV, NT>& S) {
+                                               int n_layers, sig_gemv_lds<GV, NT>& S, Hook after_requests = Hook()) {
   constexpr int ES = (DT == SAH_F32) ? 4 : 2;
   constexpr int NW = NT / SAH_WAVE;
   constexpr int LOG_NT = 31 - __builtin_clz(NT);
@@ -147,9 +153,10 @@ __device__ __forceinline__ void sig_gemv_block(const sig_params& P, bool active,
     if (t > nl - 1) t = nl - 1;
     return sah_load<DT>(P.x, (int64_t)b * P.xs_b + (int64_t)hx * P.xs_h + (int64_t)(l0 + t) * P.xs_l + d);
   };
+  float xr = 0.f;
+  float bias_r[PF];
   if (active) {
-    const float xr = x_at(tid < GV * D ? tid : 0);
-    float bias_r[PF];
+    xr = x_at(tid < GV * D ? tid : 0);
     if (PF > 1) {
 #pragma unroll
       for (int layer = 0; layer < PF; ++layer) bias_r[layer] = layer < n_layers ? fetch_bias(layer) : 0.f;
@@ -162,6 +169,9 @@ __device__ __forceinline__ void sig_gemv_block(const sig_params& P, bool active,
         }
       }
     }
+  }
+  after_requests();
+  if (active) {
     if (tid < GV * D) {
       if (GV > 1) S.x[tid / D][tid % D] = (tid / D < nl) ? xr : 0.f;
       else S.x[0][tid] = xr;

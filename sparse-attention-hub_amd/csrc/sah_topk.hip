@@ -381,7 +381,8 @@ __global__ __launch_bounds__(HSW_NT) void k_hamming_topk_swar(sah_rows R, const 
   if (cnt0 > R.cap) cnt0 = R.cap;
   for (int i = tid; i < n_ch * 8; i += HSW_NT) s_bm[i] = i < R.n_words ? bm[i] : 0u;
   __syncthreads();
-  hsw_select_row(R, r, kcodes + (int64_t)(r / lq) * pitch, qcodes[r], k, cnt0, s_bm, s_key, S);
+  hsw_bufs buf;
+  hsw_select_row(R, r, kcodes + (int64_t)(r / lq) * pitch, qcodes[r], k, cnt0, s_bm, s_key, S, buf);
 }
 
 // kernels may use up to 160 KB of LDS; HIP needs to be told once per kernel
