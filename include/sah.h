@@ -134,6 +134,9 @@ int sah_rows_to_dense(const sah_dense_rows_args* a);
  * activation is rounded to that type exactly where torch would round it.
  * codes[((b*Hq + h) * code_pitch + code_offset + l) * 2 + {0,1}] receives
  * vector l (code_pitch and code_offset count codes, not words).
+ * Wt (all layers or none): the same matrices transposed, which lets many vectors
+ * at once (a prefill, the first decode call) go through the matrix cores when the
+ * type is 16-bit, D and the hidden widths are multiples of 32 up to 128.
  * ------------------------------------------------------------------------- */
 #define SAH_MAX_MLP_LAYERS 4
 typedef struct sah_hash_sig_args {
@@ -144,6 +147,7 @@ typedef struct sah_hash_sig_args {
   int32_t n_layers;
   const void* W[SAH_MAX_MLP_LAYERS];
   const void* bias[SAH_MAX_MLP_LAYERS];
+  const void* Wt[SAH_MAX_MLP_LAYERS];  /* optional: W_i transposed, [Hq, d_out_i, d_in_i] */
   int32_t d_out[SAH_MAX_MLP_LAYERS];  /* d_in of layer 0 is D */
   int32_t act;
   uint32_t* codes;

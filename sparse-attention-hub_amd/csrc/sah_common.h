@@ -88,6 +88,27 @@ __device__ __forceinline__ float sah_round(float f) {
   return f;
 }
 
+// The same roundings through the hardware converters (round to nearest even): for code that rounds per element
+// in an inner loop.
+template <int DT>
+__device__ __forceinline__ float sah_round_hw(float f) {
+  if (DT == SAH_BF16) return (float)(__bf16)f;
+  if (DT == SAH_F16) return (float)(_Float16)f;
+  return f;
+}
+// two values rounded to the 16-bit storage type DT and packed, lo in the low half
+template <int DT>
+__device__ __forceinline__ uint32_t sah_pack2_hw(float lo, float hi) {
+  if (DT == SAH_BF16) {
+    typedef __bf16 v2 __attribute__((ext_vector_type(2)));
+    const v2 p = {(__bf16)lo, (__bf16)hi};
+    return __builtin_bit_cast(uint32_t, p);
+  }
+  typedef _Float16 v2 __attribute__((ext_vector_type(2)));
+  const v2 p = {(_Float16)lo, (_Float16)hi};
+  return __builtin_bit_cast(uint32_t, p);
+}
+
 template <int DT>
 __device__ __forceinline__ float sah_load(const void* p, int64_t i) {
   if (DT == SAH_BF16) return sah_bf16_to_float(((const uint16_t*)p)[i]);
@@ -162,6 +183,20 @@ __device__ __forceinline__ float sah_dot2(uint32_t a, uint32_t b, float c) {
   return c + sah_f16_to_float((uint16_t)(a & 0xffffu)) * sah_f16_to_float((uint16_t)(b & 0xffffu)) +
          sah_f16_to_float((uint16_t)(a >> 16)) * sah_f16_to_float((uint16_t)(b >> 16));
 #endif
+}
+
+// D = A (32 x 16) * B (16 x 32) + C on the matrix cores, 16-bit inputs, fp32 accumulation. Per lane 8 packed
+// elements of A and of B and 16 of C (layouts checked on the hardware):
+//   A[i][k]: lane i + 32 g holds k = 8 g .. 8 g + 7;   B[k][j]: lane j + 32 g holds k = 8 g .. 8 g + 7;
+//   C[i][j]: lane j + 32 g, element v holds i = 8 (v / 4) + 4 g + v % 4.
+typedef float sah_f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 sah_bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 sah_f16x8 __attribute__((ext_vector_type(8)));
+template <int DT>
+__device__ __forceinline__ sah_f32x16 sah_mfma_32x32x16(uint4 a, uint4 b, sah_f32x16 c) {
+  if (DT == SAH_BF16)
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(sah_bf16x8, a), __builtin_bit_cast(sah_bf16x8, b), c, 0, 0, 0);
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(sah_f16x8, a), __builtin_bit_cast(sah_f16x8, b), c, 0, 0, 0);
 }
 
 // Pins a loaded value at this point of the program: the load that produced it must have

@@ -109,6 +109,203 @@ __global__ __launch_bounds__(GEMV_NT) void k_hash_sig_gemv(sig_pair PP) {
   sig_gemv_block<DT, GV, GEMV_NT, GEMV_ROWS, PF>(P, true, threadIdx.x, bh / P.Hq, bh % P.Hq, l0, nl, P.n_layers, S);
 }
 
+// ---------------------------------------------------------------------------
+// Bulk path on the matrix cores (a prefill, the first decode call of a layer: every key of the context).
+// Per head the MLP is three small GEMMs; computed transposed, Y^T = W^T X^T, so that the vectors are the
+// columns (N) of every product: a wave owns 32 vectors, the matrix-core result of one layer - lane j + 32 g
+// holds, for vector j, the features 8 (v / 4) + 4 g + v % 4 of each 32-feature tile - is, after bias and
+// activation, already laid out as the B operand of the next layer if the k-slots of a 16-feature step are
+// taken in the order [0-3][8-11] (g = 0), [4-7][12-15] (g = 1). The A operand (W^T, staged once per workgroup
+// in LDS, rows padded against bank conflicts) is stored in exactly that order for the layers after the
+// first, so no value ever moves between lanes until the sign bits are packed.
+// Needs 16-bit storage, D and the hidden widths multiples of 32 and at most 128, W^T given.
+// ---------------------------------------------------------------------------
+#define SGM_NT 512
+#define SGM_NW (SGM_NT / SAH_WAVE)
+#define SGM_TILE (32 * SGM_NW)  // vectors per workgroup tile
+#define SGM_MAXW 128            // widest layer
+#define SGM_MAXK (SGM_MAXW / 16)
+#define SGM_MAXM (SGM_MAXW / 32)
+#define SGM_PAD 8               // elements of padding per LDS row: 16 B
+
+template <int DT>
+__global__ __launch_bounds__(SGM_NT, 1) void k_hash_sig_mfma(sig_params P, int n_chunks, int tiles_per_wg) {
+  HIP_DYNAMIC_SHARED(unsigned char, sgm_dyn)
+  const int tid = threadIdx.x;
+  const int lane = tid & (SAH_WAVE - 1);
+  const int wave = tid / SAH_WAVE;
+  const int i32 = lane & 31;  // row of A / column of B and C
+  const int g = lane >> 5;    // k-group of the operands, row group of C
+  // the heads of one KV group are neighbours in the grid: they read the same vectors, which then hit in L2
+  int idx = blockIdx.x;
+  const int hq = idx % P.group;
+  idx /= P.group;
+  const int chunk = idx % n_chunks;
+  idx /= n_chunks;
+  const int Hx = P.Hq / P.group;
+  const int hx = idx % Hx;
+  const int b = idx / Hx;
+  const int h = hx * P.group + hq;
+
+  // ---- stage W^T (and the biases as fp32) in LDS
+  uint16_t* s_w[SAH_MAX_MLP_LAYERS];
+  int pitch[SAH_MAX_MLP_LAYERS];
+  int w_elems = 0;
+  {
+    int din = P.D;
+    for (int l = 0; l < P.n_layers; ++l) {
+      s_w[l] = (uint16_t*)sgm_dyn + w_elems;
+      pitch[l] = din + SGM_PAD;
+      w_elems += ((P.d_out[l] + 31) & ~31) * pitch[l];
+      din = P.d_out[l];
+    }
+  }
+  float* s_bias = (float*)((uint16_t*)sgm_dyn + ((w_elems + 1) & ~1));
+  {
+    int din = P.D;
+    for (int l = 0; l < P.n_layers; ++l) {
+      const int dout = P.d_out[l];
+      const int rows = (dout + 31) & ~31;
+      const int upr = din >> 2;  // 8-byte units per row
+      const uint16_t* wt = (const uint16_t*)P.Wt[l] + (int64_t)h * dout * din;
+      for (int u = tid; u < rows * upr; u += SGM_NT) {
+        const int row = u / upr, c4 = u - row * upr;
+        const int blk = c4 >> 2, sub = c4 & 3;
+        // layers after the first: the 4-element groups of a 16-block are kept as [0-3][8-11][4-7][12-15]
+        const int dsub = (l > 0 && (sub == 1 || sub == 2)) ? (sub ^ 3) : sub;
+        uint2 val = make_uint2(0u, 0u);
+        if (row < dout) val = *(const uint2*)(wt + (int64_t)row * din + c4 * 4);
+        *(uint2*)(s_w[l] + row * pitch[l] + blk * 16 + dsub * 4) = val;
+      }
+      for (int e = tid; e < SGM_MAXW; e += SGM_NT)
+        s_bias[l * SGM_MAXW + e] = e < dout ? sah_load<DT>(P.bias[l], (int64_t)h * dout + e) : 0.f;
+      din = dout;
+    }
+  }
+  __syncthreads();
+
+  const char* xbase = (const char*)P.x + ((int64_t)b * P.xs_b + (int64_t)hx * P.xs_h + 8 * g) * 2;
+  uint2* codes = (uint2*)P.codes + ((int64_t)b * P.Hq + h) * P.code_pitch + P.code_offset;
+
+  for (int t = 0; t < tiles_per_wg; ++t) {
+    const int v0 = (chunk * tiles_per_wg + t) * SGM_TILE + wave * 32;  // first vector of this wave
+    if (v0 >= P.L) break;                                               // uniform across the wave
+    int vec = v0 + i32;
+    const bool live = vec < P.L;
+    if (!live) vec = P.L - 1;  // computed and dropped
+    // B operand of the first layer: 8 consecutive elements of the vector per 16-element step
+    uint4 bop[SGM_MAXK];
+    const char* xrow = xbase + (int64_t)vec * P.xs_l * 2;
+    const int k0 = P.D >> 4;
+#pragma unroll
+    for (int s = 0; s < SGM_MAXK; ++s) bop[s] = s < k0 ? *(const uint4*)(xrow + s * 32) : make_uint4(0u, 0u, 0u, 0u);
+
+    int ksteps = k0;
+#pragma unroll
+    for (int l = 0; l < SAH_MAX_MLP_LAYERS; ++l) {
+      if (l >= P.n_layers) break;
+      const bool last = (l == P.n_layers - 1);
+      const int mt = (P.d_out[l] + 31) >> 5;
+      sah_f32x16 acc[SGM_MAXM];
+#pragma unroll
+      for (int q = 0; q < SGM_MAXM; ++q) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[q][v] = 0.f;
+      }
+      const uint16_t* wl = s_w[l] + i32 * pitch[l] + 8 * g;
+#pragma unroll
+      for (int q = 0; q < SGM_MAXM; ++q) {
+        if (q < mt) {
+#pragma unroll
+          for (int s = 0; s < SGM_MAXK; ++s) {
+            if (s < ksteps) {
+              const uint4 a = *(const uint4*)(wl + q * 32 * pitch[l] + s * 16);
+              acc[q] = sah_mfma_32x32x16<DT>(a, bop[s], acc[q]);
+            }
+          }
+        }
+      }
+      const float* bl = s_bias + l * SGM_MAXW + 4 * g;
+      if (!last) {
+        // bias, activation, rounding as torch rounds them; the result is the next layer's B operand
+#pragma unroll
+        for (int q = 0; q < SGM_MAXM; ++q) {
+          float y[16];
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            float z = sah_round_hw<DT>(acc[q][v]);
+            z = sah_round_hw<DT>(z + bl[q * 32 + 8 * (v >> 2) + (v & 3)]);
+            y[v] = q < mt ? sig_act_fast(P.act, z) : 0.f;  // rounded by the packing below
+          }
+          bop[2 * q] = make_uint4(sah_pack2_hw<DT>(y[0], y[1]), sah_pack2_hw<DT>(y[2], y[3]), sah_pack2_hw<DT>(y[4], y[5]),
+                                  sah_pack2_hw<DT>(y[6], y[7]));
+          bop[2 * q + 1] = make_uint4(sah_pack2_hw<DT>(y[8], y[9]), sah_pack2_hw<DT>(y[10], y[11]), sah_pack2_hw<DT>(y[12], y[13]),
+                                      sah_pack2_hw<DT>(y[14], y[15]));
+        }
+        ksteps = 2 * mt;
+      } else {
+        // sign planes: this lane holds 16 of the vector's bits, lane ^ 32 the other 16
+        uint32_t pos = 0u, nz = 0u;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          float z = sah_round_hw<DT>(acc[0][v]);
+          z = sah_round_hw<DT>(z + bl[8 * (v >> 2) + (v & 3)]);
+          const int bit = 8 * (v >> 2) + 4 * g + (v & 3);
+          pos |= (z > 0.f ? 1u : 0u) << bit;
+          nz |= (z != 0.f ? 1u : 0u) << bit;
+        }
+        pos |= __shfl_xor(pos, 32);
+        nz |= __shfl_xor(nz, 32);
+        if (g == 0 && live) codes[v0 + i32] = make_uint2(pos, nz);
+      }
+    }
+  }
+}
+
+static size_t sgm_lds_bytes(const sah_hash_sig_args* a) {
+  size_t elems = 0;
+  int din = a->D;
+  for (int l = 0; l < a->n_layers; ++l) {
+    elems += (size_t)((a->d_out[l] + 31) & ~31) * (din + SGM_PAD);
+    din = a->d_out[l];
+  }
+  elems = (elems + 1) & ~(size_t)1;
+  return elems * 2 + (size_t)a->n_layers * SGM_MAXW * 4;
+}
+
+// can the matrix-core kernel run this job?
+static bool sig_mfma_ok(const sah_hash_sig_args* a) {
+  if (a->dtype != SAH_BF16 && a->dtype != SAH_F16) return false;
+  if (a->L < 64) return false;  // a few vectors: the GEMV form is the better fit
+  if (a->D % 32 || a->D > SGM_MAXW) return false;
+  if (a->xs_b % 8 || a->xs_h % 8 || a->xs_l % 8 || ((uintptr_t)a->x % 16)) return false;
+  for (int l = 0; l < a->n_layers; ++l) {
+    if (!a->Wt[l] || ((uintptr_t)a->Wt[l] % 8)) return false;
+    const bool last = l == a->n_layers - 1;
+    if (last ? a->d_out[l] > 32 : (a->d_out[l] % 32 || a->d_out[l] > SGM_MAXW)) return false;
+  }
+  return sgm_lds_bytes(a) <= 150 * 1024;
+}
+
+template <int DT>
+static int sig_launch_mfma_t(const sah_hash_sig_args* a, const sig_params& P) {
+  static bool raised = false;
+  if (!raised) {
+    hipError_t e = hipFuncSetAttribute((const void*)k_hash_sig_mfma<DT>, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+    if (e != hipSuccess) return sah_fail((int)e, "sah_hash_signatures: cannot raise the LDS limit: %s", hipGetErrorString(e));
+    raised = true;
+  }
+  const int n_tiles = (a->L + SGM_TILE - 1) / SGM_TILE;
+  const int tiles_per_wg = n_tiles < 8 ? n_tiles : 8;   // the staged weights serve up to 8 tiles
+  const int n_chunks = (n_tiles + tiles_per_wg - 1) / tiles_per_wg;
+  const int64_t n_wg = (int64_t)a->B * a->Hq * n_chunks;
+  if (n_wg > 0x7fffffff) return sah_fail(SAH_ESHAPE, "sah_hash_signatures: too many workgroups");
+  sah_timed timed("k_hash_sig_mfma", a->stream);
+  hipLaunchKernelGGL(k_hash_sig_mfma<DT>, dim3((unsigned)n_wg), dim3(SGM_NT), sgm_lds_bytes(a), (hipStream_t)a->stream, P,
+                     n_chunks, tiles_per_wg);
+  return sah_launch_status("sah_hash_signatures");
+}
+
 static int sig_launch_gemv(const sah_hash_sig_args* a, const sah_hash_sig_args* b2) {
   sig_pair PP;
   sig_fill(a, PP.p[0]);
@@ -137,6 +334,11 @@ static int sig_launch_gemv(const sah_hash_sig_args* a, const sah_hash_sig_args* 
 
 static int sig_launch_one(const sah_hash_sig_args* a) {
   if (a->L <= 0) return SAH_OK;  // nothing to hash
+  if (sig_mfma_ok(a)) {
+    sig_params P;
+    sig_fill(a, P);
+    return a->dtype == SAH_BF16 ? sig_launch_mfma_t<SAH_BF16>(a, P) : sig_launch_mfma_t<SAH_F16>(a, P);
+  }
   if (sig_gemv_ok(a, GEMV_NT, GEMV_ROWS)) return sig_launch_gemv(a, nullptr);
   sig_params P;
   sig_fill(a, P);

@@ -99,6 +99,7 @@ class HashSigArgs(C.Structure):
         ("n_layers", C.c_int32),
         ("W", C.c_void_p * SAH_MAX_MLP_LAYERS),
         ("bias", C.c_void_p * SAH_MAX_MLP_LAYERS),
+        ("Wt", C.c_void_p * SAH_MAX_MLP_LAYERS),
         ("d_out", C.c_int32 * SAH_MAX_MLP_LAYERS),
         ("act", C.c_int32),
         ("codes", C.c_void_p),

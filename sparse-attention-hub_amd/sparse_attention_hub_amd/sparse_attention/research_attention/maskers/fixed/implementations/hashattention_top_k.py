@@ -141,31 +141,34 @@ class HashAttentionTopKMasker(TopKMasker):
             raise ValueError(f"at most {N.SAH_MAX_MLP_LAYERS} signature MLP layers are supported, got {len(mats)}")
         if self.hat_mlp_activation not in N.SAH_ACT:
             raise ValueError(f"Unsupported activation function: {self.hat_mlp_activation}")
-        self._prepared[key] = (mats, biases)
-        return mats, biases
+        # the same matrices transposed to [heads, d_out, d_in]: the matrix-core path of the bulk kernel reads them
+        mats_t = [m.transpose(1, 2).contiguous() for m in mats]
+        self._prepared[key] = (mats, biases, mats_t)
+        return mats, biases, mats_t
 
     def _hash_args(self, x: torch.Tensor, x_heads: int, n_heads: int, first: int, count: int, layer_idx: int,
                    kind: str, codes: torch.Tensor, code_pitch: int, code_offset: int) -> "N.HashSigArgs":
         """Argument block for the signatures of x[:, :, first:first+count, :] into codes[..., code_offset:]."""
-        mats, biases = self._weights_for(layer_idx, kind, x.device, x.dtype)
+        mats, biases, mats_t = self._weights_for(layer_idx, kind, x.device, x.dtype)
         if mats[0].shape[0] != n_heads or mats[0].shape[1] != x.shape[-1]:
             raise ValueError(
                 f"{kind}_matrix[0] has shape {tuple(mats[0].shape)}, expected ({n_heads}, {x.shape[-1]}, *)"
             )
         W = (N.C.c_void_p * N.SAH_MAX_MLP_LAYERS)()
         Bv = (N.C.c_void_p * N.SAH_MAX_MLP_LAYERS)()
+        Wt = (N.C.c_void_p * N.SAH_MAX_MLP_LAYERS)()
         dout = (N.C.c_int32 * N.SAH_MAX_MLP_LAYERS)()
-        for i, (m, b) in enumerate(zip(mats, biases)):
-            W[i], Bv[i], dout[i] = m.data_ptr(), b.data_ptr(), m.shape[2]
+        for i, (m, b, mt) in enumerate(zip(mats, biases, mats_t)):
+            W[i], Bv[i], Wt[i], dout[i] = m.data_ptr(), b.data_ptr(), mt.data_ptr(), m.shape[2]
         args = N.HashSigArgs(
             x.data_ptr() + first * x.stride(2) * x.element_size(),
             x.stride(0), x.stride(1), x.stride(2),
             N.dtype_code(x.dtype),
             x.shape[0], n_heads, n_heads // x_heads, count, x.shape[-1],
-            len(mats), W, Bv, dout, N.SAH_ACT[self.hat_mlp_activation],
+            len(mats), W, Bv, Wt, dout, N.SAH_ACT[self.hat_mlp_activation],
             codes.data_ptr(), code_pitch, code_offset, N.stream_ptr(x.device),
         )
-        args._keepalive = (W, Bv, dout)
+        args._keepalive = (W, Bv, Wt, dout)
         return args
 
     def _hash(self, x: torch.Tensor, x_heads: int, n_heads: int, first: int, count: int, layer_idx: int,
