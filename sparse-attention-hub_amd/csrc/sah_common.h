@@ -199,6 +199,17 @@ __device__ __forceinline__ sah_f32x16 sah_mfma_32x32x16(uint4 a, uint4 b, sah_f3
   return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(sah_f16x8, a), __builtin_bit_cast(sah_f16x8, b), c, 0, 0, 0);
 }
 
+// D = A (16 x 32) * B (32 x 16) + C, 16-bit inputs, fp32 accumulation (layouts checked on the hardware):
+//   A[i][k]: lane i + 16 g holds k = 8 g .. 8 g + 7 (g = 0..3);   B[k][j]: lane j + 16 g likewise;
+//   C[i][j]: lane j + 16 g, element v holds i = 4 g + v.
+typedef float sah_f32x4 __attribute__((ext_vector_type(4)));
+template <int DT>
+__device__ __forceinline__ sah_f32x4 sah_mfma_16x16x32(uint4 a, uint4 b, sah_f32x4 c) {
+  if (DT == SAH_BF16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(sah_bf16x8, a), __builtin_bit_cast(sah_bf16x8, b), c, 0, 0, 0);
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(sah_f16x8, a), __builtin_bit_cast(sah_f16x8, b), c, 0, 0, 0);
+}
+
 // Pins a loaded value at this point of the program: the load that produced it must have
 // been issued (and is waited for) here, so the compiler can neither sink it into a later
 // branch nor serialise a batch of independent loads one wait at a time.

@@ -19,7 +19,15 @@
 #define HDEC_GROUP 512
 #define HDEC_ROWS 4
 
-typedef sig_gemv_lds<1, HDEC_GROUP> hdec_sig_lds;
+// scratch of one signature job: the GEMV form or the matrix-core form
+template <bool MF>
+struct hdec_sig {
+  typedef sig_gemv_lds<1, HDEC_GROUP> lds;
+};
+template <>
+struct hdec_sig<true> {
+  typedef sig_mfma_lds lds;
+};
 
 struct hdec_params {
   sah_rows R;
@@ -32,8 +40,9 @@ struct hdec_params {
   int update_bitmap;
 };
 
-template <int DT>
+template <int DT, bool MF>
 __global__ __launch_bounds__(HSW_NT) void k_hash_decode(hdec_params P) {
+  typedef typename hdec_sig<MF>::lds hdec_sig_lds;
   __shared__ hsw_lds S;
   HIP_DYNAMIC_SHARED(unsigned char, hdec_dyn)
   const sah_rows& R = P.R;
@@ -68,15 +77,22 @@ __global__ __launch_bounds__(HSW_NT) void k_hash_decode(hdec_params P) {
   // ---- 2. signatures of the query and of the newest key
   // uniform across the wave, and known to be: the job's parameters are then fetched by scalar loads
   const int job = __builtin_amdgcn_readfirstlane(tid / HDEC_GROUP);
-  const bool active = job == 0 || P.has_key;
+  // without a new key the second group repeats the query job (its parameter block is a copy that stores
+  // nothing): every wave then runs the same straight-line code
+  const bool active = true;
   const int Hq = P.job[0].Hq;
   // 2-byte weights: all layers requested up-front; fp32 rows are twice as wide, one layer at a time
   constexpr int PF = (DT == SAH_F32) ? 1 : SAH_MAX_MLP_LAYERS;
   // the first half of the row's codes is requested behind the MLP's own loads and arrives while it computes
   hsw_bufs buf;
   const uint2* kc = P.kcodes + (int64_t)r * P.pitch;
-  sig_gemv_block<DT, 1, HDEC_GROUP, HDEC_ROWS, PF>(P.job[job], active, tid % HDEC_GROUP, r / Hq, r % Hq, 0, 1,
-                                                    P.job[0].n_layers, s_sig[job], [&]() { hsw_prefetch(kc, n, buf); });
+  auto prefetch = [&]() { hsw_prefetch(kc, n, buf); };
+  if constexpr (MF) {
+    sig_mfma_block<DT>(P.job[job], active, tid % HDEC_GROUP, r / Hq, r % Hq, 0, 1, P.job[0].n_layers, s_sig[job], prefetch);
+  } else {
+    sig_gemv_block<DT, 1, HDEC_GROUP, HDEC_ROWS, PF>(P.job[job], active, tid % HDEC_GROUP, r / Hq, r % Hq, 0, 1,
+                                                      P.job[0].n_layers, s_sig[job], prefetch);
+  }
   const uint2 q = s_sig[0].code[0];
   __syncthreads();  // every thread holds q (and the bitmap is complete) before the scores overwrite the scratch
 
@@ -86,21 +102,35 @@ __global__ __launch_bounds__(HSW_NT) void k_hash_decode(hdec_params P) {
 
 static size_t hdec_lds_bytes(int n_keys) {
   const int n_ch = (n_keys + 255) / 256;
-  const size_t bm = (size_t)n_ch * 8 * 4, key = (size_t)n_ch * 64 * 4, sig = 2 * sizeof(hdec_sig_lds);
+  const size_t a = sizeof(hdec_sig<false>::lds), b = sizeof(hdec_sig<true>::lds);
+  const size_t bm = (size_t)n_ch * 8 * 4, key = (size_t)n_ch * 64 * 4, sig = 2 * (a > b ? a : b);
   return bm + (key > sig ? key : sig);
 }
 
-template <int DT>
+template <int DT, bool MF>
 static int hdec_launch(const sah_hash_decode_args* a, const hdec_params& P, size_t lds) {
   static bool raised = false;
   if (!raised) {
-    hipError_t e = hipFuncSetAttribute((const void*)k_hash_decode<DT>, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+    hipError_t e = hipFuncSetAttribute((const void*)k_hash_decode<DT, MF>, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
     if (e != hipSuccess) return sah_fail((int)e, "sah_hash_decode_topk: cannot raise the LDS limit: %s", hipGetErrorString(e));
     raised = true;
   }
   sah_timed timed("k_hash_decode", a->stream);
-  hipLaunchKernelGGL(k_hash_decode<DT>, dim3(a->rows.n_rows), dim3(HSW_NT), lds, (hipStream_t)a->stream, P);
+  hipLaunchKernelGGL((k_hash_decode<DT, MF>), dim3(a->rows.n_rows), dim3(HSW_NT), lds, (hipStream_t)a->stream, P);
   return sah_launch_status("sah_hash_decode_topk");
+}
+
+// Which form of the signature MLP the stand-alone launches would take for this step's jobs: the fused kernel
+// must take the same one, so that both routes produce the same bits. 0: not fusable, 1: GEMV, 2: matrix cores.
+static int hdec_sig_kind(const sah_hash_decode_args* a, bool has_key) {
+  const sah_hash_sig_args* q = a->query_sig;
+  const sah_hash_sig_args* kk = a->key_sig;
+  const bool qm = sig_mfma_small_ok(q), km = has_key ? sig_mfma_small_ok(kk) : qm;
+  if (qm && km) return 2;
+  if (qm || km) return 0;
+  if (!sig_gemv_ok(q, HDEC_GROUP, HDEC_ROWS)) return 0;
+  if (has_key && !sig_gemv_ok(kk, HDEC_GROUP, HDEC_ROWS)) return 0;
+  return 1;
 }
 
 // can the single-kernel form run this step?
@@ -109,10 +139,12 @@ static bool hdec_fusable(const sah_hash_decode_args* a) {
   const sah_hash_sig_args* kk = a->key_sig;
   const int n = a->rows.n_keys;
   if (q->L != 1 || (int64_t)q->B * q->Hq != a->rows.n_rows) return false;
-  if (!sig_gemv_ok(q, HDEC_GROUP, HDEC_ROWS)) return false;
+  if (hdec_sig_kind(a, kk && kk->L > 0) == 0) return false;
   if (kk && kk->L > 0) {
     if (kk->L != 1 || kk->B != q->B || kk->Hq != q->Hq || kk->n_layers != q->n_layers || kk->dtype != q->dtype) return false;
-    if (!sig_gemv_ok(kk, HDEC_GROUP, HDEC_ROWS)) return false;
+    if (kk->D != q->D || kk->act != q->act) return false;
+    for (int l = 0; l < q->n_layers; ++l)
+      if (kk->d_out[l] != q->d_out[l]) return false;
     // the new code is written while the row's codes are scanned: its column must be one the scan ignores
     if ((const uint32_t*)kk->codes == a->kcodes && kk->code_offset < n - a->window) return false;
   }
@@ -162,6 +194,7 @@ extern "C" int sah_hash_decode_topk(const sah_hash_decode_args* a) {
   P.R = a->rows;
   sig_fill(a->query_sig, P.job[0]);
   sig_fill(has_key ? a->key_sig : a->query_sig, P.job[1]);
+  if (!has_key) P.job[1].codes = nullptr;
   P.has_key = has_key ? 1 : 0;
   P.kcodes = (const uint2*)a->kcodes;
   P.pitch = a->code_pitch;
@@ -170,9 +203,10 @@ extern "C" int sah_hash_decode_topk(const sah_hash_decode_args* a) {
   P.window = a->window;
   P.update_bitmap = a->skip_bitmap ? 0 : 1;
   const size_t lds = hdec_lds_bytes(a->rows.n_keys);
+  const bool mf = hdec_sig_kind(a, has_key) == 2;
   switch (a->query_sig->dtype) {
-    case SAH_F32: return hdec_launch<SAH_F32>(a, P, lds);
-    case SAH_BF16: return hdec_launch<SAH_BF16>(a, P, lds);
-    default: return hdec_launch<SAH_F16>(a, P, lds);
+    case SAH_F32: return hdec_launch<SAH_F32, false>(a, P, lds);
+    case SAH_BF16: return mf ? hdec_launch<SAH_BF16, true>(a, P, lds) : hdec_launch<SAH_BF16, false>(a, P, lds);
+    default: return mf ? hdec_launch<SAH_F16, true>(a, P, lds) : hdec_launch<SAH_F16, false>(a, P, lds);
   }
 }

@@ -306,12 +306,32 @@ static int sig_launch_mfma_t(const sah_hash_sig_args* a, const sig_params& P) {
   return sah_launch_status("sah_hash_signatures");
 }
 
+// decode-size jobs on the matrix cores: up to 16 vectors of one head per workgroup
+template <int DT>
+__global__ __launch_bounds__(SMB_NT) void k_hash_sig_small_mfma(sig_pair PP) {
+  const sig_params& P = PP.p[blockIdx.z];
+  if ((int)blockIdx.x * 16 >= P.L) return;  // the two jobs may differ in vector count
+  __shared__ sig_mfma_lds S;
+  const int bh = blockIdx.y;
+  const int l0 = blockIdx.x * 16;
+  int nl = P.L - l0;
+  if (nl > 16) nl = 16;
+  sig_mfma_block<DT>(P, true, threadIdx.x, bh / P.Hq, bh % P.Hq, l0, nl, P.n_layers, S);
+}
+
 static int sig_launch_gemv(const sah_hash_sig_args* a, const sah_hash_sig_args* b2) {
   sig_pair PP;
   sig_fill(a, PP.p[0]);
   sig_fill(b2 ? b2 : a, PP.p[1]);
   const int maxL = (b2 && b2->L > a->L) ? b2->L : a->L;
   hipStream_t st = (hipStream_t)a->stream;
+  if (sig_mfma_small_ok(a) && (!b2 || sig_mfma_small_ok(b2))) {
+    sah_timed timed("k_hash_sig_small_mfma", a->stream);
+    dim3 gg((maxL + 15) / 16, a->B * a->Hq, b2 ? 2 : 1);
+    if (a->dtype == SAH_BF16) hipLaunchKernelGGL(k_hash_sig_small_mfma<SAH_BF16>, gg, dim3(SMB_NT), 0, st, PP);
+    else hipLaunchKernelGGL(k_hash_sig_small_mfma<SAH_F16>, gg, dim3(SMB_NT), 0, st, PP);
+    return sah_launch_status("sah_hash_signatures");
+  }
   sah_timed timed("k_hash_sig_gemv", a->stream);
   dim3 gb(GEMV_NT);
   if (maxL == 1) {  // decode: one vector per head and job
@@ -339,7 +359,7 @@ static int sig_launch_one(const sah_hash_sig_args* a) {
     sig_fill(a, P);
     return a->dtype == SAH_BF16 ? sig_launch_mfma_t<SAH_BF16>(a, P) : sig_launch_mfma_t<SAH_F16>(a, P);
   }
-  if (sig_gemv_ok(a, GEMV_NT, GEMV_ROWS)) return sig_launch_gemv(a, nullptr);
+  if (sig_mfma_small_ok(a) || sig_gemv_ok(a, GEMV_NT, GEMV_ROWS)) return sig_launch_gemv(a, nullptr);
   sig_params P;
   sig_fill(a, P);
   dim3 g((a->L + SIG_TL - 1) / SIG_TL, a->B * a->Hq), b(SIG_NT);
@@ -366,7 +386,10 @@ extern "C" int sah_hash_signatures_pair(const sah_hash_sig_args* a, const sah_ha
   if (rc) return rc;
   rc = sig_validate(b);
   if (rc) return rc;
-  if (a->L > 0 && b->L > 0 && sig_gemv_ok(a, GEMV_NT, GEMV_ROWS) && sig_gemv_ok(b, GEMV_NT, GEMV_ROWS) && a->dtype == b->dtype && a->stream == b->stream &&
+  const bool both_mfma = sig_mfma_small_ok(a) && sig_mfma_small_ok(b);
+  const bool both_gemv = !sig_mfma_small_ok(a) && !sig_mfma_small_ok(b) && sig_gemv_ok(a, GEMV_NT, GEMV_ROWS) &&
+                         sig_gemv_ok(b, GEMV_NT, GEMV_ROWS);
+  if (a->L > 0 && b->L > 0 && (both_mfma || both_gemv) && a->dtype == b->dtype && a->stream == b->stream &&
       (int64_t)a->B * a->Hq == (int64_t)b->B * b->Hq)
     return sig_launch_gemv(a, b);
   rc = sig_launch_one(a);

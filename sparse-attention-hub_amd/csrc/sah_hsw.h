@@ -83,8 +83,9 @@ __device__ __forceinline__ void hsw_prefetch(const uint2* kc, int n, hsw_bufs& b
   const int lane = threadIdx.x & (SAH_WAVE - 1);
   int c0, c1;
   hsw_wave_chunks(n, threadIdx.x / SAH_WAVE, c0, c1);
-  if (c0 < c1) hsw_request(kc, n, lane, buf.a0, buf.a1, c0);
-  if (c0 + HSW_BATCH < c1) hsw_request(kc, n, lane, buf.b0, buf.b1, c0 + HSW_BATCH);
+  (void)c1;  // no conditions: a request past the row's end re-reads valid memory and is never scored
+  hsw_request(kc, n, lane, buf.a0, buf.a1, c0);
+  hsw_request(kc, n, lane, buf.b0, buf.b1, c0 + HSW_BATCH);
 }
 
 // Top-k of row r over the not-yet-active columns. On entry `s_bm` (n_ch * 8 words of dynamic LDS, zero

@@ -277,6 +277,132 @@ __device__ __forceinline__ void sig_gemv_block(const sig_params& P, bool active,
 }
 
 // ---------------------------------------------------------------------------
+// The same decode-size job on the matrix cores: up to 16 vectors of one head per call, 512 threads.
+// Transposed, Y^T = W^T X^T: wave w owns the 16 output features 16 w .. 16 w + 15 of every layer, its slice of
+// W^T (16 rows, k contiguous: one 16-byte load per lane and 32-element k-step, every layer requested up-front)
+// is the A operand, the vectors (in LDS, 16-bit) are the B operand, and column j of the result is vector j.
+// One barrier per layer. Needs 16-bit storage, W^T, D and the hidden widths multiples of 32 up to 128.
+// ---------------------------------------------------------------------------
+#define SMB_NT 512
+#define SMB_MAXW 128
+#define SMB_MAXK (SMB_MAXW / 32)
+#define SMB_PITCH (SMB_MAXW + 8)  // 16-bit elements per LDS row: 16 B of padding against bank conflicts
+
+struct sig_mfma_lds {
+  uint16_t x[2][16][SMB_PITCH];  // layer inputs, double buffered: a layer reads one and writes the other
+  float y[16][32];               // last layer's outputs
+  float bias[SAH_MAX_MLP_LAYERS][SMB_MAXW];
+  uint2 code[16];
+};
+
+template <int DT, typename Hook = sig_no_hook>
+__device__ __forceinline__ void sig_mfma_block(const sig_params& P, bool active, int tid, int b, int h, int l0, int nl,
+                                               int n_layers, sig_mfma_lds& S, Hook after_requests = Hook()) {
+  const int lane = tid & (SAH_WAVE - 1);
+  const int wave = tid / SAH_WAVE;
+  const int i16 = lane & 15;  // row of A, column (vector) of B and C
+  const int g = lane >> 4;    // k-group of the operands, row group of C
+  const int hx = active ? h / P.group : 0;
+  const int D = active ? P.D : 32;
+  const int act = active ? P.act : 0;
+
+  // ---- requests: input vectors, biases, then this wave's slice of every layer's W^T. Raw loads, nothing
+  // converted or used here, and only wave-uniform conditions: all loads are in flight together and each later
+  // wait covers little more than what it needs.
+  const int xunits = D >> 3;  // 16-byte units per vector
+  const int xt = tid / xunits, xc = tid - xt * xunits;
+  uint4 xr = make_uint4(0u, 0u, 0u, 0u);
+  uint16_t bias_raw[SAH_MAX_MLP_LAYERS];
+  uint4 wr[SAH_MAX_MLP_LAYERS][SMB_MAXK];
+  if (active) {
+    const int t = xt < nl ? xt : nl - 1;  // rows beyond nl repeat the last vector (computed and dropped)
+    xr = *(const uint4*)((const uint16_t*)P.x + (int64_t)b * P.xs_b + (int64_t)hx * P.xs_h + (int64_t)(l0 + t) * P.xs_l + 8 * xc);
+#pragma unroll
+    for (int l = 0; l < SAH_MAX_MLP_LAYERS; ++l) {
+      const int ll = l < n_layers ? l : 0;
+      const int dout = P.d_out[ll];
+      bias_raw[l] = ((const uint16_t*)P.bias[ll])[(int64_t)h * dout + (tid < dout ? tid : 0)];
+    }
+#pragma unroll
+    for (int l = 0; l < SAH_MAX_MLP_LAYERS; ++l) {
+      // uniform conditions only: a wave skips the layers that do not exist and the ones it has no rows of
+      if (l < n_layers && 16 * wave < P.d_out[l]) {
+        const int dout = P.d_out[l];
+        const int din = l == 0 ? D : P.d_out[l - 1];
+        int row = 16 * wave + i16;
+        if (row > dout - 1) row = dout - 1;  // rows beyond the width repeat the last one; their results are dropped
+        const uint16_t* wrow = (const uint16_t*)P.Wt[l] + ((int64_t)h * dout + row) * din + 8 * g;
+#pragma unroll
+        for (int s = 0; s < SMB_MAXK; ++s)
+          if (32 * s < din) wr[l][s] = *(const uint4*)(wrow + 32 * s);
+      }
+    }
+  }
+  after_requests();
+  if (active) {
+    if (xt < 16) *(uint4*)&S.x[0][xt][8 * xc] = xr;
+    if (tid < SMB_MAXW) {
+#pragma unroll
+      for (int l = 0; l < SAH_MAX_MLP_LAYERS; ++l) {
+        const int dout = P.d_out[l < n_layers ? l : 0];
+        const float bv = (DT == SAH_BF16) ? sah_bf16_to_float(bias_raw[l]) : sah_f16_to_float(bias_raw[l]);
+        S.bias[l][tid] = tid < dout ? bv : 0.f;
+      }
+    }
+  }
+  __syncthreads();
+
+  int din = D;
+#pragma unroll
+  for (int l = 0; l < SAH_MAX_MLP_LAYERS; ++l) {
+    if (l >= n_layers) break;
+    const int dout = active ? P.d_out[l] : 16;
+    const bool last = (l == n_layers - 1);
+    if (active && 16 * wave < dout) {
+      sah_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < SMB_MAXK; ++s) {
+        if (32 * s < din) {
+          const uint4 bop = *(const uint4*)&S.x[l & 1][i16][32 * s + 8 * g];
+          acc = sah_mfma_16x16x32<DT>(wr[l][s], bop, acc);
+        }
+      }
+      // lane (vector i16, group g) holds the features 16 wave + 4 g + v
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int f = 16 * wave + 4 * g + v;
+        float y = sah_round_hw<DT>(acc[v]);
+        y = sah_round_hw<DT>(y + S.bias[l][f]);
+        if (!last) {
+          if (f < dout) S.x[(l + 1) & 1][i16][f] = (uint16_t)sah_pack2_hw<DT>(sig_act_fast(act, y), 0.f);
+        } else if (f < 32) {
+          S.y[i16][f] = f < dout ? y : 0.f;
+        }
+      }
+    }
+    __syncthreads();
+    din = dout;
+  }
+
+  if (active && tid < SAH_WAVE) {
+    const int bits = din;
+    for (int t = 0; t < nl; ++t) {
+      const float y = (tid < bits && tid < 32) ? S.y[t][tid] : 0.f;
+      const uint64_t pos = __ballot(y > 0.f);
+      const uint64_t nz = __ballot(y != 0.f);
+      if (tid == 0) {
+        uint2 c;
+        c.x = (uint32_t)pos;
+        c.y = (uint32_t)nz;
+        S.code[t] = c;
+        if (P.codes) ((uint2*)P.codes)[((int64_t)b * P.Hq + h) * P.code_pitch + P.code_offset + l0 + t] = c;
+      }
+    }
+  }
+  __syncthreads();  // S.code is visible to the whole workgroup
+}
+
+// ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
 // can the block-level GEMV with `nt` threads and `max_rows` row slots per thread run this job?
@@ -294,6 +420,22 @@ static inline bool sig_gemv_ok(const sah_hash_sig_args* a, int nt, int max_rows)
     if (((uintptr_t)a->W[i]) % (8 * es)) return false;
     din = dout;
   }
+  return true;
+}
+
+// can the matrix-core form of the decode-size job (sig_mfma_block) run this?
+static inline bool sig_mfma_small_ok(const sah_hash_sig_args* a) {
+  if (a->dtype != SAH_BF16 && a->dtype != SAH_F16) return false;
+  if (a->L > 64 || a->D % 32 || a->D > SMB_MAXW) return false;
+  if (a->xs_b % 8 || a->xs_h % 8 || a->xs_l % 8 || ((uintptr_t)a->x % 16)) return false;
+  int din = a->D;
+  for (int l = 0; l < a->n_layers; ++l) {
+    if (!a->Wt[l] || ((uintptr_t)a->Wt[l] % 16)) return false;
+    const bool last = l == a->n_layers - 1;
+    if (last ? a->d_out[l] > 32 : (a->d_out[l] % 32 || a->d_out[l] > SMB_MAXW)) return false;
+    din = a->d_out[l];
+  }
+  (void)din;
   return true;
 }
 
