@@ -31,11 +31,11 @@ __device__ __forceinline__ float sig_act(int act, float v) {
 __device__ __forceinline__ float sig_act_fast(int act, float v) {
   switch (act) {
     case SAH_ACT_RELU: return v > 0.f ? v : 0.f;
-    case SAH_ACT_SILU: return v * __frcp_rn(1.0f + __expf(-v));
+    case SAH_ACT_SILU: return v * __builtin_amdgcn_rcpf(1.0f + __expf(-v));
     case SAH_ACT_GELU: return 0.5f * v * (1.0f + erff(v * 0.70710678118654752440f));
     default: {
       const float e = __expf(-2.0f * fabsf(v));  // tanh |v| = (1 - e) / (1 + e)
-      const float t = (1.0f - e) * __frcp_rn(1.0f + e);
+      const float t = (1.0f - e) * __builtin_amdgcn_rcpf(1.0f + e);
       return v < 0.f ? -t : t;
     }
   }
@@ -289,12 +289,13 @@ __device__ __forceinline__ void sig_gemv_block(const sig_params& P, bool active,
 #define SMB_PITCH (SMB_MAXW + 8)  // 16-bit elements per LDS row: 16 B of padding against bank conflicts
 
 struct sig_mfma_lds {
-  uint16_t x[2][16][SMB_PITCH];  // layer inputs, double buffered: a layer reads one and writes the other
+  uint16_t x[2][16][SMB_PITCH];  // inputs of the layers after the first, double buffered
   float y[16][32];               // last layer's outputs
-  float bias[SAH_MAX_MLP_LAYERS][SMB_MAXW];
   uint2 code[16];
 };
 
+// `after_requests` runs once every load of the MLP has been requested: the place for a caller to put loads of
+// its own on their way without delaying the MLP's.
 template <int DT, typename Hook = sig_no_hook>
 __device__ __forceinline__ void sig_mfma_block(const sig_params& P, bool active, int tid, int b, int h, int l0, int nl,
                                                int n_layers, sig_mfma_lds& S, Hook after_requests = Hook()) {
@@ -305,52 +306,40 @@ __device__ __forceinline__ void sig_mfma_block(const sig_params& P, bool active,
   const int hx = active ? h / P.group : 0;
   const int D = active ? P.D : 32;
   const int act = active ? P.act : 0;
+  const int f0 = 16 * wave + 4 * g;  // this lane's 4 output features of every layer: f0 .. f0 + 3
 
-  // ---- requests: input vectors, biases, then this wave's slice of every layer's W^T. Raw loads, nothing
-  // converted or used here, and only wave-uniform conditions: all loads are in flight together and each later
-  // wait covers little more than what it needs.
-  const int xunits = D >> 3;  // 16-byte units per vector
-  const int xt = tid / xunits, xc = tid - xt * xunits;
-  uint4 xr = make_uint4(0u, 0u, 0u, 0u);
-  uint16_t bias_raw[SAH_MAX_MLP_LAYERS];
+  // ---- first requests, only what the first layer needs, so that it can start as early as possible: the
+  // vector itself straight into the B operand (no LDS round, no barrier), the biases (8 bytes per lane and
+  // layer), this wave's slice of the first W^T. Raw loads and wave-uniform conditions only.
+  uint4 bop0[SMB_MAXK];
+  uint2 bias_raw[SAH_MAX_MLP_LAYERS];
   uint4 wr[SAH_MAX_MLP_LAYERS][SMB_MAXK];
+  auto request_weights = [&](int l) {
+    if (l < n_layers && 16 * wave < P.d_out[l]) {  // a wave skips the layers it has no rows of
+      const int dout = P.d_out[l];
+      const int din = l == 0 ? D : P.d_out[l - 1];
+      int row = 16 * wave + i16;
+      if (row > dout - 1) row = dout - 1;  // rows beyond the width repeat the last one; their results are dropped
+      const uint16_t* wrow = (const uint16_t*)P.Wt[l] + ((int64_t)h * dout + row) * din + 8 * g;
+#pragma unroll
+      for (int s = 0; s < SMB_MAXK; ++s)
+        if (32 * s < din) wr[l][s] = *(const uint4*)(wrow + 32 * s);
+    }
+  };
   if (active) {
-    const int t = xt < nl ? xt : nl - 1;  // rows beyond nl repeat the last vector (computed and dropped)
-    xr = *(const uint4*)((const uint16_t*)P.x + (int64_t)b * P.xs_b + (int64_t)hx * P.xs_h + (int64_t)(l0 + t) * P.xs_l + 8 * xc);
+    const int t = i16 < nl ? i16 : nl - 1;  // columns beyond nl repeat the last vector (computed and dropped)
+    const uint16_t* xrow = (const uint16_t*)P.x + (int64_t)b * P.xs_b + (int64_t)hx * P.xs_h + (int64_t)(l0 + t) * P.xs_l + 8 * g;
+#pragma unroll
+    for (int s = 0; s < SMB_MAXK; ++s)
+      if (32 * s < D) bop0[s] = *(const uint4*)(xrow + 32 * s);
 #pragma unroll
     for (int l = 0; l < SAH_MAX_MLP_LAYERS; ++l) {
       const int ll = l < n_layers ? l : 0;
       const int dout = P.d_out[ll];
-      bias_raw[l] = ((const uint16_t*)P.bias[ll])[(int64_t)h * dout + (tid < dout ? tid : 0)];
+      bias_raw[l] = *(const uint2*)((const uint16_t*)P.bias[ll] + (int64_t)h * dout + (f0 + 4 <= dout ? f0 : 0));
     }
-#pragma unroll
-    for (int l = 0; l < SAH_MAX_MLP_LAYERS; ++l) {
-      // uniform conditions only: a wave skips the layers that do not exist and the ones it has no rows of
-      if (l < n_layers && 16 * wave < P.d_out[l]) {
-        const int dout = P.d_out[l];
-        const int din = l == 0 ? D : P.d_out[l - 1];
-        int row = 16 * wave + i16;
-        if (row > dout - 1) row = dout - 1;  // rows beyond the width repeat the last one; their results are dropped
-        const uint16_t* wrow = (const uint16_t*)P.Wt[l] + ((int64_t)h * dout + row) * din + 8 * g;
-#pragma unroll
-        for (int s = 0; s < SMB_MAXK; ++s)
-          if (32 * s < din) wr[l][s] = *(const uint4*)(wrow + 32 * s);
-      }
-    }
+    request_weights(0);
   }
-  after_requests();
-  if (active) {
-    if (xt < 16) *(uint4*)&S.x[0][xt][8 * xc] = xr;
-    if (tid < SMB_MAXW) {
-#pragma unroll
-      for (int l = 0; l < SAH_MAX_MLP_LAYERS; ++l) {
-        const int dout = P.d_out[l < n_layers ? l : 0];
-        const float bv = (DT == SAH_BF16) ? sah_bf16_to_float(bias_raw[l]) : sah_f16_to_float(bias_raw[l]);
-        S.bias[l][tid] = tid < dout ? bv : 0.f;
-      }
-    }
-  }
-  __syncthreads();
 
   int din = D;
 #pragma unroll
@@ -358,26 +347,47 @@ __device__ __forceinline__ void sig_mfma_block(const sig_params& P, bool active,
     if (l >= n_layers) break;
     const int dout = active ? P.d_out[l] : 16;
     const bool last = (l == n_layers - 1);
-    if (active && 16 * wave < dout) {
-      sah_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    sah_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    const bool mine = active && 16 * wave < dout;
+    if (mine) {
 #pragma unroll
       for (int s = 0; s < SMB_MAXK; ++s) {
         if (32 * s < din) {
-          const uint4 bop = *(const uint4*)&S.x[l & 1][i16][32 * s + 8 * g];
+          const uint4 bop = l == 0 ? bop0[s] : *(const uint4*)&S.x[l & 1][i16][32 * s + 8 * g];
           acc = sah_mfma_16x16x32<DT>(wr[l][s], bop, acc);
         }
       }
-      // lane (vector i16, group g) holds the features 16 wave + 4 g + v
+    }
+    if (l == 0) {
+      // the rest goes out behind the first layer's operands: it has the first layer's epilogue and a barrier
+      // to arrive in
+      __builtin_amdgcn_sched_barrier(0);
+      if (active) {
+#pragma unroll
+        for (int k = 1; k < SAH_MAX_MLP_LAYERS; ++k) request_weights(k);
+      }
+      after_requests();
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (mine) {
+      // lane (vector i16, group g) holds the features f0 + v
+      const uint32_t braw[2] = {bias_raw[l].x, bias_raw[l].y};
+      float y[4];
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
-        const int f = 16 * wave + 4 * g + v;
-        float y = sah_round_hw<DT>(acc[v]);
-        y = sah_round_hw<DT>(y + S.bias[l][f]);
-        if (!last) {
-          if (f < dout) S.x[(l + 1) & 1][i16][f] = (uint16_t)sah_pack2_hw<DT>(sig_act_fast(act, y), 0.f);
-        } else if (f < 32) {
-          S.y[i16][f] = f < dout ? y : 0.f;
+        const uint16_t bb = (uint16_t)(braw[v >> 1] >> (16 * (v & 1)));
+        const float bv = (f0 + 4 <= dout) ? ((DT == SAH_BF16) ? sah_bf16_to_float(bb) : sah_f16_to_float(bb)) : 0.f;
+        y[v] = sah_round_hw<DT>(sah_round_hw<DT>(acc[v]) + bv);
+      }
+      if (!last) {
+        if (f0 + 4 <= dout) {
+          const uint2 packed = make_uint2(sah_pack2_hw<DT>(sig_act_fast(act, y[0]), sig_act_fast(act, y[1])),
+                                          sah_pack2_hw<DT>(sig_act_fast(act, y[2]), sig_act_fast(act, y[3])));
+          *(uint2*)&S.x[(l + 1) & 1][i16][f0] = packed;
         }
+      } else if (f0 < 32) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) S.y[i16][f0 + v] = (f0 + 4 <= dout) ? y[v] : 0.f;
       }
     }
     __syncthreads();
@@ -432,7 +442,8 @@ static inline bool sig_mfma_small_ok(const sah_hash_sig_args* a) {
   for (int l = 0; l < a->n_layers; ++l) {
     if (!a->Wt[l] || ((uintptr_t)a->Wt[l] % 16)) return false;
     const bool last = l == a->n_layers - 1;
-    if (last ? a->d_out[l] > 32 : (a->d_out[l] % 32 || a->d_out[l] > SMB_MAXW)) return false;
+    if (last ? (a->d_out[l] > 32 || a->d_out[l] % 4) : (a->d_out[l] % 32 || a->d_out[l] > SMB_MAXW)) return false;
+    if ((uintptr_t)a->bias[l] % 8) return false;
     din = a->d_out[l];
   }
   (void)din;
