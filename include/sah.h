@@ -285,6 +285,8 @@ int sah_select_topk(const sah_select_topk_args* a);
  * accumulation; emitted as sortable keys like sah_qk_scores for candidates
  * n in [0, n_cand) at keys_out[r * key_pitch + n]. centres are the fp32
  * widening of the stored (`dtype`-rounded) centroids, [n_groups, n_cent, d_sub].
+ * The table is built once per call in `lut` (caller's scratch of
+ * sah_pq_adc_lut_bytes(...) bytes) and read from LDS by the scoring kernel.
  * ------------------------------------------------------------------------- */
 typedef struct sah_pq_assign_args {
   const void* k; int64_t ks_b, ks_h, ks_l;
@@ -323,8 +325,10 @@ typedef struct sah_pq_adc_args {
   const uint8_t* codes; int64_t code_pitch;
   int32_t n_cand;
   void* keys_out; int64_t key_pitch;
+  void* lut; int64_t lut_bytes;   /* scratch: sah_pq_adc_lut_bytes(...) bytes */
   void* stream;
 } sah_pq_adc_args;
+int64_t sah_pq_adc_lut_bytes(int32_t B, int32_t Hq, int32_t Hkv, int32_t Lq, int32_t n_sub, int32_t n_cent, int32_t dtype);
 int sah_pq_adc_scores(const sah_pq_adc_args* a);
 
 /* ---------------------------------------------------------------------------

@@ -105,6 +105,73 @@ __global__ __launch_bounds__(PQ_NT) void k_pq_assign(pq_assign_params P) {
   }
 }
 
+// Quantisation of a handful of keys (a decode step appends one): the work of one key and sub-space is a
+// 256-way argmin, so the centres take the threads - one centre per thread, read straight from memory - and
+// the keys take the grid. Same distances, same order of operations and the same lowest-index rule as the
+// one-thread-per-key kernel above.
+template <int DT>
+__global__ __launch_bounds__(PQ_NT) void k_pq_assign_few(pq_assign_params P) {
+  __shared__ float s_d[PQ_NT / SAH_WAVE];
+  __shared__ int s_i[PQ_NT / SAH_WAVE];
+  const int tid = threadIdx.x;
+  const int lane = tid & (SAH_WAVE - 1);
+  const int wave = tid / SAH_WAVE;
+  const int s = blockIdx.x;
+  const int bh = blockIdx.y;
+  const int n = blockIdx.z;
+  const int hk = bh % P.Hkv;
+  const int b = bh / P.Hkv;
+  const int g = bh * P.n_sub + s;
+  const int d_sub = P.d_sub, n_cent = P.n_cent;
+  const int64_t off = (int64_t)b * P.ks_b + (int64_t)hk * P.ks_h + (int64_t)s * d_sub + (int64_t)(P.key_offset + n) * P.ks_l;
+  float dist = INFINITY;
+  int best = 0x7fffffff;
+  for (int c = tid; c < n_cent; c += PQ_NT) {
+    const float* cc = P.centres + ((int64_t)g * n_cent + c) * d_sub;
+    float dd = 0.f;
+    if (P.round_dist) {
+      for (int d = 0; d < d_sub; ++d) {
+        const float df = sah_round<DT>(sah_load<DT>(P.k, off + d) - cc[d]);
+        dd += sah_round<DT>(df * df);
+      }
+      dd = sah_round<DT>(dd);
+    } else {
+      for (int d = 0; d < d_sub; ++d) {
+        const float df = sah_load<DT>(P.k, off + d) - cc[d];
+        dd = fmaf(df, df, dd);
+      }
+    }
+    if (dd < dist) {  // c ascends: the first minimum is kept
+      dist = dd;
+      best = c;
+    }
+  }
+  // smallest distance, lowest centre among equals
+#pragma unroll
+  for (int o = 1; o < SAH_WAVE; o <<= 1) {
+    const float od = __shfl_xor(dist, o);
+    const int oi = __shfl_xor(best, o);
+    if (od < dist || (od == dist && oi < best)) {
+      dist = od;
+      best = oi;
+    }
+  }
+  if (lane == 0) {
+    s_d[wave] = dist;
+    s_i[wave] = best;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    for (int w = 1; w < PQ_NT / SAH_WAVE; ++w) {
+      if (s_d[w] < dist || (s_d[w] == dist && s_i[w] < best)) {
+        dist = s_d[w];
+        best = s_i[w];
+      }
+    }
+    P.codes[(((int64_t)bh * P.code_pitch) + P.code_offset + n) * P.n_sub + s] = (uint8_t)best;
+  }
+}
+
 struct pq_update_params {
   const void* k; int64_t ks_b, ks_h, ks_l;
   int Hkv, n_sub, d_sub, n_cent, key_offset;
@@ -184,70 +251,124 @@ struct pq_adc_params {
   void* keys_out; int64_t key_pitch;
 };
 
-#define ADC_TILES 8
 #define ADC_MAX_LUT 4096  // n_sub * n_cent
+#define ADC_KEYS 2048     // candidates per workgroup of the scoring kernel
 
+// Lookup table of one decode step: lut[bh][vg][s][c][i] = round(q_v . centre[bh][s][c]) for the NQ query vectors
+// v = vg * NQ + i of the KV head's group, in the storage type (fp32: NQ = 2, 16-bit: NQ = 4, i.e. 8 bytes per
+// (s, c): one LDS read serves all the query vectors a workgroup scores).
 template <int DT>
-__global__ __launch_bounds__(PQ_NT) void k_pq_adc(pq_adc_params P) {
+__global__ __launch_bounds__(PQ_NT) void k_pq_lut(pq_adc_params P, void* lut) {
   constexpr int NQ = (DT == SAH_F32) ? 2 : 4;
-  typedef typename std::conditional<DT == SAH_F32, float, uint16_t>::type lut_t;
-  typedef typename std::conditional<DT == SAH_F32, uint32_t, uint16_t>::type key_t;
-  __shared__ lut_t s_lut[NQ * ADC_MAX_LUT];
-  const int tid = threadIdx.x;
+  const int s = blockIdx.x;
   const int bh = blockIdx.y;
+  const int vg = blockIdx.z;
   const int hk = bh % P.Hkv;
   const int b = bh / P.Hkv;
   const int G = P.Hq / P.Hkv;
   const int nvec = G * P.Lq;
-  const int v0 = blockIdx.z * NQ;
-  const int n_sub = P.n_sub, d_sub = P.d_sub, n_cent = P.n_cent;
+  const int n_vg = (nvec + NQ - 1) / NQ;
+  const int d_sub = P.d_sub, n_cent = P.n_cent;
+  for (int c = threadIdx.x; c < n_cent; c += PQ_NT) {
+    const float* cc = P.centres + (((int64_t)bh * P.n_sub + s) * n_cent + c) * d_sub;
+    float val[NQ];
+#pragma unroll
+    for (int i = 0; i < NQ; ++i) {
+      const int v = vg * NQ + i;
+      val[i] = 0.f;
+      if (v < nvec) {
+        const int h = hk * G + v / P.Lq, qi = v % P.Lq;
+        const int64_t qo = (int64_t)b * P.qs_b + (int64_t)h * P.qs_h + (int64_t)qi * P.qs_l + (int64_t)s * d_sub;
+        float acc = 0.f;
+        for (int d = 0; d < d_sub; ++d) acc = fmaf(sah_load<DT>(P.q, qo + d), cc[d], acc);
+        val[i] = sah_round<DT>(acc);
+      }
+    }
+    const int64_t e = (((int64_t)bh * n_vg + vg) * P.n_sub + s) * n_cent + c;
+    if (DT == SAH_F32) {
+      ((float2*)lut)[e] = make_float2(val[0], val[1]);
+    } else {
+      uint2 pk;
+      if (DT == SAH_BF16) {
+        pk.x = (uint32_t)sah_float_to_bf16(val[0]) | ((uint32_t)sah_float_to_bf16(val[1]) << 16);
+        pk.y = (uint32_t)sah_float_to_bf16(val[2]) | ((uint32_t)sah_float_to_bf16(val[3]) << 16);
+      } else {
+        pk.x = (uint32_t)sah_float_to_f16(val[0]) | ((uint32_t)sah_float_to_f16(val[1]) << 16);
+        pk.y = (uint32_t)sah_float_to_f16(val[2]) | ((uint32_t)sah_float_to_f16(val[3]) << 16);
+      }
+      ((uint2*)lut)[e] = pk;
+    }
+  }
+}
+
+// Scores of ADC_KEYS candidates for the NQ query vectors of one group: the table slab (8 bytes per (s, c))
+// in LDS, one thread per candidate, the candidate's codes as 4-byte words.
+template <int DT>
+__global__ __launch_bounds__(PQ_NT) void k_pq_adc(pq_adc_params P, const void* lut) {
+  constexpr int NQ = (DT == SAH_F32) ? 2 : 4;
+  typedef typename std::conditional<DT == SAH_F32, uint32_t, uint16_t>::type key_t;
+  __shared__ uint2 s_lut[ADC_MAX_LUT];
+  const int tid = threadIdx.x;
+  const int bh = blockIdx.y;
+  const int vg = blockIdx.z;
+  const int hk = bh % P.Hkv;
+  const int b = bh / P.Hkv;
+  const int G = P.Hq / P.Hkv;
+  const int nvec = G * P.Lq;
+  const int n_vg = (nvec + NQ - 1) / NQ;
+  const int n_sub = P.n_sub, n_cent = P.n_cent;
   const int lut_n = n_sub * n_cent;
 
   int row[NQ];
 #pragma unroll
   for (int i = 0; i < NQ; ++i) {
-    const int v = v0 + i;
+    const int v = vg * NQ + i;
     row[i] = -1;
     if (v < nvec) row[i] = (b * P.Hq + hk * G + v / P.Lq) * P.Lq + v % P.Lq;
   }
-  for (int idx = tid; idx < NQ * lut_n; idx += PQ_NT) {
-    const int i = idx / lut_n;
-    const int rem = idx % lut_n;
-    const int s = rem / n_cent, c = rem % n_cent;
-    const int v = v0 + i;
-    float val = 0.f;
-    if (v < nvec) {
-      const int h = hk * G + v / P.Lq, qi = v % P.Lq;
-      const int64_t qo = (int64_t)b * P.qs_b + (int64_t)h * P.qs_h + (int64_t)qi * P.qs_l + (int64_t)s * d_sub;
-      const float* cc = P.centres + (((int64_t)bh * n_sub + s) * n_cent + c) * d_sub;
-      float acc = 0.f;
-      for (int d = 0; d < d_sub; ++d) acc = fmaf(sah_load<DT>(P.q, qo + d), cc[d], acc);
-      val = sah_round<DT>(acc);
-    }
-    if (DT == SAH_F32) s_lut[idx] = (lut_t)val;
-    else if (DT == SAH_BF16) s_lut[idx] = (lut_t)sah_float_to_bf16(val);
-    else s_lut[idx] = (lut_t)sah_float_to_f16(val);
-  }
+  const uint2* slab = (const uint2*)lut + ((int64_t)bh * n_vg + vg) * lut_n;
+  for (int i = tid; i < lut_n; i += PQ_NT) s_lut[i] = slab[i];
   __syncthreads();
 
-  for (int t = 0; t < ADC_TILES; ++t) {
-    const int n = (blockIdx.x * ADC_TILES + t) * PQ_NT + tid;
+  const bool words = (n_sub & 3) == 0 && ((P.code_pitch * n_sub) & 3) == 0 && ((uintptr_t)P.codes & 3) == 0;
+  for (int t = 0; t < ADC_KEYS / PQ_NT; ++t) {
+    const int n = blockIdx.x * ADC_KEYS + t * PQ_NT + tid;
     if (n >= P.n_cand) continue;
     const uint8_t* code = P.codes + ((int64_t)bh * P.code_pitch + n) * n_sub;
     float acc[NQ];
 #pragma unroll
     for (int i = 0; i < NQ; ++i) acc[i] = 0.f;
-    for (int s = 0; s < n_sub; ++s) {
-      const int c = code[s];
-#pragma unroll
-      for (int i = 0; i < NQ; ++i) {
-        const lut_t raw = s_lut[i * lut_n + s * n_cent + c];
-        float lv;
-        if (DT == SAH_F32) lv = (float)raw;
-        else if (DT == SAH_BF16) lv = sah_bf16_to_float((uint16_t)raw);
-        else lv = sah_f16_to_float((uint16_t)raw);
-        acc[i] += lv;
+    auto add = [&](int s, int c) {
+      const uint2 e = s_lut[s * n_cent + c];
+      if (DT == SAH_F32) {
+        acc[0] += sah_bits_to_float(e.x);
+        acc[1] += sah_bits_to_float(e.y);
+      } else if (DT == SAH_BF16) {
+        acc[0] += sah_bits_to_float(e.x << 16);
+        acc[1] += sah_bits_to_float(e.x & 0xffff0000u);
+        if (NQ > 2) {
+          acc[2] += sah_bits_to_float(e.y << 16);
+          acc[3] += sah_bits_to_float(e.y & 0xffff0000u);
+        }
+      } else {
+        acc[0] += sah_f16_to_float((uint16_t)(e.x & 0xffffu));
+        acc[1] += sah_f16_to_float((uint16_t)(e.x >> 16));
+        if (NQ > 2) {
+          acc[2] += sah_f16_to_float((uint16_t)(e.y & 0xffffu));
+          acc[3] += sah_f16_to_float((uint16_t)(e.y >> 16));
+        }
       }
+    };
+    if (words) {
+      for (int s4 = 0; s4 < n_sub; s4 += 4) {
+        const uint32_t w = *(const uint32_t*)(code + s4);
+        add(s4, (int)(w & 0xffu));
+        add(s4 + 1, (int)((w >> 8) & 0xffu));
+        add(s4 + 2, (int)((w >> 16) & 0xffu));
+        add(s4 + 3, (int)(w >> 24));
+      }
+    } else {
+      for (int s = 0; s < n_sub; ++s) add(s, (int)code[s]);
     }
 #pragma unroll
     for (int i = 0; i < NQ; ++i) {
@@ -284,9 +405,20 @@ extern "C" int sah_pq_kmeans_assign(const sah_pq_assign_args* a) {
   P.sums = a->sums; P.counts = a->counts;
   P.round_dist = a->round_dist;
   P.skip_flag = a->skip_flag;
+  hipStream_t st = (hipStream_t)a->stream;
+  if (!a->sums && !a->skip_flag && a->n_keys <= 32) {  // new keys of a decode step
+    dim3 gf(a->n_sub, a->B * a->Hkv, a->n_keys), blk(PQ_NT);
+    sah_timed timed("k_pq_assign_few", a->stream);
+    switch (a->dtype) {
+      case SAH_F32: hipLaunchKernelGGL(k_pq_assign_few<SAH_F32>, gf, blk, 0, st, P); break;
+      case SAH_BF16: hipLaunchKernelGGL(k_pq_assign_few<SAH_BF16>, gf, blk, 0, st, P); break;
+      case SAH_F16: hipLaunchKernelGGL(k_pq_assign_few<SAH_F16>, gf, blk, 0, st, P); break;
+      default: return sah_fail(SAH_EDTYPE, "sah_pq_kmeans_assign: dtype %d", a->dtype);
+    }
+    return sah_launch_status("sah_pq_kmeans_assign");
+  }
   const int per_wg = PQ_NT * PQ_TILES;
   dim3 g(((a->n_keys + per_wg - 1) / per_wg) * a->n_sub, a->B * a->Hkv), blk(PQ_NT);
-  hipStream_t st = (hipStream_t)a->stream;
   sah_timed timed("k_pq_assign", a->stream);
   switch (a->dtype) {
     case SAH_F32: hipLaunchKernelGGL(k_pq_assign<SAH_F32>, g, blk, 0, st, P); break;
@@ -326,6 +458,14 @@ extern "C" int sah_pq_kmeans_update(const sah_pq_update_args* a) {
   return sah_launch_status("sah_pq_kmeans_update(promote)");
 }
 
+extern "C" int64_t sah_pq_adc_lut_bytes(int32_t B, int32_t Hq, int32_t Hkv, int32_t Lq, int32_t n_sub, int32_t n_cent,
+                                        int32_t dtype) {
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || Lq <= 0 || n_sub <= 0 || n_cent <= 0 || Hq % Hkv) return 0;
+  const int nq = dtype == SAH_F32 ? 2 : 4;
+  const int n_vg = ((Hq / Hkv) * Lq + nq - 1) / nq;
+  return (int64_t)B * Hkv * n_vg * n_sub * n_cent * 8;
+}
+
 extern "C" int sah_pq_adc_scores(const sah_pq_adc_args* a) {
   if (!a) return sah_fail(SAH_ENULL, "sah_pq_adc_scores: args is NULL");
   int rc = pq_check_common("sah_pq_adc_scores", a->B, a->Hkv, a->n_sub, a->d_sub, a->n_cent);
@@ -342,15 +482,31 @@ extern "C" int sah_pq_adc_scores(const sah_pq_adc_args* a) {
   P.keys_out = a->keys_out; P.key_pitch = a->key_pitch;
   const int nvec = (a->Hq / a->Hkv) * a->Lq;
   const int nq = a->dtype == SAH_F32 ? 2 : 4;
-  const int per_wg = PQ_NT * ADC_TILES;
-  dim3 g((a->n_cand + per_wg - 1) / per_wg, a->B * a->Hkv, (nvec + nq - 1) / nq), blk(PQ_NT);
+  const int n_vg = (nvec + nq - 1) / nq;
+  const int64_t need = (int64_t)a->B * a->Hkv * n_vg * a->n_sub * a->n_cent * 8;
+  if (!a->lut || a->lut_bytes < need)
+    return sah_fail(SAH_ECAPACITY, "sah_pq_adc_scores: lut holds %lld bytes, need %lld", (long long)(a->lut ? a->lut_bytes : 0),
+                    (long long)need);
+  if (n_vg > 65535) return sah_fail(SAH_ESHAPE, "sah_pq_adc_scores: too many query vectors per KV head");
   hipStream_t st = (hipStream_t)a->stream;
+  {
+    dim3 g(a->n_sub, a->B * a->Hkv, n_vg), blk(PQ_NT);
+    sah_timed timed("k_pq_lut", a->stream);
+    switch (a->dtype) {
+      case SAH_F32: hipLaunchKernelGGL(k_pq_lut<SAH_F32>, g, blk, 0, st, P, a->lut); break;
+      case SAH_BF16: hipLaunchKernelGGL(k_pq_lut<SAH_BF16>, g, blk, 0, st, P, a->lut); break;
+      case SAH_F16: hipLaunchKernelGGL(k_pq_lut<SAH_F16>, g, blk, 0, st, P, a->lut); break;
+      default: return sah_fail(SAH_EDTYPE, "sah_pq_adc_scores: dtype %d", a->dtype);
+    }
+    rc = sah_launch_status("sah_pq_adc_scores(lut)");
+    if (rc) return rc;
+  }
+  dim3 g((a->n_cand + ADC_KEYS - 1) / ADC_KEYS, a->B * a->Hkv, n_vg), blk(PQ_NT);
   sah_timed timed("k_pq_adc", a->stream);
   switch (a->dtype) {
-    case SAH_F32: hipLaunchKernelGGL(k_pq_adc<SAH_F32>, g, blk, 0, st, P); break;
-    case SAH_BF16: hipLaunchKernelGGL(k_pq_adc<SAH_BF16>, g, blk, 0, st, P); break;
-    case SAH_F16: hipLaunchKernelGGL(k_pq_adc<SAH_F16>, g, blk, 0, st, P); break;
-    default: return sah_fail(SAH_EDTYPE, "sah_pq_adc_scores: dtype %d", a->dtype);
+    case SAH_F32: hipLaunchKernelGGL(k_pq_adc<SAH_F32>, g, blk, 0, st, P, (const void*)a->lut); break;
+    case SAH_BF16: hipLaunchKernelGGL(k_pq_adc<SAH_BF16>, g, blk, 0, st, P, (const void*)a->lut); break;
+    default: hipLaunchKernelGGL(k_pq_adc<SAH_F16>, g, blk, 0, st, P, (const void*)a->lut); break;
   }
   return sah_launch_status("sah_pq_adc_scores");
 }

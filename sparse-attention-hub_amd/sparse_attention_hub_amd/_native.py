@@ -41,6 +41,7 @@ EXPECTED_SYMBOLS = (
     "sah_pq_kmeans_assign",
     "sah_pq_kmeans_update",
     "sah_pq_adc_scores",
+    "sah_pq_adc_lut_bytes",
     "sah_adaptive_budget",
     "sah_adaptive_sample",
     "sah_sparse_attention_work_floats",
@@ -203,6 +204,7 @@ class PqAdcArgs(C.Structure):
         ("codes", C.c_void_p), ("code_pitch", C.c_int64),
         ("n_cand", C.c_int32),
         ("keys_out", C.c_void_p), ("key_pitch", C.c_int64),
+        ("lut", C.c_void_p), ("lut_bytes", C.c_int64),
         ("stream", C.c_void_p),
     ]
 
@@ -336,8 +338,10 @@ def lib() -> C.CDLL:
     handle.sah_last_error.restype = C.c_char_p
     handle.sah_sparse_attention_work_floats.restype = C.c_int64
     handle.sah_sparse_attention_work_floats.argtypes = [C.c_int32, C.c_int32, C.c_int32]
+    handle.sah_pq_adc_lut_bytes.restype = C.c_int64
+    handle.sah_pq_adc_lut_bytes.argtypes = [C.c_int32] * 7
     for name in EXPECTED_SYMBOLS:
-        if name in ("sah_version", "sah_last_error", "sah_sparse_attention_work_floats",
+        if name in ("sah_version", "sah_last_error", "sah_sparse_attention_work_floats", "sah_pq_adc_lut_bytes",
                     "sah_timing_enable", "sah_timing_collect"):
             continue
         if name == "sah_hash_signatures_pair":

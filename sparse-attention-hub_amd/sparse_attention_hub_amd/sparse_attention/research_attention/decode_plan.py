@@ -29,7 +29,7 @@ from .maskers.fixed.base import sortable_key_of
 from .maskers.fixed.implementations.basic_fixed import LocalMasker, SinkMasker
 from .maskers.fixed.implementations.hashattention_top_k import HashAttentionTopKMasker, PackedSignatureCache
 from .maskers.fixed.implementations.oracle_top_k import OracleTopK
-from .maskers.fixed.implementations.pq_top_k import PQCache, PQCodebook
+from .maskers.fixed.implementations.pq_top_k import PQCache, PQCodebook, adc_lut_buffer
 
 _MAX_NEW_KEYS = 64  # more than this many unseen keys => not a decode step, take the general path
 
@@ -88,6 +88,7 @@ class DecodePlan:
         self.qk = N.QkScoresArgs()
         self.pq_assign = N.PqAssignArgs()
         self.pq_adc = N.PqAdcArgs()
+        self.adc_lut = None
         self.select = N.SelectTopkArgs()
         self.att = N.AttentionArgs()
         self.chain = N.ChainArgs()
@@ -238,6 +239,9 @@ class DecodePlan:
             ad.n_sub, ad.d_sub, ad.n_cent = n_sub, d_sub, n_cent
             ad.centres, ad.codes, ad.code_pitch, ad.n_cand = cf32.data_ptr(), book.codes.data_ptr(), book.capacity, current
             ad.keys_out, ad.key_pitch, ad.stream = self.keybuf.data_ptr(), self.keybuf_pitch, stream
+            if self.adc_lut is None:
+                self.adc_lut = adc_lut_buffer(self.B, self.Hq, self.Hkv, Lq, n_sub, n_cent, self.dtype, self.device)
+            ad.lut, ad.lut_bytes = self.adc_lut.data_ptr(), self.adc_lut.numel()
             chain.pq_adc = C.addressof(ad)
             se = self.select
             se.rows, se.keys, se.key_pitch, se.key_bits = rows, self.keybuf.data_ptr(), self.keybuf_pitch, self.key_bits

@@ -86,6 +86,13 @@ class PQCodebook:
         return self.codes[:, :, : self.n].permute(0, 2, 1, 3).to(torch.int64)
 
 
+def adc_lut_buffer(B: int, Hq: int, Hkv: int, Lq: int, n_sub: int, n_cent: int, dtype: torch.dtype,
+                   device: torch.device) -> torch.Tensor:
+    """Scratch for the per-step lookup table of the ADC scoring (bytes)."""
+    n = int(N.lib().sah_pq_adc_lut_bytes(B, Hq, Hkv, Lq, n_sub, n_cent, N.dtype_code(dtype)))
+    return torch.empty((max(n, 8),), dtype=torch.uint8, device=device)
+
+
 @MaskerRegistry.register(PQCacheConfig)
 class PQCache(TopKMasker):
     def __init__(self, config: PQCacheConfig) -> None:
@@ -194,11 +201,12 @@ class PQCache(TopKMasker):
         rows = previous_mask.to_rows(extra=k_eff)
         keybuf = score_key_buffer(rows.n_rows, n_cand, q.dtype, q.device)
         cf32 = sparse_meta_data["pq_centroids_f32"][layer_idx]
+        lut = adc_lut_buffer(B, Hq, Hkv, Lq, n_sub, n_cent, q.dtype, q.device)
         a = N.PqAdcArgs(
             q.data_ptr(), q.stride(0), q.stride(1), q.stride(2), N.dtype_code(q.dtype),
             B, Hq, Hkv, Lq, n_sub, d_sub, n_cent,
             cf32.data_ptr(), book.codes.data_ptr(), book.capacity, n_cand,
-            keybuf.data_ptr(), keybuf.stride(0), N.stream_ptr(q.device),
+            keybuf.data_ptr(), keybuf.stride(0), lut.data_ptr(), lut.numel(), N.stream_ptr(q.device),
         )
         N.call("sah_pq_adc_scores", a)
         excluded = sortable_key_of(torch.finfo(q.dtype).min, q.dtype)

@@ -35,7 +35,13 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert lib.sah_sparse_attention(None) == -2
     assert b"sah_sparse_attention" in lib.sah_last_error()
     assert lib.sah_select_topk(None) == -2
-    assert N.work_floats(256, 2688, 128) == 256 * 11 * 130
+    # whole rows per workgroup (many short rows): no workspace; few or long rows: (m, l, acc[D]) per split
+    assert N.work_floats(256, 2688, 128) == 0
+    assert N.work_floats(128, 2278, 128) == 128 * 9 * 130
+    assert N.work_floats(512, 131072, 128) == 512 * 32 * 130
+    for fn in ("sah_hash_decode_topk", "sah_adaptive_budget", "sah_adaptive_sample", "sah_pq_adc_scores"):
+        assert getattr(lib, fn)(None) == -2 and fn.encode() in lib.sah_last_error()
+    assert lib.sah_pq_adc_lut_bytes(4, 32, 8, 1, 16, 256, 1) == 4 * 8 * 1 * 16 * 256 * 8
 
 
 def test_struct_layouts_match_header_sizes():
