@@ -483,6 +483,19 @@ def adaptive_sampling(prev: OMask, q, k, attention_mask, scaling: float, rate: S
     return adaptive_merge(prev, draws, prob), budget, prob
 
 
+def random_sampling(prev: OMask, rate: float, seed: int, offset: int) -> OMask:
+    """RandomSamplingMasker.add_mask — random_sampling.py:95-193: int(rate * n_keys) uniform draws per row on
+    [0, n_keys) with replacement (here: Philox call `offset`), weight `rate` in the mask dtype, dense merge."""
+    if prev.kind == "full":
+        return prev
+    B, H, Lq, Lk = prev.shape
+    n = int(rate * Lk)
+    R = B * H * Lq
+    draws = [philox_columns(seed, offset, r, n, 0, Lk) for r in range(R)]
+    prob = torch.full((R,), rate, dtype=prev.dtype)
+    return adaptive_merge(prev, draws, prob)
+
+
 # ----------------------------------------------------------------------- attention
 def masked_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, attention_mask: Optional[torch.Tensor],
                      sinks: Optional[torch.Tensor], scaling: float, mask: OMask,
@@ -519,7 +532,7 @@ def research_attention(masker_specs: Sequence[Tuple], q, k, v, attention_mask, s
     """ResearchAttention.custom_attention — research_attention/base.py:63-170.
     masker_specs: ("sink", size) | ("local", size) | ("oracle_topk", heavy) |
     ("hash_topk", heavy, weights, activation) | ("pq_topk", heavy, init_offset, centroids, codebook) |
-    ("adaptive", rate, epsilon, delta, init_offset, local_offset, seed, offset).
+    ("adaptive", rate, epsilon, delta, init_offset, local_offset, seed, offset) | ("random", rate, seed, offset).
     Returns (out, weights, final OMask)."""
     shape = (q.shape[0], q.shape[1], q.shape[2], k.shape[2])
     m = OMask.empty(shape, q.dtype)
@@ -550,6 +563,8 @@ def research_attention(masker_specs: Sequence[Tuple], q, k, v, attention_mask, s
             m, budget, _ = adaptive_sampling(m, q, k, attention_mask, scaling, spec[1], spec[2], spec[3], spec[4],
                                              spec[5], spec[6], spec[7], state.get("budget"))
             state["budget_oracle"] = budget
+        elif kind == "random":
+            m = random_sampling(m, spec[1], spec[2], spec[3])  # ("random", rate, seed, offset)
         else:
             raise ValueError(kind)
     out, w = masked_attention(q, k, v, attention_mask, sinks, scaling, m)

@@ -8,7 +8,8 @@ from .research_attention.maskers.fixed import (
     SinkMaskerConfig, TopKMasker, TopKMaskerConfig,
 )
 from .research_attention.maskers.sampling import (
-    AdaptiveSamplingMasker, AdaptiveSamplingMaskerConfig, SamplingMasker, SamplingMaskerConfig,
+    AdaptiveSamplingMasker, AdaptiveSamplingMaskerConfig, RandomSamplingMasker, RandomSamplingMaskerConfig,
+    SamplingMasker, SamplingMaskerConfig,
 )
 from .utils.mask import Mask
 
@@ -19,5 +20,6 @@ __all__ = [
     "CausalMasker", "LocalMasker", "LocalMaskerConfig", "SinkMasker", "SinkMaskerConfig",
     "OracleTopK", "OracleTopKConfig", "HashAttentionTopKMasker", "HashAttentionTopKMaskerConfig",
     "PQCache", "PQCacheConfig", "SamplingMasker", "SamplingMaskerConfig",
-    "AdaptiveSamplingMasker", "AdaptiveSamplingMaskerConfig", "Mask",
+    "AdaptiveSamplingMasker", "AdaptiveSamplingMaskerConfig", "RandomSamplingMasker", "RandomSamplingMaskerConfig",
+    "Mask",
 ]

@@ -6,7 +6,8 @@ from .fixed import (  # noqa: F401  (importing registers the maskers)
     SinkMaskerConfig, TopKMasker, TopKMaskerConfig,
 )
 from .sampling import (  # noqa: F401
-    AdaptiveSamplingMasker, AdaptiveSamplingMaskerConfig, SamplingMasker, SamplingMaskerConfig,
+    AdaptiveSamplingMasker, AdaptiveSamplingMaskerConfig, RandomSamplingMasker, RandomSamplingMaskerConfig,
+    SamplingMasker, SamplingMaskerConfig,
 )
 
 __all__ = ["AttentionTensorDimensions", "MaskerConfig", "MaskerRegistry", "ResearchMasker"]

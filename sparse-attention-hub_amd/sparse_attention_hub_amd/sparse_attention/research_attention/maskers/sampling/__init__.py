@@ -1,5 +1,8 @@
 """Sampling maskers."""
 from .base import SamplingMasker, SamplingMaskerConfig
-from .implementations import AdaptiveSamplingMasker, AdaptiveSamplingMaskerConfig
+from .implementations import (
+    AdaptiveSamplingMasker, AdaptiveSamplingMaskerConfig, RandomSamplingMasker, RandomSamplingMaskerConfig,
+)
 
-__all__ = ["SamplingMasker", "SamplingMaskerConfig", "AdaptiveSamplingMasker", "AdaptiveSamplingMaskerConfig"]
+__all__ = ["SamplingMasker", "SamplingMaskerConfig", "AdaptiveSamplingMasker", "AdaptiveSamplingMaskerConfig",
+           "RandomSamplingMasker", "RandomSamplingMaskerConfig"]

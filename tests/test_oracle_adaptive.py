@@ -227,3 +227,38 @@ def test_only_one_sampling_masker_per_chain():
     sa = _sa()
     with pytest.raises(ValueError, match="Only one sampling masker supported"):
         sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=[_cfg(), _cfg()]))
+
+
+# ----------------------------------------------------------------- random sampling
+def test_random_sampling_oracle_and_masker_host_logic():
+    """int(rate * n_keys) draws per row on [0, n_keys), weight = rate, clamp(previous + rate); full mask untouched;
+    config validation of the reference (random_sampling.py:38-44)."""
+    sa = _sa()
+    shape = (1, 2, 1, 50)
+    prev = O.sink(O.OMask.empty(shape, torch.float32), 3)
+    m = O.random_sampling(prev, 0.2, seed=5, offset=0)
+    d = m.to_dense()
+    for h in range(2):
+        draws = O.philox_columns(5, 0, h, 10, 0, 50)
+        assert int(draws.min()) >= 0 and int(draws.max()) < 50
+        new = set(draws.tolist()) - {0, 1, 2}
+        assert set(torch.nonzero(d[0, h, 0]).flatten().tolist()) == new | {0, 1, 2}
+        for c in new:
+            assert float(d[0, h, 0, c]) == pytest.approx(0.2)
+        assert torch.all(d[0, h, 0, :3] == 1.0)
+    full = O.OMask.full(shape, torch.float32)
+    assert O.random_sampling(full, 0.2, 5, 0) is full
+    for bad in (0.0, -0.1, 1.5):
+        with pytest.raises(ValueError, match=r"sampling_rate must be in range \(0, 1\]"):
+            sa.RandomSamplingMaskerConfig(sampling_rate=bad)
+    masker = sa.ResearchMasker.create_masker_from_config(sa.RandomSamplingMaskerConfig(sampling_rate=0.5))
+    assert isinstance(masker, sa.RandomSamplingMasker) and masker.sampling_rate == 0.5
+    fm = sa.Mask.create_full_mask(shape, torch.float32, torch.device("cpu"))
+    q = torch.randn(1, 2, 1, 8)
+    k = torch.randn(1, 2, 50, 8)
+    assert masker.add_mask(k, q, k, None, 1.0, 0.0, {}, fm) is fm
+    tiny = sa.RandomSamplingMasker(sa.RandomSamplingMaskerConfig(sampling_rate=0.01))
+    em = sa.Mask.create_empty_mask(shape, torch.float32, torch.device("cpu"))
+    assert tiny.add_mask(k, q, k, None, 1.0, 0.0, {}, em) is em   # int(0.01 * 50) = 0 draws
+    with pytest.raises(ValueError, match="Invalid config type"):
+        sa.RandomSamplingMasker.create_from_config(sa.SinkMaskerConfig(sink_size=1))
