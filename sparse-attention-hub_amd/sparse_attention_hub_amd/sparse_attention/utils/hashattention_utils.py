@@ -62,3 +62,48 @@ def random_hat_weights(
                 entry[f"{kind}_bias"].append(b.to(dtype).to(device))
         out[layer] = entry
     return out
+
+
+def convert_usa_weights_to_hash_attention(usa_checkpoint, num_layers: int = 32, num_heads: int = 32,
+                                          num_mlp_layers: int = 3, device: str = "cpu") -> HatWeights:
+    """USA-module weights -> the HashAttention layout (reference: hashattention_utils.py:9-116).
+
+    `usa_checkpoint` is a state dict or the path of one (read with torch.load(..., weights_only=True), which
+    executes nothing from the file). Its entries are the per-head torch.nn.Sequential MLPs of the USA module,
+    `{layer}.learning_to_hash_transformation_{q|k}.{head}.{2 i}.{weight|bias}` for MLP layer i (the odd indices are
+    the activations). nn.Linear stores (out, in): matrices are transposed to (in, out) and stacked over the heads;
+    a missing bias becomes zeros. Layers or heads absent from the checkpoint are skipped, like in the reference."""
+    if isinstance(usa_checkpoint, (str, bytes)) or hasattr(usa_checkpoint, "__fspath__"):
+        state = torch.load(usa_checkpoint, map_location=device, weights_only=True)
+    else:
+        state = usa_checkpoint
+    hat_weights: HatWeights = {}
+    for layer_idx in range(num_layers):
+        layer: Dict[str, List[torch.Tensor]] = {"query_matrix": [], "query_bias": [], "key_matrix": [], "key_bias": []}
+        for i in range(num_mlp_layers):
+            per_kind = {}
+            for kind, tag in (("query", "q"), ("key", "k")):
+                mats, biases = [], []
+                for head in range(num_heads):
+                    prefix = f"{layer_idx}.learning_to_hash_transformation_{tag}.{head}.{2 * i}"
+                    weight = state.get(f"{prefix}.weight")
+                    if weight is None:
+                        continue
+                    mats.append(weight.t().to(device))
+                    bias = state.get(f"{prefix}.bias")
+                    biases.append(torch.zeros(weight.shape[0], device=device) if bias is None else bias.to(device))
+                per_kind[kind] = (mats, biases)
+            if per_kind["query"][0]:
+                layer["query_matrix"].append(torch.stack(per_kind["query"][0]))
+                layer["query_bias"].append(torch.stack(per_kind["query"][1]))
+                layer["key_matrix"].append(torch.stack(per_kind["key"][0]))
+                layer["key_bias"].append(torch.stack(per_kind["key"][1]))
+        hat_weights[layer_idx] = layer
+    return hat_weights
+
+
+def create_hat_weights_file_from_usa(usa_checkpoint, target_hat_path: str, num_layers: int = 32, num_heads: int = 32,
+                                     num_mlp_layers: int = 3, device: str = "cpu") -> None:
+    """Convert and save in the reference's HAT file format (hashattention_utils.py:119-152)."""
+    save_hat_weights(convert_usa_weights_to_hash_attention(usa_checkpoint, num_layers, num_heads, num_mlp_layers, device),
+                     target_hat_path)

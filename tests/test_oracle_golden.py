@@ -352,3 +352,40 @@ def test_chain_composition_on_brute_forceable_size():
             want = (p.unsqueeze(1) * vv[sel]).sum(0)
             assert torch.allclose(out[b, 0, h].double(), want, atol=1e-5)
             assert torch.nonzero(m.to_dense()[b, h, 0]).squeeze(-1).tolist() == sel
+
+
+def test_usa_checkpoint_conversion_matches_the_linear_modules(tmp_path):
+    """A USA-style state dict of per-head nn.Sequential MLPs converts to matrices that reproduce the modules'
+    outputs (y = x W^T + b -> x @ matrix + bias) and survives the HAT file round trip (hashattention_utils.py:9-180)."""
+    from sparse_attention_hub_amd.sparse_attention.utils.hashattention_utils import (
+        convert_usa_weights_to_hash_attention, create_hat_weights_file_from_usa, load_hat_weights)
+
+    torch.manual_seed(0)
+    layers, heads, d, hidden, bits = 2, 3, 8, 16, 4
+    state, modules = {}, {}
+    for layer in range(layers):
+        for tag in ("q", "k"):
+            for head in range(heads):
+                seq = torch.nn.Sequential(torch.nn.Linear(d, hidden), torch.nn.SiLU(), torch.nn.Linear(hidden, hidden),
+                                          torch.nn.SiLU(), torch.nn.Linear(hidden, bits, bias=(tag == "q")))
+                modules[(layer, tag, head)] = seq
+                for name, value in seq.state_dict().items():
+                    state[f"{layer}.learning_to_hash_transformation_{tag}.{head}.{name}"] = value
+    hat = convert_usa_weights_to_hash_attention(state, num_layers=layers, num_heads=heads, num_mlp_layers=3)
+    assert sorted(hat) == [0, 1]
+    assert [tuple(m.shape) for m in hat[0]["key_matrix"]] == [(heads, d, hidden), (heads, hidden, hidden), (heads, hidden, bits)]
+    assert torch.all(hat[1]["key_bias"][2] == 0)           # the key MLPs' last layer has no bias: zeros
+    x = torch.randn(1, heads, 5, d)
+    for layer in range(layers):
+        for tag, kind in (("q", "query"), ("k", "key")):
+            sig = O.hash_signatures(x, hat[layer][f"{kind}_matrix"], hat[layer][f"{kind}_bias"], "silu")
+            for head in range(heads):
+                want = torch.sign(modules[(layer, tag, head)](x[0, head]))
+                assert torch.equal(sig[0, head], want)
+    path = tmp_path / "hat.pkl"
+    create_hat_weights_file_from_usa(state, str(path), num_layers=layers, num_heads=heads)
+    again = load_hat_weights(str(path))
+    for layer in range(layers):
+        for name in ("query_matrix", "query_bias", "key_matrix", "key_bias"):
+            for a, b in zip(hat[layer][name], again[layer][name]):
+                assert torch.equal(a, b)
