@@ -199,6 +199,12 @@ __device__ __forceinline__ sah_f32x16 sah_mfma_32x32x16(uint4 a, uint4 b, sah_f3
   return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(sah_f16x8, a), __builtin_bit_cast(sah_f16x8, b), c, 0, 0, 0);
 }
 
+// D = A (32 x 2) * B (2 x 32) + C in fp32 (layouts checked on the hardware): A[i][k]: lane i + 32 k;
+// B[k][j]: lane j + 32 k; C as for the 32 x 32 x 16 form above.
+__device__ __forceinline__ sah_f32x16 sah_mfma_32x32x2_f32(float a, float b, sah_f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+}
+
 // D = A (16 x 32) * B (32 x 16) + C, 16-bit inputs, fp32 accumulation (layouts checked on the hardware):
 //   A[i][k]: lane i + 16 g holds k = 8 g .. 8 g + 7 (g = 0..3);   B[k][j]: lane j + 16 g likewise;
 //   C[i][j]: lane j + 16 g, element v holds i = 4 g + v.

@@ -172,6 +172,134 @@ __global__ __launch_bounds__(PQ_NT) void k_pq_assign_few(pq_assign_params P) {
   }
 }
 
+// ---------------------------------------------------------------------------
+// Lloyd assignment on the matrix cores. argmin_c ||x - c||^2 = argmin_c (||c||^2 - 2 x.c): the key x centre
+// contraction is an fp32 MFMA (32 centres x 32 keys x 2 dims per instruction) whose accumulator starts at
+// ||c||^2 and whose A operand is -2 c, so the accumulator IS the quantity to minimise. A lane owns one key
+// (column) and, per centre tile, 16 centres (rows) in ascending order: the running argmin needs no cross-lane
+// work until the two lanes of a key are merged at the end. Centres (pre-scaled, in operand order) and their
+// norms sit in LDS; per-centre sums for the update step are accumulated in LDS and flushed once.
+// The expansion rounds differently from the difference form of the reference ((A - B)^2 summed,
+// pq_utils.py:220-257): a key whose two nearest centres tie to the last bits may take the other one.
+// ---------------------------------------------------------------------------
+#define PQM_NT 256
+#define PQM_NW (PQM_NT / SAH_WAVE)
+#define PQM_KEY_TILES 16  // 32-key tiles per wave and workgroup: 2048 keys per workgroup
+
+template <int DT, int KS>  // KS = d_sub / 2 k-steps
+__global__ __launch_bounds__(PQM_NT) void k_pq_assign_mfma(pq_assign_params P) {
+  constexpr int DS = 2 * KS;
+  __shared__ __attribute__((aligned(16))) float s_a[(PQ_MAX_CENT / 32) * 2 * 32 * KS];  // -2 c, [tile][g][i][s]
+  __shared__ __attribute__((aligned(16))) float s_cn[(PQ_MAX_CENT / 32) * 2 * 16];      // ||c||^2, [tile][g][v]
+  __shared__ float s_sum[PQ_MAX_CENT * DS];
+  __shared__ int s_cnt[PQ_MAX_CENT];
+  if (P.skip_flag && *P.skip_flag) return;
+  const int tid = threadIdx.x;
+  const int lane = tid & (SAH_WAVE - 1);
+  const int wave = tid / SAH_WAVE;
+  const int j = lane & 31, g = lane >> 5;
+  const int s_idx = blockIdx.x % P.n_sub;
+  const int tg = blockIdx.x / P.n_sub;
+  const int bh = blockIdx.y;
+  const int hk = bh % P.Hkv;
+  const int b = bh / P.Hkv;
+  const int grp = bh * P.n_sub + s_idx;
+  const int n_cent = P.n_cent;
+  const int n_tiles = (n_cent + 31) >> 5;
+  const float* cbase = P.centres + (int64_t)grp * n_cent * DS;
+
+  for (int idx = tid; idx < n_tiles * 2 * 32 * KS; idx += PQM_NT) {
+    const int s = idx % KS, i = (idx / KS) & 31, gg = (idx / (KS * 32)) & 1, t = idx / (KS * 64);
+    const int c = t * 32 + i;
+    s_a[idx] = c < n_cent ? -2.0f * cbase[c * DS + 2 * s + gg] : 0.f;
+  }
+  for (int idx = tid; idx < n_tiles * 32; idx += PQM_NT) {
+    const int v = idx & 15, gg = (idx >> 4) & 1, t = idx >> 5;
+    const int c = t * 32 + 8 * (v >> 2) + 4 * gg + (v & 3);
+    float nn = INFINITY;  // centres beyond n_cent never win
+    if (c < n_cent) {
+      nn = 0.f;
+      for (int d = 0; d < DS; ++d) nn = fmaf(cbase[c * DS + d], cbase[c * DS + d], nn);
+    }
+    s_cn[idx] = nn;
+  }
+  if (P.sums) {
+    for (int i = tid; i < n_cent * DS; i += PQM_NT) s_sum[i] = 0.f;
+    for (int i = tid; i < n_cent; i += PQM_NT) s_cnt[i] = 0;
+  }
+  __syncthreads();
+
+  const int64_t kbase = (int64_t)b * P.ks_b + (int64_t)hk * P.ks_h + (int64_t)s_idx * DS;
+  for (int kt = 0; kt < PQM_KEY_TILES; ++kt) {
+    const int n0 = ((tg * PQM_KEY_TILES + kt) * PQM_NW + wave) * 32;
+    if (n0 >= P.n_keys) break;  // uniform across the wave
+    const int n = n0 + j;
+    const bool valid = n < P.n_keys;
+    const int64_t off = kbase + (int64_t)(P.key_offset + (valid ? n : P.n_keys - 1)) * P.ks_l;
+    float xs[KS];  // this lane's dims 2 s + g of its key
+#pragma unroll
+    for (int s = 0; s < KS; ++s) xs[s] = sah_load<DT>(P.k, off + 2 * s + g);
+    float best = INFINITY;
+    int bidx = 0;
+    for (int t = 0; t < n_tiles; ++t) {
+      sah_f32x16 acc;
+      const float4* cn4 = (const float4*)(s_cn + (t * 2 + g) * 16);
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const float4 c4 = cn4[q4];
+        acc[4 * q4] = c4.x; acc[4 * q4 + 1] = c4.y; acc[4 * q4 + 2] = c4.z; acc[4 * q4 + 3] = c4.w;
+      }
+      const float* ap = s_a + ((t * 2 + g) * 32 + j) * KS;
+#pragma unroll
+      for (int s = 0; s < KS; ++s) acc = sah_mfma_32x32x2_f32(ap[s], xs[s], acc);
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {  // ascending centre index: the first minimum is kept
+        if (acc[v] < best) {
+          best = acc[v];
+          bidx = t * 32 + 8 * (v >> 2) + 4 * g + (v & 3);
+        }
+      }
+    }
+    const float ob = __shfl_xor(best, 32);
+    const int oi = __shfl_xor(bidx, 32);
+    if (ob < best || (ob == best && oi < bidx)) {
+      best = ob;
+      bidx = oi;
+    }
+    if (valid) {
+      if (g == 0) P.codes[(((int64_t)bh * P.code_pitch) + P.code_offset + n) * P.n_sub + s_idx] = (uint8_t)bidx;
+      if (P.sums) {
+#pragma unroll
+        for (int s = 0; s < KS; ++s) atomicAdd(&s_sum[bidx * DS + 2 * s + g], xs[s]);
+        if (g == 0) atomicAdd(&s_cnt[bidx], 1);
+      }
+    }
+  }
+  if (!P.sums) return;
+  __syncthreads();
+  for (int c = tid; c < n_cent; c += PQM_NT) {
+    const int cn = s_cnt[c];
+    if (cn) {
+      atomicAdd(&P.counts[(int64_t)grp * n_cent + c], cn);
+      for (int d = 0; d < DS; ++d) atomicAdd(&P.sums[(int64_t)grp * n_cent * DS + c * DS + d], s_sum[c * DS + d]);
+    }
+  }
+}
+
+template <int DT>
+static int pq_launch_mfma(const sah_pq_assign_args* a, const pq_assign_params& P) {
+  const int per_wg = PQM_NW * 32 * PQM_KEY_TILES;
+  dim3 g(((a->n_keys + per_wg - 1) / per_wg) * a->n_sub, a->B * a->Hkv), blk(PQM_NT);
+  hipStream_t st = (hipStream_t)a->stream;
+  sah_timed timed("k_pq_assign_mfma", a->stream);
+  switch (a->d_sub) {
+    case 4: hipLaunchKernelGGL((k_pq_assign_mfma<DT, 2>), g, blk, 0, st, P); break;
+    case 8: hipLaunchKernelGGL((k_pq_assign_mfma<DT, 4>), g, blk, 0, st, P); break;
+    default: hipLaunchKernelGGL((k_pq_assign_mfma<DT, 8>), g, blk, 0, st, P); break;
+  }
+  return sah_launch_status("sah_pq_kmeans_assign");
+}
+
 struct pq_update_params {
   const void* k; int64_t ks_b, ks_h, ks_l;
   int Hkv, n_sub, d_sub, n_cent, key_offset;
@@ -416,6 +544,15 @@ extern "C" int sah_pq_kmeans_assign(const sah_pq_assign_args* a) {
       default: return sah_fail(SAH_EDTYPE, "sah_pq_kmeans_assign: dtype %d", a->dtype);
     }
     return sah_launch_status("sah_pq_kmeans_assign");
+  }
+  if (!a->round_dist && a->n_keys >= 1024 && (a->d_sub == 4 || a->d_sub == 8 || a->d_sub == 16)) {
+    // Lloyd iterations over a whole context: the contraction goes to the matrix cores
+    switch (a->dtype) {
+      case SAH_F32: return pq_launch_mfma<SAH_F32>(a, P);
+      case SAH_BF16: return pq_launch_mfma<SAH_BF16>(a, P);
+      case SAH_F16: return pq_launch_mfma<SAH_F16>(a, P);
+      default: return sah_fail(SAH_EDTYPE, "sah_pq_kmeans_assign: dtype %d", a->dtype);
+    }
   }
   const int per_wg = PQ_NT * PQ_TILES;
   dim3 g(((a->n_keys + per_wg - 1) / per_wg) * a->n_sub, a->B * a->Hkv), blk(PQ_NT);
