@@ -1,0 +1,330 @@
+// Row-wise top-k over 16-bit sortable keys (bf16 / fp16 scores), eight candidates per lane.
+//
+// One workgroup of 1024 threads per mask row. A lane owns eight consecutive candidates of a
+// 512-candidate chunk: one 16-byte load brings their keys, one byte of the bitmap row tells
+// which of them are already active. The k-th largest key is found by two 256-bin histogram
+// levels (high byte in wave-private LDS histograms, then the low byte of the keys inside the
+// chosen bin), so the pass count is fixed: level 1, level 2, count, write; rows of up to
+// 131072 candidates stay in registers from the first pass on.
+// Winners above the threshold are written by every wave independently; only the wave that
+// holds the last accepted tie walks its candidates in column order, which keeps the
+// canonical rule "equal keys: lowest column first" at the cost of one ordered wave.
+// The output list is unordered inside a row (its order is still a pure function of the
+// inputs), as the attention kernel does not need sorted columns.
+#pragma once
+#include "sah_common.h"
+
+#define SF_NT 1024
+#define SF_NW (SF_NT / SAH_WAVE)
+#define SF_CHUNK 512  // candidates a wave covers with one load per lane
+#define SF_BATCH 4    // chunks a wave has in flight
+#define SF_COPIES 32  // counters per high-byte bin (lanes l and l + 32 share one, and a bank anyway)
+
+struct sf_lds {
+  int part[SF_NW];
+  int eq[SF_NW];
+  int out[SF_NW];
+  int sel_bin, sel_need;
+};
+
+struct sf_chunk {
+  uint32_t k[4];   // eight effective keys, candidate 2p in the low half of k[p]
+  uint32_t excl;   // bit t: candidate t is already active (ranks with the excluded key, emits nothing)
+  uint32_t valid;  // bit t: candidate t exists
+};
+
+__device__ __forceinline__ uint32_t sf_key(const sf_chunk& c, int t) {
+  return (t & 1) ? (c.k[t >> 1] >> 16) : (c.k[t >> 1] & 0xffffu);
+}
+// two flag bits -> two 16-bit lane masks
+__device__ __forceinline__ uint32_t sf_mask2(uint32_t bits) {
+  return (0u - (bits & 1u)) & 0xffffu | ((0u - ((bits >> 1) & 1u)) & 0xffff0000u);
+}
+
+// active / existing flags of the eight candidates starting at `cand`
+__device__ __forceinline__ void sf_flags(const uint32_t* s_bm, int n_words, int cand, int n_cand, int col_offset,
+                                         uint32_t& excl, uint32_t& valid) {
+  int nv = n_cand - cand;
+  nv = nv < 0 ? 0 : (nv > 8 ? 8 : nv);
+  valid = (1u << nv) - 1u;
+  const int col = cand + col_offset;
+  int wi = col >> 5;
+  wi = wi < n_words ? wi : n_words - 1;  // s_bm has one zero word of padding behind the row
+  const uint64_t two = ((uint64_t)s_bm[wi + 1] << 32) | s_bm[wi];
+  excl = (uint32_t)(two >> (col & 31)) & valid;
+}
+
+// keys straight from memory -> effective keys (active candidates take `ek2`, missing ones 0)
+__device__ __forceinline__ void sf_effective(sf_chunk& c, uint4 raw, uint32_t ek2) {
+  const uint32_t r[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    const uint32_t me = sf_mask2(c.excl >> (2 * p));
+    const uint32_t mv = sf_mask2(c.valid >> (2 * p));
+    c.k[p] = ((r[p] & ~me) | (ek2 & me)) & mv;
+  }
+}
+
+// k-th largest bin of a 256-bin histogram. Thread t brings a partial count of bin 255 - t/4
+// (the four threads of a quad split the copies of that bin); all SF_NT threads call.
+__device__ __forceinline__ void sf_pick(int partial, int k, sf_lds& S, int& bin, int& need) {
+  const int tid = threadIdx.x;
+  const int lane = tid & (SAH_WAVE - 1);
+  const int wave = tid / SAH_WAVE;
+  int tot = partial + sah_dpp_i<0xB1, 0xF, true>(partial);  // quad_perm [1,0,3,2]
+  tot += sah_dpp_i<0x4E, 0xF, true>(tot);                   // quad_perm [2,3,0,1]
+  const int v = (tid & 3) == 0 ? tot : 0;
+  const int incl = sah_wave_incl_scan(v);
+  if (lane == SAH_WAVE - 1) S.part[wave] = incl;
+  __syncthreads();
+  if ((tid & 3) == 0) {
+    int above = incl - v;
+    for (int w = 0; w < wave; ++w) above += S.part[w];
+    if (above < k && k <= above + tot) {
+      S.sel_bin = 255 - (tid >> 2);
+      S.sel_need = k - above;
+    }
+  }
+  __syncthreads();
+  bin = S.sel_bin;
+  need = S.sel_need;
+}
+
+// the `allowed` lowest set bits of an 8-bit mask
+__device__ __forceinline__ uint32_t sf_lowest(uint32_t m, int allowed) {
+  uint32_t take = 0;
+  while (allowed > 0 && m) {
+    const uint32_t b = m & (0u - m);
+    take |= b;
+    m ^= b;
+    --allowed;
+  }
+  return take;
+}
+
+// CPW > 0: a wave keeps the effective keys of its (at most CPW) chunks in registers through
+// all passes; CPW == 0: rows too long for that re-read their keys from memory in every pass.
+template <int CPW>
+__device__ __forceinline__ void sf_select_row(sf_lds& S, unsigned char* dyn, const sah_rows& R, int r,
+                                              const uint16_t* keys, int n_cand, int col_offset, int k,
+                                              uint32_t excluded_key) {
+  constexpr bool REG = CPW > 0;
+  constexpr int NREG = REG ? CPW : 1;
+  const int tid = threadIdx.x;
+  const int lane = tid & (SAH_WAVE - 1);
+  const int wave = tid / SAH_WAVE;
+  const int n_chunks = (n_cand + SF_CHUNK - 1) / SF_CHUNK;
+  const int cpw = (n_chunks + SF_NW - 1) / SF_NW;  // <= CPW when REG (the host picks CPW)
+  const int c0 = wave * cpw;
+  const int c1 = c0 + cpw < n_chunks ? c0 + cpw : n_chunks;
+
+  // Histograms: SF_COPIES counters per bin, indexed by lane, so that the lanes of one atomic
+  // instruction never meet on an address however few bins the keys fall into (the high byte
+  // of a float key is sign + exponent: a handful of bins hold everything).
+  uint32_t* s_bm = (uint32_t*)dyn;                     // n_words + 2
+  uint32_t* s_h1 = s_bm + ((R.n_words + 2 + 3) & ~3);  // high byte: [256][SF_COPIES]
+  uint32_t* s_h2 = s_h1 + 256 * SF_COPIES;             // low byte inside the chosen bin
+  uint32_t* bm = R.bitmap + (int64_t)r * R.n_words;
+  const uint32_t ek = excluded_key & 0xffffu;
+  const uint32_t ek2 = ek * 0x00010001u;
+
+  auto raw_load = [&](int c) -> uint4 {
+    int cand = c * SF_CHUNK + lane * 8;
+    if (cand >= n_cand) cand = 0;  // a group with no candidate: any valid address will do
+    return *(const uint4*)(keys + cand);
+  };
+  auto effective = [&](int c, uint4 raw) -> uint4 {
+    sf_chunk ch;
+    sf_flags(s_bm, R.n_words, c * SF_CHUNK + lane * 8, n_cand, col_offset, ch.excl, ch.valid);
+    sf_effective(ch, raw, ek2);
+    return make_uint4(ch.k[0], ch.k[1], ch.k[2], ch.k[3]);
+  };
+
+  uint4 kreg[NREG];
+  if (REG) {
+    // the key loads go out first and land while the bitmap row and the counters are set up
+#pragma unroll
+    for (int u = 0; u < NREG; ++u) kreg[u] = raw_load(c0 + u);
+  }
+  int cnt0 = R.cnt[r];  // read before the first barrier: rewritten at the end
+  if (cnt0 > R.cap) cnt0 = R.cap;
+  for (int i = tid; i < R.n_words + 2; i += SF_NT) s_bm[i] = i < R.n_words ? bm[i] : 0u;
+  for (int i = tid; i < 2 * 256 * SF_COPIES / 4; i += SF_NT) ((uint4*)s_h1)[i] = make_uint4(0u, 0u, 0u, 0u);
+  __syncthreads();
+  if (REG) {
+#pragma unroll
+    for (int u = 0; u < NREG; ++u) kreg[u] = effective(c0 + u, kreg[u]);
+  }
+
+  // run f(c, keys) over this wave's chunks in ascending order
+  auto for_chunks = [&](auto&& f) {
+    if (REG) {
+#pragma unroll
+      for (int u = 0; u < NREG; ++u)
+        if (c0 + u < c1) {
+          // opaque to the optimiser: values derived from the keys in one pass are not kept
+          // alive for the next, they are cheaper to recompute than to hold in registers
+          sah_keep(kreg[u].x), sah_keep(kreg[u].y), sah_keep(kreg[u].z), sah_keep(kreg[u].w);
+          const uint32_t kk[4] = {kreg[u].x, kreg[u].y, kreg[u].z, kreg[u].w};
+          f(c0 + u, kk);
+        }
+    } else {
+      for (int cb = c0; cb < c1; cb += SF_BATCH) {
+        uint4 raw[SF_BATCH];
+#pragma unroll
+        for (int u = 0; u < SF_BATCH; ++u) raw[u] = raw_load(cb + u < c1 ? cb + u : c1 - 1);
+#pragma unroll
+        for (int u = 0; u < SF_BATCH; ++u)
+          if (cb + u < c1) {
+            const uint4 e = effective(cb + u, raw[u]);
+            const uint32_t kk[4] = {e.x, e.y, e.z, e.w};
+            f(cb + u, kk);
+          }
+      }
+    }
+  };
+  auto key_of = [](const uint32_t (&kk)[4], int t) -> uint32_t {
+    return (t & 1) ? (kk[t >> 1] >> 16) : (kk[t >> 1] & 0xffffu);
+  };
+  // thread t sums a quarter of the counters of bin 255 - t/4, then the block picks the bin
+  auto pick = [&](const uint32_t* hist, int kk, int& bin, int& nd) {
+    const uint4* h = (const uint4*)(hist + (255 - (tid >> 2)) * SF_COPIES + (tid & 3) * (SF_COPIES / 4));
+    int partial = 0;
+#pragma unroll
+    for (int i = 0; i < SF_COPIES / 16; ++i) {
+      const uint4 q = h[i];
+      partial += (int)(q.x + q.y + q.z + q.w);
+    }
+    sf_pick(partial, kk, S, bin, nd);
+  };
+
+  // ---- pass 1: histogram of the high byte ------------------------------------------------
+  uint32_t* my_h1 = s_h1 + (lane & (SF_COPIES - 1));
+  uint32_t* my_h2 = s_h2 + (lane & (SF_COPIES - 1));
+  for_chunks([&](int, const uint32_t (&kk)[4]) {
+#pragma unroll
+    for (int t = 0; t < 8; ++t) atomicAdd(&my_h1[(key_of(kk, t) >> 8) * SF_COPIES], 1u);
+  });
+  __syncthreads();
+  int b1, need1;
+  pick(s_h1, k, b1, need1);
+
+  // ---- pass 2: histogram of the low byte inside bin b1 ---------------------------------
+  for_chunks([&](int, const uint32_t (&kk)[4]) {
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      const uint32_t key = key_of(kk, t);
+      atomicAdd(&my_h2[(key & 0xffu) * SF_COPIES], (int)(key >> 8) == b1 ? 1u : 0u);
+    }
+  });
+  __syncthreads();
+  int b2, need;
+  pick(s_h2, need1, b2, need);
+  const uint32_t T = ((uint32_t)b1 << 8) | (uint32_t)b2;
+  // Active candidates carry the excluded key. While that ranks below the threshold they are
+  // neither winners nor ties and their flags are not needed again; otherwise (a row with
+  // fewer than k better inactive candidates) they take rank but are never emitted.
+  const bool slow = ek >= T;
+
+  // 8-bit masks of one chunk: emittable keys above the threshold, ties, active candidates
+  auto masks = [&](int c, const uint32_t (&kk)[4], uint32_t& gt, uint32_t& eq, uint32_t& ex) {
+    gt = 0, eq = 0, ex = 0;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      const uint32_t key = key_of(kk, t);
+      gt |= (key > T ? 1u : 0u) << t;
+      eq |= (key == T ? 1u : 0u) << t;
+    }
+    if (slow) {
+      uint32_t valid;
+      sf_flags(s_bm, R.n_words, c * SF_CHUNK + lane * 8, n_cand, col_offset, ex, valid);
+      eq &= valid;  // a missing candidate has key 0, which ties when T is 0
+      gt &= ~ex;
+    }
+  };
+
+  // ---- pass 3: winners and ties per lane and wave --------------------------------------------
+  int n_gt = 0, n_eq = 0;
+  for_chunks([&](int c, const uint32_t (&kk)[4]) {
+    uint32_t gt, eq, ex;
+    masks(c, kk, gt, eq, ex);
+    n_gt += __popc(gt);
+    n_eq += __popc(eq);
+  });
+  const int wave_eq = sah_wave_sum_i(n_eq);
+  if (lane == 0) S.eq[wave] = wave_eq;
+  __syncthreads();
+  int tie_base = 0;
+  for (int w = 0; w < wave; ++w) tie_base += S.eq[w];
+  // 0: no tie of this wave is taken, 1: all are, 2: the boundary lies inside the wave
+  const int mode = tie_base >= need ? 0 : (tie_base + wave_eq <= need ? 1 : 2);
+
+  // emission mask of a chunk; `tie_run` counts the wave's ties seen so far (mode 2 only)
+  int tie_run = tie_base;
+  auto emit_mask = [&](int c, const uint32_t (&kk)[4]) -> uint32_t {
+    uint32_t gt, eq, ex;
+    masks(c, kk, gt, eq, ex);
+    uint32_t take = 0;
+    if (mode == 1) take = eq;
+    if (mode == 2) {
+      const int ne = __popc(eq);
+      const int incl = sah_wave_incl_scan(ne);
+      take = sf_lowest(eq, need - tie_run - (incl - ne));
+      tie_run += __builtin_amdgcn_readlane(incl, SAH_WAVE - 1);
+    }
+    return gt | (take & ~ex);
+  };
+
+  // what each lane emits: known from the counts, except where ties are cut or may be active
+  int mine = n_gt + (mode == 1 ? n_eq : 0);
+  if (mode == 2 || slow) {
+    mine = 0;
+    for_chunks([&](int c, const uint32_t (&kk)[4]) { mine += __popc(emit_mask(c, kk)); });
+  }
+  const int incl = sah_wave_incl_scan(mine);
+  if (lane == SAH_WAVE - 1) S.out[wave] = incl;
+  __syncthreads();
+  int out_base = 0, total = 0;
+  for (int w = 0; w < SF_NW; ++w) {
+    const int v = S.out[w];
+    out_base += w < wave ? v : 0;
+    total += v;
+  }
+
+  // ---- pass 4: write ---------------------------------------------------------------------------
+  int* cols = R.cols + (int64_t)r * R.cap;
+  float* wgt = R.w ? R.w + (int64_t)r * R.cap : nullptr;
+  int pos = cnt0 + out_base + incl - mine;
+  tie_run = tie_base;
+  for_chunks([&](int c, const uint32_t (&kk)[4]) {
+    uint32_t em = emit_mask(c, kk);
+    if (em) {
+      const int col0 = c * SF_CHUNK + lane * 8 + col_offset;
+      atomicOr(&s_bm[col0 >> 5], em << (col0 & 31));
+      if ((col0 & 31) > 24) atomicOr(&s_bm[(col0 >> 5) + 1], em >> (32 - (col0 & 31)));
+      while (em) {
+        const int t = __builtin_ctz(em);
+        em &= em - 1;
+        if (pos < R.cap) {
+          cols[pos] = col0 + t;
+          if (wgt) wgt[pos] = 1.0f;
+        }
+        ++pos;
+      }
+    }
+  });
+  __syncthreads();
+  if (total > 0)
+    for (int i = tid; i < R.n_words; i += SF_NT) bm[i] = s_bm[i];
+  if (tid == 0) R.cnt[r] = cnt0 + total;
+}
+
+// dynamic LDS bytes of one launch
+static inline size_t sf_lds_bytes(int n_words) {
+  return (size_t)((n_words + 2 + 3) & ~3) * 4 + (size_t)2 * 256 * SF_COPIES * 4;
+}
+// chunks per wave of a row of n_cand candidates
+static inline int sf_chunks_per_wave(int n_cand) {
+  const int n_chunks = (n_cand + SF_CHUNK - 1) / SF_CHUNK;
+  return (n_chunks + SF_NW - 1) / SF_NW;
+}

@@ -11,6 +11,7 @@
 // touched by no other wave and need no atomics.
 #include "sah_common.h"
 #include "sah_hsw.h"
+#include "sah_sel16.h"
 
 #define SEL_NT 1024
 #define SEL_NW (SEL_NT / SAH_WAVE)
@@ -385,6 +386,16 @@ __global__ __launch_bounds__(HSW_NT) void k_hamming_topk_swar(sah_rows R, const 
   hsw_select_row(R, r, kcodes + (int64_t)(r / lq) * pitch, qcodes[r], k, cnt0, s_bm, s_key, S, buf);
 }
 
+template <int CPW>
+__global__ __launch_bounds__(SF_NT) void k_select16(sah_rows R, const uint16_t* keys, int64_t pitch, int n_cand,
+                                                    int col_offset, int k, uint32_t excluded_key) {
+  __shared__ sf_lds S;
+  HIP_DYNAMIC_SHARED(unsigned char, sf_dyn)
+  const int r = blockIdx.x;
+  sf_select_row<CPW>(S, sf_dyn, R, r, keys + (int64_t)r * pitch, n_cand, col_offset, k < n_cand ? k : n_cand,
+                     excluded_key);
+}
+
 // kernels may use up to 160 KB of LDS; HIP needs to be told once per kernel
 template <typename K>
 static int sel_allow_lds(K kernel, size_t bytes, const char* what) {
@@ -458,6 +469,26 @@ extern "C" int sah_select_topk(const sah_select_topk_args* a) {
   if (a->k <= 0) return sah_fail(SAH_EINVAL, "sah_select_topk: k must be > 0");
   if (a->key_pitch < a->n_cand) return sah_fail(SAH_EINVAL, "sah_select_topk: key_pitch < n_cand");
   hipStream_t st = (hipStream_t)a->stream;
+  if (a->key_bits == 16 && a->key_pitch % 8 == 0 && ((uintptr_t)a->keys % 16) == 0) {
+    // eight keys per lane: needs 16-byte aligned key rows
+    const size_t lds = sf_lds_bytes(a->rows.n_words);
+    if (lds > 150 * 1024) return sah_fail(SAH_ESHAPE, "sah_select_topk: %d keys need %zu bytes of LDS", a->rows.n_keys, lds);
+    const int cpw = sf_chunks_per_wave(a->n_cand);
+    sah_timed timed("k_select_topk", a->stream);
+#define SAH_SEL16(CPW)                                                                                      \
+  do {                                                                                                      \
+    rc = sel_allow_lds(k_select16<CPW>, lds, "sah_select_topk");                                            \
+    if (rc) return rc;                                                                                      \
+    hipLaunchKernelGGL(k_select16<CPW>, dim3(a->rows.n_rows), dim3(SF_NT), lds, st, a->rows,                \
+                       (const uint16_t*)a->keys, a->key_pitch, a->n_cand, a->col_offset, a->k, a->excluded_key); \
+  } while (0)
+    if (cpw <= 4) SAH_SEL16(4);
+    else if (cpw <= 8) SAH_SEL16(8);
+    else if (cpw <= 16) SAH_SEL16(16);
+    else SAH_SEL16(0);
+#undef SAH_SEL16
+    return sah_launch_status("sah_select_topk");
+  }
   sel_layout L;
   const size_t lds = sel_plan(a->key_bits, a->key_bits / 8, a->rows.n_words, a->n_cand, a->col_offset, &L);
   if (lds > 159 * 1024) return sah_fail(SAH_ESHAPE, "sah_select_topk: %d keys need %zu bytes of LDS", a->rows.n_keys, lds);
