@@ -230,6 +230,29 @@ __device__ __forceinline__ void sah_keep(float& v) {
 #endif
 }
 
+// Two unsigned 16-bit compares per instruction pair, for keys packed two to a word.
+// Result per half: 1 where a > b, else 0 (saturating packed subtract, then min with 1).
+__device__ __forceinline__ uint32_t sah_pk_gt01_u16(uint32_t a, uint32_t b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  uint32_t d;
+  asm("v_pk_sub_u16 %0, %1, %2 clamp" : "=v"(d) : "v"(a), "v"(b));
+  asm("v_pk_min_u16 %0, %1, %2" : "=v"(d) : "v"(d), "v"(0x00010001u));
+  return d;
+#else
+  return ((a & 0xffffu) > (b & 0xffffu) ? 1u : 0u) | ((a >> 16) > (b >> 16) ? 0x10000u : 0u);
+#endif
+}
+// Result per half: 1 where a != b, else 0
+__device__ __forceinline__ uint32_t sah_pk_ne01_u16(uint32_t a, uint32_t b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  uint32_t d;
+  asm("v_pk_min_u16 %0, %1, %2" : "=v"(d) : "v"(a ^ b), "v"(0x00010001u));
+  return d;
+#else
+  return ((a ^ b) & 0xffffu ? 1u : 0u) | ((a ^ b) >> 16 ? 0x10000u : 0u);
+#endif
+}
+
 // ---------------------------------------------------------------------------
 // device side: cross-lane helpers
 // ---------------------------------------------------------------------------

@@ -18,7 +18,8 @@
 #define SF_NW (SF_NT / SAH_WAVE)
 #define SF_CHUNK 512  // candidates a wave covers with one load per lane
 #define SF_BATCH 4    // chunks a wave has in flight
-#define SF_COPIES 32  // counters per high-byte bin (lanes l and l + 32 share one, and a bank anyway)
+#define SF_COPIES 64  // counters per bin: one per lane
+static_assert(SF_COPIES == 64, "sf_pick reads one row of 16 lanes x 4 counters per bin");
 
 struct sf_lds {
   int part[SF_NW];
@@ -28,18 +29,17 @@ struct sf_lds {
 };
 
 struct sf_chunk {
-  uint32_t k[4];   // eight effective keys, candidate 2p in the low half of k[p]
+  uint32_t k[4];   // eight effective keys: candidate p in the low half of k[p], candidate p + 4 in the high half
   uint32_t excl;   // bit t: candidate t is already active (ranks with the excluded key, emits nothing)
   uint32_t valid;  // bit t: candidate t exists
 };
 
-__device__ __forceinline__ uint32_t sf_key(const sf_chunk& c, int t) {
-  return (t & 1) ? (c.k[t >> 1] >> 16) : (c.k[t >> 1] & 0xffffu);
+// flag bits p and p + 4 -> the two 16-bit masks of word p
+__device__ __forceinline__ uint32_t sf_mask2(uint32_t flags, int p) {
+  return ((0u - ((flags >> p) & 1u)) & 0xffffu) | ((0u - ((flags >> (p + 4)) & 1u)) & 0xffff0000u);
 }
-// two flag bits -> two 16-bit lane masks
-__device__ __forceinline__ uint32_t sf_mask2(uint32_t bits) {
-  return (0u - (bits & 1u)) & 0xffffu | ((0u - ((bits >> 1) & 1u)) & 0xffff0000u);
-}
+// split mask (bit p: low half of word p, bit 16 + p: high half) -> one bit per candidate
+__device__ __forceinline__ uint32_t sf_join(uint32_t split) { return (split | (split >> 12)) & 0xffu; }
 
 // active / existing flags of the eight candidates starting at `cand`
 __device__ __forceinline__ void sf_flags(const uint32_t* s_bm, int n_words, int cand, int n_cand, int col_offset,
@@ -54,35 +54,64 @@ __device__ __forceinline__ void sf_flags(const uint32_t* s_bm, int n_words, int 
   excl = (uint32_t)(two >> (col & 31)) & valid;
 }
 
-// keys straight from memory -> effective keys (active candidates take `ek2`, missing ones 0)
+// keys straight from memory -> effective keys (active candidates take `ek2`, missing ones 0),
+// re-paired so that one packed compare yields mask bits in candidate order
 __device__ __forceinline__ void sf_effective(sf_chunk& c, uint4 raw, uint32_t ek2) {
-  const uint32_t r[4] = {raw.x, raw.y, raw.z, raw.w};
+  c.k[0] = (raw.x & 0xffffu) | (raw.z << 16);
+  c.k[1] = (raw.x >> 16) | (raw.z & 0xffff0000u);
+  c.k[2] = (raw.y & 0xffffu) | (raw.w << 16);
+  c.k[3] = (raw.y >> 16) | (raw.w & 0xffff0000u);
+  if (c.excl) {
 #pragma unroll
-  for (int p = 0; p < 4; ++p) {
-    const uint32_t me = sf_mask2(c.excl >> (2 * p));
-    const uint32_t mv = sf_mask2(c.valid >> (2 * p));
-    c.k[p] = ((r[p] & ~me) | (ek2 & me)) & mv;
+    for (int p = 0; p < 4; ++p) {
+      const uint32_t me = sf_mask2(c.excl, p);
+      c.k[p] = (c.k[p] & ~me) | (ek2 & me);
+    }
+  }
+  if (c.valid != 0xffu) {
+#pragma unroll
+    for (int p = 0; p < 4; ++p) c.k[p] &= sf_mask2(c.valid, p);
   }
 }
 
-// k-th largest bin of a 256-bin histogram. Thread t brings a partial count of bin 255 - t/4
-// (the four threads of a quad split the copies of that bin); all SF_NT threads call.
-__device__ __forceinline__ void sf_pick(int partial, int k, sf_lds& S, int& bin, int& need) {
+// k-th largest bin of a 256-bin histogram of [256][SF_COPIES] counters; all SF_NT threads call.
+// Wave w owns the 16 bins 255 - 16w .. 240 - 16w. One 16-byte read per lane covers four
+// bins (a row of 16 lanes per bin, 1 KB contiguous per instruction, no bank conflict); the
+// row sums become wave-uniform scalars, so the scan over the wave's bins is scalar work.
+__device__ __forceinline__ void sf_pick(const uint32_t* hist, int k, sf_lds& S, int& bin, int& need) {
   const int tid = threadIdx.x;
   const int lane = tid & (SAH_WAVE - 1);
   const int wave = tid / SAH_WAVE;
-  int tot = partial + sah_dpp_i<0xB1, 0xF, true>(partial);  // quad_perm [1,0,3,2]
-  tot += sah_dpp_i<0x4E, 0xF, true>(tot);                   // quad_perm [2,3,0,1]
-  const int v = (tid & 3) == 0 ? tot : 0;
-  const int incl = sah_wave_incl_scan(v);
-  if (lane == SAH_WAVE - 1) S.part[wave] = incl;
+  int cnt[16];  // cnt[4 * i + row]: bin 255 - (16 * wave + 4 * i + row)
+  int wave_total = 0;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int b = 255 - (16 * wave + 4 * i + (lane >> 4));
+    const uint4 q = *(const uint4*)(hist + b * SF_COPIES + (lane & 15) * 4);
+    int v = (int)(q.x + q.y + q.z + q.w);
+    v += sah_dpp_i<0xB1, 0xF, true>(v);   // quad_perm [1,0,3,2]
+    v += sah_dpp_i<0x4E, 0xF, true>(v);   // quad_perm [2,3,0,1]
+    v += sah_dpp_i<0x141, 0xF, true>(v);  // row_half_mirror
+    v += sah_dpp_i<0x140, 0xF, true>(v);  // row_mirror
+#pragma unroll
+    for (int row = 0; row < 4; ++row) {
+      cnt[4 * i + row] = __builtin_amdgcn_readlane(v, 16 * row);
+      wave_total += cnt[4 * i + row];
+    }
+  }
+  if (lane == 0) S.part[wave] = wave_total;
   __syncthreads();
-  if ((tid & 3) == 0) {
-    int above = incl - v;
-    for (int w = 0; w < wave; ++w) above += S.part[w];
-    if (above < k && k <= above + tot) {
-      S.sel_bin = 255 - (tid >> 2);
-      S.sel_need = k - above;
+  int above = 0;
+#pragma unroll
+  for (int w = 0; w < SF_NW; ++w) above += w < wave ? S.part[w] : 0;
+  if (above < k && k <= above + wave_total) {  // wave-uniform: the bin lies in this wave's range
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      if (above < k && k <= above + cnt[j] && lane == 0) {
+        S.sel_bin = 255 - (16 * wave + j);
+        S.sel_need = k - above;
+      }
+      above += cnt[j];
     }
   }
   __syncthreads();
@@ -148,8 +177,9 @@ __device__ __forceinline__ void sf_select_row(sf_lds& S, unsigned char* dyn, con
   }
   int cnt0 = R.cnt[r];  // read before the first barrier: rewritten at the end
   if (cnt0 > R.cap) cnt0 = R.cap;
-  for (int i = tid; i < R.n_words + 2; i += SF_NT) s_bm[i] = i < R.n_words ? bm[i] : 0u;
+  // clear the counters first: these stores do not wait for the loads above, the bitmap copy does
   for (int i = tid; i < 2 * 256 * SF_COPIES / 4; i += SF_NT) ((uint4*)s_h1)[i] = make_uint4(0u, 0u, 0u, 0u);
+  for (int i = tid; i < R.n_words + 2; i += SF_NT) s_bm[i] = i < R.n_words ? bm[i] : 0u;
   __syncthreads();
   if (REG) {
 #pragma unroll
@@ -184,20 +214,8 @@ __device__ __forceinline__ void sf_select_row(sf_lds& S, unsigned char* dyn, con
     }
   };
   auto key_of = [](const uint32_t (&kk)[4], int t) -> uint32_t {
-    return (t & 1) ? (kk[t >> 1] >> 16) : (kk[t >> 1] & 0xffffu);
+    return t < 4 ? (kk[t] & 0xffffu) : (kk[t - 4] >> 16);
   };
-  // thread t sums a quarter of the counters of bin 255 - t/4, then the block picks the bin
-  auto pick = [&](const uint32_t* hist, int kk, int& bin, int& nd) {
-    const uint4* h = (const uint4*)(hist + (255 - (tid >> 2)) * SF_COPIES + (tid & 3) * (SF_COPIES / 4));
-    int partial = 0;
-#pragma unroll
-    for (int i = 0; i < SF_COPIES / 16; ++i) {
-      const uint4 q = h[i];
-      partial += (int)(q.x + q.y + q.z + q.w);
-    }
-    sf_pick(partial, kk, S, bin, nd);
-  };
-
   // ---- pass 1: histogram of the high byte ------------------------------------------------
   uint32_t* my_h1 = s_h1 + (lane & (SF_COPIES - 1));
   uint32_t* my_h2 = s_h2 + (lane & (SF_COPIES - 1));
@@ -207,7 +225,7 @@ __device__ __forceinline__ void sf_select_row(sf_lds& S, unsigned char* dyn, con
   });
   __syncthreads();
   int b1, need1;
-  pick(s_h1, k, b1, need1);
+  sf_pick(s_h1, k, S, b1, need1);
 
   // ---- pass 2: histogram of the low byte inside bin b1 ---------------------------------
   for_chunks([&](int, const uint32_t (&kk)[4]) {
@@ -219,7 +237,7 @@ __device__ __forceinline__ void sf_select_row(sf_lds& S, unsigned char* dyn, con
   });
   __syncthreads();
   int b2, need;
-  pick(s_h2, need1, b2, need);
+  sf_pick(s_h2, need1, S, b2, need);
   const uint32_t T = ((uint32_t)b1 << 8) | (uint32_t)b2;
   // Active candidates carry the excluded key. While that ranks below the threshold they are
   // neither winners nor ties and their flags are not needed again; otherwise (a row with
@@ -227,14 +245,17 @@ __device__ __forceinline__ void sf_select_row(sf_lds& S, unsigned char* dyn, con
   const bool slow = ek >= T;
 
   // 8-bit masks of one chunk: emittable keys above the threshold, ties, active candidates
+  const uint32_t T2 = T * 0x00010001u;
   auto masks = [&](int c, const uint32_t (&kk)[4], uint32_t& gt, uint32_t& eq, uint32_t& ex) {
-    gt = 0, eq = 0, ex = 0;
+    uint32_t g = 0, n = 0;
 #pragma unroll
-    for (int t = 0; t < 8; ++t) {
-      const uint32_t key = key_of(kk, t);
-      gt |= (key > T ? 1u : 0u) << t;
-      eq |= (key == T ? 1u : 0u) << t;
+    for (int p = 0; p < 4; ++p) {
+      g |= sah_pk_gt01_u16(kk[p], T2) << p;
+      n |= sah_pk_ne01_u16(kk[p], T2) << p;
     }
+    gt = sf_join(g);
+    eq = sf_join(~n & 0x000f000fu);
+    ex = 0;
     if (slow) {
       uint32_t valid;
       sf_flags(s_bm, R.n_words, c * SF_CHUNK + lane * 8, n_cand, col_offset, ex, valid);
@@ -255,7 +276,8 @@ __device__ __forceinline__ void sf_select_row(sf_lds& S, unsigned char* dyn, con
   if (lane == 0) S.eq[wave] = wave_eq;
   __syncthreads();
   int tie_base = 0;
-  for (int w = 0; w < wave; ++w) tie_base += S.eq[w];
+#pragma unroll
+  for (int w = 0; w < SF_NW; ++w) tie_base += w < wave ? S.eq[w] : 0;
   // 0: no tie of this wave is taken, 1: all are, 2: the boundary lies inside the wave
   const int mode = tie_base >= need ? 0 : (tie_base + wave_eq <= need ? 1 : 2);
 

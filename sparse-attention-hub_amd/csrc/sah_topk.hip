@@ -469,10 +469,10 @@ extern "C" int sah_select_topk(const sah_select_topk_args* a) {
   if (a->k <= 0) return sah_fail(SAH_EINVAL, "sah_select_topk: k must be > 0");
   if (a->key_pitch < a->n_cand) return sah_fail(SAH_EINVAL, "sah_select_topk: key_pitch < n_cand");
   hipStream_t st = (hipStream_t)a->stream;
-  if (a->key_bits == 16 && a->key_pitch % 8 == 0 && ((uintptr_t)a->keys % 16) == 0) {
+  if (a->key_bits == 16 && a->key_pitch % 8 == 0 && ((uintptr_t)a->keys % 16) == 0 &&
+      sf_lds_bytes(a->rows.n_words) <= 150 * 1024) {
     // eight keys per lane: needs 16-byte aligned key rows
     const size_t lds = sf_lds_bytes(a->rows.n_words);
-    if (lds > 150 * 1024) return sah_fail(SAH_ESHAPE, "sah_select_topk: %d keys need %zu bytes of LDS", a->rows.n_keys, lds);
     const int cpw = sf_chunks_per_wave(a->n_cand);
     sah_timed timed("k_select_topk", a->stream);
 #define SAH_SEL16(CPW)                                                                                      \
