@@ -253,6 +253,14 @@ __device__ __forceinline__ uint32_t sah_pk_ne01_u16(uint32_t a, uint32_t b) {
 #endif
 }
 
+// Orders the LDS traffic of ONE wave: what its lanes wrote before is visible to its lanes after.
+// For LDS regions that a single wave owns; costs a wait on the wave's own LDS queue, no workgroup barrier.
+__device__ __forceinline__ void sah_wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 // ---------------------------------------------------------------------------
 // device side: cross-lane helpers
 // ---------------------------------------------------------------------------

@@ -13,7 +13,10 @@
 #define SC_NW (SC_NT / SAH_WAVE)
 #define SC_NQ 4          // query vectors per workgroup
 #define SC_TILE 256      // keys per workgroup iteration
-#define SC_ITERS 8       // tiles per workgroup => 2048 keys per workgroup
+#ifndef SC_MIN_WGS
+#define SC_MIN_WGS 4096  // workgroups wanted before a workgroup takes more than one tile
+#endif
+#define SC_ITERS 2       // most tiles per workgroup; one when that would leave CUs without work
 
 struct qk_params {
   const void* q; int64_t qs_b, qs_h, qs_l;
@@ -21,6 +24,7 @@ struct qk_params {
   const void* amask; int64_t ms_b, ms_h, ms_l;
   int B, Hq, Hkv, Lq, Lk;
   void* keys_out; int64_t key_pitch;
+  int iters;  // tiles of SC_TILE keys per workgroup
 };
 
 template <int LPK>
@@ -146,26 +150,39 @@ __global__ __launch_bounds__(SC_NT) void k_qk_scores(qk_params P) {
   // which of the four totals this lane ends up with after sc_reduce4
   const int mine = FAST4 ? (2 * (sub & 1) + ((sub >> 1) & 1)) : 0;
 
-  for (int iter = 0; iter < SC_ITERS; ++iter) {
-    const int j0 = (blockIdx.x * SC_ITERS + iter) * SC_TILE;
-    if (j0 >= P.Lk) break;  // uniform across the workgroup
-    // every load of the tile is requested before the first use; rows past the end re-read the last row
-    sc_raw<DT> kv[IT];
+  // A wave owns 64 consecutive keys of every tile and the matching columns of s_out: no workgroup
+  // barrier anywhere. The rows come in half-slices of HB iterations through two register buffers;
+  // the next half-slice is requested before the current one is scored, so every wave keeps
+  // HB..2*HB row loads in flight all the time instead of alternating between loading and computing.
+  // iterations per part of a wave's 64-key slice: half of it, a quarter for fp32 rows (twice the registers)
+  constexpr int HB = (DT == SAH_F32 && IT >= 4) ? IT / 4 : (IT >= 2 ? IT / 2 : 1);
+  constexpr int NH = IT / HB;                // parts per tile
+  const int tile0 = blockIdx.x * P.iters;
+  int n_tiles = (P.Lk - tile0 * SC_TILE + SC_TILE - 1) / SC_TILE;
+  if (n_tiles > P.iters) n_tiles = P.iters;
+  if (n_tiles <= 0) return;
+  const int n_half = n_tiles * NH;
+  auto request = [&](sc_raw<DT> (&buf)[HB], int hs) {
+    const int j0 = (tile0 + hs / NH) * SC_TILE + wave * SAH_WAVE + (hs % NH) * HB * KPI;
 #pragma unroll
-    for (int it = 0; it < IT; ++it) {
-      int j = j0 + wave * SAH_WAVE + it * KPI + grp;
-      if (j > P.Lk - 1) j = P.Lk - 1;
-      sc_load<DT>(kbase + (int64_t)j * krow, kv[it]);
+    for (int it = 0; it < HB; ++it) {
+      int j = j0 + it * KPI + grp;
+      if (j > P.Lk - 1) j = P.Lk - 1;  // rows past the end re-read the last row
+      sc_load<DT>(kbase + (int64_t)j * krow, buf[it]);
     }
+  };
+  auto score = [&](sc_raw<DT> (&buf)[HB], int hs) {
+    const int tile = tile0 + hs / NH;
+    const int jl0 = wave * SAH_WAVE + (hs % NH) * HB * KPI;  // first key of the half-slice within the tile
 #pragma unroll
-    for (int it = 0; it < IT; ++it) sc_keep<DT>(kv[it]);
+    for (int it = 0; it < HB; ++it) sc_keep<DT>(buf[it]);
 #pragma unroll
-    for (int it = 0; it < IT; ++it) {
-      const int jl = wave * SAH_WAVE + it * KPI + grp;  // key within the tile
-      const int j = j0 + jl;
+    for (int it = 0; it < HB; ++it) {
+      const int jl = jl0 + it * KPI + grp;
+      const int j = tile * SC_TILE + jl;
       if constexpr (FAST4) {
-        const float d = sc_reduce4<LPK>(sc_dot<DT>(qv[0], kv[it]), sc_dot<DT>(qv[1], kv[it]), sc_dot<DT>(qv[2], kv[it]),
-                                        sc_dot<DT>(qv[3], kv[it]), sub);
+        const float d = sc_reduce4<LPK>(sc_dot<DT>(qv[0], buf[it]), sc_dot<DT>(qv[1], buf[it]), sc_dot<DT>(qv[2], buf[it]),
+                                         sc_dot<DT>(qv[3], buf[it]), sub);
         int rr = row[0];
         int64_t mo = moff[0];
 #pragma unroll
@@ -183,7 +200,7 @@ __global__ __launch_bounds__(SC_NT) void k_qk_scores(qk_params P) {
       } else {
 #pragma unroll
         for (int i = 0; i < SC_NQ; ++i) {
-          const float d = sc_group_sum<LPK>(sc_dot<DT>(qv[i], kv[it]));
+          const float d = sc_group_sum<LPK>(sc_dot<DT>(qv[i], buf[it]));
           if (sub == (i % LPK) && j < P.Lk && row[i] >= 0) {
             float s = sah_round<DT>(d);
             if (P.amask) s = sah_round<DT>(s + sah_load<DT>(P.amask, moff[i] + j));
@@ -192,14 +209,24 @@ __global__ __launch_bounds__(SC_NT) void k_qk_scores(qk_params P) {
         }
       }
     }
-    __syncthreads();
-    int nk = P.Lk - j0;
-    if (nk > SC_TILE) nk = SC_TILE;
+    if (hs % NH == NH - 1) {
+      // the wave's 64 keys of this tile are scored: write them out, one key per lane and query vector
+      sah_wave_lds_sync();
+      const int j = tile * SC_TILE + wave * SAH_WAVE + lane;
 #pragma unroll
-    for (int i = 0; i < SC_NQ; ++i) {
-      if (row[i] >= 0 && tid < nk) ((key_t*)P.keys_out)[(int64_t)row[i] * P.key_pitch + j0 + tid] = s_out[i][tid];
+      for (int i = 0; i < SC_NQ; ++i) {
+        if (row[i] >= 0 && j < P.Lk) ((key_t*)P.keys_out)[(int64_t)row[i] * P.key_pitch + j] = s_out[i][wave * SAH_WAVE + lane];
+      }
+      sah_wave_lds_sync();  // the columns are free again for the next tile
     }
-    __syncthreads();
+  };
+  sc_raw<DT> ka[HB], kb[HB];
+  request(ka, 0);
+  for (int hs = 0; hs < n_half; hs += 2) {
+    if (hs + 1 < n_half) request(kb, hs + 1);
+    score(ka, hs);
+    if (hs + 2 < n_half) request(ka, hs + 2);
+    if (hs + 1 < n_half) score(kb, hs + 1);
   }
 }
 
@@ -207,9 +234,16 @@ template <int DT, int D>
 static int qk_launch(const sah_qk_scores_args* a, const qk_params& P) {
   const int G = a->Hq / a->Hkv;
   const int nvec = G * a->Lq;
-  dim3 g((a->Lk + SC_TILE * SC_ITERS - 1) / (SC_TILE * SC_ITERS), a->B * a->Hkv, (nvec + SC_NQ - 1) / SC_NQ);
+  // enough workgroups for several waves per SIMD on all 256 CUs, as long as a workgroup keeps at least one tile
+  const int64_t tiles = (a->Lk + SC_TILE - 1) / SC_TILE;
+  const int64_t streams = (int64_t)a->B * a->Hkv * ((nvec + SC_NQ - 1) / SC_NQ);
+  int iters = SC_ITERS;
+  while (iters > 1 && streams * ((tiles + iters - 1) / iters) < SC_MIN_WGS) iters >>= 1;
+  qk_params Q = P;
+  Q.iters = iters;
+  dim3 g((unsigned)((tiles + iters - 1) / iters), a->B * a->Hkv, (nvec + SC_NQ - 1) / SC_NQ);
   sah_timed timed("k_qk_scores", a->stream);
-  hipLaunchKernelGGL((k_qk_scores<DT, D>), g, dim3(SC_NT), 0, (hipStream_t)a->stream, P);
+  hipLaunchKernelGGL((k_qk_scores<DT, D>), g, dim3(SC_NT), 0, (hipStream_t)a->stream, Q);
   return sah_launch_status("sah_qk_scores");
 }
 
