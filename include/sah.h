@@ -246,6 +246,9 @@ typedef struct sah_select_topk_args {
   int32_t col_offset;
   int32_t k;
   uint32_t excluded_key;
+  int32_t fresh;          /* != 0: the rows are taken to be empty and are first given the sink and local   */
+  int32_t fresh_sink;     /* columns of one query per row - what sah_sink_local_indices(lq = 1, fresh = 1) */
+  int32_t fresh_window;   /* writes - in the same launch when the keys are 16-bit and 16-byte aligned      */
   void* stream;
 } sah_select_topk_args;
 int sah_select_topk(const sah_select_topk_args* a);

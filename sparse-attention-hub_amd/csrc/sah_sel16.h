@@ -136,7 +136,7 @@ __device__ __forceinline__ uint32_t sf_lowest(uint32_t m, int allowed) {
 template <int CPW>
 __device__ __forceinline__ void sf_select_row(sf_lds& S, unsigned char* dyn, const sah_rows& R, int r,
                                               const uint16_t* keys, int n_cand, int col_offset, int k,
-                                              uint32_t excluded_key) {
+                                              uint32_t excluded_key, int fresh, int sink, int window) {
   constexpr bool REG = CPW > 0;
   constexpr int NREG = REG ? CPW : 1;
   const int tid = threadIdx.x;
@@ -175,11 +175,36 @@ __device__ __forceinline__ void sf_select_row(sf_lds& S, unsigned char* dyn, con
 #pragma unroll
     for (int u = 0; u < NREG; ++u) kreg[u] = raw_load(c0 + u);
   }
-  int cnt0 = R.cnt[r];  // read before the first barrier: rewritten at the end
-  if (cnt0 > R.cap) cnt0 = R.cap;
-  // clear the counters first: these stores do not wait for the loads above, the bitmap copy does
-  for (int i = tid; i < 2 * 256 * SF_COPIES / 4; i += SF_NT) ((uint4*)s_h1)[i] = make_uint4(0u, 0u, 0u, 0u);
-  for (int i = tid; i < R.n_words + 2; i += SF_NT) s_bm[i] = i < R.n_words ? bm[i] : 0u;
+  int cnt0;
+  if (fresh) {
+    // rows still empty: the sink and local columns of one query per row in closed form, as
+    // k_sink_local would have left them (basic_fixed.py:354-363, :48-67), without a launch of their own
+    const int n = R.n_keys;
+    const int s_hi = sink < n ? sink : n;
+    int lo = 0, hi = 0;
+    if (window > 0) {
+      lo = n - window;
+      hi = n;
+      if (lo < 0) lo = 0;
+    }
+    const int lo2 = lo > s_hi ? lo : s_hi;
+    const int fixed = s_hi + (hi > lo2 ? hi - lo2 : 0);
+    int* cols0 = R.cols + (int64_t)r * R.cap;
+    for (int i = tid; i < fixed && i < R.cap; i += SF_NT) {
+      cols0[i] = i < s_hi ? i : lo2 + (i - s_hi);
+      if (R.w) R.w[(int64_t)r * R.cap + i] = 1.0f;
+    }
+    cnt0 = fixed < R.cap ? fixed : R.cap;
+    for (int i = tid; i < 2 * 256 * SF_COPIES / 4; i += SF_NT) ((uint4*)s_h1)[i] = make_uint4(0u, 0u, 0u, 0u);
+    for (int i = tid; i < R.n_words + 2; i += SF_NT)
+      s_bm[i] = i < R.n_words ? (sah_range_bits(i, 0, s_hi) | sah_range_bits(i, lo, hi)) : 0u;
+  } else {
+    cnt0 = R.cnt[r];  // read before the first barrier: rewritten at the end
+    if (cnt0 > R.cap) cnt0 = R.cap;
+    // clear the counters first: these stores do not wait for the loads above, the bitmap copy does
+    for (int i = tid; i < 2 * 256 * SF_COPIES / 4; i += SF_NT) ((uint4*)s_h1)[i] = make_uint4(0u, 0u, 0u, 0u);
+    for (int i = tid; i < R.n_words + 2; i += SF_NT) s_bm[i] = i < R.n_words ? bm[i] : 0u;
+  }
   __syncthreads();
   if (REG) {
 #pragma unroll
@@ -336,7 +361,7 @@ __device__ __forceinline__ void sf_select_row(sf_lds& S, unsigned char* dyn, con
     }
   });
   __syncthreads();
-  if (total > 0)
+  if (total > 0 || fresh)
     for (int i = tid; i < R.n_words; i += SF_NT) bm[i] = s_bm[i];
   if (tid == 0) R.cnt[r] = cnt0 + total;
 }

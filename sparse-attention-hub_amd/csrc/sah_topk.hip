@@ -388,12 +388,13 @@ __global__ __launch_bounds__(HSW_NT) void k_hamming_topk_swar(sah_rows R, const 
 
 template <int CPW>
 __global__ __launch_bounds__(SF_NT) void k_select16(sah_rows R, const uint16_t* keys, int64_t pitch, int n_cand,
-                                                    int col_offset, int k, uint32_t excluded_key) {
+                                                    int col_offset, int k, uint32_t excluded_key, int fresh, int sink,
+                                                    int window) {
   __shared__ sf_lds S;
   HIP_DYNAMIC_SHARED(unsigned char, sf_dyn)
   const int r = blockIdx.x;
   sf_select_row<CPW>(S, sf_dyn, R, r, keys + (int64_t)r * pitch, n_cand, col_offset, k < n_cand ? k : n_cand,
-                     excluded_key);
+                     excluded_key, fresh, sink, window);
 }
 
 // kernels may use up to 160 KB of LDS; HIP needs to be told once per kernel
@@ -468,6 +469,14 @@ extern "C" int sah_select_topk(const sah_select_topk_args* a) {
                     a->col_offset + a->n_cand, a->rows.n_keys);
   if (a->k <= 0) return sah_fail(SAH_EINVAL, "sah_select_topk: k must be > 0");
   if (a->key_pitch < a->n_cand) return sah_fail(SAH_EINVAL, "sah_select_topk: key_pitch < n_cand");
+  if (a->fresh && (a->fresh_sink < 0 || a->fresh_window < 0))
+    return sah_fail(SAH_EINVAL, "sah_select_topk: fresh_sink / fresh_window must be >= 0");
+  if (a->fresh) {
+    int64_t worst = (int64_t)a->fresh_sink + a->fresh_window;
+    if (worst > a->rows.n_keys) worst = a->rows.n_keys;
+    if (worst > a->rows.cap)
+      return sah_fail(SAH_ECAPACITY, "sah_select_topk: cap %d < sink+window %lld", a->rows.cap, (long long)worst);
+  }
   hipStream_t st = (hipStream_t)a->stream;
   if (a->key_bits == 16 && a->key_pitch % 8 == 0 && ((uintptr_t)a->keys % 16) == 0 &&
       sf_lds_bytes(a->rows.n_words) <= 150 * 1024) {
@@ -480,7 +489,8 @@ extern "C" int sah_select_topk(const sah_select_topk_args* a) {
     rc = sel_allow_lds(k_select16<CPW>, lds, "sah_select_topk");                                            \
     if (rc) return rc;                                                                                      \
     hipLaunchKernelGGL(k_select16<CPW>, dim3(a->rows.n_rows), dim3(SF_NT), lds, st, a->rows,                \
-                       (const uint16_t*)a->keys, a->key_pitch, a->n_cand, a->col_offset, a->k, a->excluded_key); \
+                       (const uint16_t*)a->keys, a->key_pitch, a->n_cand, a->col_offset, a->k, a->excluded_key, \
+                       a->fresh ? 1 : 0, a->fresh_sink, a->fresh_window);                                   \
   } while (0)
     if (cpw <= 4) SAH_SEL16(4);
     else if (cpw <= 8) SAH_SEL16(8);
@@ -488,6 +498,12 @@ extern "C" int sah_select_topk(const sah_select_topk_args* a) {
     else SAH_SEL16(0);
 #undef SAH_SEL16
     return sah_launch_status("sah_select_topk");
+  }
+  if (a->fresh) {
+    // the general kernel starts from rows in memory: build the sink + local rows with their own launch
+    sah_sink_local_args sl = {a->rows, 1, a->fresh_sink, a->fresh_window, 1, 0, a->stream};
+    rc = sah_sink_local_indices(&sl);
+    if (rc) return rc;
   }
   sel_layout L;
   const size_t lds = sel_plan(a->key_bits, a->key_bits / 8, a->rows.n_words, a->n_cand, a->col_offset, &L);

@@ -159,6 +159,9 @@ class SelectTopkArgs(C.Structure):
         ("col_offset", C.c_int32),
         ("k", C.c_int32),
         ("excluded_key", C.c_uint32),
+        ("fresh", C.c_int32),
+        ("fresh_sink", C.c_int32),
+        ("fresh_window", C.c_int32),
         ("stream", C.c_void_p),
     ]
 

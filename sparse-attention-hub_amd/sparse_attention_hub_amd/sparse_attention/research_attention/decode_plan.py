@@ -209,6 +209,12 @@ class DecodePlan:
             se.rows, se.keys, se.key_pitch, se.key_bits = rows, self.keybuf.data_ptr(), self.keybuf_pitch, self.key_bits
             se.n_cand, se.col_offset, se.k, se.excluded_key, se.stream = Lk, 0, k_eff, self._excluded_min, stream
             chain.select = C.addressof(se)
+            if Lq == 1:
+                # one query per row: the selection kernel writes the sink + local rows itself
+                se.fresh, se.fresh_sink, se.fresh_window = 1, sink, window
+                chain.sink_local = None
+            else:
+                se.fresh = 0
         elif self.kind == "pq":
             off = top.init_offset
             if Lk <= k_eff + off + Lq + 2 ** top.pq_bits:
@@ -247,6 +253,12 @@ class DecodePlan:
             se.rows, se.keys, se.key_pitch, se.key_bits = rows, self.keybuf.data_ptr(), self.keybuf_pitch, self.key_bits
             se.n_cand, se.col_offset, se.k, se.excluded_key, se.stream = current, off, k_eff, self._excluded_min, stream
             chain.select = C.addressof(se)
+            if Lq == 1:
+                # one query per row: the selection kernel writes the sink + local rows itself
+                se.fresh, se.fresh_sink, se.fresh_window = 1, sink, window
+                chain.sink_local = None
+            else:
+                se.fresh = 0
 
         out = torch.empty((self.B, Lq, self.Hq, self.D), dtype=self.dtype, device=self.device)
         work = _workspace(self.device, N.work_floats(self.n_rows, cap, self.D))

@@ -80,7 +80,7 @@ class TopKMasker(FixedMasker):
         rows.zero_if_fresh()
         args = N.SelectTopkArgs(
             rows.as_struct(), keys_buf.data_ptr(), keys_buf.stride(0), key_bits, n_cand, col_offset, k,
-            excluded_key, N.stream_ptr(rows.device),
+            excluded_key, 0, 0, 0, N.stream_ptr(rows.device),
         )
         N.call("sah_select_topk", args)
         # every row gains exactly k entries when it certainly has k inactive candidates left

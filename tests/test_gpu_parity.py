@@ -385,6 +385,40 @@ def test_fused_hash_decode_kernel_matches_separate_launches(cuda, dtype, Lk):
     assert bool((srt[:, 1:] != srt[:, :-1]).all()) and int(cols.min()) == 0 and int(cols.max()) == Lk + 2 - 1
 
 
+@pytest.mark.parametrize("key_bits", [16, 32])
+def test_select_topk_on_fresh_rows_equals_sink_local_then_select(cuda, key_bits):
+    """sah_select_topk with fresh != 0 writes the sink + local rows itself (inside the selection kernel for
+    16-bit keys, by a launch of its own otherwise): same rows, counts and bitmap as the two calls."""
+    from sparse_attention_hub_amd import _native as N
+    from sparse_attention_hub_amd.sparse_attention.utils.native_rows import NativeRows
+
+    n_rows, n_keys, sink, window, k = 6, 3001, 37, 211, 150
+    g = torch.Generator().manual_seed(5)
+    hi = 1 << (key_bits - 4)
+    keys = torch.randint(0, hi, (n_rows, 3008), generator=g, dtype=torch.int64)
+    kdev = keys.to(torch.int16 if key_bits == 16 else torch.int32).to(cuda)
+    results = []
+    for fused in (True, False):
+        rows = NativeRows(n_rows, n_keys, sink + window + k, cuda)
+        if not fused:
+            N.call("sah_sink_local_indices", N.SinkLocalArgs(rows.as_struct(), 1, sink, window, 1, 0, N.stream_ptr(cuda)))
+        args = N.SelectTopkArgs(rows.as_struct(), kdev.data_ptr(), kdev.stride(0), key_bits, n_keys, 0, k, 0,
+                                1 if fused else 0, sink if fused else 0, window if fused else 0, N.stream_ptr(cuda))
+        N.call("sah_select_topk", args)
+        torch.cuda.synchronize()
+        results.append((rows.cnt.cpu(), torch.sort(rows.cols.cpu(), dim=1).values, rows.bitmap.cpu()))
+    (c1, s1, b1), (c2, s2, b2) = results
+    assert bool((c1 == sink + window + k).all()) and torch.equal(c1, c2)
+    assert torch.equal(s1, s2) and torch.equal(b1, b2)
+    # and against a plain restatement: best k of the columns outside sink and window, lowest column on ties
+    kk = keys[:, :n_keys].clone()
+    kk[:, :sink] = -1
+    kk[:, n_keys - window:] = -1
+    want = torch.argsort(kk, dim=1, descending=True, stable=True)[:, :k]
+    got = torch.stack([row[(row >= sink) & (row < n_keys - window)] for row in s1])
+    assert torch.equal(got, torch.sort(want, dim=1).values.to(got.dtype))
+
+
 # ------------------------------------------------------------------------ adaptive sampling
 def _adaptive_case(cuda, pre_cfgs, pre_specs, rate, eps, delta, io, lo, B, Hq, Hkv, Lq, Lk, D, dtype, amask=None,
                    seed=1234, outliers=False):
