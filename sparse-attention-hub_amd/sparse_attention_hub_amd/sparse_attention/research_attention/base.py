@@ -15,14 +15,20 @@ import torch
 from torch import nn
 
 from ... import _native
+from ...metric_logging import MicroMetricLogger
 from ..base import SparseAttention, SparseAttentionConfig
 from ..utils.mask import Mask
-from ..utils.mask_attention_utils import get_masked_attention_output
+from ..utils.mask_attention_utils import get_masked_attention_output, get_true_attention_output
 from ..utils.native_rows import NativeRows
 from .decode_plan import DecodePlan, plan_kind
 from .maskers.base import MaskerConfig, ResearchMasker
 from .maskers.fixed.implementations.basic_fixed import LocalMasker, SinkMasker, fused_sink_local
 from .maskers.sampling.base import SamplingMasker
+
+
+# the two metrics of the reference (research_attention/base.py:20-21)
+MicroMetricLogger.register_metric("research_attention_density", float)
+MicroMetricLogger.register_metric("research_attention_output_error", float)
 
 
 @dataclass
@@ -75,7 +81,12 @@ class ResearchAttention(SparseAttention):
             raise ValueError("sparse_meta_data must be provided in kwargs while calling custom_attention()")
         sparse_meta_data: Dict[Any, Any] = kwargs.pop("sparse_meta_data")
 
-        if (not self.return_attention_weights and attention_mask is None and self._plan_kind is not None
+        metrics = MicroMetricLogger()
+        want_density = metrics.is_metric_enabled("research_attention_density")
+        want_error = metrics.is_metric_enabled("research_attention_output_error")
+
+        if (not (want_density or want_error)  # the metrics read the finished mask: masker-by-masker path
+                and not self.return_attention_weights and attention_mask is None and self._plan_kind is not None
                 and not isinstance(kwargs.get("s_aux"), torch.Tensor) and queries.dim() == 4
                 and (queries.is_cuda or not _native.REQUIRE_DEVICE_TENSORS)
                 and not (dropout > 0.0 and module is not None and getattr(module, "training", False))):
@@ -121,21 +132,31 @@ class ResearchAttention(SparseAttention):
                 **kwargs,
             )
 
+        if want_density:
+            # active fraction of the (B, Hq, Lq, Lk) mask, from the per-row counts (reference :121-126)
+            metrics.log("research_attention_density", mask.get_density(), metadata={"layer_idx": kwargs["layer_idx"]})
+
         s_aux_raw: Any = kwargs.pop("s_aux", None)
         s_aux: Optional[torch.Tensor] = s_aux_raw if isinstance(s_aux_raw, torch.Tensor) else None
+        weights: Optional[torch.Tensor] = None
         if self.return_attention_weights:
             out, weights = get_masked_attention_output(
                 module=module, queries=queries, keys=keys, values=values, attention_mask=attention_mask,
                 sinks=s_aux, scaling=scaling, dropout=dropout, sparse_attention_mask=mask,
                 return_attention_weights=True, **kwargs,
             )
-            return out, weights
-        out = get_masked_attention_output(
-            module=module, queries=queries, keys=keys, values=values, attention_mask=attention_mask,
-            sinks=s_aux, scaling=scaling, dropout=dropout, sparse_attention_mask=mask,
-            return_attention_weights=False, **kwargs,
-        )
-        return out, None
+        else:
+            out = get_masked_attention_output(
+                module=module, queries=queries, keys=keys, values=values, attention_mask=attention_mask,
+                sinks=s_aux, scaling=scaling, dropout=dropout, sparse_attention_mask=mask,
+                return_attention_weights=False, **kwargs,
+            )
+        if want_error:
+            # relative distance to dense attention over all keys, by the same kernel in dense mode (reference :150-168)
+            true_out, _ = get_true_attention_output(module, queries, keys, values, attention_mask, scaling, dropout, **kwargs)
+            error = torch.norm(true_out.float() - out.float()) / torch.norm(true_out.float())
+            metrics.log("research_attention_output_error", float(error.item()), metadata={"layer_idx": kwargs["layer_idx"]})
+        return out, weights
 
     @classmethod
     def create_from_config(cls, config: SparseAttentionConfig) -> "ResearchAttention":

@@ -419,6 +419,40 @@ def test_select_topk_on_fresh_rows_equals_sink_local_then_select(cuda, key_bits)
     assert torch.equal(got, torch.sort(want, dim=1).values.to(got.dtype))
 
 
+def test_density_and_output_error_metrics(cuda, tmp_path):
+    """research_attention_density and research_attention_output_error (reference research_attention/base.py:
+    121-126, 150-168) through the kernels: density = entries / (rows * keys) exactly, error = relative
+    distance between the sparse output and dense attention, against the oracle's two outputs."""
+    import json
+
+    from sparse_attention_hub_amd.metric_logging import MicroMetricLogger
+
+    sa = _sa()
+    B, Hq, Hkv, Lk, D = 2, 8, 2, 900, 64
+    q, k, v = make_qkv(B, Hq, Hkv, 1, Lk, D, torch.float32, seed=21)
+    cfgs = [sa.SinkMaskerConfig(sink_size=8), sa.LocalMaskerConfig(window_size=32), sa.OracleTopKConfig(heavy_size=60)]
+    ra = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=cfgs))
+    ra.return_attention_weights = False   # the metrics must also work when the fast decode plan would apply
+    lg = MicroMetricLogger()
+    saved = (lg.log_path, set(lg.enabled_metrics), lg.max_records, lg.sampling_factor)
+    try:
+        lg.configure_logging(str(tmp_path), enabled_metrics=["research_attention_density", "research_attention_output_error"])
+        out, _ = ra.custom_attention(None, q.to(cuda), k.to(cuda), v.to(cuda), None, D ** -0.5, 0.0, sparse_meta_data={}, layer_idx=3)
+        lg.flush()
+    finally:
+        lg.log_path, lg.enabled_metrics, lg.max_records, lg.sampling_factor = saved
+    recs = [json.loads(line) for line in (tmp_path / "micro_metrics.jsonl").read_text().splitlines()]
+    assert [r["metric"] for r in recs] == ["research_attention_density", "research_attention_output_error"]
+    assert all(r["metadata"] == {"layer_idx": 3} for r in recs)
+    assert all(r["location"].endswith("ResearchAttention.custom_attention") for r in recs)
+    assert recs[0]["value"] == pytest.approx((8 + 32 + 60) / Lk, rel=1e-6)
+    o_sparse, _, _ = O.research_attention([("sink", 8), ("local", 32), ("oracle_topk", 60)], q, k, v, None, D ** -0.5, None)
+    o_dense, _, _ = O.research_attention([], q, k, v, None, D ** -0.5, None)
+    want = (torch.norm(o_dense - o_sparse) / torch.norm(o_dense)).item()
+    assert recs[1]["value"] == pytest.approx(want, rel=1e-3)
+    assert torch.allclose(out.cpu(), o_sparse, rtol=1e-4, atol=1e-6)
+
+
 # ------------------------------------------------------------------------ adaptive sampling
 def _adaptive_case(cuda, pre_cfgs, pre_specs, rate, eps, delta, io, lo, B, Hq, Hkv, Lq, Lk, D, dtype, amask=None,
                    seed=1234, outliers=False):
