@@ -292,12 +292,37 @@ def pq_split(keys: torch.Tensor, init_offset: int, n_sub: int) -> torch.Tensor:
     return kc.reshape(B, H, L - init_offset, n_sub, d).transpose(2, 3).reshape(-1, L - init_offset, d)
 
 
+def ip2l2_augment(xb: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(n_groups, n, d) -> (n_groups, n, d + 1) with the extra column sqrt(phi - ||x||^2),
+    phi = largest squared norm of the group; phi (n_groups, 1, 1) — pq_utils.py:585-612."""
+    norms_sq = (xb ** 2).sum(dim=2, keepdim=True)
+    phi = norms_sq.max(dim=1, keepdim=True)[0]
+    return torch.cat([xb, torch.sqrt(phi - norms_sq)], dim=2), phi
+
+
+def ip2l2_augment_queries(xq: torch.Tensor) -> torch.Tensor:
+    """Queries (and keys quantised later) get a zero column — pq_utils.py:615-640."""
+    return torch.cat([xq, torch.zeros(xq.shape[0], xq.shape[1], 1, dtype=xq.dtype)], dim=2)
+
+
+def pq_split_ip(keys: torch.Tensor, init_offset: int, n_sub: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """The vectors metric="ip" clusters: sub-vectors of keys[:, :, init_offset:] per (b, kv head,
+    sub-space) group, augmented in the key dtype — pq_top_k.py:219-236. Returns (X, phi)."""
+    B, H, Lk, D = keys.shape
+    d = D // n_sub
+    flat = keys[:, :, init_offset:, :].reshape(B, H, Lk - init_offset, n_sub, d).transpose(2, 3).reshape(-1, Lk - init_offset, d)
+    return ip2l2_augment(flat)
+
+
 def pq_quantize_new(new_keys: torch.Tensor, centroids: torch.Tensor) -> torch.Tensor:
-    """codes (B, n_new, Hkv, n_sub) in the key dtype's arithmetic — pq_top_k.py:343-404 (euclidean)."""
+    """codes (B, n_new, Hkv, n_sub) in the key dtype's arithmetic — pq_top_k.py:343-404. Centroids one
+    dimension wider than the sub-vectors are those of metric="ip": the new keys then get a zero column."""
     B, H, n_new, D = new_keys.shape
     n_sub = centroids.shape[2]
     d = D // n_sub
     nk = new_keys.reshape(B, H, n_new, n_sub, d).transpose(2, 3)
+    if centroids.shape[-1] == d + 1:
+        nk = ip2l2_augment_queries(nk.reshape(-1, n_new, d)).reshape(B, H, n_sub, n_new, d + 1)
     dist = torch.sum((nk.unsqueeze(4) - centroids.unsqueeze(3)) ** 2, dim=-1)
     return torch.argmin(dist, dim=-1).permute(0, 3, 1, 2)
 

@@ -12,7 +12,7 @@
 #include "sah_common.h"
 
 #define PQ_NT 256
-#define PQ_MAX_D 16
+#define PQ_MAX_D 17  // 16 plus the extra coordinate of inner-product search done as L2 search
 #define PQ_MAX_CENT 256
 #define PQ_TILES 8  // key tiles of PQ_NT per workgroup
 

@@ -46,7 +46,7 @@ def plan_kind(maskers) -> Optional[str]:
             return "hash"
         if t is OracleTopK:
             return "oracle"
-        if t is PQCache:
+        if t is PQCache and maskers[2].metric == "euclidean":  # "ip" augments the keys first: masker path
             return "pq"
     return None
 

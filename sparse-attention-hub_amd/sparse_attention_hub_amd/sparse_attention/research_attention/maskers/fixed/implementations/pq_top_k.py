@@ -131,9 +131,24 @@ class PQCache(TopKMasker):
             raise ValueError(f"head_dim {head_dim} is not divisible by pq_group_factor {n_sub}")
         if self.pq_bits > 8:
             raise ValueError(f"pq_bits {self.pq_bits} > 8: codes are stored as uint8")
-        if self.metric != "euclidean":
-            raise NotImplementedError("PQCache metric 'ip' (IP->L2 augmentation) is not implemented by the MI355X kernels yet")
         return n_sub, head_dim // n_sub, 2 ** self.pq_bits
+
+    def _augmented(self, keys: torch.Tensor, first: int, n_sub: int, d_sub: int, phi: Optional[torch.Tensor]):
+        """metric="ip": keys[:, :, first:] as (B, Hkv, n, n_sub * (d_sub + 1)) in the key dtype, every sub-vector
+        followed by its extra coordinate - sqrt(phi - ||x||^2) with phi the largest squared norm of the
+        (b, kv head, sub-space) group when the keys are clustered (phi=None; pq_utils.py:585-612), 0 for keys
+        quantised later (pq_utils.py:615-640). Returns (augmented keys, phi [n_groups, 1, 1])."""
+        B, Hkv, Lk, _ = keys.shape
+        n = Lk - first
+        sub = keys[:, :, first:, :].reshape(B, Hkv, n, n_sub, d_sub)
+        if phi is None:
+            norms_sq = (sub ** 2).sum(dim=-1, keepdim=True)
+            phi5 = norms_sq.max(dim=2, keepdim=True)[0]
+            extra = torch.sqrt(phi5 - norms_sq)
+            phi = phi5.permute(0, 1, 3, 2, 4).reshape(-1, 1, 1)
+        else:
+            extra = torch.zeros((B, Hkv, n, n_sub, 1), dtype=keys.dtype, device=keys.device)
+        return torch.cat([sub, extra], dim=-1).reshape(B, Hkv, n, n_sub * (d_sub + 1)).contiguous(), phi
 
     def _perform_kmeans_clustering(self, keys: torch.Tensor, layer_idx: int, sparse_meta_data: Dict[str, Any]):
         """First call of a layer: cluster keys[:, :, init_offset:] and store centroids + codes."""
@@ -141,14 +156,25 @@ class PQCache(TopKMasker):
         n_sub, d_sub, n_cent = self._geometry(keys)
         n_keys = Lk - self.init_offset
         book = PQCodebook(B, Hkv, n_sub, n_keys + 4096, keys.device)
+        source, first, d_fit = keys, self.init_offset, d_sub
+        if self.metric == "ip":
+            # inner-product search as L2 search: cluster the augmented sub-vectors (one more dimension)
+            source, phi = self._augmented(keys, self.init_offset, n_sub, d_sub, None)
+            first, d_fit = 0, d_sub + 1
+            sparse_meta_data["pq_ip2l2_phi"][layer_idx] = phi
         centres, _ = kmeans_keys_batched(
-            keys, self.init_offset, n_sub, n_cent, self.kmeans_iter, book.codes, book.capacity, 0,
+            source, first, n_sub, n_cent, self.kmeans_iter, book.codes, book.capacity, 0,
             tol=1e-4, seed=self.kmeans_seed + 7919 * int(layer_idx),
         )
         book.n = n_keys
-        stored = centres.to(keys.dtype).reshape(B, Hkv, n_sub, n_cent, d_sub)
+        stored = centres.to(keys.dtype).reshape(B, Hkv, n_sub, n_cent, d_fit)
         sparse_meta_data["pq_centroids"][layer_idx] = stored
-        sparse_meta_data["pq_centroids_f32"][layer_idx] = stored.to(torch.float32).reshape(-1, n_cent, d_sub).contiguous()
+        # the scoring table uses the original dimensions only (pq_top_k.py:457-458); new keys are quantised
+        # against the full, possibly augmented centroids
+        sparse_meta_data["pq_centroids_f32"][layer_idx] = (
+            stored[..., :d_sub].to(torch.float32).reshape(-1, n_cent, d_sub).contiguous())
+        sparse_meta_data.setdefault("pq_centroids_fit_f32", {})[layer_idx] = (
+            stored.to(torch.float32).reshape(-1, n_cent, d_fit).contiguous())
         sparse_meta_data["pq_codebook"][layer_idx] = book
         return stored, book
 
@@ -163,10 +189,14 @@ class PQCache(TopKMasker):
         if current > book.n:
             n_new = current - book.n
             book.reserve(current)
-            cf32 = sparse_meta_data["pq_centroids_f32"][layer_idx]
+            cf32 = sparse_meta_data["pq_centroids_fit_f32"][layer_idx]
+            first = self.init_offset + book.n
+            if self.metric == "ip":
+                keys, _ = self._augmented(keys, first, n_sub, d_sub, sparse_meta_data["pq_ip2l2_phi"][layer_idx])
+                first, d_sub = 0, d_sub + 1
             a = N.PqAssignArgs(
                 keys.data_ptr(), keys.stride(0), keys.stride(1), keys.stride(2), N.dtype_code(keys.dtype),
-                B, Hkv, n_sub, d_sub, n_cent, self.init_offset + book.n, n_new,
+                B, Hkv, n_sub, d_sub, n_cent, first, n_new,
                 cf32.data_ptr(), book.codes.data_ptr(), book.capacity, book.n,
                 None, None, 1, None, N.stream_ptr(keys.device),
             )

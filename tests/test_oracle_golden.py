@@ -219,6 +219,41 @@ def test_kmeans_recovers_two_blobs_and_returns_pre_update_codes():
     assert torch.allclose(cent1[0, 0], X[0][codes1[0] == 0].mean(0), atol=1e-6)
 
 
+def test_ip2l2_augmentation_known_answers():
+    # test_pq_utils.py:25-147: phi = largest squared norm of the group, extra column sqrt(phi - ||x||^2),
+    # queries get a zero column, and ||x~ - q~||^2 = phi + ||q||^2 - 2 <x, q> (their x = [1,2], q = [3,4])
+    g = torch.Generator().manual_seed(8)
+    xb = torch.randn(3, 10, 4, generator=g)
+    aug, phi = O.ip2l2_augment(xb)
+    assert aug.shape == (3, 10, 5) and phi.shape == (3, 1, 1)
+    assert torch.equal(aug[..., :4], xb)
+    n2 = (xb ** 2).sum(-1)
+    assert torch.allclose(phi[:, 0, 0], n2.max(1).values)
+    assert torch.allclose(aug[..., 4], (phi[:, :, 0] - n2).sqrt(), atol=1e-6)
+    assert torch.allclose((aug ** 2).sum(-1), phi[:, :, 0].expand(3, 10), rtol=1e-5)   # every augmented key has norm^2 phi
+    xq = torch.randn(3, 2, 4, generator=g)
+    qa = O.ip2l2_augment_queries(xq)
+    assert qa.shape == (3, 2, 5) and torch.equal(qa[..., :4], xq) and bool((qa[..., 4] == 0).all())
+    x = torch.tensor([[[1.0, 2.0]]])
+    q = torch.tensor([[[3.0, 4.0]]])
+    xa, ph = O.ip2l2_augment(x)
+    l2 = ((xa - O.ip2l2_augment_queries(q)) ** 2).sum().item()
+    assert l2 == pytest.approx(ph.item() + 25.0 - 2 * 11.0, rel=1e-5)
+    # hence the nearest augmented key is the key of largest inner product
+    d = ((aug.unsqueeze(1) - qa.unsqueeze(2)) ** 2).sum(-1)
+    assert torch.equal(d.argmin(-1), torch.einsum("gqd,gnd->gqn", xq, xb).argmax(-1))
+    # new keys against (d + 1)-wide centroids: zero column appended, plain squared L2, first minimum
+    cent = torch.randn(1, 2, 2, 4, 3, generator=g)          # B, Hkv, n_sub, k, d + 1 with d = 2
+    nk = torch.randn(1, 2, 3, 4, generator=g)               # B, Hkv, n_new, D = 4
+    codes = O.pq_quantize_new(nk, cent)
+    assert codes.shape == (1, 3, 2, 2)
+    for h in range(2):
+        for j in range(3):
+            for s_ in range(2):
+                v = torch.cat([nk[0, h, j, 2 * s_:2 * s_ + 2], torch.zeros(1)])
+                assert int(codes[0, j, h, s_]) == int(((cent[0, h, s_] - v) ** 2).sum(-1).argmin())
+
+
 def test_pq_scores_manual_and_gqa():
     # test_pq_top_k.py:741-873: score = sum_s q_s . centroid[code]; q head h uses kv head h // G;
     # an augmented last centroid dimension is ignored
