@@ -435,6 +435,68 @@ def test_fused_hash_decode_kernel_matches_separate_launches(cuda, dtype, Lk):
     assert bool((srt[:, 1:] != srt[:, :-1]).all()) and int(cols.min()) == 0 and int(cols.max()) == Lk + 2 - 1
 
 
+@pytest.mark.parametrize("case", [
+    # n_keys, n_cand, col_offset, k, distinct key values (0 = all 65536), active per row, excluded key
+    (700, 700, 0, 50, 0, 30, 0x0080),
+    (700, 690, 10, 50, 20, 30, 0),          # heavy ties, candidate range not aligned to anything
+    (1300, 1283, 17, 200, 5, 100, 3),        # the excluded key lies inside the tie range: active columns take rank
+    (5000, 4872, 128, 600, 300, 640, 0),
+    (100, 100, 0, 100, 9, 40, 4),            # k = all candidates
+    (37, 30, 7, 3, 9, 0, 0),
+    (40000, 39990, 10, 2048, 3000, 640, 0x0080),   # 5 chunks per wave
+    (70016, 70000, 16, 3000, 40, 700, 7),          # 9 chunks per wave, ties everywhere
+    (140000, 139999, 1, 5000, 0, 300, 0x0080),     # too long for registers: keys re-read per pass
+])
+def test_select_topk_16bit_keys_against_stable_sort(cuda, case):
+    """sah_select_topk on 16-bit keys, straight through the C ABI: the k best candidates in the order
+    (key descending, column ascending), columns already active ranking with the excluded key and never
+    emitted again; rows, counts and bitmap against a stable sort on the host."""
+    import numpy as np
+
+    from sparse_attention_hub_amd import _native as N
+
+    n_keys, n_cand, off, k, n_vals, n_active, ek = case
+    n_rows = 3 if n_keys < 20000 else 2
+    rng = np.random.default_rng(n_keys + k)
+    pitch = (n_cand + 7) // 8 * 8
+    keys = (rng.integers(1, n_vals + 1, size=(n_rows, pitch)) if n_vals else rng.integers(0, 65536, size=(n_rows, pitch))).astype(np.uint16)
+    n_words = (n_keys + 31) // 32
+    cap = min(n_keys, n_active + k)
+    cols = np.full((n_rows, cap), -1, np.int32)
+    bm = np.zeros((n_rows, n_words), np.uint32)
+    active = []
+    for r in range(n_rows):
+        a = rng.choice(n_keys, size=n_active, replace=False) if n_active else np.zeros(0, np.int64)
+        active.append(set(a.tolist()))
+        cols[r, :n_active] = a
+        for c in a:
+            bm[r, c >> 5] |= np.uint32(1 << (c & 31))
+    tk = torch.from_numpy(keys.view(np.int16)).to(cuda)
+    tc = torch.from_numpy(cols).to(cuda)
+    tn = torch.full((n_rows,), n_active, dtype=torch.int32, device=cuda)
+    tb = torch.from_numpy(bm.view(np.int32)).to(cuda)
+    rows = N.Rows(tc.data_ptr(), tn.data_ptr(), None, tb.data_ptr(), n_rows, cap, n_keys, n_words)
+    N.call("sah_select_topk", N.SelectTopkArgs(rows, tk.data_ptr(), pitch, 16, n_cand, off, k, ek, 0, 0, 0, N.stream_ptr(cuda)))
+    torch.cuda.synchronize()
+    got_cols, got_cnt, got_bm = tc.cpu().numpy(), tn.cpu().numpy(), tb.cpu().numpy().view(np.uint32)
+    for r in range(n_rows):
+        eff = keys[r, :n_cand].astype(np.int64)
+        excl = np.zeros(n_cand, bool)
+        for c in active[r]:
+            if off <= c < off + n_cand:
+                excl[c - off] = True
+        eff[excl] = ek
+        order = np.argsort(-eff, kind="stable")[: min(k, n_cand)]
+        want = set((order[~excl[order]] + off).tolist())
+        new = got_cols[r, n_active:got_cnt[r]].tolist()
+        assert got_cnt[r] == n_active + len(want) and set(new) == want and len(new) == len(want), f"row {r}"
+        assert set(got_cols[r, :n_active].tolist()) == active[r]
+        exp = bm[r].copy()
+        for c in want:
+            exp[c >> 5] |= np.uint32(1 << (c & 31))
+        assert np.array_equal(got_bm[r], exp), f"bitmap, row {r}"
+
+
 @pytest.mark.parametrize("key_bits", [16, 32])
 def test_select_topk_on_fresh_rows_equals_sink_local_then_select(cuda, key_bits):
     """sah_select_topk with fresh != 0 writes the sink + local rows itself (inside the selection kernel for
