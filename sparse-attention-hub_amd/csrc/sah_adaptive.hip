@@ -94,6 +94,7 @@ struct ad_budget_params {
   float eps, ppf;
   uint32_t k0, k1, o0, o1;
   int prev_empty;
+  int vec_keys;  // 1: every row of keys starts 16-byte aligned (vector loads in the row-maximum pass)
   int* budget;
   float* prob;
   float* stats;
@@ -125,7 +126,44 @@ __global__ __launch_bounds__(AD_NT) void k_adaptive_budget(ad_budget_params P) {
 
   // ---- row maximum of z over ALL keys (adaptive_sampling.py:195-196)
   float zm = -INFINITY;
-  for (int j = tid; j < Lk; j += AD_NT) zm = fmaxf(zm, row.z(j));
+  if (!P.amask && P.vec_keys && P.scaling > 0.f) {
+    // Without an additive mask z is a non-decreasing function of the score, and the keys keep the
+    // scores' order: the row maximum is z of the largest key. 16 bytes of keys per load, integer max.
+    constexpr int KPV = (DT == SAH_F32) ? 4 : 8;  // keys per 16-byte vector
+    const uint4* kv = (const uint4*)row.keys;
+    const int n_vec = Lk / KPV;
+    uint32_t best = 0u;
+    for (int base = 0; base < n_vec; base += 4 * AD_NT) {
+      uint4 q[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int i = base + u * AD_NT + tid;
+        q[u] = i < n_vec ? kv[i] : make_uint4(0u, 0u, 0u, 0u);  // key 0 is the smallest key
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const uint32_t w[4] = {q[u].x, q[u].y, q[u].z, q[u].w};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          if (DT == SAH_F32) {
+            best = w[t] > best ? w[t] : best;
+          } else {
+            const uint32_t lo = w[t] & 0xffffu, hi = w[t] >> 16;
+            best = lo > best ? lo : best;
+            best = hi > best ? hi : best;
+          }
+        }
+      }
+    }
+    for (int j = n_vec * KPV + tid; j < Lk; j += AD_NT) {
+      const uint32_t kj = (uint32_t)row.keys[j];
+      best = kj > best ? kj : best;
+    }
+    float s = sah_round<DT>(ad_key_score<DT>(best) * row.scaling);
+    zm = s;
+  } else {
+    for (int j = tid; j < Lk; j += AD_NT) zm = fmaxf(zm, row.z(j));
+  }
   row.zmax = ad_block_max(zm, s_red);
 
   // ---- static denominator: numerators of the active entries times their inverse weight
@@ -365,6 +403,10 @@ extern "C" int sah_adaptive_budget(const sah_adaptive_budget_args* a) {
   P.k0 = (uint32_t)a->seed; P.k1 = (uint32_t)(a->seed >> 32);
   P.o0 = (uint32_t)a->offset; P.o1 = (uint32_t)(a->offset >> 32);
   P.prev_empty = a->prev_empty;
+  {
+    const int es = a->dtype == SAH_F32 ? 4 : 2;
+    P.vec_keys = (((uintptr_t)a->keys % 16) == 0 && (a->key_pitch * es) % 16 == 0) ? 1 : 0;
+  }
   P.budget = a->budget; P.prob = a->prob; P.stats = a->stats;
   switch (a->dtype) {
     case SAH_F32: return ad_budget_launch<SAH_F32>(a, P);
