@@ -56,6 +56,21 @@ __device__ __forceinline__ void sc_load(const char* p, sc_raw<DT>& r) {
   }
 }
 
+// the K stream is read once per step: a load that does not displace what the caches hold
+template <int DT>
+__device__ __forceinline__ void sc_load_stream(const char* p, sc_raw<DT>& r) {
+  typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+  if constexpr (DT == SAH_F32) {
+    const u4 a = __builtin_nontemporal_load((const u4*)p);
+    const u4 b = __builtin_nontemporal_load((const u4*)p + 1);
+    r.a = make_float4(sah_bits_to_float(a.x), sah_bits_to_float(a.y), sah_bits_to_float(a.z), sah_bits_to_float(a.w));
+    r.b = make_float4(sah_bits_to_float(b.x), sah_bits_to_float(b.y), sah_bits_to_float(b.z), sah_bits_to_float(b.w));
+  } else {
+    const u4 a = __builtin_nontemporal_load((const u4*)p);
+    r.a = make_uint4(a.x, a.y, a.z, a.w);
+  }
+}
+
 template <int DT>
 __device__ __forceinline__ void sc_keep(sc_raw<DT>& r) {
   if constexpr (DT == SAH_F32) {
@@ -168,7 +183,7 @@ __global__ __launch_bounds__(SC_NT) void k_qk_scores(qk_params P) {
     for (int it = 0; it < HB; ++it) {
       int j = j0 + it * KPI + grp;
       if (j > P.Lk - 1) j = P.Lk - 1;  // rows past the end re-read the last row
-      sc_load<DT>(kbase + (int64_t)j * krow, buf[it]);
+      sc_load_stream<DT>(kbase + (int64_t)j * krow, buf[it]);
     }
   };
   auto score = [&](sc_raw<DT> (&buf)[HB], int hs) {
