@@ -288,8 +288,9 @@ int sah_select_topk(const sah_select_topk_args* a);
  * accumulation; emitted as sortable keys like sah_qk_scores for candidates
  * n in [0, n_cand) at keys_out[r * key_pitch + n]. centres are the fp32
  * widening of the stored (`dtype`-rounded) centroids, [n_groups, n_cent, d_sub].
- * The table is built once per call in `lut` (caller's scratch of
- * sah_pq_adc_lut_bytes(...) bytes) and read from LDS by the scoring kernel.
+ * The table is read from LDS by the scoring kernel. Up to 65536 candidates every
+ * workgroup computes its slab itself (one launch, `lut` is not touched); beyond that it
+ * is built once per call in `lut` (caller's scratch of sah_pq_adc_lut_bytes(...) bytes).
  * ------------------------------------------------------------------------- */
 typedef struct sah_pq_assign_args {
   const void* k; int64_t ks_b, ks_h, ks_l;

@@ -381,10 +381,56 @@ struct pq_adc_params {
 
 #define ADC_MAX_LUT 4096  // n_sub * n_cent
 #define ADC_KEYS 2048     // candidates per workgroup of the scoring kernel
+#define ADC_MAX_HEAD_DIM 512  // widest query vector a workgroup stages in LDS when it builds its own table
+#define ADC_OWN_LUT_WGS 32 // up to this many workgroups per KV head each build the lookup table themselves
 
 // Lookup table of one decode step: lut[bh][vg][s][c][i] = round(q_v . centre[bh][s][c]) for the NQ query vectors
 // v = vg * NQ + i of the KV head's group, in the storage type (fp32: NQ = 2, 16-bit: NQ = 4, i.e. 8 bytes per
 // (s, c): one LDS read serves all the query vectors a workgroup scores).
+// NQ dot products -> one 8-byte table entry, each rounded to the storage type
+template <int DT, int NQ>
+__device__ __forceinline__ uint2 pq_pack_entry(const float (&acc)[NQ]) {
+  float val[NQ];
+#pragma unroll
+  for (int i = 0; i < NQ; ++i) val[i] = sah_round<DT>(acc[i]);
+  uint2 pk;
+  if (DT == SAH_F32) {
+    pk.x = sah_float_to_bits(val[0]);
+    pk.y = sah_float_to_bits(val[1]);
+  } else if (DT == SAH_BF16) {
+    pk.x = (uint32_t)sah_float_to_bf16(val[0]) | ((uint32_t)sah_float_to_bf16(val[1]) << 16);
+    pk.y = (uint32_t)sah_float_to_bf16(val[NQ > 2 ? 2 : 0]) | ((uint32_t)sah_float_to_bf16(val[NQ > 2 ? 3 : 0]) << 16);
+  } else {
+    pk.x = (uint32_t)sah_float_to_f16(val[0]) | ((uint32_t)sah_float_to_f16(val[1]) << 16);
+    pk.y = (uint32_t)sah_float_to_f16(val[NQ > 2 ? 2 : 0]) | ((uint32_t)sah_float_to_f16(val[NQ > 2 ? 3 : 0]) << 16);
+  }
+  return pk;
+}
+
+// One table entry: the NQ rounded dot products of sub-space s, centre c, packed into 8 bytes.
+template <int DT>
+__device__ __forceinline__ uint2 pq_lut_entry(const pq_adc_params& P, int b, int hk, int bh, int vg, int s, int c) {
+  constexpr int NQ = (DT == SAH_F32) ? 2 : 4;
+  const int G = P.Hq / P.Hkv;
+  const int nvec = G * P.Lq;
+  const int d_sub = P.d_sub;
+  const float* cc = P.centres + (((int64_t)bh * P.n_sub + s) * P.n_cent + c) * d_sub;
+  float val[NQ];
+#pragma unroll
+  for (int i = 0; i < NQ; ++i) {
+    const int v = vg * NQ + i;
+    val[i] = 0.f;
+    if (v < nvec) {
+      const int h = hk * G + v / P.Lq, qi = v % P.Lq;
+      const int64_t qo = (int64_t)b * P.qs_b + (int64_t)h * P.qs_h + (int64_t)qi * P.qs_l + (int64_t)s * d_sub;
+      float acc = 0.f;
+      for (int d = 0; d < d_sub; ++d) acc = fmaf(sah_load<DT>(P.q, qo + d), cc[d], acc);
+      val[i] = acc;
+    }
+  }
+  return pq_pack_entry<DT>(val);
+}
+
 template <int DT>
 __global__ __launch_bounds__(PQ_NT) void k_pq_lut(pq_adc_params P, void* lut) {
   constexpr int NQ = (DT == SAH_F32) ? 2 : 4;
@@ -393,45 +439,19 @@ __global__ __launch_bounds__(PQ_NT) void k_pq_lut(pq_adc_params P, void* lut) {
   const int vg = blockIdx.z;
   const int hk = bh % P.Hkv;
   const int b = bh / P.Hkv;
-  const int G = P.Hq / P.Hkv;
-  const int nvec = G * P.Lq;
+  const int nvec = (P.Hq / P.Hkv) * P.Lq;
   const int n_vg = (nvec + NQ - 1) / NQ;
-  const int d_sub = P.d_sub, n_cent = P.n_cent;
-  for (int c = threadIdx.x; c < n_cent; c += PQ_NT) {
-    const float* cc = P.centres + (((int64_t)bh * P.n_sub + s) * n_cent + c) * d_sub;
-    float val[NQ];
-#pragma unroll
-    for (int i = 0; i < NQ; ++i) {
-      const int v = vg * NQ + i;
-      val[i] = 0.f;
-      if (v < nvec) {
-        const int h = hk * G + v / P.Lq, qi = v % P.Lq;
-        const int64_t qo = (int64_t)b * P.qs_b + (int64_t)h * P.qs_h + (int64_t)qi * P.qs_l + (int64_t)s * d_sub;
-        float acc = 0.f;
-        for (int d = 0; d < d_sub; ++d) acc = fmaf(sah_load<DT>(P.q, qo + d), cc[d], acc);
-        val[i] = sah_round<DT>(acc);
-      }
-    }
-    const int64_t e = (((int64_t)bh * n_vg + vg) * P.n_sub + s) * n_cent + c;
-    if (DT == SAH_F32) {
-      ((float2*)lut)[e] = make_float2(val[0], val[1]);
-    } else {
-      uint2 pk;
-      if (DT == SAH_BF16) {
-        pk.x = (uint32_t)sah_float_to_bf16(val[0]) | ((uint32_t)sah_float_to_bf16(val[1]) << 16);
-        pk.y = (uint32_t)sah_float_to_bf16(val[2]) | ((uint32_t)sah_float_to_bf16(val[3]) << 16);
-      } else {
-        pk.x = (uint32_t)sah_float_to_f16(val[0]) | ((uint32_t)sah_float_to_f16(val[1]) << 16);
-        pk.y = (uint32_t)sah_float_to_f16(val[2]) | ((uint32_t)sah_float_to_f16(val[3]) << 16);
-      }
-      ((uint2*)lut)[e] = pk;
-    }
+  for (int c = threadIdx.x; c < P.n_cent; c += PQ_NT) {
+    const int64_t e = (((int64_t)bh * n_vg + vg) * P.n_sub + s) * P.n_cent + c;
+    ((uint2*)lut)[e] = pq_lut_entry<DT>(P, b, hk, bh, vg, s, c);
   }
 }
 
 // Scores of ADC_KEYS candidates for the NQ query vectors of one group: the table slab (8 bytes per (s, c))
-// in LDS, one thread per candidate, the candidate's codes as 4-byte words.
-template <int DT>
+// in LDS, one thread per candidate, the candidate's codes as 4-byte words. OWN_LUT: the workgroup computes
+// its slab itself (every workgroup of a KV head repeats that work, which is cheaper than a launch of its own
+// as long as a head is covered by a few dozen workgroups).
+template <int DT, bool OWN_LUT>
 __global__ __launch_bounds__(PQ_NT) void k_pq_adc(pq_adc_params P, const void* lut) {
   constexpr int NQ = (DT == SAH_F32) ? 2 : 4;
   typedef typename std::conditional<DT == SAH_F32, uint32_t, uint16_t>::type key_t;
@@ -454,11 +474,104 @@ __global__ __launch_bounds__(PQ_NT) void k_pq_adc(pq_adc_params P, const void* l
     row[i] = -1;
     if (v < nvec) row[i] = (b * P.Hq + hk * G + v / P.Lq) * P.Lq + v % P.Lq;
   }
-  const uint2* slab = (const uint2*)lut + ((int64_t)bh * n_vg + vg) * lut_n;
-  for (int i = tid; i < lut_n; i += PQ_NT) s_lut[i] = slab[i];
+  if (OWN_LUT) {
+    // the group's query vectors once into LDS (as floats), then every thread builds lut_n / PQ_NT entries
+    // from one centre each: the centre's d_sub floats from memory, the query elements as LDS broadcasts
+    __shared__ __attribute__((aligned(16))) float s_q[NQ][ADC_MAX_HEAD_DIM];
+    const int d_sub = P.d_sub;
+    const int D = n_sub * d_sub;
+    for (int i = tid; i < NQ * D; i += PQ_NT) {
+      const int qn = i / D, e = i % D;
+      const int v = vg * NQ + qn;
+      float x = 0.f;
+      if (v < nvec) {
+        const int h = hk * G + v / P.Lq, qi = v % P.Lq;
+        x = sah_load<DT>(P.q, (int64_t)b * P.qs_b + (int64_t)h * P.qs_h + (int64_t)qi * P.qs_l + e);
+      }
+      s_q[qn][e] = x;
+    }
+    __syncthreads();
+    for (int i = tid; i < lut_n; i += PQ_NT) {
+      const int s = i / n_cent, c = i % n_cent;
+      const float* cc = P.centres + (((int64_t)bh * n_sub + s) * n_cent + c) * d_sub;
+      float acc[NQ];
+#pragma unroll
+      for (int qn = 0; qn < NQ; ++qn) acc[qn] = 0.f;
+      if ((d_sub & 3) == 0) {
+        // 16-byte reads of the centre and of the staged queries (the same fused multiply-adds in the same order)
+        for (int d = 0; d < d_sub; d += 4) {
+          const float4 cv = *(const float4*)(cc + d);
+#pragma unroll
+          for (int qn = 0; qn < NQ; ++qn) {
+            const float4 qv = *(const float4*)&s_q[qn][s * d_sub + d];
+            acc[qn] = fmaf(qv.x, cv.x, acc[qn]);
+            acc[qn] = fmaf(qv.y, cv.y, acc[qn]);
+            acc[qn] = fmaf(qv.z, cv.z, acc[qn]);
+            acc[qn] = fmaf(qv.w, cv.w, acc[qn]);
+          }
+        }
+      } else {
+        for (int d = 0; d < d_sub; ++d) {
+          const float cv = cc[d];
+#pragma unroll
+          for (int qn = 0; qn < NQ; ++qn) acc[qn] = fmaf(s_q[qn][s * d_sub + d], cv, acc[qn]);
+        }
+      }
+      s_lut[i] = pq_pack_entry<DT>(acc);
+    }
+  } else {
+    const uint2* slab = (const uint2*)lut + ((int64_t)bh * n_vg + vg) * lut_n;
+    for (int i = tid; i < lut_n; i += PQ_NT) s_lut[i] = slab[i];
+  }
   __syncthreads();
 
   const bool words = (n_sub & 3) == 0 && ((P.code_pitch * n_sub) & 3) == 0 && ((uintptr_t)P.codes & 3) == 0;
+  if (n_sub == 16 && ((uintptr_t)P.codes & 15) == 0) {
+    // 16 one-byte codes per candidate = one 16-byte load: all of the thread's candidates are requested
+    // before the first table lookup
+    constexpr int T = ADC_KEYS / PQ_NT;
+    uint4 cw[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      int n = blockIdx.x * ADC_KEYS + t * PQ_NT + tid;
+      if (n >= P.n_cand) n = P.n_cand - 1;
+      cw[t] = *(const uint4*)(P.codes + ((int64_t)bh * P.code_pitch + n) * 16);
+    }
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      const int n = blockIdx.x * ADC_KEYS + t * PQ_NT + tid;
+      const uint32_t w4[4] = {cw[t].x, cw[t].y, cw[t].z, cw[t].w};
+      float acc[NQ];
+#pragma unroll
+      for (int i = 0; i < NQ; ++i) acc[i] = 0.f;
+#pragma unroll
+      for (int s = 0; s < 16; ++s) {
+        const uint2 e = s_lut[s * n_cent + (int)((w4[s >> 2] >> (8 * (s & 3))) & 0xffu)];
+        if (DT == SAH_F32) {
+          acc[0] += sah_bits_to_float(e.x);
+          acc[1] += sah_bits_to_float(e.y);
+        } else if (DT == SAH_BF16) {
+          acc[0] += sah_bits_to_float(e.x << 16);
+          acc[1] += sah_bits_to_float(e.x & 0xffff0000u);
+          acc[NQ > 2 ? 2 : 0] += sah_bits_to_float(e.y << 16);
+          acc[NQ > 2 ? 3 : 1] += sah_bits_to_float(e.y & 0xffff0000u);
+        } else {
+          acc[0] += sah_f16_to_float((uint16_t)(e.x & 0xffffu));
+          acc[1] += sah_f16_to_float((uint16_t)(e.x >> 16));
+          acc[NQ > 2 ? 2 : 0] += sah_f16_to_float((uint16_t)(e.y & 0xffffu));
+          acc[NQ > 2 ? 3 : 1] += sah_f16_to_float((uint16_t)(e.y >> 16));
+        }
+      }
+      if (n < P.n_cand) {
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) {
+          if (row[i] >= 0)
+            ((key_t*)P.keys_out)[(int64_t)row[i] * P.key_pitch + n] = (key_t)sah_sort_key<DT>(sah_round<DT>(acc[i]));
+        }
+      }
+    }
+    return;
+  }
   for (int t = 0; t < ADC_KEYS / PQ_NT; ++t) {
     const int n = blockIdx.x * ADC_KEYS + t * PQ_NT + tid;
     if (n >= P.n_cand) continue;
@@ -620,30 +733,42 @@ extern "C" int sah_pq_adc_scores(const sah_pq_adc_args* a) {
   const int nvec = (a->Hq / a->Hkv) * a->Lq;
   const int nq = a->dtype == SAH_F32 ? 2 : 4;
   const int n_vg = (nvec + nq - 1) / nq;
+  if (n_vg > 65535) return sah_fail(SAH_ESHAPE, "sah_pq_adc_scores: too many query vectors per KV head");
+  hipStream_t st = (hipStream_t)a->stream;
+  const int wgs_per_head = (a->n_cand + ADC_KEYS - 1) / ADC_KEYS;
+  dim3 g(wgs_per_head, a->B * a->Hkv, n_vg), blk(PQ_NT);
+  if (wgs_per_head <= ADC_OWN_LUT_WGS && a->n_sub * a->d_sub <= ADC_MAX_HEAD_DIM) {
+    // short contexts: no table in memory, no second launch
+    sah_timed timed("k_pq_adc", a->stream);
+    switch (a->dtype) {
+      case SAH_F32: hipLaunchKernelGGL((k_pq_adc<SAH_F32, true>), g, blk, 0, st, P, (const void*)nullptr); break;
+      case SAH_BF16: hipLaunchKernelGGL((k_pq_adc<SAH_BF16, true>), g, blk, 0, st, P, (const void*)nullptr); break;
+      case SAH_F16: hipLaunchKernelGGL((k_pq_adc<SAH_F16, true>), g, blk, 0, st, P, (const void*)nullptr); break;
+      default: return sah_fail(SAH_EDTYPE, "sah_pq_adc_scores: dtype %d", a->dtype);
+    }
+    return sah_launch_status("sah_pq_adc_scores");
+  }
   const int64_t need = (int64_t)a->B * a->Hkv * n_vg * a->n_sub * a->n_cent * 8;
   if (!a->lut || a->lut_bytes < need)
     return sah_fail(SAH_ECAPACITY, "sah_pq_adc_scores: lut holds %lld bytes, need %lld", (long long)(a->lut ? a->lut_bytes : 0),
                     (long long)need);
-  if (n_vg > 65535) return sah_fail(SAH_ESHAPE, "sah_pq_adc_scores: too many query vectors per KV head");
-  hipStream_t st = (hipStream_t)a->stream;
   {
-    dim3 g(a->n_sub, a->B * a->Hkv, n_vg), blk(PQ_NT);
+    dim3 gl(a->n_sub, a->B * a->Hkv, n_vg);
     sah_timed timed("k_pq_lut", a->stream);
     switch (a->dtype) {
-      case SAH_F32: hipLaunchKernelGGL(k_pq_lut<SAH_F32>, g, blk, 0, st, P, a->lut); break;
-      case SAH_BF16: hipLaunchKernelGGL(k_pq_lut<SAH_BF16>, g, blk, 0, st, P, a->lut); break;
-      case SAH_F16: hipLaunchKernelGGL(k_pq_lut<SAH_F16>, g, blk, 0, st, P, a->lut); break;
+      case SAH_F32: hipLaunchKernelGGL(k_pq_lut<SAH_F32>, gl, blk, 0, st, P, a->lut); break;
+      case SAH_BF16: hipLaunchKernelGGL(k_pq_lut<SAH_BF16>, gl, blk, 0, st, P, a->lut); break;
+      case SAH_F16: hipLaunchKernelGGL(k_pq_lut<SAH_F16>, gl, blk, 0, st, P, a->lut); break;
       default: return sah_fail(SAH_EDTYPE, "sah_pq_adc_scores: dtype %d", a->dtype);
     }
     rc = sah_launch_status("sah_pq_adc_scores(lut)");
     if (rc) return rc;
   }
-  dim3 g((a->n_cand + ADC_KEYS - 1) / ADC_KEYS, a->B * a->Hkv, n_vg), blk(PQ_NT);
   sah_timed timed("k_pq_adc", a->stream);
   switch (a->dtype) {
-    case SAH_F32: hipLaunchKernelGGL(k_pq_adc<SAH_F32>, g, blk, 0, st, P, (const void*)a->lut); break;
-    case SAH_BF16: hipLaunchKernelGGL(k_pq_adc<SAH_BF16>, g, blk, 0, st, P, (const void*)a->lut); break;
-    default: hipLaunchKernelGGL(k_pq_adc<SAH_F16>, g, blk, 0, st, P, (const void*)a->lut); break;
+    case SAH_F32: hipLaunchKernelGGL((k_pq_adc<SAH_F32, false>), g, blk, 0, st, P, (const void*)a->lut); break;
+    case SAH_BF16: hipLaunchKernelGGL((k_pq_adc<SAH_BF16, false>), g, blk, 0, st, P, (const void*)a->lut); break;
+    default: hipLaunchKernelGGL((k_pq_adc<SAH_F16, false>), g, blk, 0, st, P, (const void*)a->lut); break;
   }
   return sah_launch_status("sah_pq_adc_scores");
 }

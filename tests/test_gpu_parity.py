@@ -212,15 +212,17 @@ def test_hash_signatures_bits_and_cache_growth(cuda):
             masker._update_key_signatures(kc[:, :, :100].contiguous(), Hq, meta, 0)
 
 
+@pytest.mark.parametrize("geometry", [(64, 8), (128, 16)])   # (head_dim, sub-spaces); 16 one-byte codes = one 16-byte load
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_pq_chain_cold_and_warm(cuda, dtype):
+def test_pq_chain_cold_and_warm(cuda, dtype, geometry):
     sa = _sa()
     from sparse_attention_hub_amd.sparse_attention.research_attention.maskers.fixed.implementations.utils.pq_utils import (
         gather_sub_vectors, seeded_initial_centres,
     )
 
-    B, Hq, Hkv, Lk, D = 2, 8, 2, 1200, 64
-    n_sub, bits, off, iters, heavy = 8, 4, 16, 5, 64
+    D, n_sub = geometry
+    B, Hq, Hkv, Lk = 2, 8, 2, 1200
+    bits, off, iters, heavy = 4, 16, 5, 64
     n_cent = 2 ** bits
     q, k, v = make_qkv(B, Hq, Hkv, 1, Lk, D, dtype, outliers=True)
     cfg = sa.PQCacheConfig(heavy_size=heavy, pq_group_factor=n_sub, pq_bits=bits, kmeans_iter=iters, init_offset=off,
