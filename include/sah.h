@@ -494,6 +494,14 @@ typedef struct sah_hash_decode_args {
 } sah_hash_decode_args;
 int sah_hash_decode_topk(const sah_hash_decode_args* a);
 
+/* sah_hash_decode_topk(a) followed by sah_sparse_attention(t) on the same rows, with the same
+ * results. When the single-kernel form of the former applies and the attention is the plain
+ * decode case (one workgroup per row, Lq = 1, no additive mask, unit weights, no logits
+ * output, head_dim 64 or 128, same stream and dtype) both run in ONE kernel: the workgroup
+ * that selected a row goes straight on to gather that row's K / V, from a column list kept in
+ * LDS (rows.cols / rows.cnt are still written). Otherwise the two calls are made. */
+int sah_hash_decode_attention(const sah_hash_decode_args* a, const sah_attention_args* t);
+
 /* ---------------------------------------------------------------------------
  * One decode layer-step as a single call: runs, in this order and on the stream
  * each block names, every stage whose pointer is not NULL -
@@ -504,6 +512,7 @@ int sah_hash_decode_topk(const sah_hash_decode_args* a);
  * (tensor pointers, key count). Replaces the per-masker Python dispatch of
  * ResearchAttention.custom_attention (research_attention/base.py:108-148) on the
  * decode path; stops at the first stage that fails and returns its code.
+ * hash_decode directly followed by attention runs as sah_hash_decode_attention.
  * ------------------------------------------------------------------------- */
 typedef struct sah_chain_args {
   const sah_sink_local_args* sink_local;

@@ -10,154 +10,11 @@
 // A second small kernel merges the splits, applies the optional sink logit and
 // writes out[b, q, h, :].
 #include "sah_common.h"
+#include "sah_attn.h"
 
-#define ATT_NT 256
-#define ATT_NW (ATT_NT / SAH_WAVE)
-#define ATT_ROW_NT 1024  // threads of the whole-row form
-#define ATT_CHUNK (ATT_NT)  // keys per workgroup iteration: 64 per wave
-#define ATT_XCDS 8           // accelerator complex dies of an MI355X, one L2 each
-#define ATT_MAX_SPLIT 64
-
-struct att_params {
-  sah_rows rows;
-  const void* q; int64_t qs_b, qs_h, qs_l;
-  const void* k; int64_t ks_b, ks_h, ks_l;
-  const void* v; int64_t vs_b, vs_h, vs_l;
-  const void* amask; int64_t ms_b, ms_h, ms_l;
-  int Hq, Hkv, Lq, Lk;
-  float scaling, unit_inv_w;
-  int dense;
-  int n_split;
-  const float* sinks;
-  void* out;
-  float* stats;
-  float* work;
-  float* logits_out;
-  int64_t logits_pitch;
-};
-
-// exact expf for fp32 storage (1e-5 output tolerance), hardware exp2 path otherwise
-template <int DT>
-__device__ __forceinline__ float att_exp(float x) {
-  return DT == SAH_F32 ? expf(x) : __expf(x);
-}
-
-template <int LPK>
-__device__ __forceinline__ float att_group_sum(float v) {
-  // sum over each aligned group of LPK lanes (LPK in {2,4,8,16})
-  v += sah_dpp<0xB1>(v);
-  if (LPK >= 4) v += sah_dpp<0x4E>(v);
-  if (LPK >= 8) v += sah_dpp<0x141>(v);
-  if (LPK >= 16) v += sah_dpp<0x140>(v);
-  return v;
-}
-
-// raw 8-element row slice as loaded (16 B for 2-byte types, 32 B for fp32)
-template <int DT>
-struct att_raw {
-  uint4 lo;
-  uint4 hi;  // only used for fp32
-};
-
-template <int DT>
-__device__ __forceinline__ void att_load_raw(const char* p, att_raw<DT>& r) {
-  r.lo = *(const uint4*)p;
-  if (DT == SAH_F32) r.hi = *(const uint4*)(p + 16);
-}
-
-template <int DT>
-__device__ __forceinline__ void att_unpack(const att_raw<DT>& r, float (&o)[8]) {
-  const uint32_t w[4] = {r.lo.x, r.lo.y, r.lo.z, r.lo.w};
-  if (DT == SAH_F32) {
-    const uint32_t v[4] = {r.hi.x, r.hi.y, r.hi.z, r.hi.w};
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      o[t] = sah_bits_to_float(w[t]);
-      o[4 + t] = sah_bits_to_float(v[t]);
-    }
-  } else {
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      if (DT == SAH_BF16) {
-        o[2 * t] = sah_bits_to_float(w[t] << 16);
-        o[2 * t + 1] = sah_bits_to_float(w[t] & 0xffff0000u);
-      } else {
-        o[2 * t] = sah_f16_to_float((uint16_t)(w[t] & 0xffffu));
-        o[2 * t + 1] = sah_f16_to_float((uint16_t)(w[t] >> 16));
-      }
-    }
-  }
-}
-
-// Each wave keeps its own online-softmax state (m uniform across the wave, l and acc
-// per lane group) and walks its 64-key slices in batches of UB iterations; the K and V
-// rows of a batch are requested together so 2*UB row loads are in flight per lane.
-// merge the splits of one row: out = sum_s acc_s e^(m_s-M) / sum_s l_s e^(m_s-M).
-// The (m, l) pairs go through LDS and each thread's partial values are requested together,
-// so the merge costs about two memory round trips whatever the number of splits. Every thread of the
-// workgroup calls it (one barrier inside); thread d < D produces output element d.
-template <int DT, int D>
-__device__ __forceinline__ void att_combine_row(const float* work, int n_split, int r, int Hq, int Lq, const float* sinks,
-                                                void* out, float* stats, float* s_m, float* s_l) {
-  const int d = threadIdx.x;
-  const float* w = work + (int64_t)r * n_split * (D + 2);
-  if (d < n_split) {
-    s_m[d] = w[(int64_t)d * (D + 2)];
-    s_l[d] = w[(int64_t)d * (D + 2) + 1];
-  }
-  float part[ATT_MAX_SPLIT / 4];
-  float a = 0.f;
-  float M = -INFINITY, L = 0.f;
-  for (int s0 = 0; s0 < n_split; s0 += ATT_MAX_SPLIT / 4) {
-#pragma unroll
-    for (int u = 0; u < ATT_MAX_SPLIT / 4; ++u) {
-      const int sidx = s0 + u;
-      part[u] = (sidx < n_split && d < D) ? w[(int64_t)sidx * (D + 2) + 2 + d] : 0.f;
-    }
-    if (s0 == 0) {
-      __syncthreads();
-      for (int sidx = 0; sidx < n_split; ++sidx) M = fmaxf(M, s_m[sidx]);
-      for (int sidx = 0; sidx < n_split; ++sidx)
-        if (s_m[sidx] != -INFINITY) L = fmaf(s_l[sidx], att_exp<DT>(s_m[sidx] - M), L);
-    }
-#pragma unroll
-    for (int u = 0; u < ATT_MAX_SPLIT / 4; ++u) {
-      const int sidx = s0 + u;
-      if (sidx < n_split && s_m[sidx] != -INFINITY) a = fmaf(part[u], att_exp<DT>(s_m[sidx] - M), a);
-    }
-  }
-  const int qi = r % Lq;
-  const int h = (r / Lq) % Hq;
-  const int b = r / (Lq * Hq);
-  float Mf = M, den = L;
-  if (sinks) {
-    const float sk = sinks[h];
-    Mf = fmaxf(M, sk);
-    const float sc = (M == -INFINITY) ? 0.f : att_exp<DT>(M - Mf);
-    a *= sc;
-    den = L * sc + att_exp<DT>(sk - Mf);
-  }
-  if (d < D) sah_store<DT>(out, (((int64_t)b * Lq + qi) * Hq + h) * D + d, a / den);
-  if (stats && d == 0) {
-    stats[2 * (int64_t)r] = Mf;
-    stats[2 * (int64_t)r + 1] = den;
-  }
-}
-
-// ROW = false: a workgroup of 4 waves handles one (row, split) tile and leaves (m, l, acc) in the workspace
-//   for the merge kernel - the form for few or very uneven rows.
-// ROW = true: a workgroup of 16 waves handles a whole row, every wave an equal share of the row's entries,
-//   and merges the 16 partial results itself: no workspace, no second kernel, every CU gets the same
-//   amount of work when there are at least as many rows as CUs.
 template <int DT, int D, bool ROW>
 __global__ __launch_bounds__(ROW ? ATT_ROW_NT : ATT_NT, ROW ? 1 : 5) void k_sparse_attn(att_params P) {
   constexpr int NW = (ROW ? ATT_ROW_NT : ATT_NT) / SAH_WAVE;
-  constexpr int LPK = D / 8;            // lanes per key
-  constexpr int KPI = SAH_WAVE / LPK;   // keys per wave iteration
-  constexpr int IT = SAH_WAVE / KPI;    // iterations per 64-key wave slice (== LPK)
-  constexpr int UB = IT < 4 ? IT : 4;   // iterations per batch
-  constexpr int ES = (DT == SAH_F32) ? 4 : 2;
-
   __shared__ float s_m[NW];
   __shared__ float s_l[NW];
   __shared__ float s_acc[NW][D];
@@ -180,180 +37,7 @@ __global__ __launch_bounds__(ROW ? ATT_ROW_NT : ATT_NT, ROW ? 1 : 5) void k_spar
   const int b = gidx / (P.Lq * P.Hkv);
   const int h = hk * G + slot % G;
   const int r = (b * P.Hq + h) * P.Lq + qi;
-  const int tid = threadIdx.x;
-  const int lane = tid & (SAH_WAVE - 1);
-  const int wave = tid / SAH_WAVE;
-  const int sub = lane % LPK;   // which 8-element slice of the row
-  const int grp = lane / LPK;   // which key of the iteration
-
-  int cnt = P.dense ? P.Lk : P.rows.cnt[r];
-  if (!P.dense && cnt > P.rows.cap) cnt = P.rows.cap;
-  // the row's own entry count decides the slices, so rows of very different lengths all spread evenly;
-  // the host picks n_split from an upper bound only
-  int first, bound, stride;  // this wave's slices start at first, first + stride, ... and stop at bound
-  float* wout = nullptr;
-  if constexpr (ROW) {
-    const int per = (((cnt + NW - 1) / NW) + KPI - 1) / KPI * KPI;  // entries per wave
-    first = wave * per;
-    bound = first + per < cnt ? first + per : cnt;
-    stride = SAH_WAVE;
-  } else {
-    const int row_chunks = (cnt + ATT_CHUNK - 1) / ATT_CHUNK;
-    const int kps = ((row_chunks + n_split - 1) / n_split) * ATT_CHUNK;
-    const int begin = split * kps;
-    bound = begin + kps < cnt ? begin + kps : cnt;
-    first = begin + wave * SAH_WAVE;
-    stride = ATT_CHUNK;
-    wout = P.work + ((int64_t)r * n_split + split) * (D + 2);
-    if (begin >= bound) {
-      if (tid == 0) {
-        wout[0] = -INFINITY;
-        wout[1] = 0.f;
-      }
-      return;
-    }
-  }
-
-  const int* cols = P.dense ? nullptr : P.rows.cols + (int64_t)r * P.rows.cap;
-  const float* wts = (!P.dense && P.rows.w) ? P.rows.w + (int64_t)r * P.rows.cap : nullptr;
-  const char* kbase = (const char*)P.k + ((int64_t)b * P.ks_b + (int64_t)hk * P.ks_h + sub * 8) * ES;
-  const char* vbase = (const char*)P.v + ((int64_t)b * P.vs_b + (int64_t)hk * P.vs_h + sub * 8) * ES;
-  const int64_t krow = P.ks_l * ES, vrow = P.vs_l * ES;
-  const int64_t moff = P.amask ? ((int64_t)b * P.ms_b + (int64_t)h * P.ms_h + (int64_t)qi * P.ms_l) : 0;
-
-  float qv[8];
-  sah_load8<DT>(P.q, (int64_t)b * P.qs_b + (int64_t)h * P.qs_h + (int64_t)qi * P.qs_l + sub * 8, qv);
-
-  float acc[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-  float l_run = 0.f;
-  float m_run = -INFINITY;
-
-  for (int cbase = first; cbase < bound; cbase += stride) {
-    // one column (and its inverse weight) per lane: this wave's next 64 keys
-    const int my = cbase + lane;
-    int idx_l = -1;
-    float invw_l = P.unit_inv_w;
-    if (my < bound) {
-      idx_l = P.dense ? my : cols[my];
-      // the reference evaluates 1/(w + 1e-6) in the mask dtype (utils/mask.py:737-740)
-      if (wts) invw_l = sah_round<DT>(1.0f / sah_round<DT>(wts[my] + 1e-6f));
-      if (idx_l < 0 || idx_l >= P.Lk) idx_l = -1;
-    }
-#pragma unroll
-    for (int ib = 0; ib < IT; ib += UB) {
-      if (cbase + ib * KPI >= bound) break;  // uniform across the wave
-      att_raw<DT> kr[UB], vr[UB];
-      int id[UB];
-#pragma unroll
-      for (int u = 0; u < UB; ++u) {
-        id[u] = __shfl(idx_l, (ib + u) * KPI + grp);
-        const int safe = id[u] >= 0 ? id[u] : 0;  // invalid lanes read row 0 and are masked below
-        att_load_raw<DT>(kbase + (int64_t)safe * krow, kr[u]);
-        att_load_raw<DT>(vbase + (int64_t)safe * vrow, vr[u]);
-      }
-      float z[UB];
-      float mb = -INFINITY;
-#pragma unroll
-      for (int u = 0; u < UB; ++u) {
-        float kf[8];
-        att_unpack<DT>(kr[u], kf);
-        float d = 0.f;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) d = fmaf(qv[e], kf[e], d);
-        d = att_group_sum<LPK>(d) * P.scaling;
-        if (id[u] >= 0) {
-          if (P.amask) d += sah_load<DT>(P.amask, moff + id[u]);
-        } else {
-          d = -INFINITY;
-        }
-        z[u] = d;
-        mb = fmaxf(mb, d);
-      }
-      if (P.logits_out && sub == 0) {
-#pragma unroll
-        for (int u = 0; u < UB; ++u) {
-          const int pos = cbase + (ib + u) * KPI + grp;
-          if (pos < bound) P.logits_out[(int64_t)r * P.logits_pitch + pos] = z[u];
-        }
-      }
-      // batch max over the lane groups of the wave: m stays uniform across the wave
-#pragma unroll
-      for (int o = LPK; o < SAH_WAVE; o <<= 1) mb = fmaxf(mb, __shfl_xor(mb, o));
-      const float m_new = fmaxf(m_run, mb);
-      if (m_new != -INFINITY) {
-        const float rescale = (m_run == -INFINITY) ? 0.f : att_exp<DT>(m_run - m_new);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[e] *= rescale;
-        l_run *= rescale;
-        m_run = m_new;
-#pragma unroll
-        for (int u = 0; u < UB; ++u) {
-          const float iw = __shfl(invw_l, (ib + u) * KPI + grp);
-          float p = 0.f;
-          if (z[u] != -INFINITY) p = att_exp<DT>(z[u] - m_new) * iw;
-          l_run += p;
-          float vf[8];
-          att_unpack<DT>(vr[u], vf);
-#pragma unroll
-          for (int e = 0; e < 8; ++e) acc[e] = fmaf(p, vf[e], acc[e]);
-        }
-      }
-    }
-  }
-
-  // ---- reduce the KPI lane groups of the wave, then the waves (rescaled to a common max)
-#pragma unroll
-  for (int o = LPK; o < SAH_WAVE; o <<= 1) {
-#pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] += __shfl_xor(acc[e], o);
-    l_run += __shfl_xor(l_run, o);
-  }
-  if (lane < LPK) {
-#pragma unroll
-    for (int e = 0; e < 8; ++e) s_acc[wave][sub * 8 + e] = acc[e];
-  }
-  if (lane == 0) {
-    s_l[wave] = l_run;
-    s_m[wave] = m_run;
-  }
-  __syncthreads();
-  float M = s_m[0];
-#pragma unroll
-  for (int wv = 1; wv < NW; ++wv) M = fmaxf(M, s_m[wv]);
-  float sc[NW];
-#pragma unroll
-  for (int wv = 0; wv < NW; ++wv) sc[wv] = (s_m[wv] == -INFINITY) ? 0.f : att_exp<DT>(s_m[wv] - M);
-  float a = 0.f, l = 0.f;
-  if (tid < D) {
-#pragma unroll
-    for (int wv = 0; wv < NW; ++wv) a = fmaf(s_acc[wv][tid], sc[wv], a);
-  }
-#pragma unroll
-  for (int wv = 0; wv < NW; ++wv) l = fmaf(s_l[wv], sc[wv], l);
-  if constexpr (ROW) {
-    // the row is complete: normalise (with the optional sink logit, mask_attention_utils.py:357-402) and store
-    float Mf = M, den = l;
-    if (P.sinks) {
-      const float sk = P.sinks[h];
-      Mf = fmaxf(M, sk);
-      const float rs = (M == -INFINITY) ? 0.f : att_exp<DT>(M - Mf);
-      a *= rs;
-      den = l * rs + att_exp<DT>(sk - Mf);
-    }
-    if (tid < D) sah_store<DT>(P.out, (((int64_t)b * P.Lq + qi) * P.Hq + h) * D + tid, a / den);
-    if (P.stats && tid == 0) {
-      P.stats[2 * (int64_t)r] = Mf;
-      P.stats[2 * (int64_t)r + 1] = den;
-    }
-  } else {
-    if (tid < D) wout[2 + tid] = a;
-    if (tid == 0) {
-      wout[0] = M;
-      wout[1] = l;
-    }
-  }
+  att_tile<DT, D, ROW>(P, r, b, h, hk, qi, split, n_split, nullptr, -1, s_m, s_l, s_acc);
 }
 
 template <int DT, int D>
@@ -384,12 +68,6 @@ __global__ __launch_bounds__(256) void k_attn_weights(sah_rows R, const float* l
   const float z = logits[(int64_t)r * pitch + i];
   const float p = (z == -INFINITY) ? 0.f : att_exp<DT>(z - m) * iw / den;
   sah_store<DT>(weights, (int64_t)r * R.n_keys + c, p);
-}
-
-// Whole-row form when every CU can be given rows of its own (or the rows are so short that splitting them
-// only adds a second launch), and rows are not long enough for their spread in length to matter.
-static bool att_use_row_form(int n_rows, int max_cnt) {
-  return max_cnt <= 8192 && (n_rows >= 192 || max_cnt <= 1024);
 }
 
 // Splits per row, from an upper bound of the row lengths: enough workgroups to cover 256 CUs several times,
@@ -450,7 +128,8 @@ static int att_dispatch_d(const sah_attention_args* a, const att_params& P) {
   }
 }
 
-extern "C" int sah_sparse_attention(const sah_attention_args* a) {
+// checks of sah_sparse_attention and the kernels' parameter block (also used by the fused decode kernel)
+int att_prepare(const sah_attention_args* a, att_params& P) {
   if (!a) return sah_fail(SAH_ENULL, "sah_sparse_attention: args is NULL");
   if (!a->q || !a->k || !a->v || !a->out) return sah_fail(SAH_ENULL, "sah_sparse_attention: NULL tensor");
   if (a->B <= 0 || a->Hq <= 0 || a->Hkv <= 0 || a->Lq <= 0 || a->Lk <= 0)
@@ -473,7 +152,6 @@ extern "C" int sah_sparse_attention(const sah_attention_args* a) {
   if (max_cnt <= 0) return sah_fail(SAH_EINVAL, "sah_sparse_attention: max_cnt must be > 0");
   if (!a->dense && max_cnt > a->rows.cap) max_cnt = a->rows.cap;
 
-  att_params P;
   P.rows = a->rows;
   P.q = a->q; P.qs_b = a->qs_b; P.qs_h = a->qs_h; P.qs_l = a->qs_l;
   P.k = a->k; P.ks_b = a->ks_b; P.ks_h = a->ks_h; P.ks_l = a->ks_l;
@@ -491,6 +169,13 @@ extern "C" int sah_sparse_attention(const sah_attention_args* a) {
   if (a->work_floats < need)
     return sah_fail(SAH_ECAPACITY, "sah_sparse_attention: work has %lld floats, need %lld", (long long)a->work_floats,
                     (long long)need);
+  return SAH_OK;
+}
+
+extern "C" int sah_sparse_attention(const sah_attention_args* a) {
+  att_params P;
+  const int rc = att_prepare(a, P);
+  if (rc) return rc;
   switch (a->dtype) {
     case SAH_F32: return att_dispatch_d<SAH_F32>(a, P);
     case SAH_BF16: return att_dispatch_d<SAH_BF16>(a, P);
@@ -534,6 +219,8 @@ extern "C" int sah_run_chain(const sah_chain_args* a) {
     if ((rc = sah_hash_signatures(a->sig_b))) return rc;
   }
   if (a->hamming && (rc = sah_hamming_topk(a->hamming))) return rc;
+  if (a->hash_decode && a->attention && !a->qk && !a->pq_assign && !a->pq_adc && !a->select)
+    return sah_hash_decode_attention(a->hash_decode, a->attention);  // one kernel when shapes allow
   if (a->hash_decode && (rc = sah_hash_decode_topk(a->hash_decode))) return rc;
   if (a->qk && (rc = sah_qk_scores(a->qk))) return rc;
   if (a->pq_assign && (rc = sah_pq_kmeans_assign(a->pq_assign))) return rc;

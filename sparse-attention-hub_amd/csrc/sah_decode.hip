@@ -11,8 +11,11 @@
 // Against three separate launches this saves two kernel boundaries, the bitmap round trip through
 // memory and the query-code round trip.
 #include "sah_common.h"
+#include "sah_attn.h"
 #include "sah_hsw.h"
 #include "sah_sig.h"
+
+static_assert(ATT_ROW_NT == HSW_NT, "selection and whole-row attention share one workgroup");
 
 // Threads per MLP job and weight-row slots per thread: the same geometry as the stand-alone signature
 // kernel, so that both sum in the same order and produce the same bits.
@@ -40,13 +43,12 @@ struct hdec_params {
   int update_bitmap;
 };
 
+// The mask row r of one decode step; returns its entry count. s_cols (optional, LDS, R.cap ints): copy of the
+// row's column list for a caller that continues with it in the same kernel (complete after its next barrier).
 template <int DT, bool MF>
-__global__ __launch_bounds__(HSW_NT) void k_hash_decode(hdec_params P) {
+__device__ __forceinline__ int hdec_row(const hdec_params& P, int r, hsw_lds& S, unsigned char* hdec_dyn, int* s_cols) {
   typedef typename hdec_sig<MF>::lds hdec_sig_lds;
-  __shared__ hsw_lds S;
-  HIP_DYNAMIC_SHARED(unsigned char, hdec_dyn)
   const sah_rows& R = P.R;
-  const int r = blockIdx.x;
   const int tid = threadIdx.x;
   const int n = R.n_keys;
   const int n_ch = (n + 255) / 256;
@@ -69,6 +71,7 @@ __global__ __launch_bounds__(HSW_NT) void k_hash_decode(hdec_params P) {
   int* cols = R.cols + (int64_t)r * R.cap;
   for (int i = tid; i < fixed && i < R.cap; i += HSW_NT) {
     cols[i] = i < s_hi ? i : lo2 + (i - s_hi);
+    if (s_cols) s_cols[i] = i < s_hi ? i : lo2 + (i - s_hi);
     if (R.w) R.w[(int64_t)r * R.cap + i] = 1.0f;
   }
   for (int wi = tid; wi < n_ch * 8; wi += HSW_NT)
@@ -97,7 +100,41 @@ __global__ __launch_bounds__(HSW_NT) void k_hash_decode(hdec_params P) {
   __syncthreads();  // every thread holds q (and the bitmap is complete) before the scores overwrite the scratch
 
   // ---- 3. top-k over the remaining columns
-  hsw_select_row(R, r, kc, q, P.k, fixed < R.cap ? fixed : R.cap, s_bm, s_key, S, buf, true, P.update_bitmap != 0);
+  return hsw_select_row(R, r, kc, q, P.k, fixed < R.cap ? fixed : R.cap, s_bm, s_key, S, buf, true, P.update_bitmap != 0,
+                        s_cols);
+}
+
+template <int DT, bool MF>
+__global__ __launch_bounds__(HSW_NT) void k_hash_decode(hdec_params P) {
+  __shared__ hsw_lds S;
+  HIP_DYNAMIC_SHARED(unsigned char, hdec_dyn)
+  hdec_row<DT, MF>(P, blockIdx.x, S, hdec_dyn, nullptr);
+}
+
+// Selection and attention of a row in one workgroup: as soon as a row's columns are chosen its K / V rows are
+// gathered, from a column list that never leaves LDS. No kernel boundary between the two halves: a CU whose row
+// was selected early starts streaming while others still select, and the attention's start-up latency is paid
+// while the memory system would otherwise idle. Workgroup -> row mapping as in k_sparse_attn (the query heads
+// of a GQA group on one XCD).
+template <int DT, bool MF, int D>
+__global__ __launch_bounds__(HSW_NT) void k_hash_decode_attn(hdec_params P, att_params A, int cols_offset) {
+  __shared__ hsw_lds S;
+  __shared__ float s_m[HSW_NW];
+  __shared__ float s_l[HSW_NW];
+  __shared__ float s_acc[HSW_NW][D];
+  HIP_DYNAMIC_SHARED(unsigned char, hdec_dyn)
+  const int G = A.Hq / A.Hkv;
+  const int slot = blockIdx.x / ATT_XCDS;
+  const int tile = (slot / G) * ATT_XCDS + (int)(blockIdx.x % ATT_XCDS);  // b * Hkv + hk
+  if (tile >= P.R.n_rows / G) return;  // padding to a multiple of 8 tiles
+  const int hk = tile % A.Hkv;
+  const int b = tile / A.Hkv;
+  const int h = hk * G + slot % G;
+  const int r = b * A.Hq + h;
+  int* s_cols = (int*)(hdec_dyn + cols_offset);
+  const int cnt = hdec_row<DT, MF>(P, r, S, hdec_dyn, s_cols);
+  __syncthreads();  // the column list in LDS is complete
+  att_tile<DT, D, true>(A, r, b, h, hk, 0, 0, 1, s_cols, cnt, s_m, s_l, s_acc);
 }
 
 static size_t hdec_lds_bytes(int n_keys) {
@@ -153,7 +190,7 @@ static bool hdec_fusable(const sah_hash_decode_args* a) {
   return true;
 }
 
-extern "C" int sah_hash_decode_topk(const sah_hash_decode_args* a) {
+static int hdec_validate(const sah_hash_decode_args* a) {
   if (!a) return sah_fail(SAH_ENULL, "sah_hash_decode_topk: args is NULL");
   int rc = sah_check_rows(a->rows, "sah_hash_decode_topk");
   if (rc) return rc;
@@ -175,6 +212,28 @@ extern "C" int sah_hash_decode_topk(const sah_hash_decode_args* a) {
   if (worst > a->rows.cap)
     return sah_fail(SAH_ECAPACITY, "sah_hash_decode_topk: cap %d < sink + window + k = %lld", a->rows.cap, (long long)worst);
 
+  return SAH_OK;
+}
+
+static void hdec_fill(const sah_hash_decode_args* a, hdec_params& P) {
+  const bool has_key = a->key_sig && a->key_sig->L > 0;
+  P.R = a->rows;
+  sig_fill(a->query_sig, P.job[0]);
+  sig_fill(has_key ? a->key_sig : a->query_sig, P.job[1]);
+  if (!has_key) P.job[1].codes = nullptr;
+  P.has_key = has_key ? 1 : 0;
+  P.kcodes = (const uint2*)a->kcodes;
+  P.pitch = a->code_pitch;
+  P.k = a->k;
+  P.sink = a->sink;
+  P.window = a->window;
+  P.update_bitmap = a->skip_bitmap ? 0 : 1;
+}
+
+extern "C" int sah_hash_decode_topk(const sah_hash_decode_args* a) {
+  int rc = hdec_validate(a);
+  if (rc) return rc;
+  const bool has_key = a->key_sig && a->key_sig->L > 0;
   if (!hdec_fusable(a)) {
     // same step as three launches
     sah_sink_local_args sl;
@@ -191,17 +250,7 @@ extern "C" int sah_hash_decode_topk(const sah_hash_decode_args* a) {
   }
 
   hdec_params P;
-  P.R = a->rows;
-  sig_fill(a->query_sig, P.job[0]);
-  sig_fill(has_key ? a->key_sig : a->query_sig, P.job[1]);
-  if (!has_key) P.job[1].codes = nullptr;
-  P.has_key = has_key ? 1 : 0;
-  P.kcodes = (const uint2*)a->kcodes;
-  P.pitch = a->code_pitch;
-  P.k = a->k;
-  P.sink = a->sink;
-  P.window = a->window;
-  P.update_bitmap = a->skip_bitmap ? 0 : 1;
+  hdec_fill(a, P);
   const size_t lds = hdec_lds_bytes(a->rows.n_keys);
   const bool mf = hdec_sig_kind(a, has_key) == 2;
   switch (a->query_sig->dtype) {
@@ -209,4 +258,53 @@ extern "C" int sah_hash_decode_topk(const sah_hash_decode_args* a) {
     case SAH_BF16: return mf ? hdec_launch<SAH_BF16, true>(a, P, lds) : hdec_launch<SAH_BF16, false>(a, P, lds);
     default: return mf ? hdec_launch<SAH_F16, true>(a, P, lds) : hdec_launch<SAH_F16, false>(a, P, lds);
   }
+}
+
+template <int DT, bool MF, int D>
+static int hdec_attn_launch(const sah_hash_decode_args* a, const hdec_params& P, const att_params& A, size_t lds, int cols_offset) {
+  static bool raised = false;
+  if (!raised) {
+    hipError_t e = hipFuncSetAttribute((const void*)k_hash_decode_attn<DT, MF, D>, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+    if (e != hipSuccess) return sah_fail((int)e, "sah_hash_decode_attention: cannot raise the LDS limit: %s", hipGetErrorString(e));
+    raised = true;
+  }
+  const int G = A.Hq / A.Hkv;
+  const int n_tiles = P.R.n_rows / G;
+  const int n_wg = (n_tiles + ATT_XCDS - 1) / ATT_XCDS * ATT_XCDS * G;
+  sah_timed timed("k_hash_decode_attn", a->stream);
+  hipLaunchKernelGGL((k_hash_decode_attn<DT, MF, D>), dim3(n_wg), dim3(HSW_NT), lds, (hipStream_t)a->stream, P, A, cols_offset);
+  return sah_launch_status("sah_hash_decode_attention");
+}
+
+extern "C" int sah_hash_decode_attention(const sah_hash_decode_args* a, const sah_attention_args* t) {
+  if (!a || !t) return sah_fail(SAH_ENULL, "sah_hash_decode_attention: args is NULL");
+  int rc = hdec_validate(a);
+  if (rc) return rc;
+  att_params A;
+  rc = att_prepare(t, A);
+  if (rc) return rc;
+  const bool has_key = a->key_sig && a->key_sig->L > 0;
+  const size_t cols_offset = (hdec_lds_bytes(a->rows.n_keys) + 15) & ~(size_t)15;
+  const size_t lds = cols_offset + (size_t)a->rows.cap * 4;
+  const bool one_kernel =
+      hdec_fusable(a) && A.n_split == 0 && !t->dense && !t->amask && !t->logits_out && !t->rows.w && t->Lq == 1 &&
+      t->rows.cols == a->rows.cols && t->rows.cnt == a->rows.cnt && t->rows.cap == a->rows.cap &&
+      t->rows.n_rows == a->rows.n_rows && t->stream == a->stream && t->dtype == a->query_sig->dtype &&
+      (t->D == 128 || t->D == 64) && lds <= 150 * 1024 && getenv("SAH_NO_FUSED_DECODE_ATTENTION") == nullptr;
+  if (!one_kernel) {
+    if ((rc = sah_hash_decode_topk(a))) return rc;
+    return sah_sparse_attention(t);
+  }
+  hdec_params P;
+  hdec_fill(a, P);
+  const bool mf = hdec_sig_kind(a, has_key) == 2;
+#define SAH_HDA(DTC, MFC)                                                                    \
+  (t->D == 128 ? hdec_attn_launch<DTC, MFC, 128>(a, P, A, lds, (int)cols_offset)             \
+               : hdec_attn_launch<DTC, MFC, 64>(a, P, A, lds, (int)cols_offset))
+  switch (t->dtype) {
+    case SAH_F32: return SAH_HDA(SAH_F32, false);
+    case SAH_BF16: return mf ? SAH_HDA(SAH_BF16, true) : SAH_HDA(SAH_BF16, false);
+    default: return mf ? SAH_HDA(SAH_F16, true) : SAH_HDA(SAH_F16, false);
+  }
+#undef SAH_HDA
 }

@@ -92,9 +92,12 @@ __device__ __forceinline__ void hsw_prefetch(const uint2* kc, int n, hsw_bufs& b
 // padded) holds the row's bitmap and every thread of the workgroup has passed a barrier after it was
 // written; cnt0 entries of R.cols are already in place. On exit the selected columns are appended (in no
 // particular order) and cnt is updated; with update_bitmap also the bitmap row (LDS copy and global).
-__device__ __forceinline__ void hsw_select_row(const sah_rows& R, int r, const uint2* kc, const uint2 q, int k, int cnt0,
-                                               uint32_t* s_bm, uint32_t* s_key, hsw_lds& S, hsw_bufs& buf,
-                                               bool prefetched = false, bool update_bitmap = true) {
+// Returns the row's new entry count (every thread). s_cols: optional LDS copy of the row's column list (cap entries):
+// the appended columns are mirrored there for a caller that goes on to use them in the same kernel (the mirror
+// is complete only after the caller's next barrier).
+__device__ __forceinline__ int hsw_select_row(const sah_rows& R, int r, const uint2* kc, const uint2 q, int k, int cnt0,
+                                              uint32_t* s_bm, uint32_t* s_key, hsw_lds& S, hsw_bufs& buf,
+                                              bool prefetched = false, bool update_bitmap = true, int* s_cols = nullptr) {
   int* s_gt = S.gt;
   int* s_eq = S.eq;
   const int tid = threadIdx.x;
@@ -248,6 +251,7 @@ __device__ __forceinline__ void hsw_select_row(const sah_rows& R, int r, const u
         if (at < R.cap) {
           cols[at] = wi * 4 + t;
           if (wts) wts[at] = 1.0f;
+          if (s_cols) s_cols[at] = wi * 4 + t;
         }
       }
     }
@@ -300,9 +304,12 @@ __device__ __forceinline__ void hsw_select_row(const sah_rows& R, int r, const u
       out_pos += __shfl(incl, SAH_WAVE - 1);
     }
   }
-  if (tid == 0) R.cnt[r] = cnt0 + total_out;
-  if (!update_bitmap) return;
+  int cnt_new = cnt0 + total_out;
+  if (tid == 0) R.cnt[r] = cnt_new;
+  if (cnt_new > R.cap) cnt_new = R.cap;
+  if (!update_bitmap) return cnt_new;
   __syncthreads();
   for (int i = tid; i < R.n_words; i += HSW_NT) bm[i] = s_bm[i];
+  return cnt_new;
 }
 

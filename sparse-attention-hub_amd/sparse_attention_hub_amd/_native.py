@@ -36,6 +36,7 @@ EXPECTED_SYMBOLS = (
     "sah_hamming_topk",
     "sah_hamming_scores",
     "sah_hash_decode_topk",
+    "sah_hash_decode_attention",
     "sah_qk_scores",
     "sah_select_topk",
     "sah_pq_kmeans_assign",
@@ -347,7 +348,7 @@ def lib() -> C.CDLL:
         if name in ("sah_version", "sah_last_error", "sah_sparse_attention_work_floats", "sah_pq_adc_lut_bytes",
                     "sah_timing_enable", "sah_timing_collect"):
             continue
-        if name == "sah_hash_signatures_pair":
+        if name in ("sah_hash_signatures_pair", "sah_hash_decode_attention"):
             getattr(handle, name).restype = C.c_int
             getattr(handle, name).argtypes = [C.c_void_p, C.c_void_p]
             continue
