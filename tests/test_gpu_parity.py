@@ -572,6 +572,41 @@ def test_density_and_output_error_metrics(cuda, tmp_path):
     assert torch.allclose(out.cpu(), o_sparse, rtol=1e-4, atol=1e-6)
 
 
+def test_single_kernel_decode_step_head_dim_64(cuda):
+    """The one-kernel decode step (selection + attention) at head_dim 64 with 64-wide signature layers,
+    256 mask rows, a context that is not a multiple of anything: outputs and cache equal to the
+    masker-by-masker path, and against the oracle given the kernel's signatures."""
+    from sparse_attention_hub_amd import _native as N
+
+    sa = _sa()
+    dtype = torch.bfloat16
+    B, Hq, Hkv, D, Lk = 8, 32, 8, 64, 1237
+    q, k, v = make_qkv(B, Hq, Hkv, 1, Lk + 2, D, dtype, seed=13)
+    cfgs = [sa.SinkMaskerConfig(sink_size=20), sa.LocalMaskerConfig(window_size=70),
+            sa.HashAttentionTopKMaskerConfig(heavy_size=150, hat_bits=32, hat_mlp_layers=3, hat_mlp_hidden_size=64,
+                                             hat_mlp_activation="silu", hat_weights=_hat(sa, Hq, D, dtype, hidden=64))]
+    fast = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=cfgs))
+    fast.return_attention_weights = False
+    ref = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=cfgs))
+    m1, m2 = {}, {}
+    kc, vc = k.to(cuda), v.to(cuda)
+    for step in range(2):
+        n = Lk + step
+        qq = make_qkv(B, Hq, Hkv, 1, 1, D, dtype, seed=40 + step)[0].to(cuda)
+        if step == 1:
+            N.timing_enable(True)
+        o1, _ = fast.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m1, layer_idx=0)
+        if step == 1:
+            torch.cuda.synchronize()
+            names = set(N.timing_collect())
+            N.timing_enable(False)
+            assert names == {"k_hash_decode_attn"}, names
+        o2, w2 = ref.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m2, layer_idx=0)
+        assert torch.equal(o1, o2), f"step {step}"
+        assert torch.equal(m1["key"][0].codes[:, :, :n], m2["key"][0].codes[:, :, :n]), f"cache, step {step}"
+        assert bool(((w2 != 0).sum(-1) == 20 + 70 + 150).all())
+
+
 # ------------------------------------------------------------------------ adaptive sampling
 def _adaptive_case(cuda, pre_cfgs, pre_specs, rate, eps, delta, io, lo, B, Hq, Hkv, Lq, Lk, D, dtype, amask=None,
                    seed=1234, outliers=False):
