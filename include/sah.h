@@ -362,6 +362,9 @@ typedef struct sah_attention_args {
   float scaling;
   float unit_inv_w;
   int32_t dense;
+  int32_t closed_form;    /* != 0 (with dense = 0, Lq = 1, no additive mask): the rows' pointers are not read; */
+  int32_t closed_sink;    /* every row's entries are the sink and local columns of its one query, weight 1.0,  */
+  int32_t closed_window;  /* i.e. what sah_sink_local_indices(lq = 1, fresh = 1) would have written             */
   int32_t max_cnt;        /* upper bound of cnt[r] the grid is sized for */
   void* out;
   float* work; int64_t work_floats;

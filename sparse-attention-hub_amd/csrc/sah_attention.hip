@@ -137,7 +137,10 @@ int att_prepare(const sah_attention_args* a, att_params& P) {
   if (a->Hq % a->Hkv) return sah_fail(SAH_EINVAL, "sah_sparse_attention: Hq %% Hkv != 0");
   if (a->rows.n_rows != a->B * a->Hq * a->Lq || a->rows.n_keys != a->Lk)
     return sah_fail(SAH_EINVAL, "sah_sparse_attention: rows shape does not match B*Hq*Lq x Lk");
-  if (!a->dense) {
+  if (a->closed_form && (a->dense || a->Lq != 1 || a->closed_sink < 0 || a->closed_window < 0 || a->amask || a->logits_out))
+    return sah_fail(SAH_EINVAL,
+                    "sah_sparse_attention: closed_form needs Lq = 1, dense = 0, sink / window >= 0, no additive mask, no logits output");
+  if (!a->dense && !a->closed_form) {
     int rc = sah_check_rows(a->rows, "sah_sparse_attention");
     if (rc) return rc;
   }
@@ -149,8 +152,20 @@ int att_prepare(const sah_attention_args* a, att_params& P) {
   if (((uintptr_t)a->q | (uintptr_t)a->k | (uintptr_t)a->v) % (8 * es))
     return sah_fail(SAH_ESHAPE, "sah_sparse_attention: q/k/v base pointers must be %d-byte aligned", 8 * es);
   int max_cnt = a->dense ? a->Lk : a->max_cnt;
+  P.closed_sink = P.closed_lo = P.closed_cnt = 0;
+  if (a->closed_form) {
+    // the columns k_sink_local would write for one query per row (basic_fixed.py:354-363, :48-67)
+    const int s_hi = a->closed_sink < a->Lk ? a->closed_sink : a->Lk;
+    int lo = a->closed_window > 0 ? a->Lk - a->closed_window : a->Lk;
+    if (lo < 0) lo = 0;
+    if (lo < s_hi) lo = s_hi;
+    P.closed_sink = s_hi;
+    P.closed_lo = lo;
+    P.closed_cnt = s_hi + (a->closed_window > 0 ? a->Lk - lo : 0);
+    max_cnt = P.closed_cnt;
+  }
   if (max_cnt <= 0) return sah_fail(SAH_EINVAL, "sah_sparse_attention: max_cnt must be > 0");
-  if (!a->dense && max_cnt > a->rows.cap) max_cnt = a->rows.cap;
+  if (!a->dense && !a->closed_form && max_cnt > a->rows.cap) max_cnt = a->rows.cap;
 
   P.rows = a->rows;
   P.q = a->q; P.qs_b = a->qs_b; P.qs_h = a->qs_h; P.qs_l = a->qs_l;
@@ -159,7 +174,7 @@ int att_prepare(const sah_attention_args* a, att_params& P) {
   P.amask = a->amask; P.ms_b = a->ms_b; P.ms_h = a->ms_h; P.ms_l = a->ms_l;
   P.Hq = a->Hq; P.Hkv = a->Hkv; P.Lq = a->Lq; P.Lk = a->Lk;
   P.scaling = a->scaling; P.unit_inv_w = a->unit_inv_w;
-  P.dense = a->dense ? 1 : 0;
+  P.dense = a->dense ? 1 : (a->closed_form ? 2 : 0);
   P.n_split = att_use_row_form(a->rows.n_rows, max_cnt) ? 0 : att_pick_split(a->rows.n_rows, max_cnt);  // 0: whole rows
   P.work = a->work;
   P.sinks = a->sinks; P.out = a->out; P.stats = a->stats_out;

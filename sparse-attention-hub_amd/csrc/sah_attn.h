@@ -19,6 +19,7 @@ struct att_params {
   int Hq, Hkv, Lq, Lk;
   float scaling, unit_inv_w;
   int dense;
+  int closed_sink, closed_lo, closed_cnt;  // dense == 2: entries [0, closed_sink) are columns [0, closed_sink), the rest start at closed_lo
   int n_split;
   const float* sinks;
   void* out;
@@ -160,7 +161,8 @@ __device__ __forceinline__ void att_tile(const att_params& P, int r, int b, int 
   const int grp = lane / LPK;   // which key of the iteration
 
   // cnt_known >= 0: the caller holds the row's entry count (and `cols` may then point anywhere, LDS included)
-  int cnt = cnt_known >= 0 ? cnt_known : (P.dense ? P.Lk : P.rows.cnt[r]);
+  // P.dense: 0 = the rows' column lists, 1 = every key, 2 = the sink + local columns of one query in closed form
+  int cnt = cnt_known >= 0 ? cnt_known : (P.dense == 1 ? P.Lk : (P.dense == 2 ? P.closed_cnt : P.rows.cnt[r]));
   if (!P.dense && cnt > P.rows.cap) cnt = P.rows.cap;
   // the row's own entry count decides the slices, so rows of very different lengths all spread evenly;
   // the host picks n_split from an upper bound only
@@ -210,7 +212,7 @@ __device__ __forceinline__ void att_tile(const att_params& P, int r, int b, int 
     int idx_l = -1;
     float invw_l = P.unit_inv_w;
     if (my < bound) {
-      idx_l = P.dense ? my : cols[my];
+      idx_l = P.dense == 1 ? my : (P.dense == 2 ? (my < P.closed_sink ? my : P.closed_lo + (my - P.closed_sink)) : cols[my]);
       // the reference evaluates 1/(w + 1e-6) in the mask dtype (utils/mask.py:737-740)
       if (wts) invw_l = sah_round<DT>(1.0f / sah_round<DT>(wts[my] + 1e-6f));
       if (idx_l < 0 || idx_l >= P.Lk) idx_l = -1;

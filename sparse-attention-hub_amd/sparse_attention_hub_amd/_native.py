@@ -258,6 +258,9 @@ class AttentionArgs(C.Structure):
         ("scaling", C.c_float),
         ("unit_inv_w", C.c_float),
         ("dense", C.c_int32),
+        ("closed_form", C.c_int32),
+        ("closed_sink", C.c_int32),
+        ("closed_window", C.c_int32),
         ("max_cnt", C.c_int32),
         ("out", C.c_void_p),
         ("work", C.c_void_p), ("work_floats", C.c_int64),

@@ -273,6 +273,11 @@ class DecodePlan:
         at.scaling, at.unit_inv_w, at.dense, at.max_cnt = float(scaling), self.unit, 0, cap
         at.out, at.work, at.work_floats = out.data_ptr(), work.data_ptr(), work.numel()
         at.logits_out = at.stats_out = None
+        at.closed_form = 0
+        if self.kind == "fixed" and Lq == 1:
+            # Sink + Local alone: the attention kernel takes the columns in closed form, no row is ever written
+            at.closed_form, at.closed_sink, at.closed_window = 1, sink, window
+            chain.sink_local = None
         at.stream = stream
         chain.attention = C.addressof(at)
         N.call("sah_run_chain", chain)

@@ -124,6 +124,7 @@ def _run_attention(
         dt, B, Hq, Hkv, Lq, Lk, D,
         float(scaling), unit,
         1 if dense else 0,
+        0, 0, 0,
         max_cnt,
         out.data_ptr(),
         work.data_ptr(), work.numel(),
