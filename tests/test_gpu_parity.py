@@ -395,6 +395,50 @@ def test_decode_plan_matches_masker_by_masker_path(cuda, kind):
 
 
 
+def test_oracle_topk_full_size_properties(cuda):
+    """Config 2 at its full shape (B = 4, 32 query / 8 KV heads, 32768 keys, top 5 % = 1638, bf16), checked
+    through properties that need no CPU restatement of 128 x 32768 scores: every row holds sink + local +
+    k distinct columns, the sink and local columns among them, and the chosen columns dominate the rest
+    in the kernel's own order-preserving score keys (ties to the lowest column)."""
+    sa = _sa()
+    dtype = torch.bfloat16
+    B, Hq, Hkv, Lk, D = 4, 32, 8, 32768, 128
+    sink, window, k_eff = 128, 512, int(0.05 * 32768)
+    q, k, v = make_qkv(B, Hq, Hkv, 1, Lk, D, dtype, outliers=True, seed=3)
+    ra = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(
+        masker_configs=[sa.SinkMaskerConfig(sink_size=sink), sa.LocalMaskerConfig(window_size=window), sa.OracleTopKConfig(heavy_size=0.05)]))
+    ra.return_attention_weights = False
+    out, _ = ra.custom_attention(None, q.to(cuda), k.to(cuda), v.to(cuda), None, D ** -0.5, 0.0, sparse_meta_data={}, layer_idx=0)
+    plan = next(iter(ra._plans.values()))
+    n_rows = B * Hq
+    cnt = plan.cnt.cpu()
+    assert bool((cnt == sink + window + k_eff).all())
+    cols = plan.cols[:, : sink + window + k_eff].long()
+    srt = torch.sort(cols, dim=1).values
+    assert bool((srt[:, 1:] != srt[:, :-1]).all()) and int(cols.min()) == 0 and int(cols.max()) == Lk - 1
+    member = torch.zeros((n_rows, Lk), dtype=torch.bool, device=cuda)
+    member.scatter_(1, cols, True)
+    assert bool(member[:, :sink].all()) and bool(member[:, Lk - window:].all())
+    keys = (plan.keybuf[:, :Lk].to(torch.int32) & 0xFFFF)             # sortable keys: larger = better
+    cand = keys.clone()
+    cand[:, :sink] = -1
+    cand[:, Lk - window:] = -1
+    chosen = member.clone()
+    chosen[:, :sink] = False
+    chosen[:, Lk - window:] = False
+    assert bool((chosen.sum(1) == k_eff).all())
+    lowest_in = torch.where(chosen, cand, torch.full_like(cand, 1 << 20)).min(1).values
+    highest_out = torch.where(chosen, torch.full_like(cand, -1), cand).max(1).values
+    assert bool((lowest_in >= highest_out).all())
+    # ties at the threshold: every column left out with the threshold key lies behind every chosen one with that key
+    T = lowest_in.unsqueeze(1)
+    idx = torch.arange(Lk, device=cuda).unsqueeze(0).expand(n_rows, -1)
+    last_in = torch.where(chosen & (cand == T), idx, torch.full_like(idx, -1)).max(1).values
+    first_out = torch.where(~chosen & (cand == T), idx, torch.full_like(idx, Lk)).min(1).values
+    assert bool((last_in < first_out).all())
+    assert bool(torch.isfinite(out.float()).all())
+
+
 @pytest.mark.parametrize("dtype,Lk", [(torch.bfloat16, 32768), (torch.float16, 5000), (torch.float32, 3001)])
 def test_fused_hash_decode_kernel_matches_separate_launches(cuda, dtype, Lk):
     """Sink + Local + HashAttention decode steps through the single fused kernel (sink/local rows, both signature
