@@ -17,10 +17,10 @@ __device__ __forceinline__ int sig_score(uint2 q, uint2 k) {
 //       the already-active ones with a nibble of the bitmap row and parks the word in LDS;
 //   P1  the threshold T: P0 has already counted the columns at or above 8 coarse thresholds, one more
 //       pass over the staged bytes counts 7 fine ones inside the bracket (byte-parallel compares, no atomics);
-//   P2  per-wave counts of "above T" and "equal T";
-//   P3  write: one wave scan of per-lane totals, every lane appends the columns of its chunks; ties are
-//       taken lowest column first until `need` are used (the one wave where the budget runs out walks
-//       its chunks in column order); new bits are OR-ed into the LDS copy of the bitmap row, which is
+//   P2  per-lane bit masks "above T" / "equal T" of the lane's columns, per-wave counts of both;
+//   P3  write: a wave scan of per-lane counts, every lane appends the set bits of its mask; ties are
+//       taken lowest column first until `need` are used (the one wave where the budget runs out ranks
+//       its ties in column order); new bits are OR-ed into the LDS copy of the bitmap row, which is
 //       written back once at the end.
 // Active columns hold byte 0 and T >= 1 whenever k inactive columns exist, so P2/P3 never
 // look at the bitmap again.
@@ -34,6 +34,7 @@ __device__ __forceinline__ uint32_t swar_ge(uint32_t w, uint32_t t) {
   return ((w | 0x80808080u) - t * 0x01010101u) & 0x80808080u;
 }
 
+#define HSW_GC 8      // chunks per mask group of P2 / P3: 8 x 4 columns of a lane = one 32-bit mask
 #define HSW_PROBES 8  // coarse thresholds 8, 16, ... 64 counted while the scores are staged
 
 struct hsw_lds {
@@ -202,13 +203,36 @@ __device__ __forceinline__ int hsw_select_row(const sah_rows& R, int r, const ui
   // T == 0: fewer than k inactive columns exist; take them all, byte-0 "ties" emit nothing
   const int need = (T == 0) ? 0 : k - above;
 
-  // ---- P2: per-lane and per-wave counts ---------------------------------------------
+  // ---- P2: per-lane masks and per-wave counts ---------------------------------------
+  // A lane's columns of 8 chunks are one 32-bit mask (bit 8 t + u: column t of the lane's word in chunk
+  // c + u), built with byte-parallel compares: `above T` and `equal T`. The first group's masks stay in
+  // registers for P3 (a row of up to 32768 columns has no second group).
+  auto group_masks = [&](int cg, uint32_t& m_gt, uint32_t& m_eq) {
+    uint32_t ge = 0;
+    m_gt = 0;
+#pragma unroll
+    for (int u = 0; u < HSW_GC; ++u) {
+      if (cg + u < my_c1) {  // uniform across the wave
+        const uint32_t x = s_key[(cg + u) * SAH_WAVE + lane] | 0x80808080u;
+        // bit 7 of every byte of the difference is the flag; it moves to bit u of its byte
+        m_gt |= ((x - (T + 1u) * 0x01010101u) >> (7 - u)) & (0x01010101u << u);
+        ge |= ((x - T * 0x01010101u) >> (7 - u)) & (0x01010101u << u);
+      }
+    }
+    m_eq = ge & ~m_gt;
+  };
+  const int n_grp = (my_c1 - my_c0 + HSW_GC - 1) / HSW_GC;  // uniform across the wave; <= 0 for a wave without chunks
+  uint32_t mg0 = 0, me0 = 0;
   int lane_gt = 0, lane_eq = 0;
-  for (int c = my_c0; c < my_c1; ++c) {
-    const uint32_t w = s_key[c * SAH_WAVE + lane];
-    const uint32_t g = swar_ge(w, T + 1);
-    lane_gt += __popc(g);
-    lane_eq += __popc(swar_ge(w, T) & ~g);
+  for (int g = 0; g < n_grp; ++g) {
+    uint32_t m_gt, m_eq;
+    group_masks(my_c0 + g * HSW_GC, m_gt, m_eq);
+    lane_gt += __popc(m_gt);
+    lane_eq += __popc(m_eq);
+    if (g == 0) {
+      mg0 = m_gt;
+      me0 = m_eq;
+    }
   }
   const int n_gt = sah_wave_sum_i(lane_gt);
   const int n_eq = sah_wave_sum_i(lane_eq);
@@ -217,91 +241,90 @@ __device__ __forceinline__ int hsw_select_row(const sah_rows& R, int r, const ui
     s_eq[wave] = n_eq;
   }
   __syncthreads();
-  int tie_base = 0, out_base = 0, total_out = 0;
+  // lane w < 16 holds wave w's counts: two wave scans give every wave's tie and output offsets
+  int tie_base, out_base, total_out;
   {
-    int tie_run = 0, out_run = 0;
-#pragma unroll
-    for (int wv = 0; wv < HSW_NW; ++wv) {
-      if (wv == wave) {
-        tie_base = tie_run;
-        out_base = out_run;
-      }
-      int take = need - tie_run;
-      if (take < 0) take = 0;
-      if (take > s_eq[wv]) take = s_eq[wv];
-      out_run += s_gt[wv] + take;
-      tie_run += s_eq[wv];
-    }
-    total_out = out_run;
+    const int eq_w = lane < HSW_NW ? s_eq[lane] : 0;
+    const int gt_w = lane < HSW_NW ? s_gt[lane] : 0;
+    const int tie_incl = sah_wave_incl_scan(eq_w);
+    int take = need - (tie_incl - eq_w);
+    if (take < 0) take = 0;
+    if (take > eq_w) take = eq_w;
+    const int out_incl = sah_wave_incl_scan(gt_w + take);
+    tie_base = __builtin_amdgcn_readlane(tie_incl - eq_w, wave);
+    out_base = __builtin_amdgcn_readlane(out_incl - gt_w - take, wave);
+    total_out = __builtin_amdgcn_readlane(out_incl, SAH_WAVE - 1);
   }
 
   // ---- P3: write ----------------------------------------------------------------------
-  // The list of a row is unordered, so a wave whose ties are all taken or all dropped needs one scan: every
-  // lane writes the columns of all its chunks as one run. Only the wave in which the tie budget runs out
-  // has to walk its chunks in column order to keep the lowest ties.
+  // The list of a row is unordered. Per group of 8 chunks a lane's winners are the set bits of one mask: one
+  // wave scan of the per-lane counts places them, and a lane walks its own bits (a few per lane, so the walk
+  // is as long as the busiest lane's count, not the number of chunks). A wave whose ties are all taken or all
+  // dropped needs nothing else; the one wave in which the tie budget runs out first walks its chunks in
+  // column order to keep the lowest ties.
   int* cols = R.cols + (int64_t)r * R.cap;
   float* wts = R.w ? R.w + (int64_t)r * R.cap : nullptr;
   const bool ties_all = (tie_base + n_eq <= need);   // every tie of this wave is taken
   const bool ties_none = (tie_base >= need);         // none is
-  auto emit = [&](uint32_t sel, int wi, int pos) {    // sel: bits 0, 8, 16, 24 = columns 4 * wi + 0..3
+  int out_pos = cnt0 + out_base;
+  int tie_run = tie_base;
+  for (int g = 0; g < n_grp; ++g) {
+    const int cg = my_c0 + g * HSW_GC;
+    uint32_t m_gt = mg0, m_eq = me0;
+    if (g > 0) group_masks(cg, m_gt, m_eq);
+    uint32_t sel = m_gt;
+    if (ties_all) {
+      sel |= m_eq;
+    } else if (!ties_none) {
+      uint32_t kept = 0;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      if (sel & (1u << (8 * t))) {
-        const int at = pos + __popc(sel & ((1u << (8 * t)) - 1u));
-        if (at < R.cap) {
-          cols[at] = wi * 4 + t;
-          if (wts) wts[at] = 1.0f;
-          if (s_cols) s_cols[at] = wi * 4 + t;
-        }
-      }
-    }
-    if (update_bitmap) {
-      const uint32_t nib = ((sel * 0x00204081u) >> 21) & 0xFu;
-      const int j0 = wi * 4;
-      atomicOr(&s_bm[j0 >> 5], nib << (j0 & 31));
-    }
-  };
-  if (ties_all || ties_none) {
-    const int mine = lane_gt + (ties_none ? 0 : lane_eq);
-    int pos = cnt0 + out_base + sah_wave_incl_scan(mine) - mine;
-    for (int c = my_c0; c < my_c1; ++c) {
-      const int wi = c * SAH_WAVE + lane;
-      const uint32_t w = s_key[wi];
-      const uint32_t sel = swar_ge(w, ties_none ? T + 1 : T) >> 7;
-      if (sel) {
-        emit(sel, wi, pos);
-        pos += __popc(sel);
-      }
-    }
-  } else {
-    int out_pos = cnt0 + out_base;
-    int tie_run = tie_base;
-    for (int c = my_c0; c < my_c1; ++c) {
-      const int wi = c * SAH_WAVE + lane;
-      const uint32_t w = s_key[wi];
-      const uint32_t g = swar_ge(w, T + 1) >> 7;
-      uint32_t e = (swar_ge(w, T) >> 7) & ~g;
-      const int ne = __popc(e);
-      const int before = sah_wave_incl_scan(ne) - ne;     // ties in lower lanes of this chunk
-      int allowed = need - (tie_run + before);
-      if (allowed < ne) {                                  // keep only the lowest `allowed` ties
-        uint32_t kept = 0;
+      for (int u = 0; u < HSW_GC; ++u) {
+        if (cg + u < my_c1 && tie_run < need) {            // uniform across the wave
+          const uint32_t e = m_eq & (0x01010101u << u);    // this lane's ties in chunk cg + u
+          const int ne = __popc(e);
+          const int incl = sah_wave_incl_scan(ne);
+          int allowed = need - (tie_run + incl - ne);      // ties in lower chunks and lower lanes come first
+          if (allowed >= ne) {
+            kept |= e;
+          } else {
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const uint32_t bit = e & (1u << (8 * t));
-          if (bit && allowed > 0) {
-            kept |= bit;
-            --allowed;
+            for (int t = 0; t < 4; ++t) {                  // keep only the lowest `allowed` ties
+              const uint32_t bit = e & (1u << (8 * t + u));
+              if (bit && allowed > 0) {
+                kept |= bit;
+                --allowed;
+              }
+            }
           }
+          tie_run += __builtin_amdgcn_readlane(incl, SAH_WAVE - 1);
         }
-        e = kept;
       }
-      tie_run += sah_wave_sum_i(ne);
-      const uint32_t sel = g | e;
-      const int ns = __popc(sel);
-      const int incl = sah_wave_incl_scan(ns);
-      if (sel) emit(sel, wi, out_pos + incl - ns);
-      out_pos += __shfl(incl, SAH_WAVE - 1);
+      sel |= kept;
+    }
+    const int ns = __popc(sel);
+    const int incl = sah_wave_incl_scan(ns);
+    int pos = out_pos + incl - ns;
+    out_pos += __builtin_amdgcn_readlane(incl, SAH_WAVE - 1);
+    if (update_bitmap) {
+#pragma unroll
+      for (int u = 0; u < HSW_GC; ++u) {
+        const uint32_t x = (sel >> u) & 0x01010101u;
+        const uint32_t nib = (x | (x >> 7) | (x >> 14) | (x >> 21)) & 0xFu;
+        const int j0 = ((cg + u) * SAH_WAVE + lane) * 4;
+        if (nib) atomicOr(&s_bm[j0 >> 5], nib << (j0 & 31));
+      }
+    }
+    const int col0 = (cg * SAH_WAVE + lane) * 4;
+    while (sel) {
+      const int b = __ffs(sel) - 1;
+      sel &= sel - 1;
+      const int col = col0 + (b & 7) * (4 * SAH_WAVE) + (b >> 3);
+      if (pos < R.cap) {
+        cols[pos] = col;
+        if (wts) wts[pos] = 1.0f;
+        if (s_cols) s_cols[pos] = col;
+      }
+      ++pos;
     }
   }
   int cnt_new = cnt0 + total_out;
