@@ -80,9 +80,8 @@ __device__ __forceinline__ int hdec_row(const hdec_params& P, int r, hsw_lds& S,
   // ---- 2. signatures of the query and of the newest key
   // uniform across the wave, and known to be: the job's parameters are then fetched by scalar loads
   const int job = __builtin_amdgcn_readfirstlane(tid / HDEC_GROUP);
-  // without a new key the second group repeats the query job (its parameter block is a copy that stores
-  // nothing): every wave then runs the same straight-line code
-  const bool active = true;
+  // without a new key the second group only takes the barriers
+  const bool active = job == 0 || P.has_key != 0;
   const int Hq = P.job[0].Hq;
   // 2-byte weights: all layers requested up-front; fp32 rows are twice as wide, one layer at a time
   constexpr int PF = (DT == SAH_F32) ? 1 : SAH_MAX_MLP_LAYERS;

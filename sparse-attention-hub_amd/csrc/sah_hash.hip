@@ -276,7 +276,7 @@ static size_t sgm_lds_bytes(const sah_hash_sig_args* a) {
 // can the matrix-core kernel run this job?
 static bool sig_mfma_ok(const sah_hash_sig_args* a) {
   if (a->dtype != SAH_BF16 && a->dtype != SAH_F16) return false;
-  if (a->L < 64) return false;  // a few vectors: the GEMV form is the better fit
+  if (a->L < 128) return false;  // a few vectors per head: the small forms are the better fit
   if (a->D % 32 || a->D > SGM_MAXW) return false;
   if (a->xs_b % 8 || a->xs_h % 8 || a->xs_l % 8 || ((uintptr_t)a->x % 16)) return false;
   for (int l = 0; l < a->n_layers; ++l) {

@@ -32,6 +32,7 @@ from .maskers.fixed.implementations.oracle_top_k import OracleTopK
 from .maskers.fixed.implementations.pq_top_k import PQCache, PQCodebook, adc_lut_buffer
 
 _MAX_NEW_KEYS = 64  # more than this many unseen keys => not a decode step, take the general path
+_HASH_BLOCK = 64    # HashAttention decode: new keys are hashed this many at a time (never more than the local window)
 
 
 def plan_kind(maskers) -> Optional[str]:
@@ -170,7 +171,12 @@ class DecodePlan:
                 self.layers[layer_idx] = blocks
             n_new = Lk - cache.n
             cache.reserve(Lk)
-            if n_new > 0:
+            # One query per row: this step can only select columns below Lk - window, so the codes of keys still
+            # inside the local window are not needed yet. They are hashed a block at a time (one bulk launch
+            # every `lag` steps) instead of one key per step; `cache.n` is the number of keys hashed so far.
+            lag = min(window, _HASH_BLOCK) if Lq == 1 else 1
+            hash_now = n_new >= lag
+            if n_new > 0 and hash_now:
                 a = blocks.sig_a
                 a.x = k.data_ptr() + cache.n * k.stride(2) * es
                 a.xs_b, a.xs_h, a.xs_l = k.stride(0), k.stride(1), k.stride(2)
@@ -181,21 +187,26 @@ class DecodePlan:
             bq.x = q.data_ptr()
             bq.xs_b, bq.xs_h, bq.xs_l, bq.stream = q.stride(0), q.stride(1), q.stride(2), stream
             chain.sig_b = C.addressof(bq)
-            if Lq == 1 and n_new <= 1:
-                # the whole mask-building half of the step as one entry point (one kernel when shapes allow)
+            if Lq == 1:
+                # the whole mask-building half of the step as one entry point (one kernel when shapes allow);
+                # a single new key is hashed inside it, a block of them by one launch in front of it
                 hd = self.hash_decode
                 hd.rows, hd.sink, hd.window = rows, sink, window
-                hd.query_sig, hd.key_sig = chain.sig_b, chain.sig_a
+                hd.query_sig = chain.sig_b
+                hd.key_sig = chain.sig_a if n_new == 1 else None
                 hd.kcodes, hd.code_pitch, hd.k, hd.stream = cache.codes.data_ptr(), cache.capacity, k_eff, stream
                 hd.skip_bitmap = 1  # only the attention kernel reads these rows, and it reads the column lists
                 chain.hash_decode = C.addressof(hd)
-                chain.sink_local = chain.sig_a = chain.sig_b = None
+                chain.sink_local = chain.sig_b = None
+                if n_new == 1:
+                    chain.sig_a = None
             else:
                 hm = self.hamming
                 hm.rows, hm.kcodes, hm.code_pitch = rows, cache.codes.data_ptr(), cache.capacity
                 hm.qcodes, hm.lq, hm.k, hm.stream = self.qcodes.data_ptr(), Lq, k_eff, stream
                 chain.hamming = C.addressof(hm)
-            cache.n = Lk
+            if hash_now:
+                cache.n = Lk
         elif self.kind == "oracle":
             self._ensure_keybuf(Lk)
             qa = self.qk

@@ -395,6 +395,38 @@ def test_decode_plan_matches_masker_by_masker_path(cuda, kind):
 
 
 
+def test_decode_plan_hashes_new_keys_in_blocks(cuda):
+    """HashAttention decode through the plan: keys still inside the local window are hashed a block at a time
+    (one bulk launch every `window` steps here), not one per step. Over enough steps for such keys to leave the
+    window and compete, every output equals the masker-by-masker path's, which hashes one key per step, and the
+    stored codes agree."""
+    sa = _sa()
+    dtype = torch.bfloat16
+    B, Hq, Hkv, Lk, D = 2, 8, 2, 1500, 128
+    steps, window = 40, 16
+    q, k, v = make_qkv(B, Hq, Hkv, 1, Lk + steps, D, dtype, outliers=True, seed=11)
+    cfgs = [sa.SinkMaskerConfig(sink_size=8), sa.LocalMaskerConfig(window_size=window),
+            sa.HashAttentionTopKMaskerConfig(heavy_size=200, hat_bits=32, hat_mlp_layers=3, hat_mlp_hidden_size=128,
+                                             hat_mlp_activation="silu", hat_weights=_hat(sa, Hq, D, dtype, hidden=128))]
+    fast = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=cfgs))
+    fast.return_attention_weights = False
+    ref = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=cfgs))
+    m1, m2 = {}, {}
+    kc, vc = k.to(cuda), v.to(cuda)
+    hashed = []
+    for step in range(steps):
+        n = Lk + step
+        qq = make_qkv(B, Hq, Hkv, 1, 1, D, dtype, seed=150 + step)[0].to(cuda)
+        o1, _ = fast.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m1, layer_idx=0)
+        o2, _ = ref.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m2, layer_idx=0)
+        assert torch.equal(o1, o2), f"step {step}"
+        c1, c2 = m1["key"][0], m2["key"][0]
+        assert c2.n == n and n - window < c1.n <= n
+        hashed.append(c1.n)
+    assert len(set(hashed)) == 1 + (steps - 1) // window                 # the cold call, then one block per `window` steps
+    assert torch.equal(c1.codes[:, :, : c1.n], c2.codes[:, :, : c1.n])
+
+
 def test_oracle_topk_full_size_properties(cuda):
     """Config 2 at its full shape (B = 4, 32 query / 8 KV heads, 32768 keys, top 5 % = 1638, bf16), checked
     through properties that need no CPU restatement of 128 x 32768 scores: every row holds sink + local +
@@ -439,14 +471,24 @@ def test_oracle_topk_full_size_properties(cuda):
     assert bool(torch.isfinite(out.float()).all())
 
 
+def _set_hash_block(monkeypatch, block):
+    """New keys per bulk hashing launch of the decode plan; 1 = the newest key is hashed inside every step's kernel."""
+    import importlib
+
+    plan_mod = importlib.import_module("sparse_attention_hub_amd.sparse_attention.research_attention.decode_plan")
+    monkeypatch.setattr(plan_mod, "_HASH_BLOCK", block)
+
+
+@pytest.mark.parametrize("block", [1, 64])
 @pytest.mark.parametrize("dtype,Lk", [(torch.bfloat16, 32768), (torch.float16, 5000), (torch.float32, 3001)])
-def test_fused_hash_decode_kernel_matches_separate_launches(cuda, dtype, Lk):
+def test_fused_hash_decode_kernel_matches_separate_launches(cuda, monkeypatch, dtype, Lk, block):
     """Sink + Local + HashAttention decode steps through the single fused kernel (sink/local rows, both signature
     MLPs, signature top-k) against the masker-by-masker path: same outputs, same signature cache, bit for bit,
     at the headline shape (32 query heads, 8 KV heads, 32768 keys, top-2048) and at ragged sizes."""
     from sparse_attention_hub_amd import _native as N
 
     sa = _sa()
+    _set_hash_block(monkeypatch, block)
     # 256 rows at the ragged size: enough for the one-workgroup-per-row attention, so that selection and
     # attention run as ONE kernel; 64 rows at the headline length: attention in its split form, two more launches
     B, Hq, Hkv, D = (8 if Lk <= 8192 else 2), 32, 8, 128
@@ -476,7 +518,9 @@ def test_fused_hash_decode_kernel_matches_separate_launches(cuda, dtype, Lk):
                 assert names == {"k_hash_decode", "k_sparse_attn", "k_attn_combine"}, names
         o2, _ = ref.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m2, layer_idx=0)
         assert torch.equal(o1, o2), f"step {step}"
-        assert torch.equal(m1["key"][0].codes[:, :, :n], m2["key"][0].codes[:, :, :n]), f"cache, step {step}"
+        hashed = m1["key"][0].n                                       # block > 1: the newest keys are not hashed yet
+        assert hashed == (n if block == 1 else Lk)
+        assert torch.equal(m1["key"][0].codes[:, :, :hashed], m2["key"][0].codes[:, :, :hashed]), f"cache, step {step}"
     # the rows the fused kernel built: sink + local + top-k entries, all distinct
     plan = next(iter(fast._plans.values()))
     cnt = plan.cnt.cpu()
@@ -616,13 +660,15 @@ def test_density_and_output_error_metrics(cuda, tmp_path):
     assert torch.allclose(out.cpu(), o_sparse, rtol=1e-4, atol=1e-6)
 
 
-def test_single_kernel_decode_step_head_dim_64(cuda):
+@pytest.mark.parametrize("block", [1, 64])
+def test_single_kernel_decode_step_head_dim_64(cuda, monkeypatch, block):
     """The one-kernel decode step (selection + attention) at head_dim 64 with 64-wide signature layers,
     256 mask rows, a context that is not a multiple of anything: outputs and cache equal to the
     masker-by-masker path, and against the oracle given the kernel's signatures."""
     from sparse_attention_hub_amd import _native as N
 
     sa = _sa()
+    _set_hash_block(monkeypatch, block)
     dtype = torch.bfloat16
     B, Hq, Hkv, D, Lk = 8, 32, 8, 64, 1237
     q, k, v = make_qkv(B, Hq, Hkv, 1, Lk + 2, D, dtype, seed=13)
@@ -647,7 +693,9 @@ def test_single_kernel_decode_step_head_dim_64(cuda):
             assert names == {"k_hash_decode_attn"}, names
         o2, w2 = ref.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m2, layer_idx=0)
         assert torch.equal(o1, o2), f"step {step}"
-        assert torch.equal(m1["key"][0].codes[:, :, :n], m2["key"][0].codes[:, :, :n]), f"cache, step {step}"
+        hashed = m1["key"][0].n
+        assert hashed == (n if block == 1 else Lk)
+        assert torch.equal(m1["key"][0].codes[:, :, :hashed], m2["key"][0].codes[:, :, :hashed]), f"cache, step {step}"
         assert bool(((w2 != 0).sum(-1) == 20 + 70 + 150).all())
 
 
