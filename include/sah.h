@@ -493,9 +493,45 @@ typedef struct sah_hash_decode_args {
   int64_t code_pitch;
   int32_t k;
   int32_t skip_bitmap;                  /* != 0: rows.bitmap may be left stale (cols and cnt are complete) */
+  /* Optional compact form of the same codes, kept up to date with sah_hash_compact_codes (all NULL / 0:
+   * not offered). The single kernel then reads 4 bytes per column instead of 8: the sign plane, scored as
+   * if no signature component were zero, and corrects the listed columns for which that is wrong. Same
+   * results. Used only when no key is hashed inside this call (key_sig NULL or L = 0). */
+  const uint32_t* pos_codes;            /* row r: pos_codes + r * pos_pitch; pos_pitch % 4 == 0, 16-byte aligned,
+                                           readable up to ceil(n_keys / 256) * 256 + 6144 columns */
+  int64_t pos_pitch;
+  const uint32_t* exc;                  /* row r: exc + 4 * r * exc_cap; 16-byte entries, exc_cap >= 1024 */
+  const int32_t* exc_cnt;               /* [n_rows] */
+  int32_t exc_cap;
+  uint32_t full_plane;                  /* non-zero plane of a key without zero components: (1 << bits) - 1 */
   void* stream;
 } sah_hash_decode_args;
 int sah_hash_decode_topk(const sah_hash_decode_args* a);
+
+/* ---------------------------------------------------------------------------
+ * Maintains the compact form of a key-code stream (no counterpart in the reference, whose
+ * signatures are float tensors: hashattention_top_k.py:255-305 keeps (B, H, n, bits) values
+ * in {-1, 0, +1}). For the columns [from, to) of every row: pos_codes gets the sign plane of
+ * the two-plane code, and every column whose non-zero plane differs from full_plane is
+ * appended to the row's exception list as the 16-byte entry (column, non-zero plane, sign
+ * plane, 0); exc_cnt[r] counts them, also beyond exc_cap (the list has then overflowed and
+ * readers fall back to the two-plane codes). exc_cnt must be zero before the first call;
+ * call once per column range, in any order.
+ * ------------------------------------------------------------------------- */
+typedef struct sah_hash_compact_args {
+  const uint32_t* codes;   /* two-plane codes, row r: codes + 2 * r * code_pitch */
+  int64_t code_pitch;
+  int32_t n_rows;
+  int32_t from, to;
+  uint32_t* pos_codes;
+  int64_t pos_pitch;
+  uint32_t* exc;
+  int32_t exc_cap;
+  int32_t* exc_cnt;
+  uint32_t full_plane;
+  void* stream;
+} sah_hash_compact_args;
+int sah_hash_compact_codes(const sah_hash_compact_args* a);
 
 /* sah_hash_decode_topk(a) followed by sah_sparse_attention(t) on the same rows, with the same
  * results. When the single-kernel form of the former applies and the attention is the plain
@@ -508,7 +544,7 @@ int sah_hash_decode_attention(const sah_hash_decode_args* a, const sah_attention
 /* ---------------------------------------------------------------------------
  * One decode layer-step as a single call: runs, in this order and on the stream
  * each block names, every stage whose pointer is not NULL -
- *   sink_local -> (sig_a, sig_b as sah_hash_signatures_pair) -> hamming
+ *   sink_local -> (sig_a, sig_b as sah_hash_signatures_pair) -> compact -> hamming
  *   -> hash_decode -> qk -> pq_assign -> pq_adc -> select -> attention.
  * The blocks are the argument structures of the entry points above, unchanged;
  * a caller keeps them alive between steps and only patches the fields that move
@@ -528,6 +564,7 @@ typedef struct sah_chain_args {
   const sah_pq_adc_args* pq_adc;
   const sah_select_topk_args* select;
   const sah_attention_args* attention;
+  const sah_hash_compact_args* compact;
 } sah_chain_args;
 int sah_run_chain(const sah_chain_args* a);
 

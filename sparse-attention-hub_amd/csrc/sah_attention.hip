@@ -233,6 +233,7 @@ extern "C" int sah_run_chain(const sah_chain_args* a) {
   } else if (a->sig_b) {
     if ((rc = sah_hash_signatures(a->sig_b))) return rc;
   }
+  if (a->compact && (rc = sah_hash_compact_codes(a->compact))) return rc;
   if (a->hamming && (rc = sah_hamming_topk(a->hamming))) return rc;
   if (a->hash_decode && a->attention && !a->qk && !a->pq_assign && !a->pq_adc && !a->select)
     return sah_hash_decode_attention(a->hash_decode, a->attention);  // one kernel when shapes allow

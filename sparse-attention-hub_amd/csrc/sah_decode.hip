@@ -41,11 +41,19 @@ struct hdec_params {
   int k;
   int sink, window;
   int update_bitmap;
+  // compact code stream (all NULL / 0: the two-plane stream kcodes is scanned)
+  const uint32_t* pos;
+  int64_t pos_pitch;
+  const uint4* exc;
+  const int* exc_cnt;
+  int exc_cap;
+  uint32_t full_plane;
 };
 
 // The mask row r of one decode step; returns its entry count. s_cols (optional, LDS, R.cap ints): copy of the
 // row's column list for a caller that continues with it in the same kernel (complete after its next barrier).
-template <int DT, bool MF>
+// CP: the codes are read in their compact form (one sign plane per column + exception list).
+template <int DT, bool MF, bool CP>
 __device__ __forceinline__ int hdec_row(const hdec_params& P, int r, hsw_lds& S, unsigned char* hdec_dyn, int* s_cols) {
   typedef typename hdec_sig<MF>::lds hdec_sig_lds;
   const sah_rows& R = P.R;
@@ -86,9 +94,21 @@ __device__ __forceinline__ int hdec_row(const hdec_params& P, int r, hsw_lds& S,
   // 2-byte weights: all layers requested up-front; fp32 rows are twice as wide, one layer at a time
   constexpr int PF = (DT == SAH_F32) ? 1 : SAH_MAX_MLP_LAYERS;
   // the first half of the row's codes is requested behind the MLP's own loads and arrives while it computes
-  hsw_bufs buf;
+  hsw_bufs_t<CP> buf;
   const uint2* kc = P.kcodes + (int64_t)r * P.pitch;
-  auto prefetch = [&]() { hsw_prefetch(kc, n, buf); };
+  hsw_compact cs;
+  if constexpr (CP) {
+    cs.pos = P.pos + (int64_t)r * P.pos_pitch;
+    cs.exc = P.exc + (int64_t)r * P.exc_cap;
+    cs.exc_cnt = P.exc_cnt + r;
+    cs.full = kc;
+    cs.exc_cap = P.exc_cap;
+    cs.full_plane = P.full_plane;
+  }
+  auto prefetch = [&]() {
+    if constexpr (CP) hsw_prefetch(cs, n, buf);
+    else hsw_prefetch(kc, n, buf);
+  };
   if constexpr (MF) {
     sig_mfma_block<DT>(P.job[job], active, tid % HDEC_GROUP, r / Hq, r % Hq, 0, 1, P.job[0].n_layers, s_sig[job], prefetch);
   } else {
@@ -99,15 +119,15 @@ __device__ __forceinline__ int hdec_row(const hdec_params& P, int r, hsw_lds& S,
   __syncthreads();  // every thread holds q (and the bitmap is complete) before the scores overwrite the scratch
 
   // ---- 3. top-k over the remaining columns
-  return hsw_select_row(R, r, kc, q, P.k, fixed < R.cap ? fixed : R.cap, s_bm, s_key, S, buf, true, P.update_bitmap != 0,
-                        s_cols);
+  return hsw_select_row<CP>(R, r, kc, q, P.k, fixed < R.cap ? fixed : R.cap, s_bm, s_key, S, buf, true, P.update_bitmap != 0,
+                            s_cols, CP ? &cs : nullptr);
 }
 
-template <int DT, bool MF>
+template <int DT, bool MF, bool CP>
 __global__ __launch_bounds__(HSW_NT) void k_hash_decode(hdec_params P) {
   __shared__ hsw_lds S;
   HIP_DYNAMIC_SHARED(unsigned char, hdec_dyn)
-  hdec_row<DT, MF>(P, blockIdx.x, S, hdec_dyn, nullptr);
+  hdec_row<DT, MF, CP>(P, blockIdx.x, S, hdec_dyn, nullptr);
 }
 
 // Selection and attention of a row in one workgroup: as soon as a row's columns are chosen its K / V rows are
@@ -115,7 +135,7 @@ __global__ __launch_bounds__(HSW_NT) void k_hash_decode(hdec_params P) {
 // was selected early starts streaming while others still select, and the attention's start-up latency is paid
 // while the memory system would otherwise idle. Workgroup -> row mapping as in k_sparse_attn (the query heads
 // of a GQA group on one XCD).
-template <int DT, bool MF, int D>
+template <int DT, bool MF, bool CP, int D>
 __global__ __launch_bounds__(HSW_NT) void k_hash_decode_attn(hdec_params P, att_params A, int cols_offset) {
   __shared__ hsw_lds S;
   __shared__ float s_m[HSW_NW];
@@ -131,7 +151,7 @@ __global__ __launch_bounds__(HSW_NT) void k_hash_decode_attn(hdec_params P, att_
   const int h = hk * G + slot % G;
   const int r = b * A.Hq + h;
   int* s_cols = (int*)(hdec_dyn + cols_offset);
-  const int cnt = hdec_row<DT, MF>(P, r, S, hdec_dyn, s_cols);
+  const int cnt = hdec_row<DT, MF, CP>(P, r, S, hdec_dyn, s_cols);
   __syncthreads();  // the column list in LDS is complete
   att_tile<DT, D, true>(A, r, b, h, hk, 0, 0, 1, s_cols, cnt, s_m, s_l, s_acc);
 }
@@ -143,17 +163,22 @@ static size_t hdec_lds_bytes(int n_keys) {
   return bm + (key > sig ? key : sig);
 }
 
-template <int DT, bool MF>
-static int hdec_launch(const sah_hash_decode_args* a, const hdec_params& P, size_t lds) {
+template <int DT, bool MF, bool CP>
+static int hdec_launch_t(const sah_hash_decode_args* a, const hdec_params& P, size_t lds) {
   static bool raised = false;
   if (!raised) {
-    hipError_t e = hipFuncSetAttribute((const void*)k_hash_decode<DT, MF>, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+    hipError_t e = hipFuncSetAttribute((const void*)k_hash_decode<DT, MF, CP>, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
     if (e != hipSuccess) return sah_fail((int)e, "sah_hash_decode_topk: cannot raise the LDS limit: %s", hipGetErrorString(e));
     raised = true;
   }
   sah_timed timed("k_hash_decode", a->stream);
-  hipLaunchKernelGGL((k_hash_decode<DT, MF>), dim3(a->rows.n_rows), dim3(HSW_NT), lds, (hipStream_t)a->stream, P);
+  hipLaunchKernelGGL((k_hash_decode<DT, MF, CP>), dim3(a->rows.n_rows), dim3(HSW_NT), lds, (hipStream_t)a->stream, P);
   return sah_launch_status("sah_hash_decode_topk");
+}
+
+template <int DT, bool MF>
+static int hdec_launch(const sah_hash_decode_args* a, const hdec_params& P, size_t lds) {
+  return P.pos ? hdec_launch_t<DT, MF, true>(a, P, lds) : hdec_launch_t<DT, MF, false>(a, P, lds);
 }
 
 // Which form of the signature MLP the stand-alone launches would take for this step's jobs: the fused kernel
@@ -214,6 +239,17 @@ static int hdec_validate(const sah_hash_decode_args* a) {
   return SAH_OK;
 }
 
+// may the single kernel read the compact stream the caller offers? (if not it scans the two-plane stream)
+static bool hdec_compact_ok(const sah_hash_decode_args* a) {
+  if (!a->pos_codes || !a->exc || !a->exc_cnt) return false;
+  if (a->key_sig && a->key_sig->L > 0) return false;  // a key hashed inside the kernel would miss its compact entry
+  const int n_ch = (a->rows.n_keys + 255) / 256;
+  const int cpw = (n_ch + HSW_NW - 1) / HSW_NW;
+  if (a->pos_pitch % 4 || ((uintptr_t)a->pos_codes % 16) || a->pos_pitch < (int64_t)(HSW_NW * cpw + 2 * HSW_CBATCH) * 256) return false;
+  if (a->exc_cap < HSW_NT || ((uintptr_t)a->exc % 16)) return false;
+  return true;
+}
+
 static void hdec_fill(const sah_hash_decode_args* a, hdec_params& P) {
   const bool has_key = a->key_sig && a->key_sig->L > 0;
   P.R = a->rows;
@@ -227,6 +263,13 @@ static void hdec_fill(const sah_hash_decode_args* a, hdec_params& P) {
   P.sink = a->sink;
   P.window = a->window;
   P.update_bitmap = a->skip_bitmap ? 0 : 1;
+  const bool cp = hdec_compact_ok(a);
+  P.pos = cp ? a->pos_codes : nullptr;
+  P.pos_pitch = a->pos_pitch;
+  P.exc = (const uint4*)a->exc;
+  P.exc_cnt = a->exc_cnt;
+  P.exc_cap = a->exc_cap;
+  P.full_plane = a->full_plane;
 }
 
 extern "C" int sah_hash_decode_topk(const sah_hash_decode_args* a) {
@@ -259,11 +302,11 @@ extern "C" int sah_hash_decode_topk(const sah_hash_decode_args* a) {
   }
 }
 
-template <int DT, bool MF, int D>
-static int hdec_attn_launch(const sah_hash_decode_args* a, const hdec_params& P, const att_params& A, size_t lds, int cols_offset) {
+template <int DT, bool MF, bool CP, int D>
+static int hdec_attn_launch_t(const sah_hash_decode_args* a, const hdec_params& P, const att_params& A, size_t lds, int cols_offset) {
   static bool raised = false;
   if (!raised) {
-    hipError_t e = hipFuncSetAttribute((const void*)k_hash_decode_attn<DT, MF, D>, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+    hipError_t e = hipFuncSetAttribute((const void*)k_hash_decode_attn<DT, MF, CP, D>, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
     if (e != hipSuccess) return sah_fail((int)e, "sah_hash_decode_attention: cannot raise the LDS limit: %s", hipGetErrorString(e));
     raised = true;
   }
@@ -271,8 +314,14 @@ static int hdec_attn_launch(const sah_hash_decode_args* a, const hdec_params& P,
   const int n_tiles = P.R.n_rows / G;
   const int n_wg = (n_tiles + ATT_XCDS - 1) / ATT_XCDS * ATT_XCDS * G;
   sah_timed timed("k_hash_decode_attn", a->stream);
-  hipLaunchKernelGGL((k_hash_decode_attn<DT, MF, D>), dim3(n_wg), dim3(HSW_NT), lds, (hipStream_t)a->stream, P, A, cols_offset);
+  hipLaunchKernelGGL((k_hash_decode_attn<DT, MF, CP, D>), dim3(n_wg), dim3(HSW_NT), lds, (hipStream_t)a->stream, P, A, cols_offset);
   return sah_launch_status("sah_hash_decode_attention");
+}
+
+template <int DT, bool MF, int D>
+static int hdec_attn_launch(const sah_hash_decode_args* a, const hdec_params& P, const att_params& A, size_t lds, int cols_offset) {
+  return P.pos ? hdec_attn_launch_t<DT, MF, true, D>(a, P, A, lds, cols_offset)
+               : hdec_attn_launch_t<DT, MF, false, D>(a, P, A, lds, cols_offset);
 }
 
 extern "C" int sah_hash_decode_attention(const sah_hash_decode_args* a, const sah_attention_args* t) {
@@ -306,4 +355,36 @@ extern "C" int sah_hash_decode_attention(const sah_hash_decode_args* a, const sa
     default: return mf ? SAH_HDA(SAH_F16, true) : SAH_HDA(SAH_F16, false);
   }
 #undef SAH_HDA
+}
+
+// ---------------------------------------------------------------------------
+// Compact form of the key-code stream: sign planes and the list of columns with a zero component.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_hash_compact(const uint2* codes, int64_t code_pitch, int from, int to, uint32_t* pos,
+                                                      int64_t pos_pitch, uint4* exc, int exc_cap, int* exc_cnt,
+                                                      uint32_t full_plane) {
+  const int r = blockIdx.y;
+  const int j = from + blockIdx.x * 256 + threadIdx.x;
+  if (j >= to) return;
+  const uint2 c = codes[(int64_t)r * code_pitch + j];
+  pos[(int64_t)r * pos_pitch + j] = c.x;
+  if (c.y != full_plane) {
+    const int slot = atomicAdd(&exc_cnt[r], 1);
+    if (slot < exc_cap) exc[(int64_t)r * exc_cap + slot] = make_uint4((uint32_t)j, c.y, c.x, 0u);
+  }
+}
+
+extern "C" int sah_hash_compact_codes(const sah_hash_compact_args* a) {
+  if (!a) return sah_fail(SAH_ENULL, "sah_hash_compact_codes: args is NULL");
+  if (!a->codes || !a->pos_codes || !a->exc || !a->exc_cnt) return sah_fail(SAH_ENULL, "sah_hash_compact_codes: NULL buffer");
+  if (a->n_rows <= 0 || a->n_rows > 65535) return sah_fail(SAH_ESHAPE, "sah_hash_compact_codes: n_rows %d not in [1, 65535]", a->n_rows);
+  if (a->from < 0 || a->to < a->from) return sah_fail(SAH_EINVAL, "sah_hash_compact_codes: bad column range [%d, %d)", a->from, a->to);
+  if (a->code_pitch < a->to || a->pos_pitch < a->to) return sah_fail(SAH_ECAPACITY, "sah_hash_compact_codes: pitch < to");
+  if (a->exc_cap < 1 || ((uintptr_t)a->exc % 16)) return sah_fail(SAH_EINVAL, "sah_hash_compact_codes: exception list unaligned or empty");
+  if (a->to == a->from) return SAH_OK;
+  sah_timed timed("k_hash_compact", a->stream);
+  hipLaunchKernelGGL(k_hash_compact, dim3((a->to - a->from + 255) / 256, a->n_rows), dim3(256), 0, (hipStream_t)a->stream,
+                     (const uint2*)a->codes, a->code_pitch, a->from, a->to, a->pos_codes, a->pos_pitch, (uint4*)a->exc,
+                     a->exc_cap, a->exc_cnt, a->full_plane);
+  return sah_launch_status("sah_hash_compact_codes");
 }

@@ -50,10 +50,36 @@ __host__ __device__ inline size_t hsw_lds_bytes(int n_keys) {
   return (size_t)n_ch * 8 * 4 + (size_t)n_ch * 64 * 4;
 }
 
-// Register buffers of the staging pass: two batches of HSW_BATCH chunks (4 codes = 32 B per lane and chunk).
-struct hsw_bufs {
+// Compact form of a row's code stream, for rows whose keys almost never have a zero signature component: one
+// 32-bit sign plane per column (`pos`, 4 B instead of 8), scored as if every component were non-zero, plus the
+// list of the columns for which that is not true (`exc`: column, non-zero plane, sign plane, unused), whose
+// scores are corrected after staging. *exc_cnt entries exist; a count above exc_cap means the list overflowed,
+// and every column is then checked against the two-plane stream `full`.
+struct hsw_compact {
+  const uint32_t* pos;   // this row's sign planes; readable up to (16 * chunks per wave + 8) * 256 columns
+  const uint4* exc;      // this row's exception entries (exc_cap >= HSW_NT of them allocated)
+  const int* exc_cnt;    // this row's exception count
+  const uint2* full;     // this row's two-plane codes
+  int exc_cap;
+  uint32_t full_plane;   // non-zero plane of a key without zero components
+};
+
+#define HSW_CBATCH 4  // compact stream: 256-column chunks per register buffer (16 B per lane and chunk)
+
+// Register buffers of the staging pass: two batches of HSW_BATCH chunks (4 codes = 32 B per lane and chunk),
+// or, for the compact stream, two batches of HSW_CBATCH chunks (4 sign planes = 16 B) and the row's first
+// exception entry per thread.
+template <bool CP>
+struct hsw_bufs_t {
   uint4 a0[HSW_BATCH], a1[HSW_BATCH], b0[HSW_BATCH], b1[HSW_BATCH];
 };
+template <>
+struct hsw_bufs_t<true> {
+  uint4 a[HSW_CBATCH], b[HSW_CBATCH];
+  uint4 exc_first;
+  int exc_n;
+};
+typedef hsw_bufs_t<false> hsw_bufs;
 
 // wave `wave` stages the chunks [c0, c1) of a row of n columns
 __device__ __forceinline__ void hsw_wave_chunks(int n, int wave, int& c0, int& c1) {
@@ -89,6 +115,24 @@ __device__ __forceinline__ void hsw_prefetch(const uint2* kc, int n, hsw_bufs& b
   hsw_request(kc, n, lane, buf.b0, buf.b1, c0 + HSW_BATCH);
 }
 
+__device__ __forceinline__ void hsw_request_c(const uint32_t* pos, int lane, uint4 (&rc)[HSW_CBATCH], int c0) {
+#pragma unroll
+  for (int u = 0; u < HSW_CBATCH; ++u) rc[u] = *(const uint4*)(pos + ((c0 + u) * SAH_WAVE + lane) * 4);
+}
+
+// the same for the compact stream: the calling wave's first 8 chunks (a row of up to 32768 columns completely),
+// the row's exception count and the calling thread's first exception entry
+__device__ __forceinline__ void hsw_prefetch(const hsw_compact& cs, int n, hsw_bufs_t<true>& buf) {
+  const int lane = threadIdx.x & (SAH_WAVE - 1);
+  int c0, c1;
+  hsw_wave_chunks(n, threadIdx.x / SAH_WAVE, c0, c1);
+  (void)c1;
+  hsw_request_c(cs.pos, lane, buf.a, c0);
+  hsw_request_c(cs.pos, lane, buf.b, c0 + HSW_CBATCH);
+  buf.exc_n = *cs.exc_cnt;
+  buf.exc_first = cs.exc[threadIdx.x];
+}
+
 // Top-k of row r over the not-yet-active columns. On entry `s_bm` (n_ch * 8 words of dynamic LDS, zero
 // padded) holds the row's bitmap and every thread of the workgroup has passed a barrier after it was
 // written; cnt0 entries of R.cols are already in place. On exit the selected columns are appended (in no
@@ -96,9 +140,12 @@ __device__ __forceinline__ void hsw_prefetch(const uint2* kc, int n, hsw_bufs& b
 // Returns the row's new entry count (every thread). s_cols: optional LDS copy of the row's column list (cap entries):
 // the appended columns are mirrored there for a caller that goes on to use them in the same kernel (the mirror
 // is complete only after the caller's next barrier).
+// CP: the row's codes come in the compact form `cs` (kc is not used).
+template <bool CP = false>
 __device__ __forceinline__ int hsw_select_row(const sah_rows& R, int r, const uint2* kc, const uint2 q, int k, int cnt0,
-                                              uint32_t* s_bm, uint32_t* s_key, hsw_lds& S, hsw_bufs& buf,
-                                              bool prefetched = false, bool update_bitmap = true, int* s_cols = nullptr) {
+                                              uint32_t* s_bm, uint32_t* s_key, hsw_lds& S, hsw_bufs_t<CP>& buf,
+                                              bool prefetched = false, bool update_bitmap = true, int* s_cols = nullptr,
+                                              const hsw_compact* cs = nullptr) {
   int* s_gt = S.gt;
   int* s_eq = S.eq;
   const int tid = threadIdx.x;
@@ -117,53 +164,128 @@ __device__ __forceinline__ int hsw_select_row(const sah_rows& R, int r, const ui
   int pc[HSW_PROBES];
 #pragma unroll
   for (int i = 0; i < HSW_PROBES; ++i) pc[i] = 0;
-  // Two register buffers of HSW_BATCH chunks each: the next batch is requested before the current one is
-  // scored, so the memory pipe stays busy while the ALUs work.
-  auto score = [&](uint4 (&ra)[HSW_BATCH], uint4 (&rb)[HSW_BATCH], int c0) {
+  // what staging a word has in common: zero the bytes of already-active columns, park the word, count the probes
+  auto stage = [&](uint32_t word, int wi) {
+    const int j0 = wi * 4;
+    const uint32_t nib = (s_bm[j0 >> 5] >> (j0 & 31)) & 0xFu;  // nibble -> byte mask
+    const uint32_t act = ((nib * 0x00204081u) & 0x01010101u) * 0xFFu;
+    const uint32_t kw = word & ~act;
+    s_key[wi] = kw;
+    const uint32_t x = kw | 0x80808080u;
 #pragma unroll
-    for (int u = 0; u < HSW_BATCH; ++u) {
-      sah_keep(ra[u].x); sah_keep(ra[u].y); sah_keep(ra[u].z); sah_keep(ra[u].w);
-      sah_keep(rb[u].x); sah_keep(rb[u].y); sah_keep(rb[u].z); sah_keep(rb[u].w);
-    }
-#pragma unroll
-    for (int u = 0; u < HSW_BATCH; ++u) {
-      if (c0 + u >= my_c1) break;
-      const int wi = (c0 + u) * SAH_WAVE + lane;
-      const int j0 = wi * 4;
-      uint32_t word;
-      if (j0 + 4 <= n) {
-        const uint32_t s0 = (uint32_t)(sig_score(q, make_uint2(ra[u].x, ra[u].y)) + 33);
-        const uint32_t s1 = (uint32_t)(sig_score(q, make_uint2(ra[u].z, ra[u].w)) + 33);
-        const uint32_t s2 = (uint32_t)(sig_score(q, make_uint2(rb[u].x, rb[u].y)) + 33);
-        const uint32_t s3 = (uint32_t)(sig_score(q, make_uint2(rb[u].z, rb[u].w)) + 33);
-        word = s0 | (s1 << 8) | (s2 << 16) | (s3 << 24);
-      } else {
-        word = 0;  // ragged tail: the few columns of the last, partial group
-        for (int t = 0; t < 4; ++t)
-          if (j0 + t < n) word |= (uint32_t)(sig_score(q, kc[j0 + t]) + 33) << (8 * t);
-      }
-      // zero the bytes of already-active columns: nibble -> byte mask
-      const uint32_t nib = (s_bm[j0 >> 5] >> (j0 & 31)) & 0xFu;
-      const uint32_t act = ((nib * 0x00204081u) & 0x01010101u) * 0xFFu;
-      const uint32_t kw = word & ~act;
-      s_key[wi] = kw;
-      const uint32_t x = kw | 0x80808080u;
-#pragma unroll
-      for (int i = 0; i < HSW_PROBES; ++i) pc[i] += __popc((x - (uint32_t)(8 * (i + 1)) * 0x01010101u) & 0x80808080u);
-    }
+    for (int i = 0; i < HSW_PROBES; ++i) pc[i] += __popc((x - (uint32_t)(8 * (i + 1)) * 0x01010101u) & 0x80808080u);
   };
-  if (!prefetched && my_c0 < my_c1) hsw_request(kc, n, lane, buf.a0, buf.a1, my_c0);
-  for (int c0 = my_c0; c0 < my_c1; c0 += 2 * HSW_BATCH) {
-    const bool more_b = c0 + HSW_BATCH < my_c1;          // uniform across the wave
-    if (more_b && !(prefetched && c0 == my_c0)) hsw_request(kc, n, lane, buf.b0, buf.b1, c0 + HSW_BATCH);
-    score(buf.a0, buf.a1, c0);
-    if (c0 + 2 * HSW_BATCH < my_c1) hsw_request(kc, n, lane, buf.a0, buf.a1, c0 + 2 * HSW_BATCH);
-    if (more_b) score(buf.b0, buf.b1, c0 + HSW_BATCH);
-  }
+  if constexpr (CP) {
+    // ---- compact stream: every component taken as non-zero, score = popc(q.y) - 2 popc((q.x ^ k.x) & q.y)
+    const uint32_t s_full = (uint32_t)__popc(q.y) + 33u;
+    auto score1 = [&](uint32_t kx) { return s_full - 2u * (uint32_t)__popc((q.x ^ kx) & q.y); };
+    auto score_c = [&](uint4 (&rc)[HSW_CBATCH], int c0) {
 #pragma unroll
-  for (int i = 0; i < HSW_PROBES; ++i) {
-    const int t = sah_wave_sum_i(pc[i]);
-    if (lane == 0) S.probe[wave][i] = t;
+      for (int u = 0; u < HSW_CBATCH; ++u) {
+        sah_keep(rc[u].x); sah_keep(rc[u].y); sah_keep(rc[u].z); sah_keep(rc[u].w);
+      }
+#pragma unroll
+      for (int u = 0; u < HSW_CBATCH; ++u) {
+        if (c0 + u >= my_c1) break;
+        const int wi = (c0 + u) * SAH_WAVE + lane;
+        const int j0 = wi * 4;
+        uint32_t word;
+        if (j0 + 4 <= n) {
+          word = score1(rc[u].x) | (score1(rc[u].y) << 8) | (score1(rc[u].z) << 16) | (score1(rc[u].w) << 24);
+        } else {
+          word = 0;  // ragged tail
+          for (int t = 0; t < 4; ++t)
+            if (j0 + t < n) word |= score1(cs->pos[j0 + t]) << (8 * t);
+        }
+        stage(word, wi);
+      }
+    };
+    if (!prefetched) {
+      buf.exc_n = *cs->exc_cnt;
+      buf.exc_first = cs->exc[tid];
+      if (my_c0 < my_c1) hsw_request_c(cs->pos, lane, buf.a, my_c0);
+    }
+    for (int c0 = my_c0; c0 < my_c1; c0 += 2 * HSW_CBATCH) {
+      const bool more_b = c0 + HSW_CBATCH < my_c1;          // uniform across the wave
+      if (more_b && !(prefetched && c0 == my_c0)) hsw_request_c(cs->pos, lane, buf.b, c0 + HSW_CBATCH);
+      score_c(buf.a, c0);
+      if (c0 + 2 * HSW_CBATCH < my_c1) hsw_request_c(cs->pos, lane, buf.a, c0 + 2 * HSW_CBATCH);
+      if (more_b) score_c(buf.b, c0 + HSW_CBATCH);
+    }
+    // ---- the columns with a zero component: exact score from both planes, staged byte and probe counts corrected
+    __syncthreads();  // every word is staged
+    unsigned char* s_byte = (unsigned char*)s_key;
+    auto patch = [&](int col, uint32_t kx, uint32_t ky) {
+      if (col < n && !((s_bm[col >> 5] >> (col & 31)) & 1u)) {
+        const uint32_t s_new = (uint32_t)(sig_score(q, make_uint2(kx, ky)) + 33);
+        const uint32_t s_old = s_byte[col];
+        s_byte[col] = (unsigned char)s_new;
+#pragma unroll
+        for (int i = 0; i < HSW_PROBES; ++i)
+          pc[i] += (int)(s_new >= (uint32_t)(8 * (i + 1))) - (int)(s_old >= (uint32_t)(8 * (i + 1)));
+      }
+    };
+    const int n_exc = __builtin_amdgcn_readfirstlane(buf.exc_n);
+    if (n_exc <= cs->exc_cap) {
+      for (int e = tid; e < n_exc; e += HSW_NT) {
+        const uint4 en = e == tid ? buf.exc_first : cs->exc[e];
+        patch((int)en.x, en.z, en.y);
+      }
+    } else {  // the list overflowed: every column from the two-plane stream
+      for (int col = tid; col < n; col += HSW_NT) {
+        const uint2 c = cs->full[col];
+        if (c.y != cs->full_plane) patch(col, c.x, c.y);
+      }
+    }
+  } else {
+    // Two register buffers of HSW_BATCH chunks each: the next batch is requested before the current one is
+    // scored, so the memory pipe stays busy while the ALUs work.
+    auto score = [&](uint4 (&ra)[HSW_BATCH], uint4 (&rb)[HSW_BATCH], int c0) {
+#pragma unroll
+      for (int u = 0; u < HSW_BATCH; ++u) {
+        sah_keep(ra[u].x); sah_keep(ra[u].y); sah_keep(ra[u].z); sah_keep(ra[u].w);
+        sah_keep(rb[u].x); sah_keep(rb[u].y); sah_keep(rb[u].z); sah_keep(rb[u].w);
+      }
+#pragma unroll
+      for (int u = 0; u < HSW_BATCH; ++u) {
+        if (c0 + u >= my_c1) break;
+        const int wi = (c0 + u) * SAH_WAVE + lane;
+        const int j0 = wi * 4;
+        uint32_t word;
+        if (j0 + 4 <= n) {
+          const uint32_t s0 = (uint32_t)(sig_score(q, make_uint2(ra[u].x, ra[u].y)) + 33);
+          const uint32_t s1 = (uint32_t)(sig_score(q, make_uint2(ra[u].z, ra[u].w)) + 33);
+          const uint32_t s2 = (uint32_t)(sig_score(q, make_uint2(rb[u].x, rb[u].y)) + 33);
+          const uint32_t s3 = (uint32_t)(sig_score(q, make_uint2(rb[u].z, rb[u].w)) + 33);
+          word = s0 | (s1 << 8) | (s2 << 16) | (s3 << 24);
+        } else {
+          word = 0;  // ragged tail: the few columns of the last, partial group
+          for (int t = 0; t < 4; ++t)
+            if (j0 + t < n) word |= (uint32_t)(sig_score(q, kc[j0 + t]) + 33) << (8 * t);
+        }
+        stage(word, wi);
+      }
+    };
+    if (!prefetched && my_c0 < my_c1) hsw_request(kc, n, lane, buf.a0, buf.a1, my_c0);
+    for (int c0 = my_c0; c0 < my_c1; c0 += 2 * HSW_BATCH) {
+      const bool more_b = c0 + HSW_BATCH < my_c1;          // uniform across the wave
+      if (more_b && !(prefetched && c0 == my_c0)) hsw_request(kc, n, lane, buf.b0, buf.b1, c0 + HSW_BATCH);
+      score(buf.a0, buf.a1, c0);
+      if (c0 + 2 * HSW_BATCH < my_c1) hsw_request(kc, n, lane, buf.a0, buf.a1, c0 + 2 * HSW_BATCH);
+      if (more_b) score(buf.b0, buf.b1, c0 + HSW_BATCH);
+    }
+  }
+  // Wave totals, two counters to a register as signed 16-bit fields: a wave stages at most 64 * 4 * 35 columns,
+  // and the corrections a wave's lanes made (to columns anywhere in the row) can take its total a little below
+  // zero; only the workgroup's totals are counts.
+#pragma unroll
+  for (int i = 0; i < HSW_PROBES; i += 2) {
+    const int t = sah_wave_sum_i((int)((uint32_t)pc[i] + ((uint32_t)pc[i + 1] << 16)));
+    const int lo = (int)(int16_t)(t & 0xFFFF);
+    if (lane == 0) {
+      S.probe[wave][i] = lo;
+      S.probe[wave][i + 1] = (t - lo) >> 16;
+    }
   }
   __syncthreads();
 
@@ -187,9 +309,12 @@ __device__ __forceinline__ int hsw_select_row(const sah_rows& R, int r, const ui
     for (int j = 0; j < 7; ++j) fc[j] += __popc((x - (base + 1u + j) * 0x01010101u) & 0x80808080u);
   }
 #pragma unroll
-  for (int j = 0; j < 7; ++j) {
-    const int t = sah_wave_sum_i(fc[j]);
-    if (lane == 0) S.fine[wave][j] = t;
+  for (int j = 0; j < 7; j += 2) {
+    const uint32_t t = (uint32_t)sah_wave_sum_i(fc[j] + ((j + 1 < 7 ? fc[j + 1] : 0) << 16));
+    if (lane == 0) {
+      S.fine[wave][j] = (int)(t & 0xFFFFu);
+      if (j + 1 < 7) S.fine[wave][j + 1] = (int)(t >> 16);
+    }
   }
   __syncthreads();
   int ftot = 0;
@@ -234,8 +359,9 @@ __device__ __forceinline__ int hsw_select_row(const sah_rows& R, int r, const ui
       me0 = m_eq;
     }
   }
-  const int n_gt = sah_wave_sum_i(lane_gt);
-  const int n_eq = sah_wave_sum_i(lane_eq);
+  const uint32_t n_both = (uint32_t)sah_wave_sum_i(lane_gt + (lane_eq << 16));
+  const int n_gt = (int)(n_both & 0xFFFFu);
+  const int n_eq = (int)(n_both >> 16);
   if (lane == 0) {
     s_gt[wave] = n_gt;
     s_eq[wave] = n_eq;

@@ -37,6 +37,7 @@ EXPECTED_SYMBOLS = (
     "sah_hamming_scores",
     "sah_hash_decode_topk",
     "sah_hash_decode_attention",
+    "sah_hash_compact_codes",
     "sah_qk_scores",
     "sah_select_topk",
     "sah_pq_kmeans_assign",
@@ -280,6 +281,28 @@ class HashDecodeArgs(C.Structure):
         ("code_pitch", C.c_int64),
         ("k", C.c_int32),
         ("skip_bitmap", C.c_int32),
+        ("pos_codes", C.c_void_p),
+        ("pos_pitch", C.c_int64),
+        ("exc", C.c_void_p),
+        ("exc_cnt", C.c_void_p),
+        ("exc_cap", C.c_int32),
+        ("full_plane", C.c_uint32),
+        ("stream", C.c_void_p),
+    ]
+
+
+class HashCompactArgs(C.Structure):
+    _fields_ = [
+        ("codes", C.c_void_p),
+        ("code_pitch", C.c_int64),
+        ("n_rows", C.c_int32),
+        ("from_", C.c_int32), ("to", C.c_int32),
+        ("pos_codes", C.c_void_p),
+        ("pos_pitch", C.c_int64),
+        ("exc", C.c_void_p),
+        ("exc_cap", C.c_int32),
+        ("exc_cnt", C.c_void_p),
+        ("full_plane", C.c_uint32),
         ("stream", C.c_void_p),
     ]
 
@@ -296,6 +319,7 @@ class ChainArgs(C.Structure):
         ("pq_adc", C.c_void_p),
         ("select", C.c_void_p),
         ("attention", C.c_void_p),
+        ("compact", C.c_void_p),
     ]
 
 

@@ -32,6 +32,7 @@ from .maskers.fixed.implementations.oracle_top_k import OracleTopK
 from .maskers.fixed.implementations.pq_top_k import PQCache, PQCodebook, adc_lut_buffer
 
 _MAX_NEW_KEYS = 64  # more than this many unseen keys => not a decode step, take the general path
+_COMPACT_CODES = True  # HashAttention decode: the kernel scans 4-byte sign planes + an exception list instead of 8-byte codes
 _HASH_BLOCK = 64    # HashAttention decode: new keys are hashed this many at a time (never more than the local window)
 
 
@@ -86,6 +87,7 @@ class DecodePlan:
         self.sink_local = N.SinkLocalArgs()
         self.hamming = N.HammingTopkArgs()
         self.hash_decode = N.HashDecodeArgs()
+        self.compact = N.HashCompactArgs()
         self.qk = N.QkScoresArgs()
         self.pq_assign = N.PqAssignArgs()
         self.pq_adc = N.PqAdcArgs()
@@ -151,7 +153,7 @@ class DecodePlan:
         sl.rows, sl.lq, sl.sink, sl.window, sl.fresh, sl.clear_future, sl.stream = rows, Lq, sink, window, 1, 1, stream
         chain.sink_local = C.addressof(sl)
         chain.sig_a = chain.sig_b = chain.hamming = chain.qk = chain.pq_assign = chain.pq_adc = chain.select = None
-        chain.hash_decode = None
+        chain.hash_decode = chain.compact = None
 
         if self.kind == "hash":
             cache = sparse_meta_data.get("key", {}).get(layer_idx)
@@ -193,13 +195,32 @@ class DecodePlan:
                 hd = self.hash_decode
                 hd.rows, hd.sink, hd.window = rows, sink, window
                 hd.query_sig = chain.sig_b
-                hd.key_sig = chain.sig_a if n_new == 1 else None
+                use_compact = _COMPACT_CODES
+                hd.key_sig = chain.sig_a if n_new == 1 and not use_compact else None
+                hd.pos_codes = hd.exc = hd.exc_cnt = None
+                if use_compact:
+                    # keys hashed since the compact form was last brought up to date (by this step's launch in
+                    # front of the kernel, by the first call of the layer, by the general path) are added to it
+                    cache.ensure_compact_buffers()
+                    hashed = Lk if hash_now else cache.n
+                    if hashed > cache.n_compact:
+                        cp = self.compact
+                        cp.codes, cp.code_pitch, cp.n_rows = cache.codes.data_ptr(), cache.capacity, self.n_rows
+                        cp.from_, cp.to = cache.n_compact, hashed
+                        cp.pos_codes, cp.pos_pitch = cache.pos.data_ptr(), cache.pos.shape[2]
+                        cp.exc, cp.exc_cap, cp.exc_cnt = cache.exc.data_ptr(), cache.exc.shape[2], cache.exc_cnt.data_ptr()
+                        cp.full_plane, cp.stream = cache.full_plane, stream
+                        chain.compact = C.addressof(cp)
+                        cache.n_compact = hashed
+                    hd.pos_codes, hd.pos_pitch = cache.pos.data_ptr(), cache.pos.shape[2]
+                    hd.exc, hd.exc_cap, hd.exc_cnt = cache.exc.data_ptr(), cache.exc.shape[2], cache.exc_cnt.data_ptr()
+                    hd.full_plane = cache.full_plane
                 hd.kcodes, hd.code_pitch, hd.k, hd.stream = cache.codes.data_ptr(), cache.capacity, k_eff, stream
                 hd.skip_bitmap = 1  # only the attention kernel reads these rows, and it reads the column lists
                 chain.hash_decode = C.addressof(hd)
                 chain.sink_local = chain.sig_b = None
-                if n_new == 1:
-                    chain.sig_a = None
+                if hd.key_sig is not None:
+                    chain.sig_a = None  # hashed inside the kernel
             else:
                 hm = self.hamming
                 hm.rows, hm.kcodes, hm.code_pitch = rows, cache.codes.data_ptr(), cache.capacity

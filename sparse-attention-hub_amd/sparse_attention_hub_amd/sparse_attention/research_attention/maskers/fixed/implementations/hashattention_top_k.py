@@ -56,6 +56,10 @@ class PackedSignatureCache:
         self.n = 0
         capacity = (capacity + 63) // 64 * 64  # rows of codes stay 16-byte aligned for the vector loads
         self.codes = torch.empty((batch, heads, capacity, 2), dtype=torch.int32, device=device)
+        # compact form for the decode kernel (built on demand by `compact_upto`): sign planes [B, Hq, pos_pitch],
+        # columns with a zero component [B, Hq, exc_cap, 4] and their number [B, Hq]; valid for `n_compact` keys
+        self.pos = self.exc = self.exc_cnt = None
+        self.n_compact = 0
 
     @property
     def capacity(self) -> int:
@@ -73,6 +77,25 @@ class PackedSignatureCache:
         if self.n:
             grown[:, :, : self.n] = self.codes[:, :, : self.n]
         self.codes = grown
+        self.pos = self.exc = self.exc_cnt = None  # rebuilt from the codes at the next decode step
+        self.n_compact = 0
+
+    @property
+    def full_plane(self) -> int:
+        return (1 << self.bits) - 1
+
+    def ensure_compact_buffers(self) -> None:
+        """Buffers of the compact form, sized for the current capacity (8192 columns of slack for the
+        kernel's whole-chunk reads)."""
+        if self.pos is not None:
+            return
+        B, H = self.codes.shape[0], self.codes.shape[1]
+        dev = self.codes.device
+        pitch = self.capacity + 8192
+        self.pos = torch.zeros((B, H, pitch), dtype=torch.int32, device=dev)
+        self.exc = torch.empty((B, H, max(1024, self.capacity // 16), 4), dtype=torch.int32, device=dev)
+        self.exc_cnt = torch.zeros((B, H), dtype=torch.int32, device=dev)
+        self.n_compact = 0
 
     def unpack(self, dtype: torch.dtype = torch.float32) -> torch.Tensor:
         codes = self.codes[:, :, : self.n].to(torch.int64) & 0xFFFFFFFF

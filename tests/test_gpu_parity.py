@@ -427,6 +427,77 @@ def test_decode_plan_hashes_new_keys_in_blocks(cuda):
     assert torch.equal(c1.codes[:, :, : c1.n], c2.codes[:, :, : c1.n])
 
 
+def test_compact_code_stream_matches_two_plane_codes(cuda):
+    """sah_hash_compact_codes: sign planes copied, every column with a zero component listed exactly once with
+    both planes, counts right also beyond the list's capacity, ranges added in any order."""
+    from sparse_attention_hub_amd import _native as N
+
+    g = torch.Generator().manual_seed(5)
+    n_rows, n, pitch, cap = 6, 5000, 5056, 64
+    codes = torch.randint(-2**31, 2**31 - 1, (n_rows, pitch, 2), generator=g, dtype=torch.int64).to(torch.int32)
+    zero = torch.rand((n_rows, pitch), generator=g) < torch.tensor([0.0, 0.001, 0.01, 0.01, 0.5, 1.0]).view(-1, 1)
+    codes[..., 1] = torch.where(zero, codes[..., 1] & 0x7FFEFFFF, torch.full_like(codes[..., 1], -1))
+    codes[..., 0] &= codes[..., 1]
+    dc = codes.to(cuda)
+    pos = torch.zeros((n_rows, pitch + 8192), dtype=torch.int32, device=cuda)
+    exc = torch.zeros((n_rows, cap, 4), dtype=torch.int32, device=cuda)
+    cnt = torch.zeros((n_rows,), dtype=torch.int32, device=cuda)
+    for lo, hi in [(1000, 3000), (0, 1000), (3000, 3000), (3000, n)]:
+        N.call("sah_hash_compact_codes", N.HashCompactArgs(dc.data_ptr(), pitch, n_rows, lo, hi, pos.data_ptr(), pos.shape[1],
+                                                            exc.data_ptr(), cap, cnt.data_ptr(), 0xFFFFFFFF, N.stream_ptr(cuda)))
+    assert torch.equal(pos[:, :n].cpu(), codes[:, :n, 0])
+    assert not bool(pos[:, n:].any())
+    want = [torch.nonzero(codes[r, :n, 1] != -1).flatten() for r in range(n_rows)]
+    assert cnt.cpu().tolist() == [len(w) for w in want]
+    e = exc.cpu()
+    for r in range(n_rows):
+        m = min(len(want[r]), cap)
+        cols = e[r, :m, 0].long()
+        assert len(set(cols.tolist())) == m and set(cols.tolist()) <= set(want[r].tolist())
+        if len(want[r]) <= cap:
+            assert sorted(cols.tolist()) == want[r].tolist()
+        assert torch.equal(e[r, :m, 1], codes[r, cols, 1]) and torch.equal(e[r, :m, 2], codes[r, cols, 0])
+
+
+@pytest.mark.parametrize("Lk,zero_key_bits,B", [(900, [5], 8), (2300, [0, 31], 8), (2300, [0, 31], 1), (1500, [], 8)])
+def test_compact_codes_with_many_zero_components(cuda, Lk, zero_key_bits, B):
+    """The decode kernel on the compact code stream when the exception list is long (a key bit that is zero for
+    every key: all columns listed) or overflows (more than its 1024 entries: every column re-scored from the
+    two-plane codes), with zero query components as well: outputs equal the masker-by-masker path's. B = 1: the
+    selection kernel without the attention half."""
+    sa = _sa()
+    dtype = torch.bfloat16
+    Hq, Hkv, D = 32, 8, 128
+    wts = _hat(sa, Hq, D, dtype, hidden=128)
+    for e in zero_key_bits:
+        wts[0]["key_matrix"][-1][..., e] = 0
+        wts[0]["key_bias"][-1][..., e] = 0
+    wts[0]["query_matrix"][-1][..., 9] = 0
+    wts[0]["query_bias"][-1][..., 9] = 0
+    q, k, v = make_qkv(B, Hq, Hkv, 1, Lk + 3, D, dtype, outliers=True, seed=31)
+    cfgs = [sa.SinkMaskerConfig(sink_size=16), sa.LocalMaskerConfig(window_size=64),
+            sa.HashAttentionTopKMaskerConfig(heavy_size=200, hat_bits=32, hat_mlp_layers=3, hat_mlp_hidden_size=128,
+                                             hat_mlp_activation="silu", hat_weights=wts)]
+    fast = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=cfgs))
+    fast.return_attention_weights = False
+    ref = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=cfgs))
+    m1, m2 = {}, {}
+    kc, vc = k.to(cuda), v.to(cuda)
+    for step in range(3):
+        n = Lk + step
+        qq = make_qkv(B, Hq, Hkv, 1, 1, D, dtype, seed=350 + step)[0].to(cuda)
+        o1, _ = fast.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m1, layer_idx=0)
+        o2, _ = ref.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m2, layer_idx=0)
+        assert torch.equal(o1, o2), f"step {step}"
+    cache = m1["key"][0]
+    assert cache.n_compact == Lk and cache.exc.shape[2] == 1024
+    listed = cache.exc_cnt.cpu()
+    if zero_key_bits:
+        assert bool((listed == Lk).all())            # every key has a zero component: listed, or overflowed
+    else:
+        assert 0 < int(listed.max()) < 200           # bf16 outputs that round to exactly zero: a few per row
+
+
 def test_oracle_topk_full_size_properties(cuda):
     """Config 2 at its full shape (B = 4, 32 query / 8 KV heads, 32768 keys, top 5 % = 1638, bf16), checked
     through properties that need no CPU restatement of 128 x 32768 scores: every row holds sink + local +
@@ -471,24 +542,26 @@ def test_oracle_topk_full_size_properties(cuda):
     assert bool(torch.isfinite(out.float()).all())
 
 
-def _set_hash_block(monkeypatch, block):
-    """New keys per bulk hashing launch of the decode plan; 1 = the newest key is hashed inside every step's kernel."""
+def _set_hash_block(monkeypatch, block, compact=None):
+    """New keys per bulk hashing launch of the decode plan (1 = the newest key is hashed inside every step's
+    kernel) and whether the kernel scans the compact code stream (default: whenever keys are hashed in blocks)."""
     import importlib
 
     plan_mod = importlib.import_module("sparse_attention_hub_amd.sparse_attention.research_attention.decode_plan")
     monkeypatch.setattr(plan_mod, "_HASH_BLOCK", block)
+    monkeypatch.setattr(plan_mod, "_COMPACT_CODES", block != 1 if compact is None else compact)
 
 
-@pytest.mark.parametrize("block", [1, 64])
+@pytest.mark.parametrize("block,compact", [(1, False), (64, True), (64, False), (1, True)])
 @pytest.mark.parametrize("dtype,Lk", [(torch.bfloat16, 32768), (torch.float16, 5000), (torch.float32, 3001)])
-def test_fused_hash_decode_kernel_matches_separate_launches(cuda, monkeypatch, dtype, Lk, block):
+def test_fused_hash_decode_kernel_matches_separate_launches(cuda, monkeypatch, dtype, Lk, block, compact):
     """Sink + Local + HashAttention decode steps through the single fused kernel (sink/local rows, both signature
     MLPs, signature top-k) against the masker-by-masker path: same outputs, same signature cache, bit for bit,
     at the headline shape (32 query heads, 8 KV heads, 32768 keys, top-2048) and at ragged sizes."""
     from sparse_attention_hub_amd import _native as N
 
     sa = _sa()
-    _set_hash_block(monkeypatch, block)
+    _set_hash_block(monkeypatch, block, compact)
     # 256 rows at the ragged size: enough for the one-workgroup-per-row attention, so that selection and
     # attention run as ONE kernel; 64 rows at the headline length: attention in its split form, two more launches
     B, Hq, Hkv, D = (8 if Lk <= 8192 else 2), 32, 8, 128
@@ -512,6 +585,8 @@ def test_fused_hash_decode_kernel_matches_separate_launches(cuda, monkeypatch, d
             torch.cuda.synchronize()
             names = set(N.timing_collect())
             N.timing_enable(False)
+            if block == 1 and compact:   # the new key is hashed and added to the compact stream by launches of their own
+                names -= {"k_hash_compact", "k_hash_sig_small_mfma", "k_hash_sig_gemv"}
             if B * Hq >= 192:
                 assert names == {"k_hash_decode_attn"}, names   # the whole step, attention included, is one kernel
             else:
@@ -690,7 +765,7 @@ def test_single_kernel_decode_step_head_dim_64(cuda, monkeypatch, block):
             torch.cuda.synchronize()
             names = set(N.timing_collect())
             N.timing_enable(False)
-            assert names == {"k_hash_decode_attn"}, names
+            assert names - {"k_hash_compact"} == {"k_hash_decode_attn"}, names   # first plan step: the compact stream is built
         o2, w2 = ref.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m2, layer_idx=0)
         assert torch.equal(o1, o2), f"step {step}"
         hashed = m1["key"][0].n
