@@ -116,6 +116,7 @@ __device__ __forceinline__ int hdec_row(const hdec_params& P, int r, hsw_lds& S,
                                                       P.job[0].n_layers, s_sig[job], prefetch);
   }
   const uint2 q = s_sig[0].code[0];
+  hsw_lds_init(S);
   __syncthreads();  // every thread holds q (and the bitmap is complete) before the scores overwrite the scratch
 
   // ---- 3. top-k over the remaining columns

@@ -40,9 +40,17 @@ __device__ __forceinline__ uint32_t swar_ge(uint32_t w, uint32_t t) {
 struct hsw_lds {
   int gt[HSW_NW];
   int eq[HSW_NW];
-  int probe[HSW_NW][HSW_PROBES];
-  int fine[HSW_NW][HSW_PROBES];
+  int probe[HSW_PROBES];  // workgroup totals of the coarse and of the fine counts: one LDS atomic per wave and
+  int fine[HSW_PROBES];   // counter, read back by everyone after the barrier; zeroed by hsw_lds_init
 };
+
+// Clears the counters of `S`. To be called by every thread before the barrier that precedes hsw_select_row.
+__device__ __forceinline__ void hsw_lds_init(hsw_lds& S) {
+  if (threadIdx.x < HSW_PROBES) {
+    S.probe[threadIdx.x] = 0;
+    S.fine[threadIdx.x] = 0;
+  }
+}
 
 // LDS words the row needs: bitmap (padded to whole chunks) and one byte per column
 __host__ __device__ inline size_t hsw_lds_bytes(int n_keys) {
@@ -134,8 +142,8 @@ __device__ __forceinline__ void hsw_prefetch(const hsw_compact& cs, int n, hsw_b
 }
 
 // Top-k of row r over the not-yet-active columns. On entry `s_bm` (n_ch * 8 words of dynamic LDS, zero
-// padded) holds the row's bitmap and every thread of the workgroup has passed a barrier after it was
-// written; cnt0 entries of R.cols are already in place. On exit the selected columns are appended (in no
+// padded) holds the row's bitmap, hsw_lds_init(S) has run, and every thread of the workgroup has passed a
+// barrier after both; cnt0 entries of R.cols are already in place. On exit the selected columns are appended (in no
 // particular order) and cnt is updated; with update_bitmap also the bitmap row (LDS copy and global).
 // Returns the row's new entry count (every thread). s_cols: optional LDS copy of the row's column list (cap entries):
 // the appended columns are mirrored there for a caller that goes on to use them in the same kernel (the mirror
@@ -283,8 +291,8 @@ __device__ __forceinline__ int hsw_select_row(const sah_rows& R, int r, const ui
     const int t = sah_wave_sum_i((int)((uint32_t)pc[i] + ((uint32_t)pc[i + 1] << 16)));
     const int lo = (int)(int16_t)(t & 0xFFFF);
     if (lane == 0) {
-      S.probe[wave][i] = lo;
-      S.probe[wave][i + 1] = (t - lo) >> 16;
+      atomicAdd(&S.probe[i], lo);
+      atomicAdd(&S.probe[i + 1], (t - lo) >> 16);
     }
   }
   __syncthreads();
@@ -292,11 +300,7 @@ __device__ __forceinline__ int hsw_select_row(const sah_rows& R, int r, const ui
   // ---- P1: largest T with count(key >= T) >= k --------------------------------
   // counts fall as the threshold rises, so the thresholds that still reach k form a prefix
   const int n_w = n_ch * SAH_WAVE;
-  int tot = 0;
-  if (lane < HSW_PROBES) {
-#pragma unroll
-    for (int wv = 0; wv < HSW_NW; ++wv) tot += S.probe[wv][lane];
-  }
+  const int tot = lane < HSW_PROBES ? S.probe[lane] : 0;
   const int n_pass = __popcll(__ballot(lane < HSW_PROBES && tot >= k));
   const uint32_t base = 8u * (uint32_t)n_pass;                         // T is in [base, base + 8)
   const int next_probe = n_pass < HSW_PROBES ? __shfl(tot, n_pass) : 0;  // count(key >= base + 8)
@@ -312,16 +316,12 @@ __device__ __forceinline__ int hsw_select_row(const sah_rows& R, int r, const ui
   for (int j = 0; j < 7; j += 2) {
     const uint32_t t = (uint32_t)sah_wave_sum_i(fc[j] + ((j + 1 < 7 ? fc[j + 1] : 0) << 16));
     if (lane == 0) {
-      S.fine[wave][j] = (int)(t & 0xFFFFu);
-      if (j + 1 < 7) S.fine[wave][j + 1] = (int)(t >> 16);
+      atomicAdd(&S.fine[j], (int)(t & 0xFFFFu));
+      if (j + 1 < 7) atomicAdd(&S.fine[j + 1], (int)(t >> 16));
     }
   }
   __syncthreads();
-  int ftot = 0;
-  if (lane < 7) {
-#pragma unroll
-    for (int wv = 0; wv < HSW_NW; ++wv) ftot += S.fine[wv][lane];
-  }
+  const int ftot = lane < 7 ? S.fine[lane] : 0;
   const int n_fine = __popcll(__ballot(lane < 7 && ftot >= k));
   const uint32_t T = base + (uint32_t)n_fine;
   const int above = n_fine < 7 ? __shfl(ftot, n_fine) : next_probe;      // count(key >= T + 1)

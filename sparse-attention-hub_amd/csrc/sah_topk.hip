@@ -381,6 +381,7 @@ __global__ __launch_bounds__(HSW_NT) void k_hamming_topk_swar(sah_rows R, const 
   int cnt0 = R.cnt[r];  // read before the first barrier: the row's last thread rewrites it at the end
   if (cnt0 > R.cap) cnt0 = R.cap;
   for (int i = tid; i < n_ch * 8; i += HSW_NT) s_bm[i] = i < R.n_words ? bm[i] : 0u;
+  hsw_lds_init(S);
   __syncthreads();
   hsw_bufs buf;
   hsw_select_row(R, r, kcodes + (int64_t)(r / lq) * pitch, qcodes[r], k, cnt0, s_bm, s_key, S, buf);
