@@ -553,7 +553,7 @@ def _set_hash_block(monkeypatch, block, compact=None):
 
 
 @pytest.mark.parametrize("block,compact", [(1, False), (64, True), (64, False), (1, True)])
-@pytest.mark.parametrize("dtype,Lk", [(torch.bfloat16, 32768), (torch.float16, 5000), (torch.float32, 3001)])
+@pytest.mark.parametrize("dtype,Lk", [(torch.bfloat16, 32768), (torch.float16, 5000), (torch.float32, 3001), (torch.bfloat16, 70001)])
 def test_fused_hash_decode_kernel_matches_separate_launches(cuda, monkeypatch, dtype, Lk, block, compact):
     """Sink + Local + HashAttention decode steps through the single fused kernel (sink/local rows, both signature
     MLPs, signature top-k) against the masker-by-masker path: same outputs, same signature cache, bit for bit,
@@ -564,7 +564,7 @@ def test_fused_hash_decode_kernel_matches_separate_launches(cuda, monkeypatch, d
     _set_hash_block(monkeypatch, block, compact)
     # 256 rows at the ragged size: enough for the one-workgroup-per-row attention, so that selection and
     # attention run as ONE kernel; 64 rows at the headline length: attention in its split form, two more launches
-    B, Hq, Hkv, D = (8 if Lk <= 8192 else 2), 32, 8, 128
+    B, Hq, Hkv, D = (8 if Lk <= 8192 else 2 if Lk <= 32768 else 1), 32, 8, 128   # 70001 keys: 18 chunks per wave
     heavy = 2048 if Lk > 8192 else 300
     q, k, v = make_qkv(B, Hq, Hkv, 1, Lk + 3, D, dtype, seed=3)
     cfgs = [sa.SinkMaskerConfig(sink_size=128), sa.LocalMaskerConfig(window_size=512),
