@@ -76,14 +76,17 @@ __device__ __forceinline__ int hdec_row(const hdec_params& P, int r, hsw_lds& S,
   const int lo2 = lo > s_hi ? lo : s_hi;
   const int n_local = hi > lo2 ? hi - lo2 : 0;
   const int fixed = s_hi + n_local;
-  int* cols = R.cols + (int64_t)r * R.cap;
-  for (int i = tid; i < fixed && i < R.cap; i += HSW_NT) {
-    cols[i] = i < s_hi ? i : lo2 + (i - s_hi);
-    if (s_cols) s_cols[i] = i < s_hi ? i : lo2 + (i - s_hi);
-    if (R.w) R.w[(int64_t)r * R.cap + i] = 1.0f;
-  }
-  for (int wi = tid; wi < n_ch * 8; wi += HSW_NT)
-    s_bm[wi] = wi < R.n_words ? (sah_range_bits(wi, 0, s_hi) | sah_range_bits(wi, lo, hi)) : 0u;
+  // written while the loads requested below are on their way
+  auto fixed_part = [&]() {
+    int* cols = R.cols + (int64_t)r * R.cap;
+    for (int i = tid; i < fixed && i < R.cap; i += HSW_NT) {
+      cols[i] = i < s_hi ? i : lo2 + (i - s_hi);
+      if (s_cols) s_cols[i] = i < s_hi ? i : lo2 + (i - s_hi);
+      if (R.w) R.w[(int64_t)r * R.cap + i] = 1.0f;
+    }
+    for (int wi = tid; wi < n_ch * 8; wi += HSW_NT)
+      s_bm[wi] = wi < R.n_words ? (sah_range_bits(wi, 0, s_hi) | sah_range_bits(wi, lo, hi)) : 0u;
+  };
 
   // ---- 2. signatures of the query and of the newest key
   // uniform across the wave, and known to be: the job's parameters are then fetched by scalar loads
@@ -105,9 +108,17 @@ __device__ __forceinline__ int hdec_row(const hdec_params& P, int r, hsw_lds& S,
     cs.exc_cap = P.exc_cap;
     cs.full_plane = P.full_plane;
   }
+  // Compact stream with the matrix-core MLP: the waves that run the query's MLP (0-7) request their codes only
+  // after it, so that no queue of code requests stands between them and their weights (issuing 8 more loads
+  // per lane into the full memory pipe held their first layer up for 8K cycles); the idle half of the
+  // workgroup requests its codes at once and scores them while the first half's are on their way.
+  const bool early = !(MF && CP) || job != 0;
   auto prefetch = [&]() {
-    if constexpr (CP) hsw_prefetch(cs, n, buf);
-    else hsw_prefetch(kc, n, buf);
+    if (early) {
+      if constexpr (CP) hsw_prefetch(cs, n, buf);
+      else hsw_prefetch(kc, n, buf);
+    }
+    fixed_part();
   };
   if constexpr (MF) {
     sig_mfma_block<DT>(P.job[job], active, tid % HDEC_GROUP, r / Hq, r % Hq, 0, 1, P.job[0].n_layers, s_sig[job], prefetch);
@@ -120,7 +131,7 @@ __device__ __forceinline__ int hdec_row(const hdec_params& P, int r, hsw_lds& S,
   __syncthreads();  // every thread holds q (and the bitmap is complete) before the scores overwrite the scratch
 
   // ---- 3. top-k over the remaining columns
-  return hsw_select_row<CP>(R, r, kc, q, P.k, fixed < R.cap ? fixed : R.cap, s_bm, s_key, S, buf, true, P.update_bitmap != 0,
+  return hsw_select_row<CP>(R, r, kc, q, P.k, fixed < R.cap ? fixed : R.cap, s_bm, s_key, S, buf, early, P.update_bitmap != 0,
                             s_cols, CP ? &cs : nullptr);
 }
 
