@@ -498,6 +498,56 @@ def test_compact_codes_with_many_zero_components(cuda, Lk, zero_key_bits, B):
         assert 0 < int(listed.max()) < 200           # bf16 outputs that round to exactly zero: a few per row
 
 
+def test_hash_decode_plan_state_transitions(cuda):
+    """The HashAttention decode plan keeps state between steps (keys hashed so far, the compact copy of the codes).
+    Every transition that touches it: plan steps with unhashed keys pending, then a call that takes the
+    masker-by-masker path (it must hash what is missing), back to the plan (the compact copy catches up), a cache
+    that is reallocated (the compact copy is rebuilt), two layers interleaved. Outputs always equal those of a
+    second instance that never uses the plan."""
+    sa = _sa()
+    dtype = torch.bfloat16
+    B, Hq, Hkv, Lk, D = 8, 32, 8, 1200, 128
+    steps = 30
+    q, k, v = make_qkv(B, Hq, Hkv, 1, Lk + steps, D, dtype, outliers=True, seed=41)
+    wts = {0: _hat(sa, Hq, D, dtype, hidden=128, seed=1)[0], 1: _hat(sa, Hq, D, dtype, hidden=128, seed=2)[0]}
+    cfgs = [sa.SinkMaskerConfig(sink_size=8), sa.LocalMaskerConfig(window_size=8),
+            sa.HashAttentionTopKMaskerConfig(heavy_size=150, hat_bits=32, hat_mlp_layers=3, hat_mlp_hidden_size=128,
+                                             hat_mlp_activation="silu", hat_weights=wts)]
+    fast = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=cfgs))
+    ref = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=cfgs))
+    m1, m2 = {}, {}
+    kc, vc = k.to(cuda), v.to(cuda)
+    seen_lag = regrown = False
+    for step in range(steps):
+        n = Lk + step
+        general = step in (5, 6, 17)                     # these steps ask for the weights: masker-by-masker path
+        fast.return_attention_weights = general
+        for layer in (0, 1):
+            qq = make_qkv(B, Hq, Hkv, 1, 1, D, dtype, seed=450 + 2 * step + layer)[0].to(cuda)
+            o1, w1 = fast.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m1, layer_idx=layer)
+            o2, w2 = ref.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m2, layer_idx=layer)
+            assert torch.equal(o1, o2), f"step {step} layer {layer}"
+            assert (w1 is not None) == general
+            if general:
+                assert torch.equal(w1, w2)
+                assert m1["key"][layer].n == n           # the general path hashed the pending keys
+        cache = m1["key"][0]
+        seen_lag |= cache.n < n
+        if step == 11:                                   # force a reallocation of the code cache
+            cache.reserve(cache.capacity + 1)
+            assert cache.pos is None and cache.n_compact == 0
+            regrown = True
+        if step > 12 and not general:
+            assert cache.pos is not None and cache.n_compact == cache.n
+    assert seen_lag and regrown
+    for layer in (0, 1):
+        c1, c2 = m1["key"][layer], m2["key"][layer]
+        assert torch.equal(c1.codes[:, :, : c1.n], c2.codes[:, :, : c1.n])
+        assert torch.equal(c1.pos[:, :, : c1.n_compact], c1.codes[:, :, : c1.n_compact, 0])
+        zeros = (c1.codes[:, :, : c1.n_compact, 1] != -1).sum(-1)
+        assert torch.equal(zeros.to(torch.int32), c1.exc_cnt)
+
+
 def test_oracle_topk_full_size_properties(cuda):
     """Config 2 at its full shape (B = 4, 32 query / 8 KV heads, 32768 keys, top 5 % = 1638, bf16), checked
     through properties that need no CPU restatement of 128 x 32768 scores: every row holds sink + local +
