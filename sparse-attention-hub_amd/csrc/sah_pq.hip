@@ -380,9 +380,10 @@ struct pq_adc_params {
 };
 
 #define ADC_MAX_LUT 4096  // n_sub * n_cent
-#define ADC_KEYS 2048     // candidates per workgroup of the scoring kernel
+#define ADC_NT 1024       // threads of the scoring kernel
+#define ADC_KEYS 4096     // candidates per workgroup of the scoring kernel
 #define ADC_MAX_HEAD_DIM 512  // widest query vector a workgroup stages in LDS when it builds its own table
-#define ADC_OWN_LUT_WGS 32 // up to this many workgroups per KV head each build the lookup table themselves
+#define ADC_OWN_LUT_WGS 16 // up to this many workgroups per KV head each build the lookup table themselves
 
 // Lookup table of one decode step: lut[bh][vg][s][c][i] = round(q_v . centre[bh][s][c]) for the NQ query vectors
 // v = vg * NQ + i of the KV head's group, in the storage type (fp32: NQ = 2, 16-bit: NQ = 4, i.e. 8 bytes per
@@ -447,15 +448,17 @@ __global__ __launch_bounds__(PQ_NT) void k_pq_lut(pq_adc_params P, void* lut) {
   }
 }
 
-// Scores of ADC_KEYS candidates for the NQ query vectors of one group: the table slab (8 bytes per (s, c))
-// in LDS, one thread per candidate, the candidate's codes as 4-byte words. OWN_LUT: the workgroup computes
-// its slab itself (every workgroup of a KV head repeats that work, which is cheaper than a launch of its own
-// as long as a head is covered by a few dozen workgroups).
+// Scores of ADC_KEYS candidates for the NQ query vectors of one group: one 16-wave workgroup, the table in LDS
+// as fp32 (NQ floats per (s, c): one LDS read serves all the query vectors, and a lookup costs the read and NQ
+// adds, no unpacking), one thread per candidate. OWN_LUT: the workgroup computes its table itself (every
+// workgroup of a KV head repeats that work, which is cheaper than a launch of its own as long as a head is
+// covered by a few dozen workgroups); otherwise the 8-byte entries k_pq_lut wrote are widened on the way in.
 template <int DT, bool OWN_LUT>
-__global__ __launch_bounds__(PQ_NT) void k_pq_adc(pq_adc_params P, const void* lut) {
+__global__ __launch_bounds__(ADC_NT) void k_pq_adc(pq_adc_params P, const void* lut) {
   constexpr int NQ = (DT == SAH_F32) ? 2 : 4;
   typedef typename std::conditional<DT == SAH_F32, uint32_t, uint16_t>::type key_t;
-  __shared__ uint2 s_lut[ADC_MAX_LUT];
+  typedef typename std::conditional<DT == SAH_F32, float2, float4>::type entry_t;
+  HIP_DYNAMIC_SHARED(unsigned char, adc_dyn)
   const int tid = threadIdx.x;
   const int bh = blockIdx.y;
   const int vg = blockIdx.z;
@@ -466,6 +469,8 @@ __global__ __launch_bounds__(PQ_NT) void k_pq_adc(pq_adc_params P, const void* l
   const int n_vg = (nvec + NQ - 1) / NQ;
   const int n_sub = P.n_sub, n_cent = P.n_cent;
   const int lut_n = n_sub * n_cent;
+  entry_t* s_lut = (entry_t*)adc_dyn;                      // lut_n entries
+  float* s_q = (float*)(adc_dyn + (size_t)lut_n * sizeof(entry_t));  // NQ x ADC_MAX_HEAD_DIM (OWN_LUT only)
 
   int row[NQ];
 #pragma unroll
@@ -474,13 +479,29 @@ __global__ __launch_bounds__(PQ_NT) void k_pq_adc(pq_adc_params P, const void* l
     row[i] = -1;
     if (v < nvec) row[i] = (b * P.Hq + hk * G + v / P.Lq) * P.Lq + v % P.Lq;
   }
+  auto store_entry = [&](int i, const float (&val)[NQ]) {  // rounded to the storage type, kept as floats
+    if constexpr (NQ == 2) s_lut[i] = make_float2(sah_round<DT>(val[0]), sah_round<DT>(val[1]));
+    else s_lut[i] = make_float4(sah_round<DT>(val[0]), sah_round<DT>(val[1]), sah_round<DT>(val[2]), sah_round<DT>(val[3]));
+  };
+  // 16 one-byte codes per candidate = one 16-byte load: all of the thread's candidates are requested before
+  // anything else and arrive while the table is built
+  constexpr int T = ADC_KEYS / ADC_NT;
+  const bool wide = n_sub == 16 && ((uintptr_t)P.codes & 15) == 0;
+  uint4 cw[T];
+  if (wide) {
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      int n = blockIdx.x * ADC_KEYS + t * ADC_NT + tid;
+      if (n >= P.n_cand) n = P.n_cand - 1;
+      cw[t] = *(const uint4*)(P.codes + ((int64_t)bh * P.code_pitch + n) * 16);
+    }
+  }
   if (OWN_LUT) {
-    // the group's query vectors once into LDS (as floats), then every thread builds lut_n / PQ_NT entries
+    // the group's query vectors once into LDS (as floats), then every thread builds lut_n / ADC_NT entries
     // from one centre each: the centre's d_sub floats from memory, the query elements as LDS broadcasts
-    __shared__ __attribute__((aligned(16))) float s_q[NQ][ADC_MAX_HEAD_DIM];
     const int d_sub = P.d_sub;
     const int D = n_sub * d_sub;
-    for (int i = tid; i < NQ * D; i += PQ_NT) {
+    for (int i = tid; i < NQ * D; i += ADC_NT) {
       const int qn = i / D, e = i % D;
       const int v = vg * NQ + qn;
       float x = 0.f;
@@ -488,10 +509,10 @@ __global__ __launch_bounds__(PQ_NT) void k_pq_adc(pq_adc_params P, const void* l
         const int h = hk * G + v / P.Lq, qi = v % P.Lq;
         x = sah_load<DT>(P.q, (int64_t)b * P.qs_b + (int64_t)h * P.qs_h + (int64_t)qi * P.qs_l + e);
       }
-      s_q[qn][e] = x;
+      s_q[qn * ADC_MAX_HEAD_DIM + e] = x;
     }
     __syncthreads();
-    for (int i = tid; i < lut_n; i += PQ_NT) {
+    for (int i = tid; i < lut_n; i += ADC_NT) {
       const int s = i / n_cent, c = i % n_cent;
       const float* cc = P.centres + (((int64_t)bh * n_sub + s) * n_cent + c) * d_sub;
       float acc[NQ];
@@ -503,7 +524,7 @@ __global__ __launch_bounds__(PQ_NT) void k_pq_adc(pq_adc_params P, const void* l
           const float4 cv = *(const float4*)(cc + d);
 #pragma unroll
           for (int qn = 0; qn < NQ; ++qn) {
-            const float4 qv = *(const float4*)&s_q[qn][s * d_sub + d];
+            const float4 qv = *(const float4*)&s_q[qn * ADC_MAX_HEAD_DIM + s * d_sub + d];
             acc[qn] = fmaf(qv.x, cv.x, acc[qn]);
             acc[qn] = fmaf(qv.y, cv.y, acc[qn]);
             acc[qn] = fmaf(qv.z, cv.z, acc[qn]);
@@ -514,92 +535,72 @@ __global__ __launch_bounds__(PQ_NT) void k_pq_adc(pq_adc_params P, const void* l
         for (int d = 0; d < d_sub; ++d) {
           const float cv = cc[d];
 #pragma unroll
-          for (int qn = 0; qn < NQ; ++qn) acc[qn] = fmaf(s_q[qn][s * d_sub + d], cv, acc[qn]);
+          for (int qn = 0; qn < NQ; ++qn) acc[qn] = fmaf(s_q[qn * ADC_MAX_HEAD_DIM + s * d_sub + d], cv, acc[qn]);
         }
       }
-      s_lut[i] = pq_pack_entry<DT>(acc);
+      store_entry(i, acc);
     }
   } else {
     const uint2* slab = (const uint2*)lut + ((int64_t)bh * n_vg + vg) * lut_n;
-    for (int i = tid; i < lut_n; i += PQ_NT) s_lut[i] = slab[i];
+    for (int i = tid; i < lut_n; i += ADC_NT) {
+      const uint2 e = slab[i];
+      float val[NQ];
+      if (DT == SAH_F32) {
+        val[0] = sah_bits_to_float(e.x);
+        val[1] = sah_bits_to_float(e.y);
+      } else if (DT == SAH_BF16) {
+        val[0] = sah_bits_to_float(e.x << 16);
+        val[1] = sah_bits_to_float(e.x & 0xffff0000u);
+        val[NQ > 2 ? 2 : 0] = sah_bits_to_float(e.y << 16);
+        val[NQ > 2 ? 3 : 1] = sah_bits_to_float(e.y & 0xffff0000u);
+      } else {
+        val[0] = sah_f16_to_float((uint16_t)(e.x & 0xffffu));
+        val[1] = sah_f16_to_float((uint16_t)(e.x >> 16));
+        val[NQ > 2 ? 2 : 0] = sah_f16_to_float((uint16_t)(e.y & 0xffffu));
+        val[NQ > 2 ? 3 : 1] = sah_f16_to_float((uint16_t)(e.y >> 16));
+      }
+      store_entry(i, val);
+    }
   }
   __syncthreads();
 
-  const bool words = (n_sub & 3) == 0 && ((P.code_pitch * n_sub) & 3) == 0 && ((uintptr_t)P.codes & 3) == 0;
-  if (n_sub == 16 && ((uintptr_t)P.codes & 15) == 0) {
-    // 16 one-byte codes per candidate = one 16-byte load: all of the thread's candidates are requested
-    // before the first table lookup
-    constexpr int T = ADC_KEYS / PQ_NT;
-    uint4 cw[T];
-#pragma unroll
-    for (int t = 0; t < T; ++t) {
-      int n = blockIdx.x * ADC_KEYS + t * PQ_NT + tid;
-      if (n >= P.n_cand) n = P.n_cand - 1;
-      cw[t] = *(const uint4*)(P.codes + ((int64_t)bh * P.code_pitch + n) * 16);
+  float acc[NQ];
+  auto add = [&](int s, int c) {
+    const entry_t e = s_lut[s * n_cent + c];
+    acc[0] += e.x;
+    acc[1] += e.y;
+    if constexpr (NQ > 2) {
+      acc[2] += e.z;
+      acc[3] += e.w;
     }
+  };
+  auto store = [&](int n) {
+#pragma unroll
+    for (int i = 0; i < NQ; ++i) {
+      if (row[i] >= 0)
+        ((key_t*)P.keys_out)[(int64_t)row[i] * P.key_pitch + n] = (key_t)sah_sort_key<DT>(sah_round<DT>(acc[i]));
+    }
+  };
+  if (wide) {
 #pragma unroll
     for (int t = 0; t < T; ++t) {
-      const int n = blockIdx.x * ADC_KEYS + t * PQ_NT + tid;
+      const int n = blockIdx.x * ADC_KEYS + t * ADC_NT + tid;
       const uint32_t w4[4] = {cw[t].x, cw[t].y, cw[t].z, cw[t].w};
-      float acc[NQ];
 #pragma unroll
       for (int i = 0; i < NQ; ++i) acc[i] = 0.f;
 #pragma unroll
-      for (int s = 0; s < 16; ++s) {
-        const uint2 e = s_lut[s * n_cent + (int)((w4[s >> 2] >> (8 * (s & 3))) & 0xffu)];
-        if (DT == SAH_F32) {
-          acc[0] += sah_bits_to_float(e.x);
-          acc[1] += sah_bits_to_float(e.y);
-        } else if (DT == SAH_BF16) {
-          acc[0] += sah_bits_to_float(e.x << 16);
-          acc[1] += sah_bits_to_float(e.x & 0xffff0000u);
-          acc[NQ > 2 ? 2 : 0] += sah_bits_to_float(e.y << 16);
-          acc[NQ > 2 ? 3 : 1] += sah_bits_to_float(e.y & 0xffff0000u);
-        } else {
-          acc[0] += sah_f16_to_float((uint16_t)(e.x & 0xffffu));
-          acc[1] += sah_f16_to_float((uint16_t)(e.x >> 16));
-          acc[NQ > 2 ? 2 : 0] += sah_f16_to_float((uint16_t)(e.y & 0xffffu));
-          acc[NQ > 2 ? 3 : 1] += sah_f16_to_float((uint16_t)(e.y >> 16));
-        }
-      }
-      if (n < P.n_cand) {
-#pragma unroll
-        for (int i = 0; i < NQ; ++i) {
-          if (row[i] >= 0)
-            ((key_t*)P.keys_out)[(int64_t)row[i] * P.key_pitch + n] = (key_t)sah_sort_key<DT>(sah_round<DT>(acc[i]));
-        }
-      }
+      for (int s = 0; s < 16; ++s) add(s, (int)((w4[s >> 2] >> (8 * (s & 3))) & 0xffu));
+      if (n < P.n_cand) store(n);
     }
     return;
   }
-  for (int t = 0; t < ADC_KEYS / PQ_NT; ++t) {
-    const int n = blockIdx.x * ADC_KEYS + t * PQ_NT + tid;
+  const bool words = (n_sub & 3) == 0 && ((P.code_pitch * n_sub) & 3) == 0 && ((uintptr_t)P.codes & 3) == 0;
+  for (int t = 0; t < T; ++t) {
+    const int n = blockIdx.x * ADC_KEYS + t * ADC_NT + tid;
     if (n >= P.n_cand) continue;
     const uint8_t* code = P.codes + ((int64_t)bh * P.code_pitch + n) * n_sub;
-    float acc[NQ];
 #pragma unroll
     for (int i = 0; i < NQ; ++i) acc[i] = 0.f;
-    auto add = [&](int s, int c) {
-      const uint2 e = s_lut[s * n_cent + c];
-      if (DT == SAH_F32) {
-        acc[0] += sah_bits_to_float(e.x);
-        acc[1] += sah_bits_to_float(e.y);
-      } else if (DT == SAH_BF16) {
-        acc[0] += sah_bits_to_float(e.x << 16);
-        acc[1] += sah_bits_to_float(e.x & 0xffff0000u);
-        if (NQ > 2) {
-          acc[2] += sah_bits_to_float(e.y << 16);
-          acc[3] += sah_bits_to_float(e.y & 0xffff0000u);
-        }
-      } else {
-        acc[0] += sah_f16_to_float((uint16_t)(e.x & 0xffffu));
-        acc[1] += sah_f16_to_float((uint16_t)(e.x >> 16));
-        if (NQ > 2) {
-          acc[2] += sah_f16_to_float((uint16_t)(e.y & 0xffffu));
-          acc[3] += sah_f16_to_float((uint16_t)(e.y >> 16));
-        }
-      }
-    };
     if (words) {
       for (int s4 = 0; s4 < n_sub; s4 += 4) {
         const uint32_t w = *(const uint32_t*)(code + s4);
@@ -611,12 +612,27 @@ __global__ __launch_bounds__(PQ_NT) void k_pq_adc(pq_adc_params P, const void* l
     } else {
       for (int s = 0; s < n_sub; ++s) add(s, (int)code[s]);
     }
-#pragma unroll
-    for (int i = 0; i < NQ; ++i) {
-      if (row[i] >= 0)
-        ((key_t*)P.keys_out)[(int64_t)row[i] * P.key_pitch + n] = (key_t)sah_sort_key<DT>(sah_round<DT>(acc[i]));
-    }
+    store(n);
   }
+}
+
+// dynamic LDS of k_pq_adc: the fp32 table and, for OWN_LUT, the staged query vectors
+template <int DT>
+static size_t adc_lds_bytes(int lut_n) {
+  constexpr int NQ = (DT == SAH_F32) ? 2 : 4;
+  return (size_t)lut_n * NQ * 4 + (size_t)NQ * ADC_MAX_HEAD_DIM * 4;
+}
+
+template <int DT, bool OWN_LUT>
+static int adc_launch(const pq_adc_params& P, const void* lut, dim3 g, hipStream_t st) {
+  static bool raised = false;
+  if (!raised) {
+    hipError_t e = hipFuncSetAttribute((const void*)k_pq_adc<DT, OWN_LUT>, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+    if (e != hipSuccess) return sah_fail((int)e, "sah_pq_adc_scores: cannot raise the LDS limit: %s", hipGetErrorString(e));
+    raised = true;
+  }
+  hipLaunchKernelGGL((k_pq_adc<DT, OWN_LUT>), g, dim3(ADC_NT), adc_lds_bytes<DT>(P.n_sub * P.n_cent), st, P, lut);
+  return SAH_OK;
 }
 
 static int pq_check_common(const char* what, int B, int Hkv, int n_sub, int d_sub, int n_cent) {
@@ -741,11 +757,12 @@ extern "C" int sah_pq_adc_scores(const sah_pq_adc_args* a) {
     // short contexts: no table in memory, no second launch
     sah_timed timed("k_pq_adc", a->stream);
     switch (a->dtype) {
-      case SAH_F32: hipLaunchKernelGGL((k_pq_adc<SAH_F32, true>), g, blk, 0, st, P, (const void*)nullptr); break;
-      case SAH_BF16: hipLaunchKernelGGL((k_pq_adc<SAH_BF16, true>), g, blk, 0, st, P, (const void*)nullptr); break;
-      case SAH_F16: hipLaunchKernelGGL((k_pq_adc<SAH_F16, true>), g, blk, 0, st, P, (const void*)nullptr); break;
+      case SAH_F32: rc = adc_launch<SAH_F32, true>(P, nullptr, g, st); break;
+      case SAH_BF16: rc = adc_launch<SAH_BF16, true>(P, nullptr, g, st); break;
+      case SAH_F16: rc = adc_launch<SAH_F16, true>(P, nullptr, g, st); break;
       default: return sah_fail(SAH_EDTYPE, "sah_pq_adc_scores: dtype %d", a->dtype);
     }
+    if (rc) return rc;
     return sah_launch_status("sah_pq_adc_scores");
   }
   const int64_t need = (int64_t)a->B * a->Hkv * n_vg * a->n_sub * a->n_cent * 8;
@@ -766,9 +783,10 @@ extern "C" int sah_pq_adc_scores(const sah_pq_adc_args* a) {
   }
   sah_timed timed("k_pq_adc", a->stream);
   switch (a->dtype) {
-    case SAH_F32: hipLaunchKernelGGL((k_pq_adc<SAH_F32, false>), g, blk, 0, st, P, (const void*)a->lut); break;
-    case SAH_BF16: hipLaunchKernelGGL((k_pq_adc<SAH_BF16, false>), g, blk, 0, st, P, (const void*)a->lut); break;
-    default: hipLaunchKernelGGL((k_pq_adc<SAH_F16, false>), g, blk, 0, st, P, (const void*)a->lut); break;
+    case SAH_F32: rc = adc_launch<SAH_F32, false>(P, a->lut, g, st); break;
+    case SAH_BF16: rc = adc_launch<SAH_BF16, false>(P, a->lut, g, st); break;
+    default: rc = adc_launch<SAH_F16, false>(P, a->lut, g, st); break;
   }
+  if (rc) return rc;
   return sah_launch_status("sah_pq_adc_scores");
 }
