@@ -315,7 +315,7 @@ __global__ __launch_bounds__(AD_NT) void k_adaptive_sample(ad_sample_params P) {
     if (changed) w[i] = wv;
   }
 
-  // new columns, ascending: every thread owns a contiguous run of bitmap words
+  // new columns: a wave owns a contiguous run of bitmap words. Counted per thread, positions from one block scan.
   const int wpt = (nw + AD_NT - 1) / AD_NT;
   const int wa = tid * wpt;
   int wb = wa + wpt;
@@ -323,23 +323,39 @@ __global__ __launch_bounds__(AD_NT) void k_adaptive_sample(ad_sample_params P) {
   int mine = 0;
   for (int wi = wa; wi < wb; ++wi) mine += __builtin_popcount(s_bits[wi] & ~gbits[w0 + wi]);
   int total = 0;
-  int pos = cnt0 + sah_block_excl_scan<AD_NT>(mine, s_scan, &total);
-  for (int wi = wa; wi < wb; ++wi) {
-    const uint32_t drawn = s_bits[wi];
-    if (!drawn) continue;
-    const uint32_t old = gbits[w0 + wi];
-    uint32_t fresh = drawn & ~old;
-    if (fresh) gbits[w0 + wi] = old | drawn;
-    while (fresh) {
-      const int bit = __builtin_ctz(fresh);
-      fresh &= fresh - 1;
-      if (pos < cap) {
-        cols[pos] = ((w0 + wi) << 5) + bit;
-        w[pos] = p;
+  const int pos = cnt0 + sah_block_excl_scan<AD_NT>(mine, s_scan, &total);
+  // Written wave by wave, 64 words at a time (lane i: word i of the group), one bit position after the other:
+  // the lanes that hold bit b of their word store to consecutive entries, so every store instruction fills
+  // whole cache lines. (A thread appending its own columns one after the other scatters each store over 64
+  // lines; a row whose budget is most of the range writes tens of thousands of columns.) The list is unordered.
+  const int lane = tid & (SAH_WAVE - 1);
+  int out = __builtin_amdgcn_readfirstlane(pos);  // the wave's first entry
+  const int wave_w0 = (tid - lane) * wpt;
+  for (int g = 0; g < wpt; ++g) {
+    const int wi = wave_w0 + g * SAH_WAVE + lane;
+    uint32_t fresh = 0;
+    if (wi < nw) {
+      const uint32_t drawn = s_bits[wi];
+      if (drawn) {
+        const uint32_t old = gbits[w0 + wi];
+        fresh = drawn & ~old;
+        if (fresh) gbits[w0 + wi] = old | drawn;
       }
-      ++pos;
+    }
+    if (__ballot(fresh != 0) == 0) continue;  // uniform across the wave
+    for (int bit = 0; bit < 32; ++bit) {
+      const bool has = (fresh >> bit) & 1u;
+      const uint64_t m = __ballot(has);
+      if (m == 0) continue;
+      if (has) {
+        const int at = out + sah_lane_prefix(m);
+        if (at < cap) cols[at] = ((w0 + wi) << 5) + bit;
+      }
+      out += __popcll(m);
     }
   }
+  // every new entry carries the weight p: one contiguous fill instead of a second scatter
+  for (int i = cnt0 + tid; i < cnt0 + total && i < cap; i += AD_NT) w[i] = p;
   if (tid == 0) {
     int c = cnt0 + total;
     P.rows.cnt[r] = c < cap ? c : cap;
