@@ -13,7 +13,8 @@ __device__ __forceinline__ int sig_score(uint2 q, uint2 k) {
 // ---------------------------------------------------------------------------
 // Signature top-k, SWAR form. Scores fit a byte (score + 33 in [1, 65], 0 = column already
 // active or out of range), so a lane handles 4 consecutive columns as one 32-bit word:
-//   P0  each lane loads its 4 codes (32 B, whole wave: 2 KB contiguous), scores them, zeroes
+//   P0  each lane loads its 4 codes (32 B, whole wave: 2 KB contiguous; in the compact form of the stream 16 B of
+//       sign planes, with the few columns that have a zero component corrected afterwards), scores them, zeroes
 //       the already-active ones with a nibble of the bitmap row and parks the word in LDS;
 //   P1  the threshold T: P0 has already counted the columns at or above 8 coarse thresholds, one more
 //       pass over the staged bytes counts 7 fine ones inside the bracket (byte-parallel compares, no atomics);
