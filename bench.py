@@ -44,7 +44,7 @@ HQ, HKV, D = 32, 8, 128
 
 
 def algorithmic_bytes(w, sampled_per_row: float = 0.0) -> dict:
-    """Unique bytes that must cross HBM once per warm layer-step (formulas in DESIGN.md):
+    """Unique bytes that must cross HBM once per warm layer-step:
     sink/local rows shared by the 4 query heads of a KV group, top-k rows not shared,
     int32 indices written once and read once, Q and out."""
     es = 4 if w["dtype"] == "f32" else 2
@@ -57,8 +57,8 @@ def algorithmic_bytes(w, sampled_per_row: float = 0.0) -> dict:
     gather_fixed = B * HKV * fixed * row * 2
     idx = int(R * (fixed + w["k"] + 2 * sampled_per_row) * 4 * 2)   # sampled entries carry a 4-byte weight too
     qo = 2 * R * D * es
-    # one 4-byte signature per (query head, key): the packed code proper; the non-zero plane the kernels also
-    # read (another 4 bytes) is implementation traffic, not algorithmic
+    # one 4-byte signature per (query head, key): the sign plane the decode kernel scans (the non-zero plane of the
+    # two-plane cache is read only for the few keys that have a zero component)
     scan = {"none": 0, "oracle": B * HKV * Lk * row, "hash": R * Lk * 4, "pq": B * HKV * (Lk - w["sink"]) * 16}[w["kind"]]
     attn = gather_topk + gather_fixed + int(R * (fixed + w["k"] + 2 * sampled_per_row) * 4) + qo
     return dict(step=gather_topk + gather_fixed + idx + qo + scan, attention_kernel=attn, scan=scan)
