@@ -16,8 +16,8 @@ __device__ __forceinline__ int sig_score(uint2 q, uint2 k) {
 //   P0  each lane loads its 4 codes (32 B, whole wave: 2 KB contiguous; in the compact form of the stream 16 B of
 //       sign planes, with the few columns that have a zero component corrected afterwards), scores them, zeroes
 //       the already-active ones with a nibble of the bitmap row and parks the word in LDS;
-//   P1  the threshold T: P0 has already counted the columns at or above 8 coarse thresholds, one more
-//       pass over the staged bytes counts 7 fine ones inside the bracket (byte-parallel compares, no atomics);
+//   P1  the threshold T: P0 has already counted the columns at or above 8 probe thresholds, one more
+//       pass over the staged bytes counts the 3 inside the bracket (byte-parallel compares);
 //   P2  per-lane bit masks "above T" / "equal T" of the lane's columns, per-wave counts of both;
 //   P3  write: a wave scan of per-lane counts, every lane appends the set bits of its mask; ties are
 //       taken lowest column first until `need` are used (the one wave where the budget runs out ranks
@@ -36,13 +36,18 @@ __device__ __forceinline__ uint32_t swar_ge(uint32_t w, uint32_t t) {
 }
 
 #define HSW_GC 8      // chunks per mask group of P2 / P3: 8 x 4 columns of a lane = one 32-bit mask
-#define HSW_PROBES 8  // coarse thresholds 8, 16, ... 64 counted while the scores are staged
+#define HSW_PROBES 8  // thresholds counted while the scores are staged
+// Probe i: 32, 36, ... 60. Scores + 33 lie in [1, 65] around 33, and a top-k of less than half the row has its
+// threshold above that, so these eight bracket it to 4 values in the usual case; below 32 a second set
+// (4, 8, ... 28) is counted from the staged bytes, from 60 up the last bracket is resolved in one 7-way pass.
+__host__ __device__ constexpr uint32_t hsw_probe_at(int i) { return 32u + 4u * (uint32_t)i; }
 
 struct hsw_lds {
   int gt[HSW_NW];
   int eq[HSW_NW];
   int probe[HSW_PROBES];  // workgroup totals of the coarse and of the fine counts: one LDS atomic per wave and
   int fine[HSW_PROBES];   // counter, read back by everyone after the barrier; zeroed by hsw_lds_init
+  int low[HSW_PROBES];    // the second probe set (thresholds below 32), counted only when the first one misses
 };
 
 // Clears the counters of `S`. To be called by every thread before the barrier that precedes hsw_select_row.
@@ -50,6 +55,7 @@ __device__ __forceinline__ void hsw_lds_init(hsw_lds& S) {
   if (threadIdx.x < HSW_PROBES) {
     S.probe[threadIdx.x] = 0;
     S.fine[threadIdx.x] = 0;
+    S.low[threadIdx.x] = 0;
   }
 }
 
@@ -182,7 +188,7 @@ __device__ __forceinline__ int hsw_select_row(const sah_rows& R, int r, const ui
     s_key[wi] = kw;
     const uint32_t x = kw | 0x80808080u;
 #pragma unroll
-    for (int i = 0; i < HSW_PROBES; ++i) pc[i] += __popc((x - (uint32_t)(8 * (i + 1)) * 0x01010101u) & 0x80808080u);
+    for (int i = 0; i < HSW_PROBES; ++i) pc[i] += __popc((x - hsw_probe_at(i) * 0x01010101u) & 0x80808080u);
   };
   if constexpr (CP) {
     // ---- compact stream: every component taken as non-zero, score = popc(q.y) - 2 popc((q.x ^ k.x) & q.y)
@@ -231,7 +237,7 @@ __device__ __forceinline__ int hsw_select_row(const sah_rows& R, int r, const ui
         s_byte[col] = (unsigned char)s_new;
 #pragma unroll
         for (int i = 0; i < HSW_PROBES; ++i)
-          pc[i] += (int)(s_new >= (uint32_t)(8 * (i + 1))) - (int)(s_old >= (uint32_t)(8 * (i + 1)));
+          pc[i] += (int)(s_new >= hsw_probe_at(i)) - (int)(s_old >= hsw_probe_at(i));
       }
     };
     const int n_exc = __builtin_amdgcn_readfirstlane(buf.exc_n);
@@ -303,29 +309,73 @@ __device__ __forceinline__ int hsw_select_row(const sah_rows& R, int r, const ui
   const int n_w = n_ch * SAH_WAVE;
   const int tot = lane < HSW_PROBES ? S.probe[lane] : 0;
   const int n_pass = __popcll(__ballot(lane < HSW_PROBES && tot >= k));
-  const uint32_t base = 8u * (uint32_t)n_pass;                         // T is in [base, base + 8)
-  const int next_probe = n_pass < HSW_PROBES ? __shfl(tot, n_pass) : 0;  // count(key >= base + 8)
+  uint32_t base;   // T is in [base, base + n_f + 1)
+  int n_f;         // fine thresholds base + 1 .. base + n_f to count: 3, or 7 in the top bracket
+  int next_probe;  // count(key >= base + n_f + 1)
+  if (n_pass >= 1 && n_pass < HSW_PROBES) {
+    base = hsw_probe_at(n_pass - 1);
+    n_f = 3;
+    next_probe = __shfl(tot, n_pass);
+  } else if (n_pass == HSW_PROBES) {
+    base = hsw_probe_at(HSW_PROBES - 1);  // 60: scores end at 65, so count(key >= 68) = 0
+    n_f = 7;
+    next_probe = 0;
+  } else {
+    // T < 32: the second probe set, thresholds 4, 8, ... 28, from the staged bytes
+    int lc[7];
+#pragma unroll
+    for (int j = 0; j < 7; ++j) lc[j] = 0;
+    for (int i = tid; i < n_w; i += HSW_NT) {
+      const uint32_t x = s_key[i] | 0x80808080u;
+#pragma unroll
+      for (int j = 0; j < 7; ++j) lc[j] += __popc((x - (uint32_t)(4 * (j + 1)) * 0x01010101u) & 0x80808080u);
+    }
+#pragma unroll
+    for (int j = 0; j < 7; j += 2) {
+      const uint32_t t = (uint32_t)sah_wave_sum_i(lc[j] + ((j + 1 < 7 ? lc[j + 1] : 0) << 16));
+      if (lane == 0) {
+        atomicAdd(&S.low[j], (int)(t & 0xFFFFu));
+        if (j + 1 < 7) atomicAdd(&S.low[j + 1], (int)(t >> 16));
+      }
+    }
+    __syncthreads();
+    const int ltot = lane < 7 ? S.low[lane] : 0;
+    const int n_low = __popcll(__ballot(lane < 7 && ltot >= k));
+    base = 4u * (uint32_t)n_low;
+    n_f = 3;
+    next_probe = n_low < 7 ? __shfl(ltot, n_low) : __shfl(tot, 0);
+  }
   int fc[7];
 #pragma unroll
   for (int j = 0; j < 7; ++j) fc[j] = 0;
-  for (int i = tid; i < n_w; i += HSW_NT) {
-    const uint32_t x = s_key[i] | 0x80808080u;
+  if (n_f == 3) {  // uniform across the workgroup
+    for (int i = tid; i < n_w; i += HSW_NT) {
+      const uint32_t x = s_key[i] | 0x80808080u;
 #pragma unroll
-    for (int j = 0; j < 7; ++j) fc[j] += __popc((x - (base + 1u + j) * 0x01010101u) & 0x80808080u);
+      for (int j = 0; j < 3; ++j) fc[j] += __popc((x - (base + 1u + j) * 0x01010101u) & 0x80808080u);
+    }
+  } else {
+    for (int i = tid; i < n_w; i += HSW_NT) {
+      const uint32_t x = s_key[i] | 0x80808080u;
+#pragma unroll
+      for (int j = 0; j < 7; ++j) fc[j] += __popc((x - (base + 1u + j) * 0x01010101u) & 0x80808080u);
+    }
   }
 #pragma unroll
   for (int j = 0; j < 7; j += 2) {
-    const uint32_t t = (uint32_t)sah_wave_sum_i(fc[j] + ((j + 1 < 7 ? fc[j + 1] : 0) << 16));
-    if (lane == 0) {
-      atomicAdd(&S.fine[j], (int)(t & 0xFFFFu));
-      if (j + 1 < 7) atomicAdd(&S.fine[j + 1], (int)(t >> 16));
+    if (j < n_f) {
+      const uint32_t t = (uint32_t)sah_wave_sum_i(fc[j] + ((j + 1 < 7 ? fc[j + 1] : 0) << 16));
+      if (lane == 0) {
+        atomicAdd(&S.fine[j], (int)(t & 0xFFFFu));
+        if (j + 1 < 7) atomicAdd(&S.fine[j + 1], (int)(t >> 16));
+      }
     }
   }
   __syncthreads();
-  const int ftot = lane < 7 ? S.fine[lane] : 0;
-  const int n_fine = __popcll(__ballot(lane < 7 && ftot >= k));
+  const int ftot = lane < n_f ? S.fine[lane] : 0;
+  const int n_fine = __popcll(__ballot(lane < n_f && ftot >= k));
   const uint32_t T = base + (uint32_t)n_fine;
-  const int above = n_fine < 7 ? __shfl(ftot, n_fine) : next_probe;      // count(key >= T + 1)
+  const int above = n_fine < n_f ? __shfl(ftot, n_fine) : next_probe;      // count(key >= T + 1)
   // T == 0: fewer than k inactive columns exist; take them all, byte-0 "ties" emit nothing
   const int need = (T == 0) ? 0 : k - above;
 

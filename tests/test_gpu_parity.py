@@ -548,6 +548,66 @@ def test_hash_decode_plan_state_transitions(cuda):
         assert torch.equal(zeros.to(torch.int32), c1.exc_cnt)
 
 
+@pytest.mark.parametrize("case", [
+    # bits, n, k, active, columns whose code equals the query's (score 32: the highest threshold bracket)
+    (32, 5000, 5, 40, 9),          # threshold = the top score itself, ties cut among the 9
+    (32, 5000, 9, 40, 9),
+    (32, 5000, 300, 40, 9),        # usual case: threshold a few steps above the mean
+    (32, 3000, 2500, 100, 0),      # most of the row: threshold below the mean (second probe set)
+    (4, 4000, 3000, 10, 0),        # 4-bit signatures: scores + 33 in [29, 37], heavy ties
+    (32, 700, 690, 20, 0),         # more wanted than exist: every inactive column
+    (32, 40000, 2048, 640, 3),     # two mask groups per wave
+])
+def test_hamming_topk_threshold_brackets(cuda, case):
+    """sah_hamming_topk against a stable descending sort of the reference's signature score, on code sets built
+    to put the threshold in each of the ranges the kernel resolves differently (top score, usual range, below the
+    mean, nothing left), ties to the lowest column."""
+    from sparse_attention_hub_amd import _native as N
+    from sparse_attention_hub_amd.sparse_attention.utils.native_rows import NativeRows
+
+    bits, n, k, n_active, n_same = case
+    R = 3
+    g = torch.Generator().manual_seed(bits * 1000 + k)
+    mask = (1 << bits) - 1
+    pitch = n + (n % 2)
+    kc = torch.randint(0, 2**31 - 1, (R, pitch, 2), generator=g, dtype=torch.int64) * 2 + torch.randint(0, 2, (R, pitch, 2), generator=g)
+    kc &= mask
+    qc = (torch.randint(0, 2**31 - 1, (R, 2), generator=g, dtype=torch.int64) * 2 + 1) & mask
+    kc[..., 1] = mask
+    qc[..., 1] = mask
+    for r in range(R):
+        same = torch.randperm(n, generator=g)[:n_same]
+        kc[r, same, 0] = qc[r, 0]
+    rows = NativeRows(R, n, n_active + k, cuda)
+    rows.zero_if_fresh()
+    act = torch.zeros(R, n, dtype=torch.bool)
+    cols = torch.zeros((R, n_active), dtype=torch.int32)
+    for r in range(R):
+        idx = torch.randperm(n, generator=g)[:n_active]
+        act[r, idx] = True
+        cols[r] = idx.to(torch.int32)
+    rows.cols[:, :n_active] = cols.to(cuda)
+    rows.cnt.fill_(n_active)
+    words = torch.zeros((R, rows.bitmap.shape[1] * 32), dtype=torch.bool)
+    words[:, :n] = act
+    packed = (words.view(R, -1, 32).to(torch.int64) << torch.arange(32, dtype=torch.int64)).sum(-1)
+    rows.bitmap.copy_(torch.where(packed >= 2**31, packed - 2**32, packed).to(torch.int32).to(cuda))
+    rows.max_cnt = n_active
+    rows.fresh = False
+    to_i32 = lambda t: torch.where(t >= 2**31, t - 2**32, t).to(torch.int32)
+    dk, dq = to_i32(kc).contiguous().to(cuda), to_i32(qc).contiguous().to(cuda)
+    N.call("sah_hamming_topk", N.HammingTopkArgs(rows.as_struct(), dk.data_ptr(), pitch, dq.data_ptr(), 1, k, N.stream_ptr(cuda)))
+    sc = O.signature_scores_from_codes(qc.view(R, 1, 2), kc[:, :n]).view(R, n).float()
+    sc[act] = float("-inf")
+    want = O.stable_topk(sc, min(k, n))
+    got_cnt = rows.cnt.cpu()
+    got_cols = rows.cols.cpu()
+    for r in range(R):
+        exp = sorted(want[r].tolist()[: min(k, n - n_active)])     # active columns score -inf and sort last
+        got = sorted(got_cols[r, n_active: int(got_cnt[r])].tolist())
+        assert int(got_cnt[r]) == n_active + len(exp) and got == exp, f"row {r}"
+
+
 def test_oracle_topk_full_size_properties(cuda):
     """Config 2 at its full shape (B = 4, 32 query / 8 KV heads, 32768 keys, top 5 % = 1638, bf16), checked
     through properties that need no CPU restatement of 128 x 32768 scores: every row holds sink + local +
