@@ -182,9 +182,13 @@ __device__ __forceinline__ int hsw_select_row(const sah_rows& R, int r, const ui
   // what staging a word has in common: zero the bytes of already-active columns, park the word, count the probes
   auto stage = [&](uint32_t word, int wi) {
     const int j0 = wi * 4;
+    // Most chunks of a long row hold no active column at all: uniform test, the expansion is skipped
     const uint32_t nib = (s_bm[j0 >> 5] >> (j0 & 31)) & 0xFu;  // nibble -> byte mask
-    const uint32_t act = ((nib * 0x00204081u) & 0x01010101u) * 0xFFu;
-    const uint32_t kw = word & ~act;
+    uint32_t kw = word;
+    if (__ballot(nib != 0)) {
+      const uint32_t one = (nib | (nib << 7) | (nib << 14) | (nib << 21)) & 0x01010101u;
+      kw = word & ~((one << 8) - one);
+    }
     s_key[wi] = kw;
     const uint32_t x = kw | 0x80808080u;
 #pragma unroll
