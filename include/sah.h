@@ -292,6 +292,21 @@ int sah_select_topk(const sah_select_topk_args* a);
  * workgroup computes its slab itself (one launch, `lut` is not touched); beyond that it
  * is built once per call in `lut` (caller's scratch of sah_pq_adc_lut_bytes(...) bytes).
  * ------------------------------------------------------------------------- */
+/* Largest |element| of the keys [key_offset, key_offset + n_keys) of every (b, kv head), written as the bit
+ * pattern of a float into *absmax_bits, which must be zero before the call. The Lloyd kernels below take their
+ * per-centre sums in 64-bit fixed point, scaled by a power of two derived from this value: integer sums do not
+ * depend on the order of the additions, so clustering the same keys twice gives the same centroids bit for bit
+ * (the reference's one-hot sums, pq_utils.py:360-372, are reproducible too). */
+typedef struct sah_pq_absmax_args {
+  const void* k; int64_t ks_b, ks_h, ks_l;
+  int32_t dtype;
+  int32_t B, Hkv, D;
+  int32_t key_offset, n_keys;
+  uint32_t* absmax_bits;
+  void* stream;
+} sah_pq_absmax_args;
+int sah_pq_keys_absmax(const sah_pq_absmax_args* a);
+
 typedef struct sah_pq_assign_args {
   const void* k; int64_t ks_b, ks_h, ks_l;
   int32_t dtype;
@@ -299,10 +314,11 @@ typedef struct sah_pq_assign_args {
   int32_t key_offset, n_keys;
   const float* centres;
   uint8_t* codes; int64_t code_pitch; int64_t code_offset;
-  float* sums; int32_t* counts;
+  int64_t* sums; int32_t* counts;     /* [n_groups, n_cent, d_sub] fixed-point sums, [n_groups, n_cent]; both NULL: codes only */
   int32_t round_dist;
   const int32_t* skip_flag;
   void* stream;
+  const uint32_t* absmax_bits;        /* from sah_pq_keys_absmax; needed when sums is not NULL */
 } sah_pq_assign_args;
 int sah_pq_kmeans_assign(const sah_pq_assign_args* a);
 
@@ -312,12 +328,13 @@ typedef struct sah_pq_update_args {
   int32_t B, Hkv, n_sub, d_sub, n_cent;
   int32_t key_offset;
   float* centres;
-  const float* sums; const int32_t* counts;
+  const int64_t* sums; const int32_t* counts;
   const int32_t* reseed_idx;
   float* shift2;       /* [n_groups] */
   float tol;
   int32_t* state;      /* int32[4]: converged count, ticket, done flag, pending verdict */
   void* stream;
+  const uint32_t* absmax_bits;        /* the value the assignment used */
 } sah_pq_update_args;
 int sah_pq_kmeans_update(const sah_pq_update_args* a);
 

@@ -16,13 +16,32 @@
 #define PQ_MAX_CENT 256
 #define PQ_TILES 8  // key tiles of PQ_NT per workgroup
 
+// Per-centre sums of the Lloyd update are kept in 64-bit fixed point, so that their value does not depend on the
+// order in which threads and workgroups add to them (floating-point atomics would make two runs on the same keys
+// differ in a centroid's last bits). The scale is a power of two picked from the largest |key element|:
+// |x| * scale < 2^41, which leaves room for 2^20 keys per centre and costs nothing in precision (a float has 24
+// significant bits).
+__device__ __forceinline__ float pq_sum_scale(uint32_t absmax_bits) {
+  const float m = sah_bits_to_float(absmax_bits);
+  if (!(m > 0.f) || !(m < INFINITY)) return 1.f;
+  int e;
+  frexpf(m, &e);  // m = f * 2^e, f in [0.5, 1)
+  int sh = 40 - e;
+  sh = sh < -100 ? -100 : (sh > 100 ? 100 : sh);
+  return ldexpf(1.0f, sh);
+}
+__device__ __forceinline__ void pq_sum_add(long long* p, float x, float scale) {
+  atomicAdd((unsigned long long*)p, (unsigned long long)__float2ll_rn(x * scale));
+}
+
 struct pq_assign_params {
   const void* k; int64_t ks_b, ks_h, ks_l;
   int Hkv, n_sub, d_sub, n_cent;
   int key_offset, n_keys;
   const float* centres;
   uint8_t* codes; int64_t code_pitch, code_offset;
-  float* sums; int* counts;
+  long long* sums; int* counts;
+  const uint32_t* absmax_bits;
   int round_dist;
   const int* skip_flag;
 };
@@ -30,9 +49,10 @@ struct pq_assign_params {
 template <int DT>
 __global__ __launch_bounds__(PQ_NT) void k_pq_assign(pq_assign_params P) {
   __shared__ float s_c[PQ_MAX_CENT * PQ_MAX_D];
-  __shared__ float s_sum[PQ_MAX_CENT * PQ_MAX_D];
+  __shared__ long long s_sum[PQ_MAX_CENT * PQ_MAX_D];
   __shared__ int s_cnt[PQ_MAX_CENT];
   if (P.skip_flag && *P.skip_flag) return;
+  const float sum_scale = P.sums ? pq_sum_scale(*P.absmax_bits) : 1.f;
   const int tid = threadIdx.x;
   const int s = blockIdx.x % P.n_sub;
   const int tg = blockIdx.x / P.n_sub;
@@ -45,7 +65,7 @@ __global__ __launch_bounds__(PQ_NT) void k_pq_assign(pq_assign_params P) {
 
   for (int i = tid; i < cd; i += PQ_NT) {
     s_c[i] = P.centres[(int64_t)g * cd + i];
-    s_sum[i] = 0.f;
+    s_sum[i] = 0;
   }
   for (int i = tid; i < n_cent; i += PQ_NT) s_cnt[i] = 0;
   __syncthreads();
@@ -90,7 +110,7 @@ __global__ __launch_bounds__(PQ_NT) void k_pq_assign(pq_assign_params P) {
     if (P.sums) {
 #pragma unroll
       for (int d = 0; d < PQ_MAX_D; ++d)
-        if (d < d_sub) atomicAdd(&s_sum[best * d_sub + d], x[d]);
+        if (d < d_sub) pq_sum_add(&s_sum[best * d_sub + d], x[d], sum_scale);
       atomicAdd(&s_cnt[best], 1);
     }
   }
@@ -100,7 +120,8 @@ __global__ __launch_bounds__(PQ_NT) void k_pq_assign(pq_assign_params P) {
     const int cn = s_cnt[c];
     if (cn) {
       atomicAdd(&P.counts[(int64_t)g * n_cent + c], cn);
-      for (int d = 0; d < d_sub; ++d) atomicAdd(&P.sums[(int64_t)g * cd + c * d_sub + d], s_sum[c * d_sub + d]);
+      for (int d = 0; d < d_sub; ++d)
+        atomicAdd((unsigned long long*)&P.sums[(int64_t)g * cd + c * d_sub + d], (unsigned long long)s_sum[c * d_sub + d]);
     }
   }
 }
@@ -191,9 +212,10 @@ __global__ __launch_bounds__(PQM_NT) void k_pq_assign_mfma(pq_assign_params P) {
   constexpr int DS = 2 * KS;
   __shared__ __attribute__((aligned(16))) float s_a[(PQ_MAX_CENT / 32) * 2 * 32 * KS];  // -2 c, [tile][g][i][s]
   __shared__ __attribute__((aligned(16))) float s_cn[(PQ_MAX_CENT / 32) * 2 * 16];      // ||c||^2, [tile][g][v]
-  __shared__ float s_sum[PQ_MAX_CENT * DS];
+  __shared__ long long s_sum[PQ_MAX_CENT * DS];
   __shared__ int s_cnt[PQ_MAX_CENT];
   if (P.skip_flag && *P.skip_flag) return;
+  const float sum_scale = P.sums ? pq_sum_scale(*P.absmax_bits) : 1.f;
   const int tid = threadIdx.x;
   const int lane = tid & (SAH_WAVE - 1);
   const int wave = tid / SAH_WAVE;
@@ -224,7 +246,7 @@ __global__ __launch_bounds__(PQM_NT) void k_pq_assign_mfma(pq_assign_params P) {
     s_cn[idx] = nn;
   }
   if (P.sums) {
-    for (int i = tid; i < n_cent * DS; i += PQM_NT) s_sum[i] = 0.f;
+    for (int i = tid; i < n_cent * DS; i += PQM_NT) s_sum[i] = 0;
     for (int i = tid; i < n_cent; i += PQM_NT) s_cnt[i] = 0;
   }
   __syncthreads();
@@ -270,7 +292,7 @@ __global__ __launch_bounds__(PQM_NT) void k_pq_assign_mfma(pq_assign_params P) {
       if (g == 0) P.codes[(((int64_t)bh * P.code_pitch) + P.code_offset + n) * P.n_sub + s_idx] = (uint8_t)bidx;
       if (P.sums) {
 #pragma unroll
-        for (int s = 0; s < KS; ++s) atomicAdd(&s_sum[bidx * DS + 2 * s + g], xs[s]);
+        for (int s = 0; s < KS; ++s) pq_sum_add(&s_sum[bidx * DS + 2 * s + g], xs[s], sum_scale);
         if (g == 0) atomicAdd(&s_cnt[bidx], 1);
       }
     }
@@ -281,7 +303,8 @@ __global__ __launch_bounds__(PQM_NT) void k_pq_assign_mfma(pq_assign_params P) {
     const int cn = s_cnt[c];
     if (cn) {
       atomicAdd(&P.counts[(int64_t)grp * n_cent + c], cn);
-      for (int d = 0; d < DS; ++d) atomicAdd(&P.sums[(int64_t)grp * n_cent * DS + c * DS + d], s_sum[c * DS + d]);
+      for (int d = 0; d < DS; ++d)
+        atomicAdd((unsigned long long*)&P.sums[(int64_t)grp * n_cent * DS + c * DS + d], (unsigned long long)s_sum[c * DS + d]);
     }
   }
 }
@@ -304,7 +327,8 @@ struct pq_update_params {
   const void* k; int64_t ks_b, ks_h, ks_l;
   int Hkv, n_sub, d_sub, n_cent, key_offset;
   float* centres;
-  const float* sums; const int* counts;
+  const long long* sums; const int* counts;
+  const uint32_t* absmax_bits;
   const int* reseed_idx;
   float* shift2;
   float tol;
@@ -328,7 +352,8 @@ __global__ __launch_bounds__(PQ_NT) void k_pq_update(pq_update_params P) {
     const int c = tid;
     const int cn = P.counts[(int64_t)g * n_cent + c];
     float* cc = P.centres + ((int64_t)g * n_cent + c) * d_sub;
-    const float* ss = P.sums + ((int64_t)g * n_cent + c) * d_sub;
+    const long long* ss = P.sums + ((int64_t)g * n_cent + c) * d_sub;
+    const double unscale = 1.0 / ((double)pq_sum_scale(*P.absmax_bits) * (double)(cn > 0 ? cn : 1));
     float acc = 0.f;
     int64_t roff = 0;
     if (cn == 0) {
@@ -336,7 +361,7 @@ __global__ __launch_bounds__(PQ_NT) void k_pq_update(pq_update_params P) {
       roff = (int64_t)b * P.ks_b + (int64_t)hk * P.ks_h + (int64_t)(P.key_offset + ridx) * P.ks_l + (int64_t)s * d_sub;
     }
     for (int d = 0; d < d_sub; ++d) {
-      const float nv = (cn > 0) ? ss[d] / (float)cn : sah_load<DT>(P.k, roff + d);
+      const float nv = (cn > 0) ? (float)((double)ss[d] * unscale) : sah_load<DT>(P.k, roff + d);
       const float df = nv - cc[d];
       acc = fmaf(df, df, acc);
       cc[d] = nv;
@@ -643,12 +668,56 @@ static int pq_check_common(const char* what, int B, int Hkv, int n_sub, int d_su
   return SAH_OK;
 }
 
+// Largest |element| of the keys [key_offset, key_offset + n_keys) of every (b, kv head), as float bits (non-negative
+// floats order like their bit patterns, so an integer atomic max does it). *out must be zero before the launch.
+template <int DT>
+__global__ __launch_bounds__(PQ_NT) void k_pq_absmax(const void* k, int64_t ks_b, int64_t ks_h, int64_t ks_l, int Hkv, int D,
+                                                     int key_offset, int n_keys, uint32_t* out) {
+  const int bh = blockIdx.y;
+  const int64_t base = (int64_t)(bh / Hkv) * ks_b + (int64_t)(bh % Hkv) * ks_h;
+  const int64_t total = (int64_t)n_keys * D;
+  uint32_t best = 0u;
+  for (int64_t i = (int64_t)blockIdx.x * PQ_NT + threadIdx.x; i < total; i += (int64_t)gridDim.x * PQ_NT) {
+    const int n = (int)(i / D), d = (int)(i % D);
+    const uint32_t bits = sah_float_to_bits(sah_load<DT>(k, base + (int64_t)(key_offset + n) * ks_l + d)) & 0x7fffffffu;
+    if (bits <= 0x7f800000u) best = bits > best ? bits : best;  // NaN is skipped
+  }
+#pragma unroll
+  for (int o = 1; o < SAH_WAVE; o <<= 1) {
+    const uint32_t other = (uint32_t)__shfl_xor((int)best, o);
+    best = other > best ? other : best;
+  }
+  if ((threadIdx.x & (SAH_WAVE - 1)) == 0 && best) atomicMax(out, best);
+}
+
+extern "C" int sah_pq_keys_absmax(const sah_pq_absmax_args* a) {
+  if (!a) return sah_fail(SAH_ENULL, "sah_pq_keys_absmax: args is NULL");
+  if (!a->k || !a->absmax_bits) return sah_fail(SAH_ENULL, "sah_pq_keys_absmax: NULL tensor");
+  if (a->B <= 0 || a->Hkv <= 0 || a->D <= 0 || a->key_offset < 0 || a->n_keys < 0 || (int64_t)a->B * a->Hkv > 65535)
+    return sah_fail(SAH_EINVAL, "sah_pq_keys_absmax: bad B/Hkv/D/key range");
+  if (a->n_keys == 0) return SAH_OK;
+  const int64_t total = (int64_t)a->n_keys * a->D;
+  int gx = (int)((total + PQ_NT * 16 - 1) / (PQ_NT * 16));
+  gx = gx < 1 ? 1 : (gx > 64 ? 64 : gx);
+  dim3 g(gx, a->B * a->Hkv), blk(PQ_NT);
+  hipStream_t st = (hipStream_t)a->stream;
+  sah_timed timed("k_pq_absmax", a->stream);
+  switch (a->dtype) {
+    case SAH_F32: hipLaunchKernelGGL(k_pq_absmax<SAH_F32>, g, blk, 0, st, a->k, a->ks_b, a->ks_h, a->ks_l, a->Hkv, a->D, a->key_offset, a->n_keys, a->absmax_bits); break;
+    case SAH_BF16: hipLaunchKernelGGL(k_pq_absmax<SAH_BF16>, g, blk, 0, st, a->k, a->ks_b, a->ks_h, a->ks_l, a->Hkv, a->D, a->key_offset, a->n_keys, a->absmax_bits); break;
+    case SAH_F16: hipLaunchKernelGGL(k_pq_absmax<SAH_F16>, g, blk, 0, st, a->k, a->ks_b, a->ks_h, a->ks_l, a->Hkv, a->D, a->key_offset, a->n_keys, a->absmax_bits); break;
+    default: return sah_fail(SAH_EDTYPE, "sah_pq_keys_absmax: dtype %d", a->dtype);
+  }
+  return sah_launch_status("sah_pq_keys_absmax");
+}
+
 extern "C" int sah_pq_kmeans_assign(const sah_pq_assign_args* a) {
   if (!a) return sah_fail(SAH_ENULL, "sah_pq_kmeans_assign: args is NULL");
   int rc = pq_check_common("sah_pq_kmeans_assign", a->B, a->Hkv, a->n_sub, a->d_sub, a->n_cent);
   if (rc) return rc;
   if (!a->k || !a->centres || !a->codes) return sah_fail(SAH_ENULL, "sah_pq_kmeans_assign: NULL tensor");
   if ((a->sums == nullptr) != (a->counts == nullptr)) return sah_fail(SAH_EINVAL, "sah_pq_kmeans_assign: sums and counts go together");
+  if (a->sums && !a->absmax_bits) return sah_fail(SAH_ENULL, "sah_pq_kmeans_assign: sums need absmax_bits (sah_pq_keys_absmax)");
   if (a->n_keys <= 0) return SAH_OK;
   if (a->key_offset < 0 || a->code_offset < 0 || a->code_pitch < a->code_offset + a->n_keys)
     return sah_fail(SAH_ECAPACITY, "sah_pq_kmeans_assign: code_pitch %lld < code_offset %lld + n_keys %d",
@@ -659,7 +728,8 @@ extern "C" int sah_pq_kmeans_assign(const sah_pq_assign_args* a) {
   P.key_offset = a->key_offset; P.n_keys = a->n_keys;
   P.centres = a->centres;
   P.codes = a->codes; P.code_pitch = a->code_pitch; P.code_offset = a->code_offset;
-  P.sums = a->sums; P.counts = a->counts;
+  P.sums = (long long*)a->sums; P.counts = a->counts;
+  P.absmax_bits = a->absmax_bits;
   P.round_dist = a->round_dist;
   P.skip_flag = a->skip_flag;
   hipStream_t st = (hipStream_t)a->stream;
@@ -699,12 +769,13 @@ extern "C" int sah_pq_kmeans_update(const sah_pq_update_args* a) {
   if (!a) return sah_fail(SAH_ENULL, "sah_pq_kmeans_update: args is NULL");
   int rc = pq_check_common("sah_pq_kmeans_update", a->B, a->Hkv, a->n_sub, a->d_sub, a->n_cent);
   if (rc) return rc;
-  if (!a->k || !a->centres || !a->sums || !a->counts || !a->reseed_idx || !a->shift2 || !a->state)
+  if (!a->k || !a->centres || !a->sums || !a->counts || !a->reseed_idx || !a->shift2 || !a->state || !a->absmax_bits)
     return sah_fail(SAH_ENULL, "sah_pq_kmeans_update: NULL tensor");
   pq_update_params P;
   P.k = a->k; P.ks_b = a->ks_b; P.ks_h = a->ks_h; P.ks_l = a->ks_l;
   P.Hkv = a->Hkv; P.n_sub = a->n_sub; P.d_sub = a->d_sub; P.n_cent = a->n_cent; P.key_offset = a->key_offset;
-  P.centres = a->centres; P.sums = a->sums; P.counts = a->counts; P.reseed_idx = a->reseed_idx;
+  P.centres = a->centres; P.sums = (const long long*)a->sums; P.counts = a->counts; P.reseed_idx = a->reseed_idx;
+  P.absmax_bits = a->absmax_bits;
   P.shift2 = a->shift2; P.tol = a->tol; P.state = a->state;
   P.n_groups = a->B * a->Hkv * a->n_sub;
   dim3 g(P.n_groups), blk(PQ_NT);

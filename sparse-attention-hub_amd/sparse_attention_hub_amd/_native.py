@@ -40,6 +40,7 @@ EXPECTED_SYMBOLS = (
     "sah_hash_compact_codes",
     "sah_qk_scores",
     "sah_select_topk",
+    "sah_pq_keys_absmax",
     "sah_pq_kmeans_assign",
     "sah_pq_kmeans_update",
     "sah_pq_adc_scores",
@@ -180,6 +181,7 @@ class PqAssignArgs(C.Structure):
         ("round_dist", C.c_int32),
         ("skip_flag", C.c_void_p),
         ("stream", C.c_void_p),
+        ("absmax_bits", C.c_void_p),
     ]
 
 
@@ -195,6 +197,18 @@ class PqUpdateArgs(C.Structure):
         ("shift2", C.c_void_p),
         ("tol", C.c_float),
         ("state", C.c_void_p),
+        ("stream", C.c_void_p),
+        ("absmax_bits", C.c_void_p),
+    ]
+
+
+class PqAbsmaxArgs(C.Structure):
+    _fields_ = [
+        ("k", C.c_void_p), ("ks_b", C.c_int64), ("ks_h", C.c_int64), ("ks_l", C.c_int64),
+        ("dtype", C.c_int32),
+        ("B", C.c_int32), ("Hkv", C.c_int32), ("D", C.c_int32),
+        ("key_offset", C.c_int32), ("n_keys", C.c_int32),
+        ("absmax_bits", C.c_void_p),
         ("stream", C.c_void_p),
     ]
 

@@ -87,7 +87,7 @@ def kmeans_keys_batched(
                 f"cluster_centers shape mismatch. Expected ({n_groups}, {n_cent}, {d_sub}), got {tuple(cluster_centers.shape)}"
             )
         centres = cluster_centers.to(device=dev, dtype=torch.float32).contiguous().clone()
-    sums = torch.empty((n_groups, n_cent, d_sub), dtype=torch.float32, device=dev)
+    sums = torch.empty((n_groups, n_cent, d_sub), dtype=torch.int64, device=dev)  # fixed point: order-independent
     counts = torch.empty((n_groups, n_cent), dtype=torch.int32, device=dev)
     shift2 = torch.zeros((n_groups,), dtype=torch.float32, device=dev)
     state = torch.zeros((4,), dtype=torch.int32, device=dev)
@@ -95,6 +95,10 @@ def kmeans_keys_batched(
     reseed = torch.randint(0, n_keys, (max(max_iter, 1), n_groups, n_cent), generator=gen, dtype=torch.int32).to(dev)
     dt = N.dtype_code(keys.dtype)
     stream = N.stream_ptr(dev)
+    absmax = torch.zeros((1,), dtype=torch.int32, device=dev)
+    N.call("sah_pq_keys_absmax", N.PqAbsmaxArgs(
+        keys.data_ptr(), keys.stride(0), keys.stride(1), keys.stride(2), dt, B, Hkv, n_sub * d_sub, key_offset, n_keys,
+        absmax.data_ptr(), stream))
     for it in range(max_iter):
         sums.zero_()
         counts.zero_()
@@ -102,14 +106,14 @@ def kmeans_keys_batched(
             keys.data_ptr(), keys.stride(0), keys.stride(1), keys.stride(2), dt,
             B, Hkv, n_sub, d_sub, n_cent, key_offset, n_keys,
             centres.data_ptr(), codes.data_ptr(), code_pitch, code_offset,
-            sums.data_ptr(), counts.data_ptr(), 0, state[2:].data_ptr(), stream,
+            sums.data_ptr(), counts.data_ptr(), 0, state[2:].data_ptr(), stream, absmax.data_ptr(),
         )
         N.call("sah_pq_kmeans_assign", a)
         u = N.PqUpdateArgs(
             keys.data_ptr(), keys.stride(0), keys.stride(1), keys.stride(2), dt,
             B, Hkv, n_sub, d_sub, n_cent, key_offset,
             centres.data_ptr(), sums.data_ptr(), counts.data_ptr(), reseed[it].data_ptr(),
-            shift2.data_ptr(), float(tol), state.data_ptr(), stream,
+            shift2.data_ptr(), float(tol), state.data_ptr(), stream, absmax.data_ptr(),
         )
         N.call("sah_pq_kmeans_update", u)
     return centres, shift2

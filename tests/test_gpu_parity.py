@@ -615,6 +615,22 @@ def test_hamming_topk_threshold_brackets(cuda, case):
         assert int(got_cnt[r]) == n_active + len(exp) and got == exp, f"row {r}"
 
 
+def test_pq_clustering_is_reproducible(cuda):
+    """Two clusterings of the same keys give the same centroids and codes, bit for bit: the Lloyd sums are
+    order-independent (64-bit fixed point), whatever order workgroups and waves add in."""
+    from sparse_attention_hub_amd.sparse_attention.research_attention.maskers.fixed.implementations.utils.pq_utils import kmeans_keys_batched
+
+    B, Hkv, n, D, n_sub, n_cent = 2, 4, 20000, 128, 16, 256
+    k = make_qkv(B, Hkv, Hkv, 1, n, D, torch.bfloat16, outliers=True, seed=77)[1].to(cuda)
+    runs = []
+    for _ in range(3):
+        codes = torch.zeros((B, Hkv, n, n_sub), dtype=torch.uint8, device=cuda)
+        centres, _ = kmeans_keys_batched(k, 0, n_sub, n_cent, 4, codes, n, seed=3)
+        runs.append((centres.clone(), codes.clone()))
+    for c, z in runs[1:]:
+        assert torch.equal(c, runs[0][0]) and torch.equal(z, runs[0][1])
+
+
 def test_oracle_topk_full_size_properties(cuda):
     """Config 2 at its full shape (B = 4, 32 query / 8 KV heads, 32768 keys, top 5 % = 1638, bf16), checked
     through properties that need no CPU restatement of 128 x 32768 scores: every row holds sink + local +
