@@ -28,8 +28,6 @@ HIP_FLAGS = [
     "-fno-gpu-rdc",
     "-Wall",
     "-Wno-unused-function",
-    # native global/LDS float atomic add (k-means centre sums) instead of CAS loops
-    "-munsafe-fp-atomics",
     # packed fp32 VALU forms are switched off for every kernel in this library
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
