@@ -71,12 +71,14 @@ __global__ __launch_bounds__(256) void k_attn_weights(sah_rows R, const float* l
 }
 
 // Splits per row, from an upper bound of the row lengths: enough workgroups to cover 256 CUs several times,
-// at least one chunk and at most 16 chunks of keys each (the kernel divides every row's own length by it).
+// at least one chunk and at most 11 chunks of keys each (the kernel divides every row's own length by it; the
+// longest rows set the pace at the end of the launch, so their tiles must stay small: at 512 rows of 1300 to
+// 130000 entries 32 -> 47 splits took the kernel from 513 to 501 us, 64 splits gained nothing more).
 static int att_pick_split(int n_rows, int max_cnt) {
   int chunks = (max_cnt + ATT_CHUNK - 1) / ATT_CHUNK;
   if (chunks < 1) chunks = 1;
   int want = (4096 + n_rows - 1) / n_rows;  // target ~4096 workgroups
-  const int for_length = (chunks + 15) / 16;
+  const int for_length = (chunks + 10) / 11;
   if (want < for_length) want = for_length;
   int n_split = chunks < want ? chunks : want;
   if (n_split > ATT_MAX_SPLIT) n_split = ATT_MAX_SPLIT;
