@@ -37,8 +37,19 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert lib.sah_select_topk(None) == -2
     # whole rows per workgroup (many short rows): no workspace; few or long rows: (m, l, acc[D]) per split
     assert N.work_floats(256, 2688, 128) == 0
-    assert N.work_floats(128, 2278, 128) == 128 * 9 * 130
-    assert N.work_floats(512, 131072, 128) == 512 * 32 * 130
+    # split form: rows x splits x (D + 2) floats, where the library chooses the split count: never more than 64
+    # splits, never more splits than 256-key chunks, no tile of a longest row beyond 11 chunks, and enough
+    # workgroups to cover the chip while the row still has chunks to hand out
+    for n_rows, max_cnt, D in ((128, 2278, 128), (512, 131072, 128), (64, 2688, 64), (32, 1500, 128), (1, 70000, 128)):
+        floats = N.work_floats(n_rows, max_cnt, D)
+        assert floats > 0 and floats % (n_rows * (D + 2)) == 0
+        n_split = floats // (n_rows * (D + 2))
+        chunks = -(-max_cnt // 256)
+        assert 1 <= n_split <= min(64, chunks)
+        assert -(-chunks // n_split) <= 11 or n_split == 64
+        assert n_rows * n_split >= 2048 or 2 * n_split > min(64, chunks)
+    assert N.work_floats(32, 300, 128) == 0  # short rows: whole-row form
+    assert N.work_floats(0, 100, 128) == 0 and N.work_floats(16, 100, 0) == 0
     for fn in ("sah_hash_decode_topk", "sah_adaptive_budget", "sah_adaptive_sample", "sah_pq_adc_scores"):
         assert getattr(lib, fn)(None) == -2 and fn.encode() in lib.sah_last_error()
     assert lib.sah_pq_adc_lut_bytes(4, 32, 8, 1, 16, 256, 1) == 4 * 8 * 1 * 16 * 256 * 8
