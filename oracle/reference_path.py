@@ -16,16 +16,23 @@ the oracle takes a stable descending sort, i.e. ties go to the lowest key index.
 That is the canonical rule the kernels implement; parity with `torch.topk` itself
 is tie-aware (same keys strictly above the k-th score, same count at it).
 
-Pinning (tests/test_oracle_*.py): Sink/Local patterns, Mask index/ptr vectors,
-top-k known answers, ADC manual check, pairwise distances, sink-logit closed form
-and HF eager attention equality are taken from the reference's own unit tests.
-Parity unpinned (no reference vector exists, checked against closed forms and
-brute force only): the float values of the signature MLP (`hash_signatures`), the
-k-means trajectory beyond one Lloyd step from given centres (`kmeans_lloyd`), the
-adaptive-sampling index streams (torch.randint in the reference; `adaptive_budget` and
-`adaptive_merge` take the draws as inputs, `adaptive_sampling` draws them with Philox4x32-10,
-itself pinned by the published known-answer vectors), and the
-full masker-chain -> output composition (`research_attention`).
+Pinning (tests/test_oracle_golden.py, tests/test_oracle_adaptive.py): every function below has a
+check that a dropped term, a wrong sign or index or a transposed operand fails.
+* From the reference's own unit tests: Sink/Local patterns and full-mask shortcuts, Mask
+  index/ptr vectors, merge known answers, top-k known answers and invariants, pairwise distances,
+  two-blob recovery, ip->l2 augmentation, ADC manual check, PQ full-attention rule, adaptive range /
+  base count / failure-rate bar, sink-logit closed form, HF eager attention equality.
+* Where the reference holds no vector, from what the mathematics fixes: `hash_signatures` against
+  per-head `torch.nn.functional.linear` layers; `hash_topk`'s selected set against a column-by-column
+  sort by (-score, column) over the inactive columns; `pq_split` / `pq_split_ip` against explicit
+  (batch, head, sub-space) loops; `kmeans_lloyd` by hand-computed Lloyd steps including the
+  empty-cluster reseed; `adaptive_exp_scores` against an fp64 evaluation of the definition;
+  `adaptive_budget` against hand arithmetic; Philox4x32-10 against the published known-answer vectors;
+  `research_attention` (the chain) by composing the pieces on a brute-forceable size.
+Not reproducible by any restatement, because the reference leaves them to torch's RNG or to an
+unspecified library choice: which samples `torch.randint` draws (adaptive / random sampling, k-means
+initialisation and reseeding; the oracle takes the draws or the start centres as inputs, or draws
+with Philox) and which of several equal scores `torch.topk` keeps (lowest index here).
 """
 from __future__ import annotations
 

@@ -192,6 +192,60 @@ def test_hash_topk_cache_growth_and_shrink_error():
         O.hash_topk(_empty(1, H, 1, 20), q, k[:, :, :20], None, 4, w, "relu", key_signatures=sig2)
 
 
+def test_hash_topk_selected_set_against_brute_force():
+    # invariants of test_hashattention_top_k.py:444-589 (exactly k new columns per row, none inside the previous
+    # mask, previous columns kept) and the selected SET itself, rebuilt here column by column from the definition:
+    # score(j) = sum_e qsig[e] * ksig[j][e], winners = first k of the inactive columns ordered by (-score, j)
+    B, Hq, Hkv, Lk, D, k_sel = 2, 4, 2, 37, 8, 5
+    w = _tiny_hat(Hq, D, 8, 8, seed=3)
+    g = torch.Generator().manual_seed(11)
+    q = torch.randn(B, Hq, 1, D, generator=g)
+    k = torch.randn(B, Hkv, Lk, D, generator=g)
+    add = torch.randn(B, 1, 1, Lk + 3, generator=g).round()  # additive mask, wider than the keys, integer valued
+    prev = torch.zeros(B, Hq, 1, Lk)
+    prev[..., :3] = 1.0
+    prev[..., -4:] = 1.0
+    prev[0, 1, 0, 10] = 1.0
+    for attention_mask in (None, add):
+        m, ksig = O.hash_topk(O.OMask("dense", prev.shape, torch.float32, prev.clone()), q, k, attention_mask, k_sel, w, "silu")
+        got = m.to_dense()
+        qsig = O.hash_signatures(q, w["query_matrix"], w["query_bias"], "silu")
+        for b in range(B):
+            for h in range(Hq):
+                # key head of query head h is h // G: the signatures of row (b, h) come from K[b, h // 2]
+                ks = O.hash_signatures(k[b:b + 1, h // 2:h // 2 + 1].expand(1, 1, Lk, D), [mm[h:h + 1] for mm in w["key_matrix"]],
+                                       [bb[h:h + 1] for bb in w["key_bias"]], "silu")[0, 0]
+                assert torch.equal(ks, ksig[b, h])
+                sc = []
+                for j in range(Lk):
+                    if prev[b, h, 0, j] != 0:
+                        continue
+                    val = sum(float(qsig[b, h, 0, e]) * float(ks[j, e]) for e in range(8))
+                    if attention_mask is not None:
+                        val += float(attention_mask[b, 0, 0, j])
+                    sc.append((-val, j))
+                winners = {j for _, j in sorted(sc)[:k_sel]}
+                active = set(torch.nonzero(got[b, h, 0]).flatten().tolist())
+                before = set(torch.nonzero(prev[b, h, 0]).flatten().tolist())
+                assert before <= active and active - before == winners and len(winners) == k_sel
+                assert torch.all(got[b, h, 0][list(active)] == 1.0)
+
+
+def test_hash_topk_with_given_signatures_skips_the_mlps():
+    # the `key_signatures` / `query_signatures` arguments are what the GPU tests feed the kernels' own codes through
+    H, Lk = 2, 12
+    ks = torch.ones(1, H, Lk, 4)
+    ks[0, 0, 5] = -1.0            # row 0: column 5 is the worst, every other column ties at +4
+    ks[0, 1, :, :2] = -1.0        # row 1: all columns tie at 0 except column 7
+    ks[0, 1, 7] = 1.0
+    qs = torch.ones(1, H, 1, 4)
+    m, out = O.hash_topk(_empty(1, H, 1, Lk), torch.zeros(1, H, 1, 3), torch.zeros(1, H, Lk, 3), None, 3, None, "relu",
+                         key_signatures=ks, query_signatures=qs)
+    assert out is ks
+    assert torch.nonzero(m.to_dense()[0, 0, 0]).flatten().tolist() == [0, 1, 2]      # ties: lowest columns first
+    assert torch.nonzero(m.to_dense()[0, 1, 0]).flatten().tolist() == [0, 1, 7]      # the best, then the lowest ties
+
+
 # ------------------------------------------------------------------------- PQCache
 def test_pairwise_sq_dist_known_values():
     # utils/test_pq_utils.py:183-209 (and :264-295 batched): all four distances are 1
@@ -217,6 +271,68 @@ def test_kmeans_recovers_two_blobs_and_returns_pre_update_codes():
     codes1, cent1 = O.kmeans_lloyd(X, c_bad, 1)
     assert torch.equal(codes1, torch.argmin(O.pairwise_sq_dist(X, c_bad), 2))
     assert torch.allclose(cent1[0, 0], X[0][codes1[0] == 0].mean(0), atol=1e-6)
+
+
+def test_pq_split_against_explicit_loops():
+    # pq_top_k.py:216-231: group (b, h, s) holds keys[b, h, init_offset + i, s * d:(s + 1) * d] as its row i
+    B, H, Lk, D, n_sub, off = 2, 3, 11, 12, 4, 3
+    d = D // n_sub
+    keys = torch.arange(B * H * Lk * D, dtype=torch.float32).reshape(B, H, Lk, D)
+    X = O.pq_split(keys, off, n_sub)
+    assert X.shape == (B * H * n_sub, Lk - off, d)
+    for b in range(B):
+        for h in range(H):
+            for s in range(n_sub):
+                grp = (b * H + h) * n_sub + s
+                for i in range(Lk - off):
+                    assert torch.equal(X[grp, i], keys[b, h, off + i, s * d:(s + 1) * d])
+
+
+def test_pq_split_ip_against_explicit_loops():
+    # pq_top_k.py:219-236 + pq_utils.py:585-612: the same groups, one more coordinate sqrt(phi - |x|^2) with phi the
+    # group's largest squared norm; the row that attains phi gets exactly 0
+    B, H, Lk, D, n_sub, off = 1, 2, 9, 6, 3, 2
+    d = D // n_sub
+    g = torch.Generator().manual_seed(5)
+    keys = torch.randn(B, H, Lk, D, generator=g)
+    X, phi = O.pq_split_ip(keys, off, n_sub)
+    assert X.shape == (B * H * n_sub, Lk - off, d + 1) and phi.shape == (B * H * n_sub, 1, 1)
+    for h in range(H):
+        for s in range(n_sub):
+            grp = h * n_sub + s
+            sub = [keys[0, h, off + i, s * d:(s + 1) * d] for i in range(Lk - off)]
+            norms = [float((v * v).sum()) for v in sub]
+            assert math.isclose(float(phi[grp]), max(norms), rel_tol=1e-6)
+            for i, v in enumerate(sub):
+                assert torch.equal(X[grp, i, :d], v)
+                assert math.isclose(float(X[grp, i, d]), math.sqrt(max(max(norms) - norms[i], 0.0)), rel_tol=1e-4, abs_tol=1e-3)
+            assert float(X[grp, norms.index(max(norms)), d]) == 0.0
+    # keys before init_offset take no part: a huge key there leaves phi alone
+    keys2 = keys.clone()
+    keys2[:, :, 0] = 100.0
+    assert torch.equal(O.pq_split_ip(keys2, off, n_sub)[1], phi)
+
+
+def test_kmeans_empty_cluster_takes_the_reseed_sample():
+    # pq_utils.py:384-396: a cluster without points becomes X[g, random index]; every other centre is the mean of its
+    # points. Two groups: in group 0 centre 2 sits far away and stays empty, in group 1 nothing is empty.
+    X = torch.tensor([[[0.0, 0.0], [0.0, 2.0], [10.0, 0.0], [10.0, 2.0]],
+                      [[0.0, 0.0], [1.0, 0.0], [5.0, 0.0], [9.0, 0.0]]])
+    c0 = torch.tensor([[[0.0, 1.0], [9.0, 1.0], [100.0, 100.0]],
+                       [[0.0, 0.0], [5.0, 0.0], [9.0, 0.0]]])
+    reseed = torch.tensor([[[3, 3, 1], [0, 0, 0]]])      # (iteration, group, centre) -> sample index
+    codes, centres = O.kmeans_lloyd(X, c0, iter_limit=1, reseed_idx=reseed)
+    assert codes.tolist() == [[0, 0, 1, 1], [0, 0, 1, 2]]
+    assert torch.equal(centres[0], torch.tensor([[0.0, 1.0], [10.0, 1.0], [0.0, 2.0]]))   # centre 2 := X[0, 1]
+    assert torch.equal(centres[1], torch.tensor([[0.5, 0.0], [5.0, 0.0], [9.0, 0.0]]))    # untouched by the reseed
+    with pytest.raises(ValueError):
+        O.kmeans_lloyd(X, c0, iter_limit=1)
+    # second iteration: the reseeded centre now wins its own sample; codes are those of the assignment BEFORE the
+    # last update, centres after it
+    reseed2 = torch.cat([reseed, reseed], dim=0)
+    codes2, centres2 = O.kmeans_lloyd(X, c0, iter_limit=2, reseed_idx=reseed2)
+    assert codes2[0].tolist() == [0, 2, 1, 1]
+    assert torch.equal(centres2[0], torch.tensor([[0.0, 0.0], [10.0, 1.0], [0.0, 2.0]]))
 
 
 def test_ip2l2_augmentation_known_answers():
@@ -297,6 +413,30 @@ def test_pq_topk_offsets_and_exclusion():
 
 
 # ------------------------------------------------------------- adaptive sampling
+def test_adaptive_exp_scores_against_fp64_definition():
+    # adaptive_sampling.py:183-197: exp(q.k * scaling + mask - rowmax) over ALL keys, key head h // G, mask cut to Lk
+    B, Hq, Hkv, Lk, D = 2, 4, 2, 9, 6
+    g = torch.Generator().manual_seed(8)
+    q = torch.randn(B, Hq, 1, D, generator=g)
+    k = torch.randn(B, Hkv, Lk, D, generator=g)
+    add = torch.randn(B, 1, 1, Lk + 2, generator=g)
+    scaling = 0.37
+    for attention_mask in (None, add):
+        got = O.adaptive_exp_scores(q, k, scaling, attention_mask)
+        assert got.shape == (B, Hq, 1, Lk) and got.dtype == q.dtype
+        for b in range(B):
+            for h in range(Hq):
+                z = [sum(float(q[b, h, 0, e]) * float(k[b, h // 2, j, e]) for e in range(D)) * scaling for j in range(Lk)]
+                if attention_mask is not None:
+                    z = [zz + float(attention_mask[b, 0, 0, j]) for j, zz in enumerate(z)]
+                top = max(z)
+                want = torch.tensor([math.exp(zz - top) for zz in z], dtype=torch.float64)
+                assert torch.allclose(got[b, h, 0].double(), want, rtol=1e-5, atol=1e-7)
+                assert float(got[b, h, 0].max()) == 1.0
+    # the result is in the query dtype (the reference never widens here)
+    assert O.adaptive_exp_scores(q.bfloat16(), k.bfloat16(), scaling, None).dtype == torch.bfloat16
+
+
 def test_adaptive_range_and_base_count():
     # sampling/implementations/test_adaptive_sampling.py:207-272
     assert O.adaptive_sampling_range(131072, 128, 1024) == (128, 130048, 129920)
