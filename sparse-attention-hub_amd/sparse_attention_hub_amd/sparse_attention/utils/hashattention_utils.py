@@ -7,6 +7,8 @@ list entry per MLP layer.
 """
 from __future__ import annotations
 
+import collections
+import io
 import pickle
 from typing import Dict, List
 
@@ -15,15 +17,48 @@ import torch
 HatWeights = Dict[int, Dict[str, List[torch.Tensor]]]
 
 
-def load_hat_weights(hat_weights_path: str, device: str = "cpu") -> HatWeights:
-    """Load a HAT weight pickle written by this package or by the reference tools.
+def _storage_from_bytes(data: bytes):
+    """What `torch.storage._load_from_bytes` does for a pickled tensor's storage, but through the loader that
+    executes nothing from the bytes."""
+    return torch.load(io.BytesIO(data), weights_only=True)
 
-    Pickles execute code on load: only open files you wrote or trust."""
+
+class _HatUnpickler(pickle.Unpickler):
+    """Unpickler that resolves only what a dict of lists of CPU tensors needs. A tensor pickles as
+    `torch._utils._rebuild_tensor_v2(storage, ...)` with the storage as `torch.storage._load_from_bytes(bytes)`
+    (replaced here by the safe loader above) and its (empty) hooks as an OrderedDict; `nn.Parameter`s add
+    `_rebuild_parameter`. Every other global a file asks for is refused, so loading runs no code from the file."""
+
+    _ALLOWED = {
+        ("torch._utils", "_rebuild_tensor_v2"): lambda: torch._utils._rebuild_tensor_v2,
+        ("torch._utils", "_rebuild_parameter"): lambda: torch._utils._rebuild_parameter,
+        ("torch.storage", "_load_from_bytes"): lambda: _storage_from_bytes,
+        ("collections", "OrderedDict"): lambda: collections.OrderedDict,
+    }
+
+    def find_class(self, module: str, name: str):
+        try:
+            return self._ALLOWED[(module, name)]()
+        except KeyError:
+            raise pickle.UnpicklingError(
+                f"HAT weight file refers to {module}.{name}; only plain containers of tensors are accepted") from None
+
+
+def load_hat_weights(hat_weights_path: str, device: str = "cpu") -> HatWeights:
+    """Load a HAT weight pickle written by this package or by the reference tools
+    (reference: hashattention_utils.py:155-180). The file is read with an allow-list unpickler: anything but
+    dicts, lists, numbers, strings and tensors raises `pickle.UnpicklingError`."""
     with open(hat_weights_path, "rb") as f:
-        hat_weights: HatWeights = pickle.load(f)
+        hat_weights = _HatUnpickler(f).load()
+    if not isinstance(hat_weights, dict):
+        raise ValueError(f"{hat_weights_path}: expected Dict[layer] -> Dict[name] -> List[Tensor], got {type(hat_weights).__name__}")
     for layer_idx, layer_weights in hat_weights.items():
+        if not isinstance(layer_weights, dict):
+            raise ValueError(f"{hat_weights_path}: layer {layer_idx!r} is not a dict")
         for name, tensors in layer_weights.items():
-            hat_weights[layer_idx][name] = [t.to(device) for t in tensors]
+            if not all(isinstance(t, torch.Tensor) for t in tensors):
+                raise ValueError(f"{hat_weights_path}: layer {layer_idx!r} entry {name!r} holds non-tensors")
+            hat_weights[layer_idx][name] = [t.detach().to(device) for t in tensors]
     return hat_weights
 
 

@@ -74,8 +74,11 @@ def _run_attention(
     rows: Optional[NativeRows],
     return_attention_weights: bool,
     out: Optional[torch.Tensor] = None,
+    return_stats: bool = False,
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
-    """rows=None => dense attention over all keys."""
+    """rows=None => dense attention over all keys. `return_stats`: the second value is the kernel's
+    fp32 (n_rows, 2) tensor of (largest logit among the row's entries, softmax denominator relative to it)
+    instead of the dense probabilities."""
     N.require_device(queries, "queries")
     N.require_device(keys, "keys")
     N.require_device(values, "values")
@@ -113,6 +116,7 @@ def _run_attention(
     logits = stats = None
     if return_attention_weights:
         logits = torch.empty((n_rows, Lk if dense else rows.cap), dtype=torch.float32, device=dev)
+    if return_attention_weights or return_stats:
         stats = torch.empty((n_rows, 2), dtype=torch.float32, device=dev)
     args = N.AttentionArgs(
         rows_struct,
@@ -133,6 +137,8 @@ def _run_attention(
         N.stream_ptr(dev),
     )
     N.call("sah_sparse_attention", args)
+    if return_stats:
+        return out, stats
     weights = None
     if return_attention_weights:
         weights = torch.zeros((B, Hq, Lq, Lk), dtype=q.dtype, device=dev)
@@ -203,3 +209,101 @@ def get_masked_attention_output(
     if return_attention_weights:
         return out, weights
     return out
+
+
+# ------------------------------------------------------------------ numerator / denominator helpers
+def _masked_softmax_parts(queries, keys, values, attention_mask, scaling, mask: Mask):
+    """(out (B, Hq, Lq, D) fp32, den (B, Hq, Lq, 1) fp32, m_all (B, Hq, Lq, 1) fp32) of the masked softmax in the
+    reference's scale, i.e. relative to the largest logit over ALL keys of the row
+    (mask_attention_utils.py:187-240). Two launches of the attention kernel: one over the mask's rows, one dense
+    pass whose statistics give the all-key maximum."""
+    B, Hq, Lq, D = queries.shape
+    rows = None if (mask.is_full or mask.is_empty) else mask.to_rows(0)
+    out, stats = _run_attention(queries, keys, values, attention_mask, None, scaling, rows, False, return_stats=True)
+    if rows is None:
+        all_stats = stats
+    else:
+        _, all_stats = _run_attention(queries, keys, values, attention_mask, None, scaling, None, False, return_stats=True)
+    m_sel = stats[:, 0].view(B, Hq, Lq, 1)
+    m_all = all_stats[:, 0].view(B, Hq, Lq, 1)
+    den = stats[:, 1].view(B, Hq, Lq, 1) * torch.exp(m_sel - m_all)
+    return out.transpose(1, 2).to(torch.float32), den, m_all
+
+
+def get_attention_denominator(module: Optional[nn.Module], queries: torch.Tensor, keys: torch.Tensor,
+                              attention_mask: Optional[torch.Tensor], scaling: float, dropout: float,
+                              sparse_attention_mask: Mask, **kwargs: Dict[str, Any]) -> torch.Tensor:
+    """sum_j exp(z_j - max_all z) / (w_j + 1e-6) over the mask's entries, (B, Hq, Lq, 1) fp32
+    (reference: mask_attention_utils.py:271-311). The kernel needs a value tensor: the keys stand in."""
+    _reject_training_dropout(module, dropout)
+    _, den, _ = _masked_softmax_parts(queries, keys, keys, attention_mask, scaling, sparse_attention_mask)
+    return den
+
+
+def get_attention_numerator(module: Optional[nn.Module], queries: torch.Tensor, keys: torch.Tensor, values: torch.Tensor,
+                            attention_mask: Optional[torch.Tensor], scaling: float, dropout: float,
+                            sparse_attention_mask: Mask, **kwargs: Dict[str, Any]) -> torch.Tensor:
+    """sum_j exp(z_j - max_all z) / (w_j + 1e-6) * V_j, (B, Hq, Lq, D) fp32 (reference :314-355). Rebuilt as the
+    kernel's normalised output times the denominator, so for bf16 / fp16 inputs it carries the output's rounding
+    (one part in 2^8 / 2^11) where the reference's fp32 product does not."""
+    _reject_training_dropout(module, dropout)
+    out, den, _ = _masked_softmax_parts(queries, keys, values, attention_mask, scaling, sparse_attention_mask)
+    return out * den
+
+
+def apply_sink_bias(num: torch.Tensor, den: torch.Tensor, exp_attention_weights: Optional[torch.Tensor],
+                    queries: torch.Tensor, keys: torch.Tensor, attention_mask: Optional[torch.Tensor],
+                    sinks: Optional[torch.Tensor], scaling: float):
+    """Adds one attention-sink logit per query head to a softmax given as (numerator, denominator[, exp weights])
+    in the all-key-maximum scale: everything is rescaled by exp(old_max - max(old_max, sink)) and the
+    denominator gains exp(sink - new_max) (reference :357-402). The all-key maximum comes from a dense pass of
+    the attention kernel; the rest is arithmetic on (B, Hq, Lq, 1) tensors."""
+    if sinks is None:
+        return num, den, exp_attention_weights
+    assert sinks.ndim == 1, f"sinks must be 1D tensor of shape [H], got {sinks.shape}"
+    B, H, Q = queries.shape[0], queries.shape[1], queries.shape[2]
+    _, stats = _run_attention(queries, keys, keys, attention_mask, None, scaling, None, False, return_stats=True)
+    old_max = stats[:, 0].view(B, H, Q, 1)
+    sinks_row = sinks.to(device=old_max.device, dtype=torch.float32).view(1, H, 1, 1).expand(B, H, Q, 1)
+    new_max = torch.maximum(old_max, sinks_row)
+    scale = torch.exp(old_max - new_max).to(den.dtype)
+    num = num * scale
+    den = den * scale
+    if exp_attention_weights is not None:
+        exp_attention_weights = exp_attention_weights * scale
+    den = den + torch.exp(sinks_row - new_max).to(den.dtype)
+    return num, den, exp_attention_weights
+
+
+def create_sampling_mask_with_per_head_budget(budgets: torch.Tensor, sampling_probability: torch.Tensor,
+                                              seq_len_keys: int, start_idx: int, end_idx: int,
+                                              dtype: torch.dtype = torch.float32, seed: Optional[int] = None,
+                                              offset: int = 0) -> Mask:
+    """Mask (B, H, Lq, seq_len_keys) in which row r holds the DISTINCT columns among `budgets[r]` uniform draws
+    (with replacement) from [start_idx, end_idx), each with weight `sampling_probability[r]` rounded to `dtype`
+    (reference: mask_attention_utils.py:105-184, one `sah_adaptive_sample` launch here, no host
+    synchronisation). The reference lists a column once per draw in its index form; every consumer
+    (dense conversion, merge) collapses such repeats to the one weight, which is what the rows hold here.
+    Draws are Philox4x32-10 with key `seed` (default torch.initial_seed()) and stream `offset`."""
+    if budgets.dim() != 4 or budgets.shape[-1] != 1 or sampling_probability.shape != budgets.shape:
+        raise ValueError(f"budgets and sampling_probability must both be (b, h, q, 1), got {tuple(budgets.shape)} "
+                         f"and {tuple(sampling_probability.shape)}")
+    N.require_device(budgets, "budgets")
+    B, H, Lq, _ = budgets.shape
+    n = int(end_idx) - int(start_idx)
+    if n <= 0 or start_idx < 0 or end_idx > seq_len_keys:
+        raise ValueError(f"sampling range [{start_idx}, {end_idx}) is outside the {seq_len_keys} keys")
+    dev = budgets.device
+    n_rows = B * H * Lq
+    rows = NativeRows(n_rows, int(seq_len_keys), n, dev, weighted=True)
+    rows.zero_if_fresh()
+    bud = budgets.reshape(n_rows).to(torch.int32).contiguous()
+    N.dtype_code(dtype)
+    prob = sampling_probability.reshape(n_rows).to(dtype).to(torch.float32).contiguous()
+    key = (torch.initial_seed() if seed is None else int(seed)) & 0xFFFFFFFFFFFFFFFF
+    N.call("sah_adaptive_sample", N.AdaptiveSampleArgs(
+        rows.as_struct(), bud.data_ptr(), prob.data_ptr(), N.dtype_code(dtype),
+        int(start_idx), n, key, int(offset), 1, N.stream_ptr(dev),
+    ))
+    rows.note_added(n, exact=False)
+    return Mask.create_mask_from_rows((B, H, Lq, int(seq_len_keys)), rows, dtype)

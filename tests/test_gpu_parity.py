@@ -185,6 +185,38 @@ def test_hash_topk_chain(cuda, dtype, use_amask):
     assert (ksig == sig.float()).float().mean().item() >= 0.9995
 
 
+def test_hash_masker_from_weight_file_matches_in_memory_weights(cuda, tmp_path):
+    """`hat_weight_file=` (the reference's pickle layout, hashattention_utils.py:155-180) through the kernels:
+    same codes, same selected sets, same output bits as `hat_weights=` with the tensors it was written from."""
+    import pickle
+
+    sa = _sa()
+    B, Hq, Hkv, Lk, D = 2, 8, 2, 900, 128
+    dtype = torch.bfloat16
+    wts = _hat(sa, Hq, D, dtype, hidden=128)
+    path = tmp_path / "hat_weights.pkl"
+    with open(path, "wb") as f:
+        pickle.dump(wts, f)
+    q, k, v = make_qkv(B, Hq, Hkv, 1, Lk, D, dtype, seed=12)
+    results = []
+    for source in (dict(hat_weights=wts), dict(hat_weight_file=str(path))):
+        cfg = sa.HashAttentionTopKMaskerConfig(heavy_size=96, hat_bits=32, hat_mlp_layers=3, hat_mlp_hidden_size=128,
+                                               hat_mlp_activation="silu", **source)
+        ra = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(
+            masker_configs=[sa.SinkMaskerConfig(sink_size=8), sa.LocalMaskerConfig(window_size=32), cfg]))
+        meta = {}
+        out, w = ra.custom_attention(None, q.to(cuda), k.to(cuda), v.to(cuda), None, D ** -0.5, 0.0,
+                                     sparse_meta_data=meta, layer_idx=0)
+        results.append((out.cpu(), w.cpu(), meta["key"][0].unpack(torch.float32).cpu()))
+    (o1, w1, s1), (o2, w2, s2) = results
+    assert torch.equal(s1, s2) and torch.equal(w1, w2) and torch.equal(o1, o2)
+    assert torch.all((w1 != 0).sum(-1) == 8 + 32 + 96)
+    with pytest.raises(ValueError):
+        sa.ResearchMasker.create_masker_from_config(sa.HashAttentionTopKMaskerConfig(
+            heavy_size=96, hat_bits=32, hat_mlp_layers=3, hat_mlp_hidden_size=128, hat_mlp_activation="silu",
+            hat_weights=wts, hat_weight_file=str(path)))
+
+
 def test_hash_signatures_bits_and_cache_growth(cuda):
     sa = _sa()
     from sparse_attention_hub_amd.sparse_attention.research_attention.maskers.fixed.implementations.hashattention_top_k import (

@@ -564,3 +564,44 @@ def test_usa_checkpoint_conversion_matches_the_linear_modules(tmp_path):
         for name in ("query_matrix", "query_bias", "key_matrix", "key_bias"):
             for a, b in zip(hat[layer][name], again[layer][name]):
                 assert torch.equal(a, b)
+
+
+def test_hat_weight_loader_runs_no_code_from_the_file(tmp_path):
+    # file format of the reference (utils/hashattention_utils.py:155-180): a pickle of Dict[layer] -> Dict[name] ->
+    # List[Tensor]. The loader resolves tensors and plain containers only.
+    import pickle
+
+    from sparse_attention_hub_amd.sparse_attention.utils.hashattention_utils import (
+        load_hat_weights, random_hat_weights, save_hat_weights)
+
+    w = random_hat_weights(2, 3, 8, 4, 2, 6, dtype=torch.bfloat16, seed=3)
+    w[1]["key_bias"][0] = torch.nn.Parameter(w[1]["key_bias"][0].float(), requires_grad=False)  # trained files hold these
+    good = tmp_path / "hat.pkl"
+    with open(good, "wb") as f:                      # written as the reference writes it: a bare pickle.dump
+        pickle.dump(w, f)
+    back = load_hat_weights(str(good))
+    assert sorted(back) == [0, 1]
+    for layer in w:
+        for name in w[layer]:
+            assert len(back[layer][name]) == len(w[layer][name])
+            for a, b in zip(back[layer][name], w[layer][name]):
+                assert a.dtype == b.dtype and torch.equal(a, b.detach())
+    save_hat_weights(w, str(tmp_path / "again.pkl"))
+    assert torch.equal(load_hat_weights(str(tmp_path / "again.pkl"))[0]["query_matrix"][1], w[0]["query_matrix"][1])
+
+    marker = tmp_path / "ran"
+
+    class Payload:
+        def __reduce__(self):
+            return (open, (str(marker), "w"))
+
+    bad = tmp_path / "bad.pkl"
+    with open(bad, "wb") as f:
+        pickle.dump({0: {"query_matrix": [Payload()]}}, f)
+    with pytest.raises(pickle.UnpicklingError, match="only plain containers of tensors"):
+        load_hat_weights(str(bad))
+    assert not marker.exists()
+    with open(bad, "wb") as f:
+        pickle.dump([1, 2, 3], f)
+    with pytest.raises(ValueError, match="expected Dict"):
+        load_hat_weights(str(bad))
