@@ -49,6 +49,10 @@ static inline int sah_launch_status(const char* what) {
   return SAH_OK;
 }
 
+// A kernel that wants more than 48 KB of dynamic LDS needs hipFuncAttributeMaxDynamicSharedMemorySize raised
+// once per (kernel, device). Thread-safe; remembers what has been done (defined with the row builders).
+int sah_allow_lds(const void* kernel, size_t bytes, const char* what);
+
 static inline int sah_check_rows(const sah_rows& r, const char* what, bool need_cols = true) {
   if (r.n_rows <= 0 || r.n_keys <= 0) return sah_fail(SAH_EINVAL, "%s: rows.n_rows/n_keys must be > 0", what);
   if (r.n_words != (r.n_keys + 31) / 32) return sah_fail(SAH_EINVAL, "%s: rows.n_words != ceil(n_keys/32)", what);

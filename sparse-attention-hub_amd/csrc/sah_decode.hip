@@ -177,12 +177,7 @@ static size_t hdec_lds_bytes(int n_keys) {
 
 template <int DT, bool MF, bool CP>
 static int hdec_launch_t(const sah_hash_decode_args* a, const hdec_params& P, size_t lds) {
-  static bool raised = false;
-  if (!raised) {
-    hipError_t e = hipFuncSetAttribute((const void*)k_hash_decode<DT, MF, CP>, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
-    if (e != hipSuccess) return sah_fail((int)e, "sah_hash_decode_topk: cannot raise the LDS limit: %s", hipGetErrorString(e));
-    raised = true;
-  }
+  if (int rc = sah_allow_lds((const void*)k_hash_decode<DT, MF, CP>, 150 * 1024, "sah_hash_decode_topk")) return rc;
   sah_timed timed("k_hash_decode", a->stream);
   hipLaunchKernelGGL((k_hash_decode<DT, MF, CP>), dim3(a->rows.n_rows), dim3(HSW_NT), lds, (hipStream_t)a->stream, P);
   return sah_launch_status("sah_hash_decode_topk");
@@ -316,12 +311,7 @@ extern "C" int sah_hash_decode_topk(const sah_hash_decode_args* a) {
 
 template <int DT, bool MF, bool CP, int D>
 static int hdec_attn_launch_t(const sah_hash_decode_args* a, const hdec_params& P, const att_params& A, size_t lds, int cols_offset) {
-  static bool raised = false;
-  if (!raised) {
-    hipError_t e = hipFuncSetAttribute((const void*)k_hash_decode_attn<DT, MF, CP, D>, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
-    if (e != hipSuccess) return sah_fail((int)e, "sah_hash_decode_attention: cannot raise the LDS limit: %s", hipGetErrorString(e));
-    raised = true;
-  }
+  if (int rc = sah_allow_lds((const void*)k_hash_decode_attn<DT, MF, CP, D>, 150 * 1024, "sah_hash_decode_attention")) return rc;
   const int G = A.Hq / A.Hkv;
   const int n_tiles = P.R.n_rows / G;
   const int n_wg = (n_tiles + ATT_XCDS - 1) / ATT_XCDS * ATT_XCDS * G;
@@ -350,7 +340,7 @@ extern "C" int sah_hash_decode_attention(const sah_hash_decode_args* a, const sa
       hdec_fusable(a) && A.n_split == 0 && !t->dense && !t->closed_form && !t->amask && !t->logits_out && !t->rows.w && t->Lq == 1 &&
       t->rows.cols == a->rows.cols && t->rows.cnt == a->rows.cnt && t->rows.cap == a->rows.cap &&
       t->rows.n_rows == a->rows.n_rows && t->stream == a->stream && t->dtype == a->query_sig->dtype &&
-      (t->D == 128 || t->D == 64) && lds <= 150 * 1024 && getenv("SAH_NO_FUSED_DECODE_ATTENTION") == nullptr;
+      (t->D == 128 || t->D == 64) && lds <= 150 * 1024;
   if (!one_kernel) {
     if ((rc = sah_hash_decode_topk(a))) return rc;
     return sah_sparse_attention(t);

@@ -289,12 +289,7 @@ static bool sig_mfma_ok(const sah_hash_sig_args* a) {
 
 template <int DT>
 static int sig_launch_mfma_t(const sah_hash_sig_args* a, const sig_params& P) {
-  static bool raised = false;
-  if (!raised) {
-    hipError_t e = hipFuncSetAttribute((const void*)k_hash_sig_mfma<DT>, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
-    if (e != hipSuccess) return sah_fail((int)e, "sah_hash_signatures: cannot raise the LDS limit: %s", hipGetErrorString(e));
-    raised = true;
-  }
+  if (int rc = sah_allow_lds((const void*)k_hash_sig_mfma<DT>, 150 * 1024, "sah_hash_signatures")) return rc;
   const int n_tiles = (a->L + SGM_TILE - 1) / SGM_TILE;
   const int tiles_per_wg = n_tiles < 8 ? n_tiles : 8;   // the staged weights serve up to 8 tiles
   const int n_chunks = (n_tiles + tiles_per_wg - 1) / tiles_per_wg;

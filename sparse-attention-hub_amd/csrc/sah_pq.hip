@@ -650,12 +650,7 @@ static size_t adc_lds_bytes(int lut_n) {
 
 template <int DT, bool OWN_LUT>
 static int adc_launch(const pq_adc_params& P, const void* lut, dim3 g, hipStream_t st) {
-  static bool raised = false;
-  if (!raised) {
-    hipError_t e = hipFuncSetAttribute((const void*)k_pq_adc<DT, OWN_LUT>, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
-    if (e != hipSuccess) return sah_fail((int)e, "sah_pq_adc_scores: cannot raise the LDS limit: %s", hipGetErrorString(e));
-    raised = true;
-  }
+  if (int rc = sah_allow_lds((const void*)k_pq_adc<DT, OWN_LUT>, 150 * 1024, "sah_pq_adc_scores")) return rc;
   hipLaunchKernelGGL((k_pq_adc<DT, OWN_LUT>), g, dim3(ADC_NT), adc_lds_bytes<DT>(P.n_sub * P.n_cent), st, P, lut);
   return SAH_OK;
 }

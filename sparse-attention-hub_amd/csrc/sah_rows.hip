@@ -78,6 +78,21 @@ extern "C" int sah_timing_collect(const char** names, int* counts, float* total_
   return n;
 }
 
+int sah_allow_lds(const void* kernel, size_t bytes, const char* what) {
+  static std::mutex mu;
+  static std::vector<std::pair<const void*, int>> done;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return sah_fail((int)e, "%s: hipGetDevice: %s", what, hipGetErrorString(e));
+  std::lock_guard<std::mutex> lk(mu);
+  for (const auto& d : done)
+    if (d.first == kernel && d.second == dev) return SAH_OK;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  if (e != hipSuccess) return sah_fail((int)e, "%s: cannot raise the dynamic LDS limit: %s", what, hipGetErrorString(e));
+  done.emplace_back(kernel, dev);
+  return SAH_OK;
+}
+
 extern "C" int sah_version(void) { return SAH_VERSION; }
 extern "C" const char* sah_last_error(void) { return g_err; }
 

@@ -402,17 +402,7 @@ __global__ __launch_bounds__(SF_NT) void k_select16(sah_rows R, const uint16_t* 
 template <typename K>
 static int sel_allow_lds(K kernel, size_t bytes, const char* what) {
   if (bytes <= 48 * 1024) return SAH_OK;
-  static thread_local const void* raised[8];  // one instantiation per kernel type: remember what is done
-  for (const void* p : raised)
-    if (p == (const void*)kernel) return SAH_OK;
-  hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 1024);
-  if (e != hipSuccess) return sah_fail((int)e, "%s: cannot raise the dynamic LDS limit: %s", what, hipGetErrorString(e));
-  for (const void*& p : raised)
-    if (!p) {
-      p = (const void*)kernel;
-      break;
-    }
-  return SAH_OK;
+  return sah_allow_lds((const void*)kernel, 160 * 1024 - 1024, what);
 }
 
 // Signature scores as sortable float keys, for callers that pass an additive

@@ -148,6 +148,10 @@ class DecodePlan:
         rows = self._rows_struct(Lk)
         chain = self.chain
         es = self.es
+        # what this step adds to the persistent caches (keys hashed, compacted, quantised) is recorded only after
+        # the native call has returned without an error: a refused call must not leave a cache that claims codes
+        # nobody wrote
+        commit = []
 
         sl = self.sink_local
         sl.rows, sl.lq, sl.sink, sl.window, sl.fresh, sl.clear_future, sl.stream = rows, Lq, sink, window, 1, 1, stream
@@ -211,7 +215,7 @@ class DecodePlan:
                         cp.exc, cp.exc_cap, cp.exc_cnt = cache.exc.data_ptr(), cache.exc.shape[2], cache.exc_cnt.data_ptr()
                         cp.full_plane, cp.stream = cache.full_plane, stream
                         chain.compact = C.addressof(cp)
-                        cache.n_compact = hashed
+                        commit.append((cache, "n_compact", hashed))
                     hd.pos_codes, hd.pos_pitch = cache.pos.data_ptr(), cache.pos.shape[2]
                     hd.exc, hd.exc_cap, hd.exc_cnt = cache.exc.data_ptr(), cache.exc.shape[2], cache.exc_cnt.data_ptr()
                     hd.full_plane = cache.full_plane
@@ -227,7 +231,7 @@ class DecodePlan:
                 hm.qcodes, hm.lq, hm.k, hm.stream = self.qcodes.data_ptr(), Lq, k_eff, stream
                 chain.hamming = C.addressof(hm)
             if hash_now:
-                cache.n = Lk
+                commit.append((cache, "n", Lk))
         elif self.kind == "oracle":
             self._ensure_keybuf(Lk)
             qa = self.qk
@@ -269,7 +273,7 @@ class DecodePlan:
                 pa.sums = pa.counts = pa.skip_flag = None
                 pa.round_dist, pa.stream = 1, stream
                 chain.pq_assign = C.addressof(pa)
-                book.n = current
+                commit.append((book, "n", current))
             self._ensure_keybuf(current)
             ad = self.pq_adc
             ad.q, ad.qs_b, ad.qs_h, ad.qs_l = q.data_ptr(), q.stride(0), q.stride(1), q.stride(2)
@@ -313,4 +317,6 @@ class DecodePlan:
         at.stream = stream
         chain.attention = C.addressof(at)
         N.call("sah_run_chain", chain)
+        for obj, name, value in commit:
+            setattr(obj, name, value)
         return out

@@ -11,7 +11,7 @@ device flag that turns the remaining launches into no-ops.
 """
 from __future__ import annotations
 
-from typing import Optional, Tuple
+from typing import Dict, Optional, Tuple
 
 import torch
 
@@ -117,6 +117,78 @@ def kmeans_keys_batched(
         )
         N.call("sah_pq_kmeans_update", u)
     return centres, shift2
+
+
+def kmeans_batched(
+    X: torch.Tensor,
+    num_clusters: int,
+    distance: str = "euclidean",
+    cluster_centers: Optional[torch.Tensor] = None,
+    tol: float = 1e-4,
+    tqdm_flag: bool = False,
+    iter_limit: int = 0,
+    device: Optional[torch.device] = None,
+    seed: Optional[int] = None,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Batched k-means of X (b, n, d) under the reference's own name and argument list (pq_utils.py:260-438):
+    returns (cluster choice (b, n) int64, centres (b, num_clusters, d) in X's dtype). Every group b is one
+    "sub-space" of a single-head key tensor for `kmeans_keys_batched`, so the same Lloyd kernels run.
+
+    Differences a caller can observe: codes are one byte in the kernels, so `num_clusters` is at most 256;
+    `iter_limit == 0` (the reference: until convergence) runs at most 300 iterations, each a no-op once every
+    group's squared centre shift has fallen below `tol`; the start is a seeded stratified sample of distinct
+    vectors (`seed`, default 0) instead of torch's global RNG; `device` is ignored (X stays where it is)."""
+    if X.ndim != 3:
+        raise ValueError(f"Expected 3D input (b, n, d), got {X.ndim}D tensor with shape {X.shape}")
+    if distance != "euclidean":
+        raise NotImplementedError(
+            f"Distance '{distance}' not yet implemented for batched k-means. Only 'euclidean' is supported.")
+    if not 1 <= num_clusters <= 256:
+        raise ValueError(f"num_clusters must be in [1, 256] (one-byte codes), got {num_clusters}")
+    b, n, d = X.shape
+    if d > 17 or b > 65535:
+        raise ValueError(f"the Lloyd kernels cluster up to 65535 groups of vectors of at most 17 dimensions, got b={b}, d={d}")
+    if cluster_centers is not None and tuple(cluster_centers.shape) != (b, num_clusters, d):
+        raise ValueError(
+            f"cluster_centers shape mismatch. Expected ({b}, {num_clusters}, {d}), got {tuple(cluster_centers.shape)}")
+    N.require_device(X, "X")
+    data = X if X.dtype in (torch.float32, torch.bfloat16, torch.float16) else X.float()
+    # (b, n, d) read as keys (B = b, one kv head, n keys, head_dim d) with ONE sub-space of width d
+    keys = data.contiguous().view(b, 1, n, d)
+    codes = torch.empty((b, 1, n, 1), dtype=torch.uint8, device=X.device)
+    centres, _ = kmeans_keys_batched(keys, 0, 1, num_clusters, iter_limit if iter_limit > 0 else 300, codes, n, 0, tol=tol,
+                                     cluster_centers=cluster_centers, seed=0 if seed is None else int(seed))
+    return codes.view(b, n).to(torch.int64), centres.to(X.dtype)
+
+
+def kmeans_batched_pytorch(data: torch.Tensor, k: int, max_iter: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(centroids (n_groups, k, d), codes (n_groups, n_samples) int64) — the reference's wrapper
+    (pq_utils.py:547-582) over `kmeans_batched`."""
+    codes, centroids = kmeans_batched(X=data, num_clusters=k, distance="euclidean", cluster_centers=None, tol=1e-4,
+                                      tqdm_flag=False, iter_limit=max_iter, device=data.device, seed=None)
+    return centroids, codes.long()
+
+
+def compute_reconstruction_errors(original_keys: torch.Tensor, centroids: torch.Tensor, codebook: torch.Tensor,
+                                  pq_sub_dim: int, use_ip_metric: bool = False) -> Dict[str, float]:
+    """mse / l2 / relative error of keys rebuilt from their codes (reference: pq_utils.py:643-705).
+    original_keys (B, H, n, D); centroids (B, H, n_sub, n_cent, d [+1 for the ip metric]); codebook
+    (B, n, H, n_sub) integer codes (the reference's layout; a `PQCodebook` is converted). A diagnostic, not on the
+    decode path: one gather with torch indexing."""
+    if hasattr(codebook, "to_reference"):
+        codebook = codebook.to_reference()
+    B, H, n, D = original_keys.shape
+    n_sub = D // pq_sub_dim
+    original = original_keys.transpose(1, 2).reshape(B, n, H, n_sub, pq_sub_dim)
+    cents = centroids[..., :pq_sub_dim] if use_ip_metric else centroids           # (B, H, n_sub, n_cent, d)
+    idx = codebook.to(torch.int64).permute(0, 2, 3, 1)                              # (B, H, n_sub, n)
+    rebuilt = torch.gather(cents, 3, idx.unsqueeze(-1).expand(-1, -1, -1, -1, cents.shape[-1]))   # (B, H, n_sub, n, d)
+    rebuilt = rebuilt.permute(0, 3, 1, 2, 4).to(original.dtype)
+    diff = original - rebuilt
+    l2 = torch.norm(diff.float()).item()
+    norm = torch.norm(original.float()).item()
+    return {"mse_error": torch.mean(diff.float() ** 2).item(), "l2_error": l2,
+            "relative_error": l2 / norm if norm > 0 else 0.0}
 
 
 def ip2l2_augment(xb: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
