@@ -49,8 +49,10 @@ def test_config3_step_is_one_kernel_and_matches_the_oracle(cuda):
     meta = {}
     kc, vc = k.to(cuda), v.to(cuda)
     scaling = D ** -0.5
-    # cold call on all but the last key: hashes them (general path); then the warm step on all keys
-    ra.custom_attention(None, q0.to(cuda), kc[:, :, :Lk - 1], vc[:, :, :Lk - 1], None, scaling, 0.0, sparse_meta_data=meta, layer_idx=0)
+    # cold call on all but the last two keys: hashes them (general path); a first decode step brings the compact
+    # code stream up to date (one more launch, once); then the warm step on all keys
+    for n in (Lk - 2, Lk - 1):
+        ra.custom_attention(None, q0.to(cuda), kc[:, :, :n], vc[:, :, :n], None, scaling, 0.0, sparse_meta_data=meta, layer_idx=0)
     torch.cuda.synchronize()
     N.timing_enable(True)
     out, _ = ra.custom_attention(None, q.to(cuda), kc, vc, None, scaling, 0.0, sparse_meta_data=meta, layer_idx=0)
@@ -65,7 +67,7 @@ def test_config3_step_is_one_kernel_and_matches_the_oracle(cuda):
     srt = torch.sort(cols, dim=1).values
     assert bool((srt[:, 1:] != srt[:, :-1]).all()) and int(cols.min()) == 0 and int(cols.max()) == Lk - 1
     cache = meta["key"][0]
-    assert cache.n == Lk - 1          # the newest key sits inside the local window: hashed with the next block of 64
+    assert cache.n == Lk - 2          # the newest keys sit inside the local window: hashed with the next block of 64
     # the query signatures, from the stand-alone signature kernel (same order of sums, same bits as inside the step)
     qcodes = torch.empty((B * Hq, 2), dtype=torch.int32, device=cuda)
     ra.maskers[2]._hash(q.to(cuda), Hq, Hq, 0, 1, 0, "query", qcodes, 1, 0)
