@@ -392,6 +392,18 @@ typedef struct sah_attention_args {
 int64_t sah_sparse_attention_work_floats(int32_t n_rows, int32_t max_cnt, int32_t D);
 int sah_sparse_attention(const sah_attention_args* a);
 
+/* sah_sparse_attention for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc). No counterpart in the reference. Same arguments
+ * and results, except that a->work / a->work_floats are ignored: the partial results of the split form go
+ * to a buffer of SAH_ATTENTION_STATIC_WORK_FLOATS floats (16 MiB) inside the library's device image, which
+ * every GPU the library runs on holds until the process ends. A call that needs more (see
+ * sah_sparse_attention_work_floats) returns SAH_ECAPACITY and launches nothing. The call allocates nothing
+ * and records no kernel timing. All calls on one GPU share the buffer: calls that overlap on one GPU
+ * (different streams, different threads) race; calls on one stream are ordered and safe. Nothing in the
+ * buffer needs to start at zero: every launch writes each partial result before its merge kernel reads it. */
+#define SAH_ATTENTION_STATIC_WORK_FLOATS (4 * 1024 * 1024)
+int sah_sparse_attention_static(const sah_attention_args* a);
+
 /* Dense attention probabilities (the second return value of
  * get_masked_attention_output, utils/mask_attention_utils.py:482-489):
  * weights[r, j] = round_to_dtype(exp(z - m) * inv_w / den) at the row's

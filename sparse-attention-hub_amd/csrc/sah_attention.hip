@@ -12,6 +12,8 @@
 #include "sah_common.h"
 #include "sah_attn.h"
 
+#include <mutex>
+
 template <int DT, int D, bool ROW>
 __global__ __launch_bounds__(ROW ? ATT_ROW_NT : ATT_NT, ROW ? 1 : 5) void k_sparse_attn(att_params P) {
   constexpr int NW = (ROW ? ATT_ROW_NT : ATT_NT) / SAH_WAVE;
@@ -94,11 +96,11 @@ extern "C" int64_t sah_sparse_attention_work_floats(int32_t n_rows, int32_t max_
 }
 
 template <int DT, int D>
-static int att_launch(const sah_attention_args* a, const att_params& P) {
+static int att_launch(const sah_attention_args* a, const att_params& P, bool timing) {
   hipStream_t st = (hipStream_t)a->stream;
   const int G = a->Hq / a->Hkv;
   if (P.n_split == 0) {  // whole-row form
-    sah_timed timed("k_sparse_attn", a->stream);
+    sah_timed timed("k_sparse_attn", a->stream, timing);
     const int n_tiles = a->rows.n_rows / G;
     const int n_wg = (n_tiles + ATT_XCDS - 1) / ATT_XCDS * ATT_XCDS * G;
     hipLaunchKernelGGL((k_sparse_attn<DT, D, true>), dim3(n_wg), dim3(ATT_ROW_NT), 0, st, P);
@@ -106,26 +108,26 @@ static int att_launch(const sah_attention_args* a, const att_params& P) {
   }
   int rc;
   {
-    sah_timed timed("k_sparse_attn", a->stream);
+    sah_timed timed("k_sparse_attn", a->stream, timing);
     const int n_tiles = (a->rows.n_rows / G) * P.n_split;
     const int n_wg = (n_tiles + ATT_XCDS - 1) / ATT_XCDS * ATT_XCDS * G;
     hipLaunchKernelGGL((k_sparse_attn<DT, D, false>), dim3(n_wg), dim3(ATT_NT), 0, st, P);
     rc = sah_launch_status("sah_sparse_attention");
   }
   if (rc) return rc;
-  sah_timed timed("k_attn_combine", a->stream);
+  sah_timed timed("k_attn_combine", a->stream, timing);
   hipLaunchKernelGGL((k_attn_combine<DT, D>), dim3(a->rows.n_rows), dim3(D < 64 ? 64 : D), 0, st,
                      (const float*)a->work, P.n_split, a->Hq, a->Lq, a->sinks, a->out, a->stats_out);
   return sah_launch_status("sah_sparse_attention(combine)");
 }
 
 template <int DT>
-static int att_dispatch_d(const sah_attention_args* a, const att_params& P) {
+static int att_dispatch_d(const sah_attention_args* a, const att_params& P, bool timing) {
   switch (a->D) {
-    case 16: return att_launch<DT, 16>(a, P);
-    case 32: return att_launch<DT, 32>(a, P);
-    case 64: return att_launch<DT, 64>(a, P);
-    case 128: return att_launch<DT, 128>(a, P);
+    case 16: return att_launch<DT, 16>(a, P, timing);
+    case 32: return att_launch<DT, 32>(a, P, timing);
+    case 64: return att_launch<DT, 64>(a, P, timing);
+    case 128: return att_launch<DT, 128>(a, P, timing);
     default: return sah_fail(SAH_ESHAPE, "sah_sparse_attention: head_dim %d not in {16,32,64,128}", a->D);
   }
 }
@@ -189,16 +191,64 @@ int att_prepare(const sah_attention_args* a, att_params& P) {
   return SAH_OK;
 }
 
+static int att_dispatch(const sah_attention_args* a, const att_params& P, bool timing) {
+  switch (a->dtype) {
+    case SAH_F32: return att_dispatch_d<SAH_F32>(a, P, timing);
+    case SAH_BF16: return att_dispatch_d<SAH_BF16>(a, P, timing);
+    case SAH_F16: return att_dispatch_d<SAH_F16>(a, P, timing);
+    default: return sah_fail(SAH_EDTYPE, "sah_sparse_attention: dtype %d", a->dtype);
+  }
+}
+
 extern "C" int sah_sparse_attention(const sah_attention_args* a) {
   att_params P;
   const int rc = att_prepare(a, P);
   if (rc) return rc;
-  switch (a->dtype) {
-    case SAH_F32: return att_dispatch_d<SAH_F32>(a, P);
-    case SAH_BF16: return att_dispatch_d<SAH_BF16>(a, P);
-    case SAH_F16: return att_dispatch_d<SAH_F16>(a, P);
-    default: return sah_fail(SAH_EDTYPE, "sah_sparse_attention: dtype %d", a->dtype);
+  return att_dispatch(a, P, true);
+}
+
+// ---------------------------------------------------------------------------
+// The same call for callers that cannot allocate: the partial results of the split form go to a buffer that
+// lives in the library's own device image instead of a workspace the caller would have to allocate.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) float scratch[SAH_ATTENTION_STATIC_WORK_FLOATS];
+
+// Device address of `scratch` on the current device. In host code the array's name is only a handle for
+// hipGetSymbolAddress; every GPU has its own copy at its own address, looked up once per device.
+static int att_static_work(float** out) {
+  static std::mutex mu;
+  static float* ptr[64];
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return sah_fail((int)e, "sah_sparse_attention_static: hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= 64) return sah_fail(SAH_EINVAL, "sah_sparse_attention_static: device index %d not in [0, 64)", dev);
+  std::lock_guard<std::mutex> lk(mu);
+  if (!ptr[dev]) {
+    float* p = nullptr;
+    e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p)
+      return sah_fail(e != hipSuccess ? (int)e : SAH_ENULL, "sah_sparse_attention_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    ptr[dev] = p;
   }
+  *out = ptr[dev];
+  return SAH_OK;
+}
+
+extern "C" int sah_sparse_attention_static(const sah_attention_args* a) {
+  if (!a) return sah_fail(SAH_ENULL, "sah_sparse_attention_static: args is NULL");
+  sah_attention_args b = *a;
+  int rc = att_static_work(&b.work);
+  if (rc) return rc;
+  b.work_floats = SAH_ATTENTION_STATIC_WORK_FLOATS;
+  att_params P;
+  rc = att_prepare(&b, P);
+  if (rc == SAH_ECAPACITY)
+    return sah_fail(SAH_ECAPACITY,
+                    "sah_sparse_attention_static: this call needs %lld workspace floats, the built-in buffer holds %lld; "
+                    "use sah_sparse_attention with a workspace of your own",
+                    (long long)b.rows.n_rows * P.n_split * (b.D + 2), (long long)SAH_ATTENTION_STATIC_WORK_FLOATS);
+  if (rc) return rc;
+  return att_dispatch(&b, P, false);  // no kernel timing here: recording it creates events
 }
 
 extern "C" int sah_attention_weights(const sah_attention_weights_args* a) {

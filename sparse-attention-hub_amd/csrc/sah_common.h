@@ -33,7 +33,8 @@ void sah_timing_end(hipStream_t st);
 struct sah_timed {
   hipStream_t st;
   bool on;
-  sah_timed(const char* name, void* stream) : st((hipStream_t)stream), on(sah_timing_enabled()) {
+  // allow = false: never time (entry points that must not create events)
+  sah_timed(const char* name, void* stream, bool allow = true) : st((hipStream_t)stream), on(allow && sah_timing_enabled()) {
     if (on) sah_timing_begin(name, st);
   }
   ~sah_timed() {

@@ -49,6 +49,7 @@ EXPECTED_SYMBOLS = (
     "sah_adaptive_sample",
     "sah_sparse_attention_work_floats",
     "sah_sparse_attention",
+    "sah_sparse_attention_static",
     "sah_attention_weights",
     "sah_run_chain",
 )
