@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Decode layer-step benchmark of the MI355X ResearchAttention path.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 1|2|3|4]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 1|2|3|4|5]
 
 A step is one `ResearchAttention.custom_attention` call with one query token on a warm
 cache (hash signatures / PQ codes of all earlier keys already built, one new key appended
@@ -9,13 +9,24 @@ per step), on synthetic inputs that are resident in HBM before the timed region.
 workload: BASELINE config 3, the one the headline target is quoted on (Sink 128 + Local 512
 + HashAttention top-2048, batch 8, 32 query / 8 KV heads, head_dim 128, 32768 keys, bf16).
 
+Timing. K steps are timed between two synchronisations (host clock and HIP events on the
+launch stream). That bracket is repeated back to back, on a context that keeps growing by
+one key per step, until the timed steps add up to a multiple of 64 and to at least 128:
+the HashAttention plan hashes new keys 64 at a time (one extra launch pair every 64 steps),
+so a multiple of 64 steps holds exactly its share of that work whatever K is. `value` is
+the mean over all timed steps; the median and minimum over the K-step brackets are
+reported beside it.
+
 Prints ONE JSON line: whole-step microseconds (`value`), the roofline of the dominant kernel
-from HIP-event timings taken inside this run, and the CPU oracle timed on the host cores.
+from HIP-event timings taken inside this run, the parity of the last timed step against the
+CPU oracle, the oracle timed on the host cores, and short sub-runs of the other BASELINE
+configurations (`other_configs`).
 """
 from __future__ import annotations
 
 import argparse
 import json
+import math
 import os
 import sys
 import time
@@ -27,6 +38,7 @@ for p in (ROOT, os.path.join(ROOT, "sparse-attention-hub_amd")):
 
 HBM_PEAK_GBS = 8000.0
 OUTLIER_CHANNELS = (7, 33, 71, 101)
+HASH_BLOCK = 64  # the decode plan hashes new keys this many at a time
 
 WORKLOADS = {
     1: dict(name="cfg1 Sink128+Local256 fp32 B1 Lk4096", B=1, Lk=4096, dtype="f32", sink=128, local=256, kind="none", k=0),
@@ -65,18 +77,21 @@ def algorithmic_bytes(w, sampled_per_row: float = 0.0) -> dict:
 
 
 def measured_traffic(kernel: str, cfg: int):
-    """HBM bytes per launch of `kernel` from the committed rocprofv3 PMC summary, if there is one."""
-    path = os.path.join(ROOT, "profiles", f"{kernel}_cfg{cfg}_hbm_traffic.txt")
+    """(HBM bytes per launch of `kernel`, file) from the committed rocprofv3 PMC summary, if there is one."""
+    rel = os.path.join("profiles", f"{kernel}_cfg{cfg}_hbm_traffic.txt")
     try:
-        for line in open(path):
+        for line in open(os.path.join(ROOT, rel)):
             if line.startswith("hbm_bytes_per_launch"):
-                return int(line.split("=")[1])
+                return int(line.split("=")[1]), rel
     except OSError:
         pass
-    return None
+    return None, None
 
 
-def build_workload(w, device, total_keys):
+def build_workload(w, device, total_keys, host_rng=True):
+    """The chain, 64 query sets and K / V of `total_keys` keys. `host_rng`: N(0, 1) drawn on the host with seed 0
+    and cast (the headline run, reproducible everywhere); otherwise drawn on the device (the short sub-runs: config 5
+    holds 2 x 2.1 G elements)."""
     import torch
 
     from sparse_attention_hub_amd.sparse_attention import (
@@ -86,14 +101,24 @@ def build_workload(w, device, total_keys):
     from sparse_attention_hub_amd.sparse_attention.utils.hashattention_utils import random_hat_weights
 
     dtype = torch.float32 if w["dtype"] == "f32" else torch.bfloat16
-    g = torch.Generator().manual_seed(0)
     B = w["B"]
-    k = torch.randn(B, HKV, total_keys, D, generator=g)
-    v = torch.randn(B, HKV, total_keys, D, generator=g)
-    if w.get("outliers"):
-        for c in OUTLIER_CHANNELS:
-            k[..., c] *= 8.0
-    qs = torch.randn(64, B, HQ, 1, D, generator=g)
+    if host_rng:
+        g = torch.Generator().manual_seed(0)
+        k = torch.randn(B, HKV, total_keys, D, generator=g)
+        v = torch.randn(B, HKV, total_keys, D, generator=g)
+        qs = torch.randn(64, B, HQ, 1, D, generator=g)
+        if w.get("outliers"):
+            for c in OUTLIER_CHANNELS:
+                k[..., c] *= 8.0
+        k, v, qs = k.to(dtype).to(device), v.to(dtype).to(device), qs.to(dtype).to(device)
+    else:
+        g = torch.Generator(device=device).manual_seed(0)
+        k = torch.randn(B, HKV, total_keys, D, generator=g, device=device, dtype=dtype)
+        v = torch.randn(B, HKV, total_keys, D, generator=g, device=device, dtype=dtype)
+        qs = torch.randn(64, B, HQ, 1, D, generator=g, device=device, dtype=dtype)
+        if w.get("outliers"):
+            for c in OUTLIER_CHANNELS:
+                k[..., c] *= 8.0
     cfgs = [SinkMaskerConfig(sink_size=w["sink"]), LocalMaskerConfig(window_size=w["local"])]
     extra = {}
     if w["kind"] == "oracle":
@@ -114,61 +139,210 @@ def build_workload(w, device, total_keys):
     if w.get("adaptive"):
         ra.maskers[-1].seed = 0
     ra.return_attention_weights = False  # HF attention modules drop the dense probabilities in decode
-    return ra, qs.to(dtype).to(device), k.to(dtype).to(device), v.to(dtype).to(device), extra
+    return ra, qs, k, v, extra
 
 
-def cpu_baseline(w, extra, ra_meta, k_dev, v_dev, q_dev, n_keys, budget_s=25.0):
-    """The reference algorithm (dense masks, repeat_kv, full-key fp32 softmax) as restated by the
-    oracle, timed on the host cores for ONE batch row and scaled by the batch size (rows are
-    independent); the warm caches are taken from the GPU run so only the layer-step is timed."""
-    import torch
+def repeats_for(steps: int) -> int:
+    """Number of K-step brackets so that the timed steps are a multiple of 64 and at least 128."""
+    reps = HASH_BLOCK // math.gcd(steps, HASH_BLOCK)
+    while steps * reps < 2 * HASH_BLOCK:
+        reps *= 2
+    return reps
 
-    from oracle import reference_path as O
 
-    cores = os.cpu_count() or 1
-    torch.set_num_threads(cores)
-    q = q_dev[:1].cpu()
-    k = k_dev[:1, :, :n_keys].cpu()
-    v = v_dev[:1, :, :n_keys].cpu()
+def median(xs):
+    s = sorted(xs)
+    return s[len(s) // 2] if len(s) % 2 else 0.5 * (s[len(s) // 2 - 1] + s[len(s) // 2])
+
+
+class Run:
+    """One workload on the GPU: cold call, warm-up, timed brackets; keeps the last step's output and rows."""
+
+    def __init__(self, w, dev, steps, warm, reps, probe, host_rng):
+        import torch
+
+        self.torch = torch
+        self.w, self.dev, self.steps, self.warm, self.reps, self.probe = w, dev, steps, warm, reps, probe
+        self.total = steps * reps
+        self.first = w["Lk"] - (warm + self.total)         # the last timed step runs at exactly Lk keys
+        if self.first <= w["sink"] + w["local"] + w["k"] + 512:
+            raise SystemExit(f"bench.py: {warm} + {self.total} steps do not fit below {w['Lk']} keys")
+        self.ra, self.qs, self.k, self.v, self.extra = build_workload(w, dev, w["Lk"] + probe, host_rng)
+        self.meta = {}
+        self.scaling = D ** -0.5
+
+    def step(self, i, n_keys):
+        return self.ra.custom_attention(None, self.qs[i % self.qs.shape[0]], self.k[:, :, :n_keys], self.v[:, :, :n_keys], None,
+                                        self.scaling, 0.0, sparse_meta_data=self.meta, layer_idx=0)
+
+    def cold(self):
+        torch = self.torch
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        self.step(0, self.first)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3
+
+    def timed(self):
+        """(wall ms per bracket, HIP-event ms per bracket, host launch-loop ms per bracket)."""
+        torch = self.torch
+        for i in range(self.warm):
+            self.step(i, self.first + 1 + i)
+        torch.cuda.synchronize()
+        wall, gpu, host = [], [], []
+        n = self.first + self.warm
+        for _ in range(self.reps):
+            ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            ev0.record()
+            for i in range(self.steps):
+                n += 1
+                self.last_q = i % self.qs.shape[0]
+                self.last_out, _ = self.step(i, n)
+            ev1.record()
+            t1 = time.perf_counter()
+            torch.cuda.synchronize()
+            t2 = time.perf_counter()
+            wall.append((t2 - t0) * 1e3)
+            host.append((t1 - t0) * 1e3)
+            gpu.append(ev0.elapsed_time(ev1))
+        assert n == self.w["Lk"]
+        return wall, gpu, host
+
+    def last_rows(self):
+        """(cols int32 [R, cap], cnt int32 [R]) of the last step's mask, or None when no row list was written."""
+        if self.w.get("adaptive"):
+            rows = self.ra.maskers[-1].last_rows
+            return rows.cols, rows.cnt
+        plan = next(iter(self.ra._plans.values()), None)
+        if plan is None or plan.cols is None or self.w["kind"] == "none":
+            return None
+        return plan.cols, plan.cnt
+
+    def instrumented(self):
+        """Per-kernel durations: HIP events around every launch, `probe` more steps on the same buffers."""
+        from sparse_attention_hub_amd import _native as N
+
+        N.timing_enable(True)
+        for i in range(self.probe):
+            self.step(i, self.w["Lk"] + 1 + i)
+        self.torch.cuda.synchronize()
+        kt = N.timing_collect()
+        N.timing_enable(False)
+        return {name: dict(launches=c, avg_us=1e3 * ms / c) for name, (c, ms) in kt.items()}
+
+
+def oracle_specs(run, n_keys, n_hashed):
+    """Masker specs and warm state (one batch row) for `oracle.reference_path.research_attention`."""
+    w, extra, meta = run.w, run.extra, run.meta
     specs = [("sink", w["sink"]), ("local", w["local"])]
     state = {}
     if w["kind"] == "oracle":
         specs.append(("oracle_topk", w["k"]))
     elif w["kind"] == "hash":
         specs.append(("hash_topk", w["k"], extra["hat_weights"][0], "silu"))
-        cache = ra_meta["key"][0]
-        sub = type(cache).__new__(type(cache))            # one batch row, the n_keys - 1 earlier keys
-        sub.bits, sub.n, sub.codes = cache.bits, n_keys - 1, cache.codes[:1]
-        state["key_sig"] = sub.unpack(q.dtype).cpu()
+        cache = meta["key"][0]
+        sub = type(cache).__new__(type(cache))            # one batch row, the keys hashed when the step ran
+        sub.bits, sub.n, sub.codes = cache.bits, n_hashed, cache.codes[:1]
+        state["key_sig"] = sub.unpack(run.qs.dtype).cpu()
     elif w["kind"] == "pq":
-        cent = ra_meta["pq_centroids"][0][:1].cpu()
-        book = ra_meta["pq_codebook"][0].to_reference()[:1, : n_keys - w["sink"]].cpu()
+        cent = meta["pq_centroids"][0][:1].cpu()
+        book = meta["pq_codebook"][0].to_reference()[:1, : n_keys - w["sink"]].cpu()
         specs.append(("pq_topk", w["k"], w["sink"], cent, book))
     if w.get("adaptive"):
         a = w["adaptive"]
         specs.append(("adaptive", a["rate"], a["epsilon"], a["delta"], w["sink"], w["local"], 0, 0))
+    return specs, state
+
+
+def parity_and_cpu_baseline(run, last, budget_s=25.0):
+    """The reference algorithm (dense masks, repeat_kv, full-key fp32 softmax) as restated by the oracle, on ONE
+    batch row of the last timed step: first as the checker of that step's output and selected columns, then timed
+    on the host cores and scaled by the batch size (batch rows are independent). Warm caches (key signatures / PQ
+    codes) are the GPU run's, so only the layer-step is restated."""
+    import torch
+
+    from oracle import reference_path as O
+
+    w = run.w
+    n_keys = w["Lk"]
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    q = run.qs[last["q"]][:1].cpu()
+    k = run.k[:1, :, :n_keys].cpu()
+    v = run.v[:1, :, :n_keys].cpu()
+    specs, state = oracle_specs(run, n_keys, last["n_hashed"])
+    if w["kind"] == "hash":
+        # the query's signature bits as the kernels compute them (a float MLP on the host may round a borderline
+        # output to the other side of zero)
+        qcodes = torch.empty((HQ, 2), dtype=torch.int32, device=run.dev)
+        run.ra.maskers[2]._hash(run.qs[last["q"]][:1], HQ, HQ, 0, 1, 0, "query", qcodes, 1, 0)
+        c = qcodes.cpu().to(torch.int64) & 0xFFFFFFFF
+        shifts = torch.arange(32)
+        state["query_sig"] = ((((c[:, 0:1] >> shifts) & 1) * 2 - 1) * ((c[:, 1:2] >> shifts) & 1)).to(q.dtype).view(1, HQ, 1, 32)
+    parity = None
     times = []
     t_all = time.perf_counter()
     for it in range(12):
         st = dict(state)
         t0 = time.perf_counter()
-        O.research_attention(specs, q, k, v, None, D ** -0.5, state=st)
+        oo, _, om = O.research_attention(specs, q, k, v, None, D ** -0.5, state=st)
         times.append(time.perf_counter() - t0)
+        if parity is None and not w.get("adaptive"):
+            got = last["out"][:1].float().cpu()
+            err = ((got - oo.float()).norm() / oo.float().norm()).item()
+            parity = dict(rel_err=float(f"{err:.3e}"), tolerance=1e-5 if w["dtype"] == "f32" else 2e-2,
+                          rows_checked=f"batch row 0 ({HQ} of {w['B'] * HQ} mask rows) of the last timed step")
+            if last["cols"] is not None:
+                want = om.to_dense()[0, :, 0] != 0
+                member = torch.zeros_like(want)
+                cols, cnt = last["cols"][:HQ].long().cpu(), last["cnt"][:HQ].long().cpu()
+                for r in range(HQ):
+                    member[r, cols[r, : cnt[r]]] = True
+                parity["index_sets_equal"] = bool(torch.equal(member, want))
+                parity["index_set_overlap"] = round(float((member & want).sum()) / float(want.sum()), 6)
         if time.perf_counter() - t_all > budget_s and it >= 1:
             break
-    per_row = sorted(times[1:] or times)[len(times[1:] or times) // 2]
-    return dict(value=per_row * w["B"] * 1e6, unit="us/layer-step", cores=cores, kind="port",
+    per_row = median(times[1:] or times)
+    base = dict(value=per_row * w["B"] * 1e6, unit="us/layer-step", cores=cores, kind="port",
                 sample=f"oracle (torch-CPU restatement of the reference path) on 1 of {w['B']} batch rows, "
                        f"median of {max(1, len(times) - 1)} warm steps x {w['B']}; torch threads={cores}")
+    return parity, base
+
+
+def sub_run(cfg: int, dev) -> dict:
+    """A short run of another BASELINE configuration: cold call, 5 warm-up steps, one bracket of timed steps."""
+    import torch
+
+    w = dict(WORKLOADS[cfg])
+    steps = 24 if cfg == 5 else 64
+    run = Run(w, dev, steps, 5, 1, 0, host_rng=False)
+    cold_ms = run.cold()
+    wall, gpu, _ = run.timed()
+    sampled = 0.0
+    if w.get("adaptive"):
+        sampled = float(run.ra.maskers[-1].last_rows.cnt.float().mean().item()) - (w["sink"] + w["local"] + w["k"])
+    ab = algorithmic_bytes(w, sampled)["step"]
+    us, gpu_us = wall[0] / steps * 1e3, gpu[0] / steps * 1e3
+    out = dict(workload=w["name"], us=round(us, 2), gpu_us=round(gpu_us, 2), steps=steps, algorithmic_bytes=ab,
+               achieved_GBps=round(ab / (gpu_us * 1e-6) / 1e9, 1), frac=round(ab / (gpu_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+               cold_call_ms=round(cold_ms, 2), data="synthetic, drawn on the device")
+    if w.get("adaptive"):
+        out["keys_per_row"] = round(w["sink"] + w["local"] + w["k"] + sampled, 1)
+    del run
+    torch.cuda.empty_cache()
+    return out
 
 
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", type=int, default=3, choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true", help="skip the short sub-runs of the other configurations")
     ap.add_argument("--batch", type=int, default=0, help="study only: override the workload's batch size")
     ap.add_argument("--keys", type=int, default=0, help="study only: override the workload's key count")
     ap.add_argument("--pmc-probe", action="store_true",
@@ -188,32 +362,20 @@ def main() -> None:
     N.lib()
     dev = torch.device("cuda:0")
     w = dict(WORKLOADS[args.config])
-    if args.batch or args.keys:
+    study = bool(args.batch or args.keys)
+    if study:
         w["B"] = args.batch or w["B"]
         w["Lk"] = args.keys or w["Lk"]
         w["name"] += f" [size override: B={w['B']} Lk={w['Lk']}]"
     steps, warm = args.steps, args.warmup
-    probe = max(20, min(steps, 100))                      # instrumented steps for the per-kernel roofline
-    total_keys = w["Lk"] + probe
-    first = w["Lk"] - (warm + steps)                      # the last timed step runs at exactly Lk keys
-    ra, qs, k, v, extra = build_workload(w, dev, total_keys)
-    meta = {}
-    scaling = D ** -0.5
-
-    def step(i, n_keys):
-        return ra.custom_attention(None, qs[i % qs.shape[0]], k[:, :, :n_keys], v[:, :, :n_keys], None, scaling, 0.0,
-                                   sparse_meta_data=meta, layer_idx=0)
-
-    # cold call: builds all signatures / runs k-means; reported apart
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    step(0, first)
-    torch.cuda.synchronize()
-    cold_ms = (time.perf_counter() - t0) * 1e3
+    reps = repeats_for(steps)
+    probe = 2 * HASH_BLOCK                                # instrumented steps for the per-kernel durations
+    run = Run(w, dev, steps, warm, reps, probe, host_rng=True)
+    cold_ms = run.cold()
 
     if args.pmc_probe:
         for i in range(5):
-            step(i, first + 1 + i)
+            run.step(i, run.first + 1 + i)
         src = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device=dev).fill_(1)
         dst = torch.empty_like(src)
         for _ in range(3):
@@ -222,56 +384,50 @@ def main() -> None:
         print(json.dumps({"pmc_probe": True, "copy_bytes": src.numel(), "steps": 5}))
         return
 
-    for i in range(warm):
-        step(i, first + 1 + i)
-    torch.cuda.synchronize()
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    ev0.record()
-    for i in range(steps):
-        step(i, first + warm + 1 + i)
-    ev1.record()
-    host_ms = (time.perf_counter() - t0) * 1e3          # launch loop only: host cost when the GPU keeps up
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3
-    gpu_ms = ev0.elapsed_time(ev1)
-    ms_per_step = wall_ms / steps
+    wall, gpu, host = run.timed()
+    total = run.total
+    ms_per_step = sum(wall) / total
+    gpu_ms_per_step = sum(gpu) / total
+    rows = run.last_rows()
+    cache = run.meta.get("key", {}).get(0) if w["kind"] == "hash" else None
+    last = dict(out=run.last_out, q=run.last_q, n_hashed=getattr(cache, "n", 0),
+                cols=None if rows is None else rows[0].clone(), cnt=None if rows is None else rows[1].clone())
 
-    # per-kernel durations, HIP events on the launch stream, same process, same buffers
-    N.timing_enable(True)
-    for i in range(probe):
-        step(i, w["Lk"] + 1 + i)
-    torch.cuda.synchronize()
-    kt = N.timing_collect()
-    N.timing_enable(False)
-    kernels = {name: dict(launches=c, avg_us=1e3 * ms / c) for name, (c, ms) in kt.items()}
+    kernels = run.instrumented()
     sampled = 0.0
     if w.get("adaptive"):
         # mean entries per row after the last step, minus what the fixed maskers put there
-        sampled = float(ra.maskers[-1].last_rows.cnt.float().mean().item()) - (w["sink"] + w["local"] + w["k"])
+        sampled = float(run.ra.maskers[-1].last_rows.cnt.float().mean().item()) - (w["sink"] + w["local"] + w["k"])
     ab = algorithmic_bytes(w, sampled)
+    periodic = {n: d for n, d in kernels.items() if n in ("k_hash_sig_small_mfma", "k_hash_sig_gemv", "k_hash_compact")}
+    amortised_hash_us = sum(d["avg_us"] * d["launches"] for d in periodic.values()) / probe
     # the dominant kernel: the attention kernel, or - when selection and attention of a step run as one
     # kernel - that kernel, whose algorithmic bytes are then the whole step's
     if "k_hash_decode_attn" in kernels:
+        # One launch per step: the event pair around K back-to-back steps times K launches without the gaps an event
+        # pair around every single launch adds. The brackets hold exactly their share of the periodic hashing
+        # launches (one pair every 64 steps), which stays inside this figure: it errs on the long side.
         dom, dom_bytes = "k_hash_decode_attn", ab["step"]
+        dom_us = gpu_ms_per_step * 1e3
+        timing = ("HIP events around each bracket of K back-to-back steps / K, mean over all brackets (one launch per step; "
+                  "includes the amortised new-key hashing launches)")
+        del kernels[dom]                                  # per-launch event pairs measure launch gaps for this one
     else:
         dom, dom_bytes = "k_sparse_attn", ab["attention_kernel"]
-    dom_us = kernels[dom]["avg_us"]
-    timing = "HIP events around every launch"
-    if dom == "k_hash_decode_attn":
-        # One launch per step: the event pair around the K back-to-back steps of the timed region times K launches
-        # without the launch gaps an event pair around each single launch adds. The rare hashing launches of the
-        # region (one pair every 64 steps) stay inside this figure, which therefore errs on the long side.
-        dom_us = gpu_ms * 1e3 / steps
-        timing = "HIP events around the timed region / steps (one launch per step)"
+        dom_us = kernels[dom]["avg_us"]
+        timing = "HIP events around every launch"
     achieved = dom_bytes / (dom_us * 1e-6) / 1e9
+    traffic, traffic_file = measured_traffic(dom, args.config)
     roofline = dict(bound="hbm", kernel=dom, achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s",
-                    frac=round(achieved / HBM_PEAK_GBS, 4), traffic=measured_traffic(dom, args.config),
+                    frac=round(achieved / HBM_PEAK_GBS, 4), traffic=None if study else traffic,
+                    traffic_source=None if study or traffic is None else f"{traffic_file} (rocprofv3 --pmc run of this workload, committed; not re-measured here)",
                     algorithmic_bytes_per_launch=dom_bytes, avg_launch_us=round(dom_us, 2), timing=timing)
     step_gbs = ab["step"] / (ms_per_step * 1e-3) / 1e9
+    per_bracket_us = [x / steps * 1e3 for x in wall]
+    per_bracket_gpu_us = [x / steps * 1e3 for x in gpu]
 
     out = {
-        "metric": "sparse decode us/layer-step at 32K ctx; achieved HBM GB/s vs peak",
+        "metric": "sparse decode \u00b5s/layer-step at 32K/128K ctx; achieved HBM GB/s vs peak",
         "value": round(ms_per_step * 1e3, 2),
         "unit": "us/layer-step",
         "n_gpus": 1,
@@ -285,17 +441,33 @@ def main() -> None:
         "data": "synthetic",
         "config": {"workload": w["name"], "q_heads": HQ, "kv_heads": HKV, "head_dim": D, "batch": w["B"], "keys": w["Lk"],
                    "keys_per_row": round(w["sink"] + w["local"] + w["k"] + sampled, 1), "attention_weights_output": False},
-        "gpu_ms_per_step": round(gpu_ms / steps, 5),
-        "host_launch_ms_per_step": round(host_ms / steps, 5),
+        "timed_steps_total": total,
+        "brackets": reps,
+        "median_us": round(median(per_bracket_us), 2),
+        "min_us": round(min(per_bracket_us), 2),
+        "gpu_ms_per_step": round(gpu_ms_per_step, 5),
+        "gpu_median_us": round(median(per_bracket_gpu_us), 2),
+        "gpu_min_us": round(min(per_bracket_gpu_us), 2),
+        "host_launch_ms_per_step": round(sum(host) / total, 5),
         "step_algorithmic_bytes": ab["step"],
         "step_achieved_GBps": round(step_gbs, 1),
         "step_frac_of_hbm_peak": round(step_gbs / HBM_PEAK_GBS, 4),
         "cold_call_ms": round(cold_ms, 2),
+        "amortised_hash_us": round(amortised_hash_us, 3),
         "kernels_avg_us": {n: round(d["avg_us"], 2) for n, d in sorted(kernels.items())},
+        "kernels_avg_us_note": "HIP events around every single launch (they include the event markers' own gaps)",
         "roofline": roofline,
     }
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(w, extra, meta, k, v, qs[0], w["Lk"])
+        out["parity"], out["cpu_baseline"] = parity_and_cpu_baseline(run, last)
+    if not args.no_other_configs and not study:
+        del run, last, rows
+        torch.cuda.empty_cache()
+        others = {}
+        for cfg in sorted(WORKLOADS):
+            if cfg != args.config:
+                others[f"cfg{cfg}"] = sub_run(cfg, dev)
+        out["other_configs"] = others
     print(json.dumps(out))
 
 
