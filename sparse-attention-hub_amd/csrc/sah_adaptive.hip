@@ -102,6 +102,7 @@ struct ad_budget_params {
 
 template <int DT>
 __global__ __launch_bounds__(AD_NT) void k_adaptive_budget(ad_budget_params P) {
+  sah_touch_kernargs<sizeof(ad_budget_params)>();
   HIP_DYNAMIC_SHARED(uint32_t, s_bits)  // one bit per column of the sampling range (word aligned)
   __shared__ float s_red[AD_NW];
   const int tid = threadIdx.x;
@@ -267,6 +268,7 @@ struct ad_sample_params {
 
 template <int DT>
 __global__ __launch_bounds__(AD_NT) void k_adaptive_sample(ad_sample_params P) {
+  sah_touch_kernargs<sizeof(ad_sample_params)>();
   HIP_DYNAMIC_SHARED(uint32_t, s_bits)
   __shared__ int s_scan[AD_NW + 1];
   const int tid = threadIdx.x;

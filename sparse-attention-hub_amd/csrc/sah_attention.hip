@@ -16,6 +16,7 @@
 
 template <int DT, int D, bool ROW>
 __global__ __launch_bounds__(ROW ? ATT_ROW_NT : ATT_NT, ROW ? 1 : 5) void k_sparse_attn(att_params P) {
+  sah_touch_kernargs<sizeof(att_params)>();
   constexpr int NW = (ROW ? ATT_ROW_NT : ATT_NT) / SAH_WAVE;
   __shared__ float s_m[NW];
   __shared__ float s_l[NW];

@@ -63,6 +63,28 @@ static inline int sah_check_rows(const sah_rows& r, const char* what, bool need_
 }
 
 // ---------------------------------------------------------------------------
+// device side: kernel arguments
+// ---------------------------------------------------------------------------
+// A kernel's arguments live in memory and are fetched by scalar loads where the code first needs them. Each
+// first touch of a 64-byte line is a round trip of about 500 cycles, and the compiler chains them (a load, a
+// wait, the next load ...) along the kernel's control flow: 5 to 6 round trips before the first vector load of a
+// kernel with a 700-byte argument block. Called first thing in a kernel, this reads one word of every line of
+// the first BYTES of the block in ONE batch; the real loads that follow hit the scalar cache.
+template <int BYTES>
+__device__ __forceinline__ void sah_touch_kernargs() {
+  static_assert(BYTES <= 1024, "at most 16 lines");
+  typedef const int __attribute__((address_space(4))) karg_int;
+  karg_int* p = (karg_int*)__builtin_amdgcn_kernarg_segment_ptr();
+  // word o of line i, or of line 0 again when the block is shorter; one sink for all of them, so that every
+  // load is issued before the one wait
+#define SAH_KARG(i) p[(64 * (i) < BYTES ? 16 * (i) : 0)]
+  asm volatile("" ::"s"(SAH_KARG(0)), "s"(SAH_KARG(1)), "s"(SAH_KARG(2)), "s"(SAH_KARG(3)), "s"(SAH_KARG(4)), "s"(SAH_KARG(5)),
+               "s"(SAH_KARG(6)), "s"(SAH_KARG(7)), "s"(SAH_KARG(8)), "s"(SAH_KARG(9)), "s"(SAH_KARG(10)), "s"(SAH_KARG(11)),
+               "s"(SAH_KARG(12)), "s"(SAH_KARG(13)), "s"(SAH_KARG(14)), "s"(SAH_KARG(15)));
+#undef SAH_KARG
+}
+
+// ---------------------------------------------------------------------------
 // device side: dtype helpers (bf16 / f16 handled as raw bits, fp32 arithmetic)
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ float sah_bits_to_float(uint32_t u) { return __builtin_bit_cast(float, u); }

@@ -137,6 +137,7 @@ __device__ __forceinline__ int hdec_row(const hdec_params& P, int r, hsw_lds& S,
 
 template <int DT, bool MF, bool CP>
 __global__ __launch_bounds__(HSW_NT) void k_hash_decode(hdec_params P) {
+  sah_touch_kernargs<sizeof(hdec_params)>();
   __shared__ hsw_lds S;
   HIP_DYNAMIC_SHARED(unsigned char, hdec_dyn)
   hdec_row<DT, MF, CP>(P, blockIdx.x, S, hdec_dyn, nullptr);
@@ -154,6 +155,7 @@ __global__ __launch_bounds__(HSW_NT) void k_hash_decode_attn(hdec_params P, att_
   __shared__ float s_l[HSW_NW];
   __shared__ float s_acc[HSW_NW][D];
   HIP_DYNAMIC_SHARED(unsigned char, hdec_dyn)
+  sah_touch_kernargs<sizeof(hdec_params) + sizeof(att_params) + 8>();
   const int G = A.Hq / A.Hkv;
   const int slot = blockIdx.x / ATT_XCDS;
   const int tile = (slot / G) * ATT_XCDS + (int)(blockIdx.x % ATT_XCDS);  // b * Hkv + hk

@@ -304,6 +304,7 @@ static int sig_launch_mfma_t(const sah_hash_sig_args* a, const sig_params& P) {
 // decode-size jobs on the matrix cores: up to 16 vectors of one head per workgroup
 template <int DT>
 __global__ __launch_bounds__(SMB_NT) void k_hash_sig_small_mfma(sig_pair PP) {
+  sah_touch_kernargs<(sizeof(sig_pair) < 1024 ? sizeof(sig_pair) : 1024)>();
   const sig_params& P = PP.p[blockIdx.z];
   if ((int)blockIdx.x * 16 >= P.L) return;  // the two jobs may differ in vector count
   __shared__ sig_mfma_lds S;

@@ -132,6 +132,7 @@ __global__ __launch_bounds__(PQ_NT) void k_pq_assign(pq_assign_params P) {
 // one-thread-per-key kernel above.
 template <int DT>
 __global__ __launch_bounds__(PQ_NT) void k_pq_assign_few(pq_assign_params P) {
+  sah_touch_kernargs<sizeof(pq_assign_params)>();
   __shared__ float s_d[PQ_NT / SAH_WAVE];
   __shared__ int s_i[PQ_NT / SAH_WAVE];
   const int tid = threadIdx.x;
@@ -480,6 +481,7 @@ __global__ __launch_bounds__(PQ_NT) void k_pq_lut(pq_adc_params P, void* lut) {
 // covered by a few dozen workgroups); otherwise the 8-byte entries k_pq_lut wrote are widened on the way in.
 template <int DT, bool OWN_LUT>
 __global__ __launch_bounds__(ADC_NT) void k_pq_adc(pq_adc_params P, const void* lut) {
+  sah_touch_kernargs<sizeof(pq_adc_params) + 8>();
   constexpr int NQ = (DT == SAH_F32) ? 2 : 4;
   typedef typename std::conditional<DT == SAH_F32, uint32_t, uint16_t>::type key_t;
   typedef typename std::conditional<DT == SAH_F32, float2, float4>::type entry_t;

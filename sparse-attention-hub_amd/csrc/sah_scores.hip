@@ -122,6 +122,7 @@ __device__ __forceinline__ float sc_reduce4(float d0, float d1, float d2, float 
 
 template <int DT, int D>
 __global__ __launch_bounds__(SC_NT) void k_qk_scores(qk_params P) {
+  sah_touch_kernargs<sizeof(qk_params)>();
   constexpr int LPK = D / 8;
   constexpr int KPI = SAH_WAVE / LPK;
   constexpr int IT = SAH_WAVE / KPI;
