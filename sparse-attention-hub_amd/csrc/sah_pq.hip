@@ -194,6 +194,72 @@ __global__ __launch_bounds__(PQ_NT) void k_pq_assign_few(pq_assign_params P) {
   }
 }
 
+// A block of new keys (up to a few hundred) against frozen centres: one workgroup per (sub-space, batch x KV head)
+// stages the group's centres in LDS once; a wave takes every 4th key, its lanes share the centres out
+// (lane, lane + 64, ...), and the argmin of a key is a wave reduction: no workgroup barrier per key. Same
+// arithmetic per (key, centre) pair as k_pq_assign_few, same "first minimum" rule.
+#define PQB_NT 1024
+template <int DT>
+__global__ __launch_bounds__(PQB_NT) void k_pq_assign_block(pq_assign_params P) {
+  sah_touch_kernargs<sizeof(pq_assign_params)>();
+  __shared__ float s_c[PQ_MAX_CENT * PQ_MAX_D];
+  const int tid = threadIdx.x;
+  const int lane = tid & (SAH_WAVE - 1);
+  const int wave = tid / SAH_WAVE;
+  const int s = blockIdx.x;
+  const int bh = blockIdx.y;
+  const int hk = bh % P.Hkv;
+  const int b = bh / P.Hkv;
+  const int g = bh * P.n_sub + s;
+  const int d_sub = P.d_sub, n_cent = P.n_cent;
+  for (int i = tid; i < n_cent * d_sub; i += PQB_NT) s_c[i] = P.centres[(int64_t)g * n_cent * d_sub + i];
+  __syncthreads();
+  for (int n = wave; n < P.n_keys; n += PQB_NT / SAH_WAVE) {
+    const int64_t off = (int64_t)b * P.ks_b + (int64_t)hk * P.ks_h + (int64_t)s * d_sub + (int64_t)(P.key_offset + n) * P.ks_l;
+    float x[PQ_MAX_D];
+#pragma unroll
+    for (int d = 0; d < PQ_MAX_D; ++d) x[d] = d < d_sub ? sah_load<DT>(P.k, off + d) : 0.f;
+    float dist = INFINITY;
+    int best = 0x7fffffff;
+    for (int c = lane; c < n_cent; c += SAH_WAVE) {
+      const float* cc = s_c + c * d_sub;
+      float dd = 0.f;
+      if (P.round_dist) {
+#pragma unroll
+        for (int d = 0; d < PQ_MAX_D; ++d) {
+          if (d < d_sub) {
+            const float df = sah_round_hw<DT>(x[d] - cc[d]);
+            dd += sah_round_hw<DT>(df * df);
+          }
+        }
+        dd = sah_round_hw<DT>(dd);
+      } else {
+#pragma unroll
+        for (int d = 0; d < PQ_MAX_D; ++d) {
+          if (d < d_sub) {
+            const float df = x[d] - cc[d];
+            dd = fmaf(df, df, dd);
+          }
+        }
+      }
+      if (dd < dist) {  // c ascends: the first minimum is kept
+        dist = dd;
+        best = c;
+      }
+    }
+#pragma unroll
+    for (int o = 1; o < SAH_WAVE; o <<= 1) {
+      const float od = __shfl_xor(dist, o);
+      const int oi = __shfl_xor(best, o);
+      if (od < dist || (od == dist && oi < best)) {
+        dist = od;
+        best = oi;
+      }
+    }
+    if (lane == 0) P.codes[(((int64_t)bh * P.code_pitch) + P.code_offset + n) * P.n_sub + s] = (uint8_t)best;
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Lloyd assignment on the matrix cores. argmin_c ||x - c||^2 = argmin_c (||c||^2 - 2 x.c): the key x centre
 // contraction is an fp32 MFMA (32 centres x 32 keys x 2 dims per instruction) whose accumulator starts at
@@ -737,6 +803,17 @@ extern "C" int sah_pq_kmeans_assign(const sah_pq_assign_args* a) {
       case SAH_F32: hipLaunchKernelGGL(k_pq_assign_few<SAH_F32>, gf, blk, 0, st, P); break;
       case SAH_BF16: hipLaunchKernelGGL(k_pq_assign_few<SAH_BF16>, gf, blk, 0, st, P); break;
       case SAH_F16: hipLaunchKernelGGL(k_pq_assign_few<SAH_F16>, gf, blk, 0, st, P); break;
+      default: return sah_fail(SAH_EDTYPE, "sah_pq_kmeans_assign: dtype %d", a->dtype);
+    }
+    return sah_launch_status("sah_pq_kmeans_assign");
+  }
+  if (!a->sums && !a->skip_flag && a->n_keys <= 512) {  // a block of new keys of a decode plan
+    dim3 gb(a->n_sub, a->B * a->Hkv), blk(PQB_NT);
+    sah_timed timed("k_pq_assign_block", a->stream);
+    switch (a->dtype) {
+      case SAH_F32: hipLaunchKernelGGL(k_pq_assign_block<SAH_F32>, gb, blk, 0, st, P); break;
+      case SAH_BF16: hipLaunchKernelGGL(k_pq_assign_block<SAH_BF16>, gb, blk, 0, st, P); break;
+      case SAH_F16: hipLaunchKernelGGL(k_pq_assign_block<SAH_F16>, gb, blk, 0, st, P); break;
       default: return sah_fail(SAH_EDTYPE, "sah_pq_kmeans_assign: dtype %d", a->dtype);
     }
     return sah_launch_status("sah_pq_kmeans_assign");

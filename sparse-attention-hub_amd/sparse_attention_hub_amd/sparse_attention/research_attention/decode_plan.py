@@ -264,7 +264,12 @@ class DecodePlan:
                 return None
             n_sub, d_sub, n_cent = top._geometry(k)
             book.reserve(current)
-            if current > book.n:
+            # One query per row: only columns below Lk - window can be selected, so the code of a key that is still
+            # inside the local window is not needed yet. New keys are quantised a block at a time (one launch every
+            # `lag` steps); `book.n` is the number of keys quantised so far and the scoring pass covers exactly those,
+            # which always include every column outside the window.
+            lag = min(window, _HASH_BLOCK) if Lq == 1 else 1
+            if current - book.n >= lag:
                 pa = self.pq_assign
                 pa.k, pa.ks_b, pa.ks_h, pa.ks_l = k.data_ptr(), k.stride(0), k.stride(1), k.stride(2)
                 pa.dtype, pa.B, pa.Hkv, pa.n_sub, pa.d_sub, pa.n_cent = self.dt, self.B, self.Hkv, n_sub, d_sub, n_cent
@@ -274,6 +279,8 @@ class DecodePlan:
                 pa.round_dist, pa.stream = 1, stream
                 chain.pq_assign = C.addressof(pa)
                 commit.append((book, "n", current))
+            else:
+                current = book.n
             self._ensure_keybuf(current)
             ad = self.pq_adc
             ad.q, ad.qs_b, ad.qs_h, ad.qs_l = q.data_ptr(), q.stride(0), q.stride(1), q.stride(2)

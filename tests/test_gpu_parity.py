@@ -466,6 +466,39 @@ def test_decode_plan_hashes_new_keys_in_blocks(cuda):
     assert torch.equal(c1.codes[:, :, : c1.n], c2.codes[:, :, : c1.n])
 
 
+def test_decode_plan_quantises_new_keys_in_blocks(cuda):
+    """PQCache decode through the plan: keys still inside the local window are quantised a block at a time (one
+    launch every `window` steps here), and the scoring pass covers the quantised keys only. Over enough steps for
+    such keys to leave the window and compete, every output equals the masker-by-masker path's, which quantises one
+    key per step, and the stored codes agree."""
+    sa = _sa()
+    dtype = torch.bfloat16
+    B, Hq, Hkv, Lk, D = 2, 8, 2, 1500, 128
+    steps, window, off = 40, 16, 8
+    q, k, v = make_qkv(B, Hq, Hkv, 1, Lk + steps, D, dtype, outliers=True, seed=13)
+    cfgs = [sa.SinkMaskerConfig(sink_size=off), sa.LocalMaskerConfig(window_size=window),
+            sa.PQCacheConfig(heavy_size=100, pq_group_factor=16, pq_bits=6, kmeans_iter=3, init_offset=off, metric="euclidean")]
+    fast = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=cfgs))
+    fast.return_attention_weights = False
+    ref = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=cfgs))
+    m1 = {}
+    kc, vc = k.to(cuda), v.to(cuda)
+    fast.custom_attention(None, q[:, :, :1].to(cuda), kc[:, :, :Lk], vc[:, :, :Lk], None, D ** -0.5, 0.0, sparse_meta_data=m1, layer_idx=0)
+    m2 = copy.deepcopy(m1)          # both start from the same codebook
+    quantised = []
+    for step in range(1, steps):
+        n = Lk + step
+        qq = make_qkv(B, Hq, Hkv, 1, 1, D, dtype, seed=250 + step)[0].to(cuda)
+        o1, _ = fast.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m1, layer_idx=0)
+        o2, _ = ref.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m2, layer_idx=0)
+        assert torch.equal(o1, o2), f"step {step}"
+        b1, b2 = m1["pq_codebook"][0], m2["pq_codebook"][0]
+        assert b2.n == n - off and n - off - window < b1.n <= n - off
+        quantised.append(b1.n)
+    assert len(set(quantised)) == 1 + (steps - 1) // window              # the cold call's count, then one block per `window` steps
+    assert torch.equal(b1.codes[:, :, : b1.n], b2.codes[:, :, : b1.n])
+
+
 def test_compact_code_stream_matches_two_plane_codes(cuda):
     """sah_hash_compact_codes: sign planes copied, every column with a zero component listed exactly once with
     both planes, counts right also beyond the list's capacity, ranges added in any order."""
