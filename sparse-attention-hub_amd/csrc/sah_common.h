@@ -269,6 +269,18 @@ __device__ __forceinline__ uint32_t sah_pk_gt01_u16(uint32_t a, uint32_t b) {
   return ((a & 0xffffu) > (b & 0xffffu) ? 1u : 0u) | ((a >> 16) > (b >> 16) ? 0x10000u : 0u);
 #endif
 }
+// larger of the two unsigned 16-bit halves, per half
+__device__ __forceinline__ uint32_t sah_pk_max_u16(uint32_t a, uint32_t b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  uint32_t d;
+  asm("v_pk_max_u16 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b));
+  return d;
+#else
+  const uint32_t lo = (a & 0xffffu) > (b & 0xffffu) ? (a & 0xffffu) : (b & 0xffffu);
+  const uint32_t hi = (a >> 16) > (b >> 16) ? (a >> 16) : (b >> 16);
+  return lo | (hi << 16);
+#endif
+}
 // Result per half: 1 where a != b, else 0
 __device__ __forceinline__ uint32_t sah_pk_ne01_u16(uint32_t a, uint32_t b) {
 #if defined(__HIP_DEVICE_COMPILE__)

@@ -20,11 +20,14 @@
 #define SF_BATCH 4    // chunks a wave has in flight
 #define SF_COPIES 64  // counters per bin: one per lane
 static_assert(SF_COPIES == 64, "sf_pick reads one row of 16 lanes x 4 counters per bin");
+#define SF_COPIES2 8  // counters per bin of the low-byte histogram of the short path
+#define SF_TOP_BINS 4 // high-byte bins below the row's largest key that the short path looks at
 
 struct sf_lds {
   int part[SF_NW];
   int eq[SF_NW];
   int out[SF_NW];
+  int top[SF_TOP_BINS];  // short path: candidates at or above each of the top high-byte bins
   int sel_bin, sel_need;
 };
 
@@ -119,6 +122,44 @@ __device__ __forceinline__ void sf_pick(const uint32_t* hist, int k, sf_lds& S, 
   need = S.sel_need;
 }
 
+// The same for a histogram of [256][SF_COPIES2] counters: a quad of lanes per bin, two counters per lane.
+__device__ __forceinline__ void sf_pick8(const uint32_t* hist, int k, sf_lds& S, int& bin, int& need) {
+  static_assert(SF_COPIES2 == 8, "a quad of lanes reads one bin: 4 x 2 counters");
+  const int tid = threadIdx.x;
+  const int lane = tid & (SAH_WAVE - 1);
+  const int wave = tid / SAH_WAVE;
+  const int b = 255 - (16 * wave + (lane >> 2));
+  const uint2 q = *(const uint2*)(hist + b * SF_COPIES2 + (lane & 3) * 2);
+  int v = (int)(q.x + q.y);
+  v += sah_dpp_i<0xB1, 0xF, true>(v);  // quad_perm [1,0,3,2]
+  v += sah_dpp_i<0x4E, 0xF, true>(v);  // quad_perm [2,3,0,1]
+  int cnt[16];  // cnt[j]: bin 255 - (16 * wave + j)
+  int wave_total = 0;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    cnt[j] = __builtin_amdgcn_readlane(v, 4 * j);
+    wave_total += cnt[j];
+  }
+  if (lane == 0) S.part[wave] = wave_total;
+  __syncthreads();
+  int above = 0;
+#pragma unroll
+  for (int w = 0; w < SF_NW; ++w) above += w < wave ? S.part[w] : 0;
+  if (above < k && k <= above + wave_total) {  // wave-uniform: the bin lies in this wave's range
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      if (above < k && k <= above + cnt[j] && lane == 0) {
+        S.sel_bin = 255 - (16 * wave + j);
+        S.sel_need = k - above;
+      }
+      above += cnt[j];
+    }
+  }
+  __syncthreads();
+  bin = S.sel_bin;
+  need = S.sel_need;
+}
+
 // the `allowed` lowest set bits of an 8-bit mask
 __device__ __forceinline__ uint32_t sf_lowest(uint32_t m, int allowed) {
   uint32_t take = 0;
@@ -169,6 +210,18 @@ __device__ __forceinline__ void sf_select_row(sf_lds& S, unsigned char* dyn, con
     return make_uint4(ch.k[0], ch.k[1], ch.k[2], ch.k[3]);
   };
 
+  // Counters that must be zero at the first barrier. Rows held in registers try the short path first (see
+  // below), which needs the top-bin counts and a low-byte histogram of SF_COPIES2 counters per bin; the two
+  // histograms of SF_COPIES counters per bin (128 KB, slow to clear and to scan) are cleared by the long path
+  // itself when it is taken.
+  auto clear_counters = [&]() {
+    if (REG) {
+      if (tid < SF_TOP_BINS) S.top[tid] = 0;
+      for (int i = tid; i < 256 * SF_COPIES2 / 4; i += SF_NT) ((uint4*)s_h2)[i] = make_uint4(0u, 0u, 0u, 0u);
+    } else {
+      for (int i = tid; i < 2 * 256 * SF_COPIES / 4; i += SF_NT) ((uint4*)s_h1)[i] = make_uint4(0u, 0u, 0u, 0u);
+    }
+  };
   uint4 kreg[NREG];
   if (REG) {
     // the key loads go out first and land while the bitmap row and the counters are set up
@@ -195,14 +248,14 @@ __device__ __forceinline__ void sf_select_row(sf_lds& S, unsigned char* dyn, con
       if (R.w) R.w[(int64_t)r * R.cap + i] = 1.0f;
     }
     cnt0 = fixed < R.cap ? fixed : R.cap;
-    for (int i = tid; i < 2 * 256 * SF_COPIES / 4; i += SF_NT) ((uint4*)s_h1)[i] = make_uint4(0u, 0u, 0u, 0u);
+    clear_counters();
     for (int i = tid; i < R.n_words + 2; i += SF_NT)
       s_bm[i] = i < R.n_words ? (sah_range_bits(i, 0, s_hi) | sah_range_bits(i, lo, hi)) : 0u;
   } else {
     cnt0 = R.cnt[r];  // read before the first barrier: rewritten at the end
     if (cnt0 > R.cap) cnt0 = R.cap;
     // clear the counters first: these stores do not wait for the loads above, the bitmap copy does
-    for (int i = tid; i < 2 * 256 * SF_COPIES / 4; i += SF_NT) ((uint4*)s_h1)[i] = make_uint4(0u, 0u, 0u, 0u);
+    clear_counters();
     for (int i = tid; i < R.n_words + 2; i += SF_NT) s_bm[i] = i < R.n_words ? bm[i] : 0u;
   }
   __syncthreads();
@@ -241,28 +294,103 @@ __device__ __forceinline__ void sf_select_row(sf_lds& S, unsigned char* dyn, con
   auto key_of = [](const uint32_t (&kk)[4], int t) -> uint32_t {
     return t < 4 ? (kk[t] & 0xffffu) : (kk[t - 4] >> 16);
   };
-  // ---- pass 1: histogram of the high byte ------------------------------------------------
+  // ---- threshold: the k-th largest key, as (high byte b1, low byte b2) ---------------------------
   uint32_t* my_h1 = s_h1 + (lane & (SF_COPIES - 1));
   uint32_t* my_h2 = s_h2 + (lane & (SF_COPIES - 1));
-  for_chunks([&](int, const uint32_t (&kk)[4]) {
+  int b1 = 0, need1 = 0, b2 = 0, need = 0;
+  bool short_path = false;
+  if (REG) {
+    // Short path. Scores are floats: the high byte of a key is sign + seven exponent bits, and the k-th largest
+    // key of a row lies within a few such bins of the largest. The row's largest key, then the counts of the
+    // keys at or above the bottom of the SF_TOP_BINS bins below it (packed 16-bit compares, no histogram),
+    // give b1 whenever it is one of those bins; otherwise the long path runs.
+    uint32_t m2 = 0;
+    for_chunks([&](int, const uint32_t (&kk)[4]) {
 #pragma unroll
-    for (int t = 0; t < 8; ++t) atomicAdd(&my_h1[(key_of(kk, t) >> 8) * SF_COPIES], 1u);
-  });
-  __syncthreads();
-  int b1, need1;
-  sf_pick(s_h1, k, S, b1, need1);
-
-  // ---- pass 2: histogram of the low byte inside bin b1 ---------------------------------
-  for_chunks([&](int, const uint32_t (&kk)[4]) {
+      for (int p = 0; p < 4; ++p) m2 = sah_pk_max_u16(m2, kk[p]);
+    });
+    uint32_t m = (m2 & 0xffffu) > (m2 >> 16) ? (m2 & 0xffffu) : (m2 >> 16);
 #pragma unroll
-    for (int t = 0; t < 8; ++t) {
-      const uint32_t key = key_of(kk, t);
-      atomicAdd(&my_h2[(key & 0xffu) * SF_COPIES], (int)(key >> 8) == b1 ? 1u : 0u);
+    for (int o = 1; o < SAH_WAVE; o <<= 1) {
+      const uint32_t other = (uint32_t)__shfl_xor((int)m, o);
+      m = other > m ? other : m;
     }
-  });
-  __syncthreads();
-  int b2, need;
-  sf_pick(s_h2, need1, S, b2, need);
+    if (lane == 0) S.part[wave] = (int)m;
+    __syncthreads();
+    uint32_t row_max = 0;
+#pragma unroll
+    for (int w = 0; w < SF_NW; ++w) row_max = (uint32_t)S.part[w] > row_max ? (uint32_t)S.part[w] : row_max;
+    const int b_max = (int)(row_max >> 8);
+    // bin b_max - j has its bottom at key (b_max - j) << 8; bin 0 is left to the long path (a compare against
+    // "below zero" does not exist)
+    uint32_t below[SF_TOP_BINS];
+#pragma unroll
+    for (int jj = 0; jj < SF_TOP_BINS; ++jj) {
+      const int bj = b_max - jj;
+      below[jj] = bj >= 1 ? (uint32_t)((bj << 8) - 1) * 0x00010001u : 0xffffffffu;  // nothing is above 0xffff
+    }
+    uint32_t pc[SF_TOP_BINS];
+#pragma unroll
+    for (int jj = 0; jj < SF_TOP_BINS; ++jj) pc[jj] = 0;
+    for_chunks([&](int, const uint32_t (&kk)[4]) {
+#pragma unroll
+      for (int p = 0; p < 4; ++p)
+#pragma unroll
+        for (int jj = 0; jj < SF_TOP_BINS; ++jj) pc[jj] += sah_pk_gt01_u16(kk[p], below[jj]);
+    });
+#pragma unroll
+    for (int jj = 0; jj < SF_TOP_BINS; ++jj) {
+      const int c = sah_wave_sum_i((int)((pc[jj] & 0xffffu) + (pc[jj] >> 16)));
+      if (lane == 0) atomicAdd(&S.top[jj], c);
+    }
+    __syncthreads();
+    int above = 0;
+#pragma unroll
+    for (int jj = 0; jj < SF_TOP_BINS; ++jj) {
+      const int c = S.top[jj];  // candidates in the bins b_max .. b_max - jj
+      if (!short_path && b_max - jj >= 1 && c >= k) {
+        short_path = true;
+        b1 = b_max - jj;
+        need1 = k - above;
+      }
+      above = c;
+    }
+  }
+  if (short_path) {
+    // low byte inside bin b1: only the keys of that bin touch the histogram
+    uint32_t* my_h = s_h2 + (lane & (SF_COPIES2 - 1));
+    for_chunks([&](int, const uint32_t (&kk)[4]) {
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        const uint32_t key = key_of(kk, t);
+        if ((int)(key >> 8) == b1) atomicAdd(&my_h[(key & 0xffu) * SF_COPIES2], 1u);
+      }
+    });
+    __syncthreads();
+    sf_pick8(s_h2, need1, S, b2, need);
+  } else {
+    if (REG) {  // the short path left these untouched
+      for (int i = tid; i < 2 * 256 * SF_COPIES / 4; i += SF_NT) ((uint4*)s_h1)[i] = make_uint4(0u, 0u, 0u, 0u);
+      __syncthreads();
+    }
+    // ---- pass 1: histogram of the high byte
+    for_chunks([&](int, const uint32_t (&kk)[4]) {
+#pragma unroll
+      for (int t = 0; t < 8; ++t) atomicAdd(&my_h1[(key_of(kk, t) >> 8) * SF_COPIES], 1u);
+    });
+    __syncthreads();
+    sf_pick(s_h1, k, S, b1, need1);
+    // ---- pass 2: histogram of the low byte inside bin b1
+    for_chunks([&](int, const uint32_t (&kk)[4]) {
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        const uint32_t key = key_of(kk, t);
+        atomicAdd(&my_h2[(key & 0xffu) * SF_COPIES], (int)(key >> 8) == b1 ? 1u : 0u);
+      }
+    });
+    __syncthreads();
+    sf_pick(s_h2, need1, S, b2, need);
+  }
   const uint32_t T = ((uint32_t)b1 << 8) | (uint32_t)b2;
   // Active candidates carry the excluded key. While that ranks below the threshold they are
   // neither winners nor ties and their flags are not needed again; otherwise (a row with
