@@ -348,6 +348,10 @@ typedef struct sah_pq_adc_args {
   void* keys_out; int64_t key_pitch;
   void* lut; int64_t lut_bytes;   /* scratch: sah_pq_adc_lut_bytes(...) bytes */
   void* stream;
+  const void* centres_narrow;     /* optional: the same centres [n_groups, n_cent, d_sub] in `dtype` (the form the
+                                     reference stores, pq_top_k.py:246-254; `centres` is their widening). When given
+                                     with a 16-bit dtype and d_sub a multiple of 8, the table is built from these:
+                                     half the bytes, identical values */
 } sah_pq_adc_args;
 int64_t sah_pq_adc_lut_bytes(int32_t B, int32_t Hq, int32_t Hkv, int32_t Lq, int32_t n_sub, int32_t n_cent, int32_t dtype);
 int sah_pq_adc_scores(const sah_pq_adc_args* a);

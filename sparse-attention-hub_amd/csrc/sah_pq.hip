@@ -466,6 +466,7 @@ struct pq_adc_params {
   const void* q; int64_t qs_b, qs_h, qs_l;
   int Hq, Hkv, Lq, n_sub, d_sub, n_cent;
   const float* centres;
+  const void* centres_narrow;  // the same values in the storage type, or NULL
   const uint8_t* codes; int64_t code_pitch;
   int n_cand;
   void* keys_out; int64_t key_pitch;
@@ -541,16 +542,19 @@ __global__ __launch_bounds__(PQ_NT) void k_pq_lut(pq_adc_params P, void* lut) {
 }
 
 // Scores of ADC_KEYS candidates for the NQ query vectors of one group: one 16-wave workgroup, the table in LDS
-// as fp32 (NQ floats per (s, c): one LDS read serves all the query vectors, and a lookup costs the read and NQ
-// adds, no unpacking), one thread per candidate. OWN_LUT: the workgroup computes its table itself (every
-// workgroup of a KV head repeats that work, which is cheaper than a launch of its own as long as a head is
-// covered by a few dozen workgroups); otherwise the 8-byte entries k_pq_lut wrote are widened on the way in.
+// as 8-byte entries per (s, c) (two floats for fp32, four packed 16-bit values otherwise: the entries are rounded to
+// the storage type anyway, and the LDS reads are what bounds this kernel), one thread per candidate. A lookup is
+// one LDS read, NQ widenings (a shift or a mask for bf16) and NQ additions. (The packed dot-product instruction
+// against (1, 0) would widen and add in one operation, but its sum is not always the correctly rounded one: one
+// addition in 800 differed in the last bit.) OWN_LUT: the workgroup computes its table itself
+// (every workgroup of a KV head repeats that work, which is cheaper than a launch of its own as long as a head is
+// covered by a few dozen workgroups); otherwise the entries k_pq_lut wrote are copied in.
 template <int DT, bool OWN_LUT>
 __global__ __launch_bounds__(ADC_NT) void k_pq_adc(pq_adc_params P, const void* lut) {
   sah_touch_kernargs<sizeof(pq_adc_params) + 8>();
   constexpr int NQ = (DT == SAH_F32) ? 2 : 4;
   typedef typename std::conditional<DT == SAH_F32, uint32_t, uint16_t>::type key_t;
-  typedef typename std::conditional<DT == SAH_F32, float2, float4>::type entry_t;
+  typedef uint2 entry_t;
   HIP_DYNAMIC_SHARED(unsigned char, adc_dyn)
   const int tid = threadIdx.x;
   const int bh = blockIdx.y;
@@ -572,9 +576,10 @@ __global__ __launch_bounds__(ADC_NT) void k_pq_adc(pq_adc_params P, const void* 
     row[i] = -1;
     if (v < nvec) row[i] = (b * P.Hq + hk * G + v / P.Lq) * P.Lq + v % P.Lq;
   }
-  auto store_entry = [&](int i, const float (&val)[NQ]) {  // rounded to the storage type, kept as floats
-    if constexpr (NQ == 2) s_lut[i] = make_float2(sah_round<DT>(val[0]), sah_round<DT>(val[1]));
-    else s_lut[i] = make_float4(sah_round<DT>(val[0]), sah_round<DT>(val[1]), sah_round<DT>(val[2]), sah_round<DT>(val[3]));
+  // rounded to the storage type by the hardware converters (round to nearest even, as the software rounding)
+  auto store_entry = [&](int i, const float (&val)[NQ]) {
+    if constexpr (NQ == 2) s_lut[i] = make_uint2(sah_float_to_bits(val[0]), sah_float_to_bits(val[1]));
+    else s_lut[i] = make_uint2(sah_pack2_hw<DT>(val[0], val[1]), sah_pack2_hw<DT>(val[2], val[3]));
   };
   // 16 one-byte codes per candidate = one 16-byte load: all of the thread's candidates are requested before
   // anything else and arrive while the table is built
@@ -605,13 +610,36 @@ __global__ __launch_bounds__(ADC_NT) void k_pq_adc(pq_adc_params P, const void* 
       s_q[qn * ADC_MAX_HEAD_DIM + e] = x;
     }
     __syncthreads();
+    const bool pow2 = (n_cent & (n_cent - 1)) == 0;  // the usual case (2^bits centres): no integer division per entry
+    const int shift = 31 - __builtin_clz(n_cent);
     for (int i = tid; i < lut_n; i += ADC_NT) {
-      const int s = i / n_cent, c = i % n_cent;
+      const int s = pow2 ? i >> shift : i / n_cent;
+      const int c = pow2 ? i & (n_cent - 1) : i % n_cent;
       const float* cc = P.centres + (((int64_t)bh * n_sub + s) * n_cent + c) * d_sub;
       float acc[NQ];
 #pragma unroll
       for (int qn = 0; qn < NQ; ++qn) acc[qn] = 0.f;
-      if ((d_sub & 3) == 0) {
+      if (DT != SAH_F32 && P.centres_narrow) {
+        // the centres in their 16-bit storage form: every workgroup of a KV head reads the whole codebook of the
+        // head, so halving its bytes halves the larger part of this kernel's memory traffic
+        for (int d = 0; d < d_sub; d += 8) {
+          float cv[8];
+          sah_load8<DT>(P.centres_narrow, (((int64_t)bh * n_sub + s) * n_cent + c) * d_sub + d, cv);
+#pragma unroll
+          for (int qn = 0; qn < NQ; ++qn) {
+            const float4 q0 = *(const float4*)&s_q[qn * ADC_MAX_HEAD_DIM + s * d_sub + d];
+            const float4 q1 = *(const float4*)&s_q[qn * ADC_MAX_HEAD_DIM + s * d_sub + d + 4];
+            acc[qn] = fmaf(q0.x, cv[0], acc[qn]);
+            acc[qn] = fmaf(q0.y, cv[1], acc[qn]);
+            acc[qn] = fmaf(q0.z, cv[2], acc[qn]);
+            acc[qn] = fmaf(q0.w, cv[3], acc[qn]);
+            acc[qn] = fmaf(q1.x, cv[4], acc[qn]);
+            acc[qn] = fmaf(q1.y, cv[5], acc[qn]);
+            acc[qn] = fmaf(q1.z, cv[6], acc[qn]);
+            acc[qn] = fmaf(q1.w, cv[7], acc[qn]);
+          }
+        }
+      } else if ((d_sub & 3) == 0) {
         // 16-byte reads of the centre and of the staged queries (the same fused multiply-adds in the same order)
         for (int d = 0; d < d_sub; d += 4) {
           const float4 cv = *(const float4*)(cc + d);
@@ -635,36 +663,26 @@ __global__ __launch_bounds__(ADC_NT) void k_pq_adc(pq_adc_params P, const void* 
     }
   } else {
     const uint2* slab = (const uint2*)lut + ((int64_t)bh * n_vg + vg) * lut_n;
-    for (int i = tid; i < lut_n; i += ADC_NT) {
-      const uint2 e = slab[i];
-      float val[NQ];
-      if (DT == SAH_F32) {
-        val[0] = sah_bits_to_float(e.x);
-        val[1] = sah_bits_to_float(e.y);
-      } else if (DT == SAH_BF16) {
-        val[0] = sah_bits_to_float(e.x << 16);
-        val[1] = sah_bits_to_float(e.x & 0xffff0000u);
-        val[NQ > 2 ? 2 : 0] = sah_bits_to_float(e.y << 16);
-        val[NQ > 2 ? 3 : 1] = sah_bits_to_float(e.y & 0xffff0000u);
-      } else {
-        val[0] = sah_f16_to_float((uint16_t)(e.x & 0xffffu));
-        val[1] = sah_f16_to_float((uint16_t)(e.x >> 16));
-        val[NQ > 2 ? 2 : 0] = sah_f16_to_float((uint16_t)(e.y & 0xffffu));
-        val[NQ > 2 ? 3 : 1] = sah_f16_to_float((uint16_t)(e.y >> 16));
-      }
-      store_entry(i, val);
-    }
+    for (int i = tid; i < lut_n; i += ADC_NT) s_lut[i] = slab[i];
   }
   __syncthreads();
 
   float acc[NQ];
   auto add = [&](int s, int c) {
     const entry_t e = s_lut[s * n_cent + c];
-    acc[0] += e.x;
-    acc[1] += e.y;
-    if constexpr (NQ > 2) {
-      acc[2] += e.z;
-      acc[3] += e.w;
+    if constexpr (NQ == 2) {
+      acc[0] += sah_bits_to_float(e.x);
+      acc[1] += sah_bits_to_float(e.y);
+    } else if constexpr (DT == SAH_BF16) {
+      acc[0] += sah_bits_to_float(e.x << 16);
+      acc[1] += sah_bits_to_float(e.x & 0xffff0000u);
+      acc[2] += sah_bits_to_float(e.y << 16);
+      acc[3] += sah_bits_to_float(e.y & 0xffff0000u);
+    } else {
+      acc[0] += sah_f16_to_float((uint16_t)(e.x & 0xffffu));
+      acc[1] += sah_f16_to_float((uint16_t)(e.x >> 16));
+      acc[2] += sah_f16_to_float((uint16_t)(e.y & 0xffffu));
+      acc[3] += sah_f16_to_float((uint16_t)(e.y >> 16));
     }
   };
   auto store = [&](int n) {
@@ -709,11 +727,11 @@ __global__ __launch_bounds__(ADC_NT) void k_pq_adc(pq_adc_params P, const void* 
   }
 }
 
-// dynamic LDS of k_pq_adc: the fp32 table and, for OWN_LUT, the staged query vectors
+// dynamic LDS of k_pq_adc: the table (8 bytes per entry) and, for OWN_LUT, the staged query vectors
 template <int DT>
 static size_t adc_lds_bytes(int lut_n) {
   constexpr int NQ = (DT == SAH_F32) ? 2 : 4;
-  return (size_t)lut_n * NQ * 4 + (size_t)NQ * ADC_MAX_HEAD_DIM * 4;
+  return (size_t)lut_n * 8 + (size_t)NQ * ADC_MAX_HEAD_DIM * 4;
 }
 
 template <int DT, bool OWN_LUT>
@@ -890,6 +908,7 @@ extern "C" int sah_pq_adc_scores(const sah_pq_adc_args* a) {
   P.q = a->q; P.qs_b = a->qs_b; P.qs_h = a->qs_h; P.qs_l = a->qs_l;
   P.Hq = a->Hq; P.Hkv = a->Hkv; P.Lq = a->Lq; P.n_sub = a->n_sub; P.d_sub = a->d_sub; P.n_cent = a->n_cent;
   P.centres = a->centres; P.codes = a->codes; P.code_pitch = a->code_pitch; P.n_cand = a->n_cand;
+  P.centres_narrow = (a->dtype != SAH_F32 && a->d_sub % 8 == 0 && ((uintptr_t)a->centres_narrow % 16) == 0) ? a->centres_narrow : nullptr;
   P.keys_out = a->keys_out; P.key_pitch = a->key_pitch;
   const int nvec = (a->Hq / a->Hkv) * a->Lq;
   const int nq = a->dtype == SAH_F32 ? 2 : 4;

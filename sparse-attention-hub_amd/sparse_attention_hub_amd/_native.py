@@ -226,6 +226,7 @@ class PqAdcArgs(C.Structure):
         ("keys_out", C.c_void_p), ("key_pitch", C.c_int64),
         ("lut", C.c_void_p), ("lut_bytes", C.c_int64),
         ("stream", C.c_void_p),
+        ("centres_narrow", C.c_void_p),
     ]
 
 

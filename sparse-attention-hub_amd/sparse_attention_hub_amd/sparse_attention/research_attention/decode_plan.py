@@ -291,6 +291,9 @@ class DecodePlan:
             if self.adc_lut is None:
                 self.adc_lut = adc_lut_buffer(self.B, self.Hq, self.Hkv, Lq, n_sub, n_cent, self.dtype, self.device)
             ad.lut, ad.lut_bytes = self.adc_lut.data_ptr(), self.adc_lut.numel()
+            narrow = sparse_meta_data.get("pq_centroids", {}).get(layer_idx)
+            ad.centres_narrow = (narrow.data_ptr() if narrow is not None and narrow.dtype == self.dtype and narrow.is_contiguous()
+                                 and narrow.shape[-1] == d_sub and narrow.dtype != torch.float32 else None)
             chain.pq_adc = C.addressof(ad)
             se = self.select
             se.rows, se.keys, se.key_pitch, se.key_bits = rows, self.keybuf.data_ptr(), self.keybuf_pitch, self.key_bits

@@ -238,6 +238,9 @@ class PQCache(TopKMasker):
             cf32.data_ptr(), book.codes.data_ptr(), book.capacity, n_cand,
             keybuf.data_ptr(), keybuf.stride(0), lut.data_ptr(), lut.numel(), N.stream_ptr(q.device),
         )
+        stored = sparse_meta_data["pq_centroids"][layer_idx]
+        if stored.dtype == q.dtype and stored.dtype != torch.float32 and stored.shape[-1] == d_sub and stored.is_contiguous():
+            a.centres_narrow = stored.data_ptr()   # the table is built from the 16-bit centroids: half the bytes
         N.call("sah_pq_adc_scores", a)
         excluded = sortable_key_of(torch.finfo(q.dtype).min, q.dtype)
         self._select_into_rows(rows, keybuf, 32 if q.dtype == torch.float32 else 16, n_cand, self.init_offset, k_eff, excluded)
