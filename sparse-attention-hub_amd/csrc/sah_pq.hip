@@ -612,7 +612,63 @@ __global__ __launch_bounds__(ADC_NT) void k_pq_adc(pq_adc_params P, const void* 
     __syncthreads();
     const bool pow2 = (n_cent & (n_cent - 1)) == 0;  // the usual case (2^bits centres): no integer division per entry
     const int shift = 31 - __builtin_clz(n_cent);
-    for (int i = tid; i < lut_n; i += ADC_NT) {
+    int first = tid;  // first entry the general loop below still has to build
+    if (DT != SAH_F32 && P.centres_narrow && d_sub == 8 && pow2 && n_cent >= SAH_WAVE) {
+      // Sub-vectors of 8 in 16-bit storage. A wave takes whole sub-spaces (wave w: s = w, w + 16, ...), so the
+      // query elements of a sub-space are read from LDS once per wave and lane instead of once per entry (those
+      // broadcast reads were most of the table's cost); a lane builds the entries of centres lane, lane + 64, ...:
+      // one 16-byte load per centre, up to four of them requested together.
+      const int lane = tid & (SAH_WAVE - 1);
+      constexpr int LE = 4;
+      for (int s = tid / SAH_WAVE; s < n_sub; s += ADC_NT / SAH_WAVE) {
+        float qv[NQ][8];
+#pragma unroll
+        for (int qn = 0; qn < NQ; ++qn) {
+          const float4 q0 = *(const float4*)&s_q[qn * ADC_MAX_HEAD_DIM + s * 8];
+          const float4 q1 = *(const float4*)&s_q[qn * ADC_MAX_HEAD_DIM + s * 8 + 4];
+          qv[qn][0] = q0.x; qv[qn][1] = q0.y; qv[qn][2] = q0.z; qv[qn][3] = q0.w;
+          qv[qn][4] = q1.x; qv[qn][5] = q1.y; qv[qn][6] = q1.z; qv[qn][7] = q1.w;
+        }
+        for (int c0 = lane; c0 < n_cent; c0 += LE * SAH_WAVE) {
+          uint4 raw[LE];
+#pragma unroll
+          for (int u = 0; u < LE; ++u) {
+            int c = c0 + u * SAH_WAVE;
+            if (c >= n_cent) c = n_cent - 1;
+            raw[u] = *(const uint4*)((const uint16_t*)P.centres_narrow + (((int64_t)bh * n_sub + s) * n_cent + c) * 8);
+          }
+#pragma unroll
+          for (int u = 0; u < LE; ++u) {
+            const int c = c0 + u * SAH_WAVE;
+            if (c < n_cent) {
+              const uint32_t w[4] = {raw[u].x, raw[u].y, raw[u].z, raw[u].w};
+              float cv[8];
+#pragma unroll
+              for (int t = 0; t < 4; ++t) {
+                if (DT == SAH_BF16) {
+                  cv[2 * t] = sah_bits_to_float(w[t] << 16);
+                  cv[2 * t + 1] = sah_bits_to_float(w[t] & 0xffff0000u);
+                } else {
+                  cv[2 * t] = sah_f16_to_float((uint16_t)(w[t] & 0xffffu));
+                  cv[2 * t + 1] = sah_f16_to_float((uint16_t)(w[t] >> 16));
+                }
+              }
+              float acc[NQ];
+#pragma unroll
+              for (int qn = 0; qn < NQ; ++qn) {
+                float a = 0.f;
+#pragma unroll
+                for (int d = 0; d < 8; ++d) a = fmaf(qv[qn][d], cv[d], a);
+                acc[qn] = a;
+              }
+              store_entry(s * n_cent + c, acc);
+            }
+          }
+        }
+      }
+      first = lut_n;
+    }
+    for (int i = first; i < lut_n; i += ADC_NT) {
       const int s = pow2 ? i >> shift : i / n_cent;
       const int c = pow2 ? i & (n_cent - 1) : i % n_cent;
       const float* cc = P.centres + (((int64_t)bh * n_sub + s) * n_cent + c) * d_sub;
