@@ -335,6 +335,50 @@ def sub_run(cfg: int, dev) -> dict:
     return out
 
 
+def cold_probe(dev) -> dict:
+    """The matrix-core kernels of the cold calls at their BASELINE shapes, timed with HIP events: two Lloyd iterations
+    of the config-4 k-means (4 x 8 KV heads x 16 sub-spaces, 32640 keys, 256 centres, sub-vectors of 8) and the
+    config-3 bulk signature build (8 x 32 heads x 32768 keys, MLP 128-128-128-32)."""
+    import torch
+
+    from sparse_attention_hub_amd.sparse_attention import HashAttentionTopKMasker, HashAttentionTopKMaskerConfig
+    from sparse_attention_hub_amd.sparse_attention.research_attention.maskers.fixed.implementations.utils.pq_utils import kmeans_keys_batched
+    from sparse_attention_hub_amd.sparse_attention.utils.hashattention_utils import random_hat_weights
+
+    dtype = torch.bfloat16
+    g = torch.Generator(device=dev).manual_seed(0)
+    k4 = torch.randn(4, HKV, 32768, D, generator=g, device=dev, dtype=dtype)
+    for c in OUTLIER_CHANNELS:
+        k4[..., c] *= 8.0
+    codes = torch.zeros((4, HKV, 32768 - 128, 16), dtype=torch.uint8, device=dev)
+    from sparse_attention_hub_amd import _native as N
+
+    kmeans_keys_batched(k4, 128, 16, 256, 1, codes, 32768 - 128, seed=0)       # warm-up (module load)
+    k3 = torch.randn(8, HKV, 32768, D, generator=g, device=dev, dtype=dtype)
+    wts = random_hat_weights(1, HQ, D, 32, 3, 128, dtype=dtype, seed=1)
+    m = HashAttentionTopKMasker(HashAttentionTopKMaskerConfig(heavy_size=2048, hat_bits=32, hat_mlp_layers=3, hat_mlp_hidden_size=128,
+                                                             hat_mlp_activation="silu", hat_weights=wts))
+    m._update_key_signatures(k3[:, :, :4096], HQ, {}, 0)                       # warm-up
+    torch.cuda.synchronize()
+    N.timing_enable(True)                                                      # HIP events around every launch of the library
+    kmeans_keys_batched(k4, 128, 16, 256, 2, codes, 32768 - 128, seed=0)
+    m._update_key_signatures(k3, HQ, {}, 0)
+    torch.cuda.synchronize()
+    kt = N.timing_collect()
+    N.timing_enable(False)
+    lloyd_ms = kt["k_pq_assign_mfma"][1] / kt["k_pq_assign_mfma"][0]
+    sig_ms = kt["k_hash_sig_mfma"][1] / kt["k_hash_sig_mfma"][0]
+    lloyd_flop = 2.0 * 4 * HKV * 16 * (32768 - 128) * 256 * 8
+    sig_flop = 2.0 * 8 * HQ * 32768 * (128 * 128 + 128 * 128 + 128 * 32)
+    return {"cold_probe": True,
+            "k_pq_assign_mfma_ms": round(lloyd_ms, 3), "k_pq_assign_mfma_TFLOPs": round(lloyd_flop / lloyd_ms / 1e9, 1),
+            "k_pq_assign_mfma_frac_of_fp32_mfma_peak": round(lloyd_flop / lloyd_ms / 1e9 / 157.3, 4),
+            "k_hash_sig_mfma_ms": round(sig_ms, 3), "k_hash_sig_mfma_TFLOPs": round(sig_flop / sig_ms / 1e9, 1),
+            "k_hash_sig_mfma_frac_of_bf16_mfma_peak": round(sig_flop / sig_ms / 1e9 / 2500.0, 4),
+            "kernels_avg_ms": {n: round(ms / c, 4) for n, (c, ms) in sorted(kt.items())},
+            "note": "HIP events around every launch; flops = 2 x keys x centres x dims (k-means), 2 x MLP multiply-adds (signatures)"}
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -345,6 +389,9 @@ def main() -> None:
     ap.add_argument("--no-other-configs", action="store_true", help="skip the short sub-runs of the other configurations")
     ap.add_argument("--batch", type=int, default=0, help="study only: override the workload's batch size")
     ap.add_argument("--keys", type=int, default=0, help="study only: override the workload's key count")
+    ap.add_argument("--cold-probe", action="store_true",
+                    help="short run for `rocprofv3 --pmc` / `--kernel-trace` of the two matrix-core kernels of the cold calls: "
+                         "two Lloyd iterations of the config-4 k-means and the config-3 bulk signature build")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="short run for `rocprofv3 --pmc`: a few layer-steps plus three 256 MiB copy kernels of known size")
     args = ap.parse_args()
@@ -361,6 +408,9 @@ def main() -> None:
         sys.exit(3)
     N.lib()
     dev = torch.device("cuda:0")
+    if args.cold_probe:
+        print(json.dumps(cold_probe(dev)))
+        return
     w = dict(WORKLOADS[args.config])
     study = bool(args.batch or args.keys)
     if study:

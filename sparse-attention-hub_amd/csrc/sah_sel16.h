@@ -180,6 +180,9 @@ __device__ __forceinline__ void sf_select_row(sf_lds& S, unsigned char* dyn, con
                                               uint32_t excluded_key, int fresh, int sink, int window) {
   constexpr bool REG = CPW > 0;
   constexpr int NREG = REG ? CPW : 1;
+  // The short way to the threshold (below) costs four packed compares per key word and pays up to 64 keys per
+  // thread; longer rows amortise the histograms' fixed cost better (512 x 131072: 134 us against 107)
+  constexpr bool SHORT = REG && CPW <= 8;
   const int tid = threadIdx.x;
   const int lane = tid & (SAH_WAVE - 1);
   const int wave = tid / SAH_WAVE;
@@ -215,7 +218,7 @@ __device__ __forceinline__ void sf_select_row(sf_lds& S, unsigned char* dyn, con
   // histograms of SF_COPIES counters per bin (128 KB, slow to clear and to scan) are cleared by the long path
   // itself when it is taken.
   auto clear_counters = [&]() {
-    if (REG) {
+    if (SHORT) {
       if (tid < SF_TOP_BINS) S.top[tid] = 0;
       for (int i = tid; i < 256 * SF_COPIES2 / 4; i += SF_NT) ((uint4*)s_h2)[i] = make_uint4(0u, 0u, 0u, 0u);
     } else {
@@ -299,7 +302,7 @@ __device__ __forceinline__ void sf_select_row(sf_lds& S, unsigned char* dyn, con
   uint32_t* my_h2 = s_h2 + (lane & (SF_COPIES - 1));
   int b1 = 0, need1 = 0, b2 = 0, need = 0;
   bool short_path = false;
-  if (REG) {
+  if (SHORT) {
     // Short path. Scores are floats: the high byte of a key is sign + seven exponent bits, and the k-th largest
     // key of a row lies within a few such bins of the largest. The row's largest key, then the counts of the
     // keys at or above the bottom of the SF_TOP_BINS bins below it (packed 16-bit compares, no histogram),
@@ -369,7 +372,7 @@ __device__ __forceinline__ void sf_select_row(sf_lds& S, unsigned char* dyn, con
     __syncthreads();
     sf_pick8(s_h2, need1, S, b2, need);
   } else {
-    if (REG) {  // the short path left these untouched
+    if (SHORT) {  // the short path left these untouched
       for (int i = tid; i < 2 * 256 * SF_COPIES / 4; i += SF_NT) ((uint4*)s_h1)[i] = make_uint4(0u, 0u, 0u, 0u);
       __syncthreads();
     }
