@@ -156,7 +156,7 @@ __device__ __forceinline__ void att_tile(const att_params& P, int r, int b, int 
   constexpr int ES = (DT == SAH_F32) ? 4 : 2;
   const int tid = threadIdx.x;
   const int lane = tid & (SAH_WAVE - 1);
-  const int wave = tid / SAH_WAVE;
+  const int wave = sah_wave_id();
   const int sub = lane % LPK;   // which 8-element slice of the row
   const int grp = lane / LPK;   // which key of the iteration
 

@@ -62,6 +62,10 @@ static inline int sah_check_rows(const sah_rows& r, const char* what, bool need_
   return SAH_OK;
 }
 
+// The calling wave's index in its (one-dimensional) workgroup, in a scalar register: loops and conditions on it
+// compile to scalar branches instead of execution-mask bookkeeping.
+__device__ __forceinline__ int sah_wave_id() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x / SAH_WAVE)); }
+
 // ---------------------------------------------------------------------------
 // device side: kernel arguments
 // ---------------------------------------------------------------------------
@@ -369,7 +373,7 @@ template <int NT>
 __device__ __forceinline__ int sah_block_excl_scan(int v, int* wsum, int* total) {
   constexpr int NW = NT / SAH_WAVE;
   const int lane = threadIdx.x & (SAH_WAVE - 1);
-  const int wave = threadIdx.x / SAH_WAVE;
+  const int wave = sah_wave_id();
   int incl = sah_wave_incl_scan(v);
   __syncthreads();  // protect wsum from a previous use
   if (lane == SAH_WAVE - 1) wsum[wave] = incl;

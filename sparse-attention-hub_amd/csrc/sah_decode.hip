@@ -131,8 +131,9 @@ __device__ __forceinline__ int hdec_row(const hdec_params& P, int r, hsw_lds& S,
   __syncthreads();  // every thread holds q (and the bitmap is complete) before the scores overwrite the scratch
 
   // ---- 3. top-k over the remaining columns
+  // the row's active columns are the sink and local ranges just built, nothing else
   return hsw_select_row<CP>(R, r, kc, q, P.k, fixed < R.cap ? fixed : R.cap, s_bm, s_key, S, buf, early, P.update_bitmap != 0,
-                            s_cols, CP ? &cs : nullptr);
+                            s_cols, CP ? &cs : nullptr, s_hi, n_local > 0 ? lo2 : n);
 }
 
 template <int DT, bool MF, bool CP>

@@ -133,7 +133,7 @@ __global__ __launch_bounds__(SGM_NT, 1) void k_hash_sig_mfma(sig_params P, int n
   HIP_DYNAMIC_SHARED(unsigned char, sgm_dyn)
   const int tid = threadIdx.x;
   const int lane = tid & (SAH_WAVE - 1);
-  const int wave = tid / SAH_WAVE;
+  const int wave = sah_wave_id();
   const int i32 = lane & 31;  // row of A / column of B and C
   const int g = lane >> 5;    // k-group of the operands, row group of C
   // the heads of one KV group are neighbours in the grid: they read the same vectors, which then hit in L2

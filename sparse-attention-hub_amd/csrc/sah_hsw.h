@@ -124,7 +124,7 @@ __device__ __forceinline__ void hsw_request(const uint2* kc, int n, int lane, ui
 __device__ __forceinline__ void hsw_prefetch(const uint2* kc, int n, hsw_bufs& buf) {
   const int lane = threadIdx.x & (SAH_WAVE - 1);
   int c0, c1;
-  hsw_wave_chunks(n, threadIdx.x / SAH_WAVE, c0, c1);
+  hsw_wave_chunks(n, sah_wave_id(), c0, c1);
   (void)c1;  // no conditions: a request past the row's end re-reads valid memory and is never scored
   hsw_request(kc, n, lane, buf.a0, buf.a1, c0);
   hsw_request(kc, n, lane, buf.b0, buf.b1, c0 + HSW_BATCH);
@@ -140,7 +140,7 @@ __device__ __forceinline__ void hsw_request_c(const uint32_t* pos, int lane, uin
 __device__ __forceinline__ void hsw_prefetch(const hsw_compact& cs, int n, hsw_bufs_t<true>& buf) {
   const int lane = threadIdx.x & (SAH_WAVE - 1);
   int c0, c1;
-  hsw_wave_chunks(n, threadIdx.x / SAH_WAVE, c0, c1);
+  hsw_wave_chunks(n, sah_wave_id(), c0, c1);
   (void)c1;
   hsw_request_c(cs.pos, lane, buf.a, c0);
   hsw_request_c(cs.pos, lane, buf.b, c0 + HSW_CBATCH);
@@ -156,16 +156,19 @@ __device__ __forceinline__ void hsw_prefetch(const hsw_compact& cs, int n, hsw_b
 // the appended columns are mirrored there for a caller that goes on to use them in the same kernel (the mirror
 // is complete only after the caller's next barrier).
 // CP: the row's codes come in the compact form `cs` (kc is not used).
+// active_below / active_from (both >= 0): the caller knows that the row's active columns are exactly
+// [0, active_below) and [active_from, n) (the sink and local columns of a fresh decode row); chunks that lie between
+// the two ranges then skip the bitmap test of every word.
 template <bool CP = false>
 __device__ __forceinline__ int hsw_select_row(const sah_rows& R, int r, const uint2* kc, const uint2 q, int k, int cnt0,
                                               uint32_t* s_bm, uint32_t* s_key, hsw_lds& S, hsw_bufs_t<CP>& buf,
                                               bool prefetched = false, bool update_bitmap = true, int* s_cols = nullptr,
-                                              const hsw_compact* cs = nullptr) {
+                                              const hsw_compact* cs = nullptr, int active_below = -1, int active_from = -1) {
   int* s_gt = S.gt;
   int* s_eq = S.eq;
   const int tid = threadIdx.x;
   const int lane = tid & (SAH_WAVE - 1);
-  const int wave = tid / SAH_WAVE;
+  const int wave = sah_wave_id();
   const int n = R.n_keys;
   const int n_ch = (n + 255) / 256;            // chunks of 256 columns = 64 words
   int my_c0, my_c1;
@@ -180,14 +183,19 @@ __device__ __forceinline__ int hsw_select_row(const sah_rows& R, int r, const ui
 #pragma unroll
   for (int i = 0; i < HSW_PROBES; ++i) pc[i] = 0;
   // what staging a word has in common: zero the bytes of already-active columns, park the word, count the probes
-  auto stage = [&](uint32_t word, int wi) {
-    const int j0 = wi * 4;
-    // Most chunks of a long row hold no active column at all: uniform test, the expansion is skipped
-    const uint32_t nib = (s_bm[j0 >> 5] >> (j0 & 31)) & 0xFu;  // nibble -> byte mask
+  const bool ranges_known = active_below >= 0 && active_from >= 0;
+  // may chunk c hold an active column? (uniform across the wave)
+  auto chunk_may_be_active = [&](int c) { return !ranges_known || c * 256 < active_below || (c + 1) * 256 > active_from; };
+  auto stage = [&](uint32_t word, int wi, bool check) {
     uint32_t kw = word;
-    if (__ballot(nib != 0)) {
-      const uint32_t one = (nib | (nib << 7) | (nib << 14) | (nib << 21)) & 0x01010101u;
-      kw = word & ~((one << 8) - one);
+    if (check) {
+      const int j0 = wi * 4;
+      // Most chunks of a long row hold no active column at all: uniform test, the expansion is skipped
+      const uint32_t nib = (s_bm[j0 >> 5] >> (j0 & 31)) & 0xFu;  // nibble -> byte mask
+      if (__ballot(nib != 0)) {
+        const uint32_t one = (nib | (nib << 7) | (nib << 14) | (nib << 21)) & 0x01010101u;
+        kw = word & ~((one << 8) - one);
+      }
     }
     s_key[wi] = kw;
     const uint32_t x = kw | 0x80808080u;
@@ -197,7 +205,19 @@ __device__ __forceinline__ int hsw_select_row(const sah_rows& R, int r, const ui
   if constexpr (CP) {
     // ---- compact stream: every component taken as non-zero, score = popc(q.y) - 2 popc((q.x ^ k.x) & q.y)
     const uint32_t s_full = (uint32_t)__popc(q.y) + 33u;
-    auto score1 = [&](uint32_t kx) { return s_full - 2u * (uint32_t)__popc((q.x ^ kx) & q.y); };
+    const uint32_t s_full4 = s_full * 0x01010101u;
+    // a query without zero components (the usual case) needs no mask on the differing bits; uniform
+    const bool q_dense = q.y == 0xFFFFFFFFu;
+    // four scores as the bytes of a word: the four mismatch counts are packed first, then one multiply-add turns
+    // them into scores (a count is at most popc(q.y), so no byte borrows from its neighbour)
+    auto word_of = [&](const uint4& k4) {
+      uint32_t m0 = q.x ^ k4.x, m1 = q.x ^ k4.y, m2 = q.x ^ k4.z, m3 = q.x ^ k4.w;
+      if (!q_dense) {
+        m0 &= q.y; m1 &= q.y; m2 &= q.y; m3 &= q.y;
+      }
+      const uint32_t p4 = (uint32_t)__popc(m0) | ((uint32_t)__popc(m1) << 8) | ((uint32_t)__popc(m2) << 16) | ((uint32_t)__popc(m3) << 24);
+      return s_full4 - 2u * p4;
+    };
     auto score_c = [&](uint4 (&rc)[HSW_CBATCH], int c0) {
 #pragma unroll
       for (int u = 0; u < HSW_CBATCH; ++u) {
@@ -208,15 +228,10 @@ __device__ __forceinline__ int hsw_select_row(const sah_rows& R, int r, const ui
         if (c0 + u >= my_c1) break;
         const int wi = (c0 + u) * SAH_WAVE + lane;
         const int j0 = wi * 4;
-        uint32_t word;
-        if (j0 + 4 <= n) {
-          word = score1(rc[u].x) | (score1(rc[u].y) << 8) | (score1(rc[u].z) << 16) | (score1(rc[u].w) << 24);
-        } else {
-          word = 0;  // ragged tail
-          for (int t = 0; t < 4; ++t)
-            if (j0 + t < n) word |= score1(cs->pos[j0 + t]) << (8 * t);
-        }
-        stage(word, wi);
+        uint32_t word = word_of(rc[u]);
+        // ragged tail: the stream is readable beyond the row, what lies there scores nothing
+        if (j0 + 4 > n) word = j0 < n ? word & ((1u << (8 * (n - j0))) - 1u) : 0u;
+        stage(word, wi, chunk_may_be_active(c0 + u));
       }
     };
     if (!prefetched) {
@@ -282,7 +297,7 @@ __device__ __forceinline__ int hsw_select_row(const sah_rows& R, int r, const ui
           for (int t = 0; t < 4; ++t)
             if (j0 + t < n) word |= (uint32_t)(sig_score(q, kc[j0 + t]) + 33) << (8 * t);
         }
-        stage(word, wi);
+        stage(word, wi, chunk_may_be_active(c0 + u));
       }
     };
     if (!prefetched && my_c0 < my_c1) hsw_request(kc, n, lane, buf.a0, buf.a1, my_c0);

@@ -137,7 +137,7 @@ __global__ __launch_bounds__(PQ_NT) void k_pq_assign_few(pq_assign_params P) {
   __shared__ int s_i[PQ_NT / SAH_WAVE];
   const int tid = threadIdx.x;
   const int lane = tid & (SAH_WAVE - 1);
-  const int wave = tid / SAH_WAVE;
+  const int wave = sah_wave_id();
   const int s = blockIdx.x;
   const int bh = blockIdx.y;
   const int n = blockIdx.z;
@@ -285,7 +285,7 @@ __global__ __launch_bounds__(PQM_NT) void k_pq_assign_mfma(pq_assign_params P) {
   const float sum_scale = P.sums ? pq_sum_scale(*P.absmax_bits) : 1.f;
   const int tid = threadIdx.x;
   const int lane = tid & (SAH_WAVE - 1);
-  const int wave = tid / SAH_WAVE;
+  const int wave = sah_wave_id();
   const int j = lane & 31, g = lane >> 5;
   const int s_idx = blockIdx.x % P.n_sub;
   const int tg = blockIdx.x / P.n_sub;
@@ -620,7 +620,7 @@ __global__ __launch_bounds__(ADC_NT) void k_pq_adc(pq_adc_params P, const void* 
       // one 16-byte load per centre, up to four of them requested together.
       const int lane = tid & (SAH_WAVE - 1);
       constexpr int LE = 4;
-      for (int s = tid / SAH_WAVE; s < n_sub; s += ADC_NT / SAH_WAVE) {
+      for (int s = sah_wave_id(); s < n_sub; s += ADC_NT / SAH_WAVE) {
         float qv[NQ][8];
 #pragma unroll
         for (int qn = 0; qn < NQ; ++qn) {

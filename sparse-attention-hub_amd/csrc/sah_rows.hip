@@ -250,7 +250,7 @@ __global__ __launch_bounds__(ROWS_NT) void k_rows_from_dense(sah_rows R, const v
   const int r = blockIdx.x;
   const int tid = threadIdx.x;
   const int lane = tid & (SAH_WAVE - 1);
-  const int wave = tid / SAH_WAVE;
+  const int wave = sah_wave_id();
   constexpr int NW = ROWS_NT / SAH_WAVE;
   const int Lk = R.n_keys;
   const int64_t rowoff = (int64_t)r * Lk;

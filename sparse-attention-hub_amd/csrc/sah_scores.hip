@@ -133,7 +133,7 @@ __global__ __launch_bounds__(SC_NT) void k_qk_scores(qk_params P) {
 
   const int tid = threadIdx.x;
   const int lane = tid & (SAH_WAVE - 1);
-  const int wave = tid / SAH_WAVE;
+  const int wave = sah_wave_id();
   const int sub = lane % LPK;
   const int grp = lane / LPK;
   const int G = P.Hq / P.Hkv;

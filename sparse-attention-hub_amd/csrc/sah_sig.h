@@ -131,7 +131,7 @@ __device__ __forceinline__ void sig_gemv_block(const sig_params& P, bool active,
   constexpr int LOG_NT = 31 - __builtin_clz(NT);
   static_assert((NT & (NT - 1)) == 0, "NT must be a power of two");
   const int lane = tid & (SAH_WAVE - 1);
-  const int wave = tid / SAH_WAVE;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / SAH_WAVE);  // tid: the caller's numbering of the block's threads
   const int hx = active ? h / P.group : 0;
   const int D = active ? P.D : 8;
 
@@ -300,7 +300,7 @@ template <int DT, typename Hook = sig_no_hook>
 __device__ __forceinline__ void sig_mfma_block(const sig_params& P, bool active, int tid, int b, int h, int l0, int nl,
                                                int n_layers, sig_mfma_lds& S, Hook after_requests = Hook()) {
   const int lane = tid & (SAH_WAVE - 1);
-  const int wave = tid / SAH_WAVE;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / SAH_WAVE);  // tid: the caller's numbering of the block's threads
   const int i16 = lane & 15;  // row of A, column (vector) of B and C
   const int g = lane >> 4;    // k-group of the operands, row group of C
   const int hx = active ? h / P.group : 0;

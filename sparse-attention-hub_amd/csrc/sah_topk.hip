@@ -87,7 +87,7 @@ __device__ __forceinline__ void select_row(sel_shared& S, unsigned char* dyn, se
                                            const SRC& src, int n_cand, int col_offset, int k, uint32_t excluded_key) {
   const int tid = threadIdx.x;
   const int lane = tid & (SAH_WAVE - 1);
-  const int wave = tid / SAH_WAVE;
+  const int wave = sah_wave_id();
   uint32_t* hist = (uint32_t*)dyn;
   uint32_t* s_bm = hist + L.hist_bins;
   STG* staged = (STG*)(s_bm + R.n_words);
