@@ -82,9 +82,6 @@ __device__ __forceinline__ void att_unpack(const att_raw<DT>& r, float (&o)[8]) 
   }
 }
 
-// Each wave keeps its own online-softmax state (m uniform across the wave, l and acc
-// per lane group) and walks its 64-key slices in batches of UB iterations; the K and V
-// rows of a batch are requested together so 2*UB row loads are in flight per lane.
 // merge the splits of one row: out = sum_s acc_s e^(m_s-M) / sum_s l_s e^(m_s-M).
 // The (m, l) pairs go through LDS and each thread's partial values are requested together,
 // so the merge costs about two memory round trips whatever the number of splits. Every thread of the
@@ -137,6 +134,223 @@ __device__ __forceinline__ void att_combine_row(const float* work, int n_split, 
   }
 }
 
+// A wave's online-softmax state: m uniform across the wave, l and acc per lane group (lane group = the D / 8
+// lanes that share a key; a lane holds 8 elements of the accumulator).
+struct att_wave_state {
+  float acc[8];
+  float l_run;
+  float m_run;
+  __device__ __forceinline__ void clear() {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+    l_run = 0.f;
+    m_run = -INFINITY;
+  }
+};
+
+// The K and V rows of one batch of a wave: UB iterations of SAH_WAVE / (D / 8) keys each, as loaded. id[u] is the
+// column of the calling lane's key in iteration u (-1: none, the lane then reads row 0 and its result is dropped).
+template <int DT, int UB>
+struct att_batch {
+  att_raw<DT> kr[UB], vr[UB];
+  int id[UB];
+};
+
+// the calling lane's slice (8 elements) of the rows of head (b, hk): addresses, and the query's elements
+template <int DT, int D>
+struct att_lane {
+  static constexpr int LPK = D / 8;            // lanes per key
+  static constexpr int KPI = SAH_WAVE / LPK;   // keys per wave iteration
+  static constexpr int ES = (DT == SAH_F32) ? 4 : 2;
+  const char* kbase;
+  const char* vbase;
+  int64_t krow, vrow;
+  int sub, grp;  // which 8-element slice of the row, which key of the iteration
+  __device__ __forceinline__ att_lane(const att_params& P, int b, int hk) {
+    const int lane = threadIdx.x & (SAH_WAVE - 1);
+    sub = lane % LPK;
+    grp = lane / LPK;
+    kbase = (const char*)P.k + ((int64_t)b * P.ks_b + (int64_t)hk * P.ks_h + sub * 8) * ES;
+    vbase = (const char*)P.v + ((int64_t)b * P.vs_b + (int64_t)hk * P.vs_h + sub * 8) * ES;
+    krow = P.ks_l * ES;
+    vrow = P.vs_l * ES;
+  }
+  __device__ __forceinline__ void load_q(const att_params& P, int b, int h, int qi, float (&qv)[8]) const {
+    sah_load8<DT>(P.q, (int64_t)b * P.qs_b + (int64_t)h * P.qs_h + (int64_t)qi * P.qs_l + sub * 8, qv);
+  }
+  // puts the batch's 2 * UB row loads on their way
+  template <int UB>
+  __device__ __forceinline__ void request(att_batch<DT, UB>& B) const {
+#pragma unroll
+    for (int u = 0; u < UB; ++u) {
+      const int safe = B.id[u] >= 0 ? B.id[u] : 0;
+      att_load_raw<DT>(kbase + (int64_t)safe * krow, B.kr[u]);
+      att_load_raw<DT>(vbase + (int64_t)safe * vrow, B.vr[u]);
+    }
+  }
+  // the batch's logits (scaled, plus the additive mask; -inf for a lane without a key), and their maximum over the wave
+  template <int UB>
+  __device__ __forceinline__ float logits(const att_params& P, int64_t moff, const float (&qv)[8], const att_batch<DT, UB>& B,
+                                          float (&z)[UB]) const {
+    float mb = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < UB; ++u) {
+      float kf[8];
+      att_unpack<DT>(B.kr[u], kf);
+      float d = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) d = fmaf(qv[e], kf[e], d);
+      d = att_group_sum<LPK>(d) * P.scaling;
+      if (B.id[u] >= 0) {
+        if (P.amask) d += sah_load<DT>(P.amask, moff + B.id[u]);
+      } else {
+        d = -INFINITY;
+      }
+      z[u] = d;
+      mb = fmaxf(mb, d);
+    }
+    // over the lane groups of the wave: m stays uniform across the wave
+#pragma unroll
+    for (int o = LPK; o < SAH_WAVE; o <<= 1) mb = fmaxf(mb, __shfl_xor(mb, o));
+    return mb;
+  }
+  // the online-softmax step of a batch: iw[u] is the inverse weight of the lane's key in iteration u
+  template <int UB>
+  __device__ __forceinline__ void accumulate(const att_batch<DT, UB>& B, const float (&z)[UB], float mb, const float (&iw)[UB],
+                                             att_wave_state& st) const {
+    const float m_new = fmaxf(st.m_run, mb);
+    if (m_new != -INFINITY) {
+      const float rescale = (st.m_run == -INFINITY) ? 0.f : att_exp<DT>(st.m_run - m_new);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) st.acc[e] *= rescale;
+      st.l_run *= rescale;
+      st.m_run = m_new;
+#pragma unroll
+      for (int u = 0; u < UB; ++u) {
+        float p = 0.f;
+        if (z[u] != -INFINITY) p = att_exp<DT>(z[u] - m_new) * iw[u];
+        st.l_run += p;
+        float vf[8];
+        att_unpack<DT>(B.vr[u], vf);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) st.acc[e] = fmaf(p, vf[e], st.acc[e]);
+      }
+    }
+  }
+};
+
+// The calling wave attends to the entries first .. first + 63, first + stride .., all below `bound`, of row r:
+// entry i is column col_of(i) (anything outside [0, Lk) is skipped) with inverse weight inv_w_of(i). Batches of UB
+// iterations: the K and V rows of a batch are requested together, so 2 * UB row loads are in flight per lane.
+template <int DT, int D, typename ColOf, typename InvWOf>
+__device__ __forceinline__ void att_walk(const att_params& P, int r, int b, int h, int hk, int qi, int first, int bound,
+                                         int stride, ColOf col_of, InvWOf inv_w_of, att_wave_state& st) {
+  typedef att_lane<DT, D> lane_t;
+  constexpr int KPI = lane_t::KPI;
+  constexpr int IT = SAH_WAVE / KPI;    // iterations per 64-key wave slice
+  constexpr int UB = IT < 4 ? IT : 4;   // iterations per batch
+  const int lane = threadIdx.x & (SAH_WAVE - 1);
+  const lane_t L(P, b, hk);
+  const int64_t moff = P.amask ? ((int64_t)b * P.ms_b + (int64_t)h * P.ms_h + (int64_t)qi * P.ms_l) : 0;
+  float qv[8];
+  L.load_q(P, b, h, qi, qv);
+
+  for (int cbase = first; cbase < bound; cbase += stride) {
+    // one column (and its inverse weight) per lane: this wave's next 64 keys
+    const int my = cbase + lane;
+    int idx_l = -1;
+    float invw_l = P.unit_inv_w;
+    if (my < bound) {
+      idx_l = col_of(my);
+      invw_l = inv_w_of(my);
+      if (idx_l < 0 || idx_l >= P.Lk) idx_l = -1;
+    }
+#pragma unroll
+    for (int ib = 0; ib < IT; ib += UB) {
+      if (cbase + ib * KPI >= bound) break;  // uniform across the wave
+      att_batch<DT, UB> B;
+#pragma unroll
+      for (int u = 0; u < UB; ++u) B.id[u] = __shfl(idx_l, (ib + u) * KPI + L.grp);
+      L.request(B);
+      float z[UB];
+      const float mb = L.logits(P, moff, qv, B, z);
+      if (P.logits_out && L.sub == 0) {
+#pragma unroll
+        for (int u = 0; u < UB; ++u) {
+          const int pos = cbase + (ib + u) * KPI + L.grp;
+          if (pos < bound) P.logits_out[(int64_t)r * P.logits_pitch + pos] = z[u];
+        }
+      }
+      float iw[UB];
+#pragma unroll
+      for (int u = 0; u < UB; ++u) iw[u] = __shfl(invw_l, (ib + u) * KPI + L.grp);
+      L.accumulate(B, z, mb, iw, st);
+    }
+  }
+}
+
+// The calling wave's state, summed over its lane groups, into slot `slot` of the workgroup's partial results.
+template <int D, int NS>
+__device__ __forceinline__ void att_park(att_wave_state& st, int slot, float (&s_m)[NS], float (&s_l)[NS], float (&s_acc)[NS][D]) {
+  constexpr int LPK = D / 8;
+  const int lane = threadIdx.x & (SAH_WAVE - 1);
+#pragma unroll
+  for (int o = LPK; o < SAH_WAVE; o <<= 1) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) st.acc[e] += __shfl_xor(st.acc[e], o);
+    st.l_run += __shfl_xor(st.l_run, o);
+  }
+  if (lane < LPK) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s_acc[slot][lane * 8 + e] = st.acc[e];
+  }
+  if (lane == 0) {
+    s_l[slot] = st.l_run;
+    s_m[slot] = st.m_run;
+  }
+}
+
+// The workgroup's NS partial results (complete, a barrier passed) rescaled to a common max and summed: thread
+// d < D gets element d of the numerator in `a`; every thread the max M and the denominator l.
+template <int DT, int D, int NS>
+__device__ __forceinline__ void att_gather(const float (&s_m)[NS], const float (&s_l)[NS], const float (&s_acc)[NS][D], float& a,
+                                           float& M, float& l) {
+  const int tid = threadIdx.x;
+  M = s_m[0];
+#pragma unroll
+  for (int wv = 1; wv < NS; ++wv) M = fmaxf(M, s_m[wv]);
+  float sc[NS];
+#pragma unroll
+  for (int wv = 0; wv < NS; ++wv) sc[wv] = (s_m[wv] == -INFINITY) ? 0.f : att_exp<DT>(s_m[wv] - M);
+  a = 0.f;
+  l = 0.f;
+  if (tid < D) {
+#pragma unroll
+    for (int wv = 0; wv < NS; ++wv) a = fmaf(s_acc[wv][tid], sc[wv], a);
+  }
+#pragma unroll
+  for (int wv = 0; wv < NS; ++wv) l = fmaf(s_l[wv], sc[wv], l);
+}
+
+// A complete row: normalise (with the optional sink logit, mask_attention_utils.py:357-402) and store
+template <int DT, int D>
+__device__ __forceinline__ void att_store_row(const att_params& P, int r, int b, int h, int qi, float a, float M, float l) {
+  const int tid = threadIdx.x;
+  float Mf = M, den = l;
+  if (P.sinks) {
+    const float sk = P.sinks[h];
+    Mf = fmaxf(M, sk);
+    const float rs = (M == -INFINITY) ? 0.f : att_exp<DT>(M - Mf);
+    a *= rs;
+    den = l * rs + att_exp<DT>(sk - Mf);
+  }
+  if (tid < D) sah_store<DT>(P.out, (((int64_t)b * P.Lq + qi) * P.Hq + h) * D + tid, a / den);
+  if (P.stats && tid == 0) {
+    P.stats[2 * (int64_t)r] = Mf;
+    P.stats[2 * (int64_t)r + 1] = den;
+  }
+}
+
 // One tile of work of a workgroup. ROW = false: a workgroup of 4 waves handles one (row, split) tile and leaves (m, l, acc) in the workspace
 //   for the merge kernel - the form for few or very uneven rows.
 // ROW = true: a workgroup of 16 waves handles a whole row, every wave an equal share of the row's entries,
@@ -149,16 +363,9 @@ __device__ __forceinline__ void att_tile(const att_params& P, int r, int b, int 
                                          float (&s_l)[(ROW ? ATT_ROW_NT : ATT_NT) / SAH_WAVE],
                                          float (&s_acc)[(ROW ? ATT_ROW_NT : ATT_NT) / SAH_WAVE][D]) {
   constexpr int NW = (ROW ? ATT_ROW_NT : ATT_NT) / SAH_WAVE;
-  constexpr int LPK = D / 8;            // lanes per key
-  constexpr int KPI = SAH_WAVE / LPK;   // keys per wave iteration
-  constexpr int IT = SAH_WAVE / KPI;    // iterations per 64-key wave slice (== LPK)
-  constexpr int UB = IT < 4 ? IT : 4;   // iterations per batch
-  constexpr int ES = (DT == SAH_F32) ? 4 : 2;
+  constexpr int KPI = SAH_WAVE / (D / 8);   // keys per wave iteration
   const int tid = threadIdx.x;
-  const int lane = tid & (SAH_WAVE - 1);
   const int wave = sah_wave_id();
-  const int sub = lane % LPK;   // which 8-element slice of the row
-  const int grp = lane / LPK;   // which key of the iteration
 
   // cnt_known >= 0: the caller holds the row's entry count (and `cols` may then point anywhere, LDS included)
   // P.dense: 0 = the rows' column lists, 1 = every key, 2 = the sink + local columns of one query in closed form
@@ -192,137 +399,21 @@ __device__ __forceinline__ void att_tile(const att_params& P, int r, int b, int 
 
   const int* cols = cols_known ? cols_known : (P.dense ? nullptr : P.rows.cols + (int64_t)r * P.rows.cap);
   const float* wts = (!P.dense && P.rows.w) ? P.rows.w + (int64_t)r * P.rows.cap : nullptr;
-  const char* kbase = (const char*)P.k + ((int64_t)b * P.ks_b + (int64_t)hk * P.ks_h + sub * 8) * ES;
-  const char* vbase = (const char*)P.v + ((int64_t)b * P.vs_b + (int64_t)hk * P.vs_h + sub * 8) * ES;
-  const int64_t krow = P.ks_l * ES, vrow = P.vs_l * ES;
-  const int64_t moff = P.amask ? ((int64_t)b * P.ms_b + (int64_t)h * P.ms_h + (int64_t)qi * P.ms_l) : 0;
-
-  float qv[8];
-  sah_load8<DT>(P.q, (int64_t)b * P.qs_b + (int64_t)h * P.qs_h + (int64_t)qi * P.qs_l + sub * 8, qv);
-
-  float acc[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-  float l_run = 0.f;
-  float m_run = -INFINITY;
-
-  for (int cbase = first; cbase < bound; cbase += stride) {
-    // one column (and its inverse weight) per lane: this wave's next 64 keys
-    const int my = cbase + lane;
-    int idx_l = -1;
-    float invw_l = P.unit_inv_w;
-    if (my < bound) {
-      idx_l = P.dense == 1 ? my : (P.dense == 2 ? (my < P.closed_sink ? my : P.closed_lo + (my - P.closed_sink)) : cols[my]);
+  att_wave_state st;
+  st.clear();
+  att_walk<DT, D>(
+      P, r, b, h, hk, qi, first, bound, stride,
+      [&](int i) { return P.dense == 1 ? i : (P.dense == 2 ? (i < P.closed_sink ? i : P.closed_lo + (i - P.closed_sink)) : cols[i]); },
       // the reference evaluates 1/(w + 1e-6) in the mask dtype (utils/mask.py:737-740)
-      if (wts) invw_l = sah_round<DT>(1.0f / sah_round<DT>(wts[my] + 1e-6f));
-      if (idx_l < 0 || idx_l >= P.Lk) idx_l = -1;
-    }
-#pragma unroll
-    for (int ib = 0; ib < IT; ib += UB) {
-      if (cbase + ib * KPI >= bound) break;  // uniform across the wave
-      att_raw<DT> kr[UB], vr[UB];
-      int id[UB];
-#pragma unroll
-      for (int u = 0; u < UB; ++u) {
-        id[u] = __shfl(idx_l, (ib + u) * KPI + grp);
-        const int safe = id[u] >= 0 ? id[u] : 0;  // invalid lanes read row 0 and are masked below
-        att_load_raw<DT>(kbase + (int64_t)safe * krow, kr[u]);
-        att_load_raw<DT>(vbase + (int64_t)safe * vrow, vr[u]);
-      }
-      float z[UB];
-      float mb = -INFINITY;
-#pragma unroll
-      for (int u = 0; u < UB; ++u) {
-        float kf[8];
-        att_unpack<DT>(kr[u], kf);
-        float d = 0.f;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) d = fmaf(qv[e], kf[e], d);
-        d = att_group_sum<LPK>(d) * P.scaling;
-        if (id[u] >= 0) {
-          if (P.amask) d += sah_load<DT>(P.amask, moff + id[u]);
-        } else {
-          d = -INFINITY;
-        }
-        z[u] = d;
-        mb = fmaxf(mb, d);
-      }
-      if (P.logits_out && sub == 0) {
-#pragma unroll
-        for (int u = 0; u < UB; ++u) {
-          const int pos = cbase + (ib + u) * KPI + grp;
-          if (pos < bound) P.logits_out[(int64_t)r * P.logits_pitch + pos] = z[u];
-        }
-      }
-      // batch max over the lane groups of the wave: m stays uniform across the wave
-#pragma unroll
-      for (int o = LPK; o < SAH_WAVE; o <<= 1) mb = fmaxf(mb, __shfl_xor(mb, o));
-      const float m_new = fmaxf(m_run, mb);
-      if (m_new != -INFINITY) {
-        const float rescale = (m_run == -INFINITY) ? 0.f : att_exp<DT>(m_run - m_new);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[e] *= rescale;
-        l_run *= rescale;
-        m_run = m_new;
-#pragma unroll
-        for (int u = 0; u < UB; ++u) {
-          const float iw = __shfl(invw_l, (ib + u) * KPI + grp);
-          float p = 0.f;
-          if (z[u] != -INFINITY) p = att_exp<DT>(z[u] - m_new) * iw;
-          l_run += p;
-          float vf[8];
-          att_unpack<DT>(vr[u], vf);
-#pragma unroll
-          for (int e = 0; e < 8; ++e) acc[e] = fmaf(p, vf[e], acc[e]);
-        }
-      }
-    }
-  }
+      [&](int i) { return wts ? sah_round<DT>(1.0f / sah_round<DT>(wts[i] + 1e-6f)) : P.unit_inv_w; }, st);
 
-  // ---- reduce the KPI lane groups of the wave, then the waves (rescaled to a common max)
-#pragma unroll
-  for (int o = LPK; o < SAH_WAVE; o <<= 1) {
-#pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] += __shfl_xor(acc[e], o);
-    l_run += __shfl_xor(l_run, o);
-  }
-  if (lane < LPK) {
-#pragma unroll
-    for (int e = 0; e < 8; ++e) s_acc[wave][sub * 8 + e] = acc[e];
-  }
-  if (lane == 0) {
-    s_l[wave] = l_run;
-    s_m[wave] = m_run;
-  }
+  // ---- reduce the lane groups of the wave, then the waves (rescaled to a common max)
+  att_park<D, NW>(st, wave, s_m, s_l, s_acc);
   __syncthreads();
-  float M = s_m[0];
-#pragma unroll
-  for (int wv = 1; wv < NW; ++wv) M = fmaxf(M, s_m[wv]);
-  float sc[NW];
-#pragma unroll
-  for (int wv = 0; wv < NW; ++wv) sc[wv] = (s_m[wv] == -INFINITY) ? 0.f : att_exp<DT>(s_m[wv] - M);
-  float a = 0.f, l = 0.f;
-  if (tid < D) {
-#pragma unroll
-    for (int wv = 0; wv < NW; ++wv) a = fmaf(s_acc[wv][tid], sc[wv], a);
-  }
-#pragma unroll
-  for (int wv = 0; wv < NW; ++wv) l = fmaf(s_l[wv], sc[wv], l);
+  float a, M, l;
+  att_gather<DT, D, NW>(s_m, s_l, s_acc, a, M, l);
   if constexpr (ROW) {
-    // the row is complete: normalise (with the optional sink logit, mask_attention_utils.py:357-402) and store
-    float Mf = M, den = l;
-    if (P.sinks) {
-      const float sk = P.sinks[h];
-      Mf = fmaxf(M, sk);
-      const float rs = (M == -INFINITY) ? 0.f : att_exp<DT>(M - Mf);
-      a *= rs;
-      den = l * rs + att_exp<DT>(sk - Mf);
-    }
-    if (tid < D) sah_store<DT>(P.out, (((int64_t)b * P.Lq + qi) * P.Hq + h) * D + tid, a / den);
-    if (P.stats && tid == 0) {
-      P.stats[2 * (int64_t)r] = Mf;
-      P.stats[2 * (int64_t)r + 1] = den;
-    }
+    att_store_row<DT, D>(P, r, b, h, qi, a, M, l);
   } else {
     if (tid < D) wout[2 + tid] = a;
     if (tid == 0) {
