@@ -122,37 +122,42 @@ __device__ __forceinline__ void sf_pick(const uint32_t* hist, int k, sf_lds& S, 
   need = S.sel_need;
 }
 
-// The same for a histogram of [256][SF_COPIES2] counters: a quad of lanes per bin, two counters per lane.
+// The same for the short path's histogram of [SF_COPIES2][256] counters (copy-major: the counters of a bin are 1 KB
+// apart), by ONE wave: lane l sums the copies of the four bins 252 - 4 l .. 255 - 4 l (one 16-byte read per copy,
+// consecutive lanes at consecutive addresses), a wave scan gives the candidates in all bins from its own up, and the
+// first lane that reaches k holds the bin. One barrier; the other waves only wait for it.
 __device__ __forceinline__ void sf_pick8(const uint32_t* hist, int k, sf_lds& S, int& bin, int& need) {
-  static_assert(SF_COPIES2 == 8, "a quad of lanes reads one bin: 4 x 2 counters");
   const int tid = threadIdx.x;
-  const int lane = tid & (SAH_WAVE - 1);
-  const int wave = tid / SAH_WAVE;
-  const int b = 255 - (16 * wave + (lane >> 2));
-  const uint2 q = *(const uint2*)(hist + b * SF_COPIES2 + (lane & 3) * 2);
-  int v = (int)(q.x + q.y);
-  v += sah_dpp_i<0xB1, 0xF, true>(v);  // quad_perm [1,0,3,2]
-  v += sah_dpp_i<0x4E, 0xF, true>(v);  // quad_perm [2,3,0,1]
-  int cnt[16];  // cnt[j]: bin 255 - (16 * wave + j)
-  int wave_total = 0;
+  if (tid < SAH_WAVE) {
+    const int lo = 4 * (SAH_WAVE - 1 - tid);  // this lane's bins: lo .. lo + 3
+    uint4 c = make_uint4(0u, 0u, 0u, 0u);
 #pragma unroll
-  for (int j = 0; j < 16; ++j) {
-    cnt[j] = __builtin_amdgcn_readlane(v, 4 * j);
-    wave_total += cnt[j];
-  }
-  if (lane == 0) S.part[wave] = wave_total;
-  __syncthreads();
-  int above = 0;
+    for (int cp = 0; cp < SF_COPIES2; ++cp) {
+      const uint4 q = *(const uint4*)(hist + cp * 256 + lo);
+      c.x += q.x; c.y += q.y; c.z += q.z; c.w += q.w;
+    }
+    const int mine = (int)(c.x + c.y + c.z + c.w);
+    const int incl = sah_wave_incl_scan(mine);  // candidates in the bins lo .. 255
+    const uint64_t reach = __ballot(incl >= k);
+    if (reach) {  // always: the caller's k is at most the histogram's total
+      const int l = __builtin_ctzll(reach);
+      if (tid == l) {
+        int above = incl - mine;
+        const int cnt[4] = {(int)c.w, (int)c.z, (int)c.y, (int)c.x};  // bins lo + 3, lo + 2, lo + 1, lo
+        int bsel = lo, nsel = k - above;
+        bool found = false;
 #pragma unroll
-  for (int w = 0; w < SF_NW; ++w) above += w < wave ? S.part[w] : 0;
-  if (above < k && k <= above + wave_total) {  // wave-uniform: the bin lies in this wave's range
-#pragma unroll
-    for (int j = 0; j < 16; ++j) {
-      if (above < k && k <= above + cnt[j] && lane == 0) {
-        S.sel_bin = 255 - (16 * wave + j);
-        S.sel_need = k - above;
+        for (int j = 0; j < 4; ++j) {
+          if (!found && k <= above + cnt[j]) {
+            found = true;
+            bsel = lo + 3 - j;
+            nsel = k - above;
+          }
+          above += cnt[j];
+        }
+        S.sel_bin = bsel;
+        S.sel_need = nsel;
       }
-      above += cnt[j];
     }
   }
   __syncthreads();
@@ -294,6 +299,20 @@ __device__ __forceinline__ void sf_select_row(sf_lds& S, unsigned char* dyn, con
       }
     }
   };
+  // the same with the chunk's register slot as third argument (REG only; 0 otherwise)
+  auto for_chunks_slot = [&](auto&& f) {
+    if (REG) {
+#pragma unroll
+      for (int u = 0; u < NREG; ++u)
+        if (c0 + u < c1) {
+          sah_keep(kreg[u].x), sah_keep(kreg[u].y), sah_keep(kreg[u].z), sah_keep(kreg[u].w);
+          const uint32_t kk[4] = {kreg[u].x, kreg[u].y, kreg[u].z, kreg[u].w};
+          f(c0 + u, kk, u);
+        }
+    } else {
+      for_chunks([&](int c, const uint32_t (&kk)[4]) { f(c, kk, 0); });
+    }
+  };
   auto key_of = [](const uint32_t (&kk)[4], int t) -> uint32_t {
     return t < 4 ? (kk[t] & 0xffffu) : (kk[t - 4] >> 16);
   };
@@ -361,12 +380,12 @@ __device__ __forceinline__ void sf_select_row(sf_lds& S, unsigned char* dyn, con
   }
   if (short_path) {
     // low byte inside bin b1: only the keys of that bin touch the histogram
-    uint32_t* my_h = s_h2 + (lane & (SF_COPIES2 - 1));
+    uint32_t* my_h = s_h2 + (lane & (SF_COPIES2 - 1)) * 256;
     for_chunks([&](int, const uint32_t (&kk)[4]) {
 #pragma unroll
       for (int t = 0; t < 8; ++t) {
         const uint32_t key = key_of(kk, t);
-        if ((int)(key >> 8) == b1) atomicAdd(&my_h[(key & 0xffu) * SF_COPIES2], 1u);
+        if ((int)(key >> 8) == b1) atomicAdd(&my_h[key & 0xffu], 1u);
       }
     });
     __syncthreads();
@@ -421,12 +440,22 @@ __device__ __forceinline__ void sf_select_row(sf_lds& S, unsigned char* dyn, con
   };
 
   // ---- pass 3: winners and ties per lane and wave --------------------------------------------
+  // Rows held in registers keep the two masks of every chunk (16 bits, two chunks to a register) for the passes
+  // below, which then do not compare a key again; not when active candidates may rank (their flags come from LDS).
+  // (up to 64 keys per thread: beyond that the registers are full)
+  constexpr bool KEEP = REG && CPW <= 8;
+  constexpr int NPM = KEEP ? (NREG + 1) / 2 : 1;
+  const bool stored = KEEP && !slow;  // uniform across the workgroup
+  uint32_t pm[NPM];
+#pragma unroll
+  for (int i = 0; i < NPM; ++i) pm[i] = 0;
   int n_gt = 0, n_eq = 0;
-  for_chunks([&](int c, const uint32_t (&kk)[4]) {
+  for_chunks_slot([&](int c, const uint32_t (&kk)[4], int u) {
     uint32_t gt, eq, ex;
     masks(c, kk, gt, eq, ex);
     n_gt += __popc(gt);
     n_eq += __popc(eq);
+    if (KEEP) pm[u >> 1] |= (gt | (eq << 8)) << (16 * (u & 1));
   });
   const int wave_eq = sah_wave_sum_i(n_eq);
   if (lane == 0) S.eq[wave] = wave_eq;
@@ -439,9 +468,16 @@ __device__ __forceinline__ void sf_select_row(sf_lds& S, unsigned char* dyn, con
 
   // emission mask of a chunk; `tie_run` counts the wave's ties seen so far (mode 2 only)
   int tie_run = tie_base;
-  auto emit_mask = [&](int c, const uint32_t (&kk)[4]) -> uint32_t {
+  auto emit_mask = [&](int c, const uint32_t (&kk)[4], int u) -> uint32_t {
     uint32_t gt, eq, ex;
-    masks(c, kk, gt, eq, ex);
+    if (stored) {
+      const uint32_t both = pm[KEEP ? u >> 1 : 0] >> (16 * (u & 1));
+      gt = both & 0xffu;
+      eq = (both >> 8) & 0xffu;
+      ex = 0;
+    } else {
+      masks(c, kk, gt, eq, ex);
+    }
     uint32_t take = 0;
     if (mode == 1) take = eq;
     if (mode == 2) {
@@ -457,7 +493,7 @@ __device__ __forceinline__ void sf_select_row(sf_lds& S, unsigned char* dyn, con
   int mine = n_gt + (mode == 1 ? n_eq : 0);
   if (mode == 2 || slow) {
     mine = 0;
-    for_chunks([&](int c, const uint32_t (&kk)[4]) { mine += __popc(emit_mask(c, kk)); });
+    for_chunks_slot([&](int c, const uint32_t (&kk)[4], int u) { mine += __popc(emit_mask(c, kk, u)); });
   }
   const int incl = sah_wave_incl_scan(mine);
   if (lane == SAH_WAVE - 1) S.out[wave] = incl;
@@ -474,8 +510,8 @@ __device__ __forceinline__ void sf_select_row(sf_lds& S, unsigned char* dyn, con
   float* wgt = R.w ? R.w + (int64_t)r * R.cap : nullptr;
   int pos = cnt0 + out_base + incl - mine;
   tie_run = tie_base;
-  for_chunks([&](int c, const uint32_t (&kk)[4]) {
-    uint32_t em = emit_mask(c, kk);
+  for_chunks_slot([&](int c, const uint32_t (&kk)[4], int u) {
+    uint32_t em = emit_mask(c, kk, u);
     if (em) {
       const int col0 = c * SF_CHUNK + lane * 8 + col_offset;
       atomicOr(&s_bm[col0 >> 5], em << (col0 & 31));

@@ -391,6 +391,7 @@ template <int CPW>
 __global__ __launch_bounds__(SF_NT) void k_select16(sah_rows R, const uint16_t* keys, int64_t pitch, int n_cand,
                                                     int col_offset, int k, uint32_t excluded_key, int fresh, int sink,
                                                     int window) {
+  sah_touch_kernargs<sizeof(sah_rows) + 56>();
   __shared__ sf_lds S;
   HIP_DYNAMIC_SHARED(unsigned char, sf_dyn)
   const int r = blockIdx.x;
