@@ -22,6 +22,7 @@
 static_assert(SF_COPIES == 64, "sf_pick reads one row of 16 lanes x 4 counters per bin");
 #define SF_COPIES2 8  // counters per bin of the low-byte histogram of the short path
 #define SF_TOP_BINS 4 // high-byte bins below the row's largest key that the short path looks at
+static_assert(SF_TOP_BINS % 2 == 0, "the short path counts its bins in pairs");
 
 struct sf_lds {
   int part[SF_NW];
@@ -344,38 +345,40 @@ __device__ __forceinline__ void sf_select_row(sf_lds& S, unsigned char* dyn, con
     for (int w = 0; w < SF_NW; ++w) row_max = (uint32_t)S.part[w] > row_max ? (uint32_t)S.part[w] : row_max;
     const int b_max = (int)(row_max >> 8);
     // bin b_max - j has its bottom at key (b_max - j) << 8; bin 0 is left to the long path (a compare against
-    // "below zero" does not exist)
-    uint32_t below[SF_TOP_BINS];
-#pragma unroll
-    for (int jj = 0; jj < SF_TOP_BINS; ++jj) {
+    // "below zero" does not exist). Two bins at a time: the threshold is nearly always in the largest key's own
+    // bin or the next, and the second pair is counted only when it is not.
+    auto bottom = [&](int jj) -> uint32_t {
       const int bj = b_max - jj;
-      below[jj] = bj >= 1 ? (uint32_t)((bj << 8) - 1) * 0x00010001u : 0xffffffffu;  // nothing is above 0xffff
-    }
-    uint32_t pc[SF_TOP_BINS];
-#pragma unroll
-    for (int jj = 0; jj < SF_TOP_BINS; ++jj) pc[jj] = 0;
-    for_chunks([&](int, const uint32_t (&kk)[4]) {
-#pragma unroll
-      for (int p = 0; p < 4; ++p)
-#pragma unroll
-        for (int jj = 0; jj < SF_TOP_BINS; ++jj) pc[jj] += sah_pk_gt01_u16(kk[p], below[jj]);
-    });
-#pragma unroll
-    for (int jj = 0; jj < SF_TOP_BINS; ++jj) {
-      const int c = sah_wave_sum_i((int)((pc[jj] & 0xffffu) + (pc[jj] >> 16)));
-      if (lane == 0) atomicAdd(&S.top[jj], c);
-    }
-    __syncthreads();
+      return bj >= 1 ? (uint32_t)((bj << 8) - 1) * 0x00010001u : 0xffffffffu;  // nothing is above 0xffff
+    };
     int above = 0;
+    for (int j0 = 0; j0 < SF_TOP_BINS && !short_path; j0 += 2) {  // uniform across the workgroup
+      const uint32_t lim0 = bottom(j0), lim1 = bottom(j0 + 1);
+      uint32_t pc0 = 0, pc1 = 0;
+      for_chunks([&](int, const uint32_t (&kk)[4]) {
 #pragma unroll
-    for (int jj = 0; jj < SF_TOP_BINS; ++jj) {
-      const int c = S.top[jj];  // candidates in the bins b_max .. b_max - jj
-      if (!short_path && b_max - jj >= 1 && c >= k) {
-        short_path = true;
-        b1 = b_max - jj;
-        need1 = k - above;
+        for (int p = 0; p < 4; ++p) {
+          pc0 += sah_pk_gt01_u16(kk[p], lim0);
+          pc1 += sah_pk_gt01_u16(kk[p], lim1);
+        }
+      });
+      // both counts in one wave sum: a wave holds at most 64 * 8 * CPW <= 4096 candidates
+      const int both = sah_wave_sum_i((int)((pc0 & 0xffffu) + (pc0 >> 16) + (((pc1 & 0xffffu) + (pc1 >> 16)) << 16)));
+      if (lane == 0) {
+        atomicAdd(&S.top[j0], both & 0xffff);
+        atomicAdd(&S.top[j0 + 1], (int)((uint32_t)both >> 16));
       }
-      above = c;
+      __syncthreads();
+#pragma unroll
+      for (int jj = 0; jj < 2; ++jj) {
+        const int c = S.top[j0 + jj];  // candidates in the bins b_max .. b_max - (j0 + jj)
+        if (!short_path && b_max - (j0 + jj) >= 1 && c >= k) {
+          short_path = true;
+          b1 = b_max - (j0 + jj);
+          need1 = k - above;
+        }
+        above = c;
+      }
     }
   }
   if (short_path) {

@@ -814,6 +814,14 @@ def test_fused_hash_decode_kernel_matches_separate_launches(cuda, monkeypatch, d
     (40000, 39990, 10, 2048, 3000, 640, 0x0080),   # 5 chunks per wave
     (70016, 70000, 16, 3000, 40, 700, 7),          # 9 chunks per wave, ties everywhere
     (140000, 139999, 1, 5000, 0, 300, 0x0080),     # too long for registers: keys re-read per pass
+    # distinct key values = -(1 + j): float-like keys, the k-th largest lies j high-byte bins below the row's largest
+    # (the threshold search looks at the largest key's bin and the next, then at two more, then builds histograms)
+    (6000, 6000, 0, 300, -1, 40, 0x0080),
+    (6000, 5990, 10, 300, -2, 40, 0x0080),
+    (6000, 6000, 0, 300, -3, 40, 0),
+    (20000, 19999, 1, 1000, -4, 640, 0x0080),
+    (6000, 6000, 0, 300, -6, 40, 0x0080),
+    (33000, 33000, 0, 300, -4, 40, 0x0080),        # the same with 5 chunks per wave
 ])
 def test_select_topk_16bit_keys_against_stable_sort(cuda, case):
     """sah_select_topk on 16-bit keys, straight through the C ABI: the k best candidates in the order
@@ -827,7 +835,20 @@ def test_select_topk_16bit_keys_against_stable_sort(cuda, case):
     n_rows = 3 if n_keys < 20000 else 2
     rng = np.random.default_rng(n_keys + k)
     pitch = (n_cand + 7) // 8 * 8
-    keys = (rng.integers(1, n_vals + 1, size=(n_rows, pitch)) if n_vals else rng.integers(0, 65536, size=(n_rows, pitch))).astype(np.uint16)
+    if n_vals < 0:
+        j, top = -n_vals - 1, 0xC9
+        # fewer than k keys in the j bins from the largest key's down, most of the row in the bin below them (low bytes
+        # from a small set, so the threshold is tied) and the rest spread over the bins further down
+        hi = rng.integers(top - j - 40, top - j + 1, size=(n_rows, pitch))
+        hi[rng.random((n_rows, pitch)) < 0.5] = top - j
+        few = rng.random((n_rows, pitch)) < (0.5 * k / n_cand)
+        hi[few] = rng.integers(top - j + 1, top + 1, size=int(few.sum())) if j else top
+        hi[:, 5] = top
+        keys = ((hi << 8) | rng.integers(0, 256, size=(n_rows, pitch)) // 8 * 8).astype(np.uint16)
+    elif n_vals:
+        keys = rng.integers(1, n_vals + 1, size=(n_rows, pitch)).astype(np.uint16)
+    else:
+        keys = rng.integers(0, 65536, size=(n_rows, pitch)).astype(np.uint16)
     n_words = (n_keys + 31) // 32
     cap = min(n_keys, n_active + k)
     cols = np.full((n_rows, cap), -1, np.int32)
