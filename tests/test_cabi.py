@@ -59,3 +59,53 @@ def test_struct_layouts_match_header_sizes():
     # sah_rows: 4 pointers + 4 int32
     assert ctypes.sizeof(N.Rows) == 4 * 8 + 4 * 4
     assert ctypes.sizeof(N.SinkLocalArgs) == ctypes.sizeof(N.Rows) + 5 * 4 + 4 + 8
+
+
+def test_every_entry_point_refuses_null_and_names_itself():
+    """Every `int sah_*(const args*)` entry point checks its argument block before touching the device."""
+    lib = N.lib()
+    one_arg = ["sah_sink_local_indices", "sah_rows_from_dense", "sah_rows_to_dense", "sah_hash_signatures", "sah_hamming_topk",
+               "sah_hamming_scores", "sah_qk_scores", "sah_select_topk", "sah_pq_keys_absmax", "sah_pq_kmeans_assign",
+               "sah_pq_kmeans_update", "sah_pq_adc_scores", "sah_sparse_attention", "sah_sparse_attention_static",
+               "sah_attention_weights", "sah_adaptive_budget", "sah_adaptive_sample", "sah_hash_decode_topk",
+               "sah_hash_compact_codes", "sah_run_chain"]
+    for fn in one_arg:
+        assert getattr(lib, fn)(None) == -2, fn
+        assert fn.replace("_static", "").encode() in lib.sah_last_error() or fn.encode() in lib.sah_last_error(), fn
+    assert lib.sah_hash_signatures_pair(None, None) == -2
+    assert lib.sah_hash_decode_attention(None, None) == -2
+    # whatever takes an argument block is in one of the two lists above
+    plain = {"sah_version", "sah_last_error", "sah_timing_enable", "sah_timing_collect", "sah_pq_adc_lut_bytes",
+             "sah_sparse_attention_work_floats"}
+    assert set(one_arg) | {"sah_hash_signatures_pair", "sah_hash_decode_attention"} | plain == set(_declared_functions())
+
+
+def test_bad_argument_blocks_are_refused_with_the_documented_codes():
+    """Validation happens on the host, before any launch: the codes of include/sah.h (no GPU needed)."""
+    lib = N.lib()
+    buf = ctypes.create_string_buffer(4096)          # stands for device memory: never dereferenced by the checks
+    ptr = ctypes.addressof(buf)
+
+    def rows(n_rows=4, n_keys=100, cap=16, n_words=None):
+        return N.Rows(ptr, ptr, None, ptr, n_rows, cap, n_keys, (n_keys + 31) // 32 if n_words is None else n_words)
+
+    # rows: empty, inconsistent bitmap width, missing arrays
+    a = N.SinkLocalArgs(rows(n_rows=0), 1, 4, 4, 1, 0, None)
+    assert lib.sah_sink_local_indices(ctypes.byref(a)) == -1
+    a = N.SinkLocalArgs(rows(n_words=1), 1, 4, 4, 1, 0, None)
+    assert lib.sah_sink_local_indices(ctypes.byref(a)) == -1 and b"n_words" in lib.sah_last_error()
+    r = rows()
+    r.cnt = None
+    a = N.SinkLocalArgs(r, 1, 4, 4, 1, 0, None)
+    assert lib.sah_sink_local_indices(ctypes.byref(a)) == -2
+    # selection: key width other than 16 / 32 bits, capacity below active + k
+    sel = N.SelectTopkArgs(rows(), ptr, 104, 8, 100, 0, 5, 0, 0, 0, 0, None)
+    assert lib.sah_select_topk(ctypes.byref(sel)) < 0 and b"sah_select_topk" in lib.sah_last_error()
+    sel = N.SelectTopkArgs(rows(cap=6), ptr, 104, 16, 100, 0, 50, 0, 1, 4, 4, None)   # fresh rows: sink + window do not fit
+    assert lib.sah_select_topk(ctypes.byref(sel)) == -4
+    sel = N.SelectTopkArgs(rows(), ptr, 104, 16, 100, 50, 5, 0, 0, 0, 0, None)         # candidates beyond the row
+    assert lib.sah_select_topk(ctypes.byref(sel)) == -1
+    sel = N.SelectTopkArgs(rows(), ptr, 96, 16, 100, 0, 5, 0, 0, 0, 0, None)           # key rows shorter than the candidates
+    assert lib.sah_select_topk(ctypes.byref(sel)) == -1
+    # what the no-allocation attention refuses is more than its built-in buffer holds
+    assert N.work_floats(1024, 131072, 128) > 4 * 1024 * 1024 >= N.work_floats(512, 131072, 128)
