@@ -392,6 +392,15 @@ typedef struct sah_attention_args {
   float* logits_out;
   float* stats_out;
   void* stream;
+  /* Training-mode dropout of the exp weights (torch.nn.functional.dropout in _compute_masked_exp_attention_weights,
+   * utils/mask_attention_utils.py:234-238): with 0 < dropout_p < 1 the entry (mask row r, column j) is dropped
+   * when word 0 of Philox4x32-10(counter (j, r, offset lo, offset hi), key (seed lo, seed hi)) is below
+   * dropout_p * 2^32, and kept entries are scaled by 1 / (1 - dropout_p), in the numerator and in the denominator
+   * (the sink term, where there is one, is not scaled). The reference draws from torch's generator: the stream
+   * differs, the distribution does not. 0: no dropout. */
+  float dropout_p;
+  uint64_t dropout_seed;
+  uint64_t dropout_offset;
 } sah_attention_args;
 int64_t sah_sparse_attention_work_floats(int32_t n_rows, int32_t max_cnt, int32_t D);
 int sah_sparse_attention(const sah_attention_args* a);
@@ -421,6 +430,9 @@ typedef struct sah_attention_weights_args {
   int32_t dtype;
   void* weights;
   void* stream;
+  float dropout_p;          /* the same three values the sah_sparse_attention call was given */
+  uint64_t dropout_seed;
+  uint64_t dropout_offset;
 } sah_attention_weights_args;
 int sah_attention_weights(const sah_attention_weights_args* a);
 

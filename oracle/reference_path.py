@@ -28,7 +28,8 @@ check that a dropped term, a wrong sign or index or a transposed operand fails.
   (batch, head, sub-space) loops; `kmeans_lloyd` by hand-computed Lloyd steps including the
   empty-cluster reseed; `adaptive_exp_scores` against an fp64 evaluation of the definition;
   `adaptive_budget` against hand arithmetic; Philox4x32-10 against the published known-answer vectors;
-  `research_attention` (the chain) by composing the pieces on a brute-forceable size.
+  `research_attention` (the chain) by composing the pieces on a brute-forceable size; the training-mode dropout of
+  `masked_attention` against the definition of `torch.nn.functional.dropout` in fp64 and single Philox calls.
 Not reproducible by any restatement, because the reference leaves them to torch's RNG or to an
 unspecified library choice: which samples `torch.randint` draws (adaptive / random sampling, k-means
 initialisation and reseeding; the oracle takes the draws or the start centres as inputs, or draws
@@ -529,12 +530,31 @@ def random_sampling(prev: OMask, rate: float, seed: int, offset: int) -> OMask:
 
 
 # ----------------------------------------------------------------------- attention
+def dropout_keep(seed: int, offset: int, n_rows: int, n_keys: int, p: float) -> torch.Tensor:
+    """(n_rows, n_keys) bool: entry (r, j) survives a dropout of probability p when word 0 of
+    Philox4x32-10(counter (j, r, offset lo, offset hi), key (seed lo, seed hi)) is at least p * 2^32."""
+    import numpy as np
+
+    ctr = np.zeros((n_rows, n_keys, 4), dtype=np.uint64)
+    ctr[:, :, 0] = np.arange(n_keys, dtype=np.uint64)[None, :]
+    ctr[:, :, 1] = np.arange(n_rows, dtype=np.uint64)[:, None]
+    ctr[:, :, 2] = offset & 0xFFFFFFFF
+    ctr[:, :, 3] = (offset >> 32) & 0xFFFFFFFF
+    u = philox4x32_10(ctr, (seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF))[..., 0].astype(np.uint64)
+    thresh = max(1, min(0xFFFFFFFF, int(np.float64(np.float32(p)) * 4294967296.0)))
+    return torch.from_numpy(u >= np.uint64(thresh))
+
+
 def masked_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, attention_mask: Optional[torch.Tensor],
                      sinks: Optional[torch.Tensor], scaling: float, mask: OMask,
-                     accumulate: torch.dtype = torch.float32) -> Tuple[torch.Tensor, torch.Tensor]:
+                     accumulate: torch.dtype = torch.float32,
+                     dropout: Optional[Tuple[float, int, int]] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """(out (B, Lq, Hq, D), weights (B, Hq, Lq, Lk)) in the query dtype —
     mask_attention_utils.py:187-240 (exp weights), :357-402 (sink logit), :406-491 (num/den).
-    `accumulate=torch.float64` gives a high-precision variant for tolerance studies."""
+    `accumulate=torch.float64` gives a high-precision variant for tolerance studies.
+    `dropout` = (p, seed, offset): training-mode dropout of the exp weights (:234-238, torch.nn.functional.dropout:
+    an element is zeroed with probability p, the others are scaled by 1 / (1 - p)), with the element's fate drawn
+    from Philox (dropout_keep) instead of torch's generator."""
     G = q.shape[1] // k.shape[1]
     kk = repeat_kv(k, G).to(accumulate)
     vv = repeat_kv(v, G).to(accumulate)
@@ -545,6 +565,11 @@ def masked_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, attentio
     e = torch.exp(logits - old_max)
     if mask.kind == "dense":
         e = apply_inv_mask_dense(e, mask.dense)
+    if dropout is not None and dropout[0] > 0.0:
+        p, seed, offset = dropout
+        B, H, Q, Lk = e.shape
+        keep = dropout_keep(seed, offset, B * H * Q, Lk, p).view(B, H, Q, Lk)
+        e = e * keep.to(accumulate) * (1.0 / (1.0 - float(torch.tensor(p, dtype=torch.float32))))
     num = torch.matmul(e, vv)
     den = e.sum(dim=-1, keepdim=True)
     if sinks is not None:
@@ -560,12 +585,13 @@ def masked_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, attentio
 
 # --------------------------------------------------------------- chain composition
 def research_attention(masker_specs: Sequence[Tuple], q, k, v, attention_mask, scaling: float,
-                       sinks: Optional[torch.Tensor] = None, state: Optional[dict] = None):
+                       sinks: Optional[torch.Tensor] = None, state: Optional[dict] = None,
+                       dropout: Optional[Tuple[float, int, int]] = None):
     """ResearchAttention.custom_attention — research_attention/base.py:63-170.
     masker_specs: ("sink", size) | ("local", size) | ("oracle_topk", heavy) |
     ("hash_topk", heavy, weights, activation) | ("pq_topk", heavy, init_offset, centroids, codebook) |
     ("adaptive", rate, epsilon, delta, init_offset, local_offset, seed, offset) | ("random", rate, seed, offset).
-    Returns (out, weights, final OMask)."""
+    `dropout` = (p, seed, offset): see masked_attention. Returns (out, weights, final OMask)."""
     shape = (q.shape[0], q.shape[1], q.shape[2], k.shape[2])
     m = OMask.empty(shape, q.dtype)
     state = {} if state is None else state
@@ -599,5 +625,5 @@ def research_attention(masker_specs: Sequence[Tuple], q, k, v, attention_mask, s
             m = random_sampling(m, spec[1], spec[2], spec[3])  # ("random", rate, seed, offset)
         else:
             raise ValueError(kind)
-    out, w = masked_attention(q, k, v, attention_mask, sinks, scaling, m)
+    out, w = masked_attention(q, k, v, attention_mask, sinks, scaling, m, dropout=dropout)
     return out, w, m

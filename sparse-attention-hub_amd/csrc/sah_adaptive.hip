@@ -14,27 +14,8 @@
 #define AD_NW (AD_NT / SAH_WAVE)
 #define AD_MAX_LDS_WORDS 36864  // 144 KB bitmap: sampling range up to ~1.17 M keys
 
-// ---------------------------------------------------------------------------
-// Philox4x32-10 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3")
-// ---------------------------------------------------------------------------
-__device__ __forceinline__ uint32_t ad_mulhi(uint32_t a, uint32_t b) { return (uint32_t)(((uint64_t)a * b) >> 32); }
-
-__device__ __forceinline__ void ad_philox(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1,
-                                          uint32_t (&out)[4]) {
-#pragma unroll
-  for (int round = 0; round < 10; ++round) {
-    const uint32_t hi0 = ad_mulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
-    const uint32_t hi1 = ad_mulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
-    const uint32_t n0 = hi1 ^ c1 ^ k0, n2 = hi0 ^ c3 ^ k1;
-    c0 = n0; c1 = lo1; c2 = n2; c3 = lo0;
-    k0 += 0x9E3779B9u;
-    k1 += 0xBB67AE85u;
-  }
-  out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
-}
-
 // uniform column of [start, start + range) from one 32-bit draw
-__device__ __forceinline__ int ad_column(uint32_t u, int start, int range) { return start + (int)ad_mulhi(u, (uint32_t)range); }
+__device__ __forceinline__ int ad_column(uint32_t u, int start, int range) { return start + (int)sah_mulhi(u, (uint32_t)range); }
 
 // ---------------------------------------------------------------------------
 // score keys -> numerators, rounded where the reference's torch ops round
@@ -191,7 +172,7 @@ __global__ __launch_bounds__(AD_NT) void k_adaptive_budget(ad_budget_params P) {
   part = 0.f;
   for (int c = tid; c < n_calls; c += AD_NT) {
     uint32_t u[4];
-    ad_philox((uint32_t)c, (uint32_t)r, P.o0, P.o1, P.k0, P.k1, u);
+    sah_philox((uint32_t)c, (uint32_t)r, P.o0, P.o1, P.k0, P.k1, u);
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       if (4 * c + t < P.n_base) {
@@ -205,7 +186,7 @@ __global__ __launch_bounds__(AD_NT) void k_adaptive_budget(ad_budget_params P) {
   part = 0.f;
   for (int c = tid; c < n_calls; c += AD_NT) {
     uint32_t u[4];
-    ad_philox((uint32_t)c, (uint32_t)r, P.o0, P.o1, P.k0, P.k1, u);
+    sah_philox((uint32_t)c, (uint32_t)r, P.o0, P.o1, P.k0, P.k1, u);
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       if (4 * c + t < P.n_base) {
@@ -290,7 +271,7 @@ __global__ __launch_bounds__(AD_NT) void k_adaptive_sample(ad_sample_params P) {
   const int n_calls = (budget + 3) >> 2;
   for (int c = tid; c < n_calls; c += AD_NT) {
     uint32_t u[4];
-    ad_philox((uint32_t)c, (uint32_t)r, P.o0, P.o1, P.k0, P.k1, u);
+    sah_philox((uint32_t)c, (uint32_t)r, P.o0, P.o1, P.k0, P.k1, u);
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       if (4 * c + t < budget) {

@@ -14,7 +14,7 @@
 
 #include <mutex>
 
-template <int DT, int D, bool ROW>
+template <int DT, int D, bool ROW, bool DROP>
 __global__ __launch_bounds__(ROW ? ATT_ROW_NT : ATT_NT, ROW ? 1 : 5) void k_sparse_attn(att_params P) {
   sah_touch_kernargs<sizeof(att_params)>();
   constexpr int NW = (ROW ? ATT_ROW_NT : ATT_NT) / SAH_WAVE;
@@ -40,7 +40,7 @@ __global__ __launch_bounds__(ROW ? ATT_ROW_NT : ATT_NT, ROW ? 1 : 5) void k_spar
   const int b = gidx / (P.Lq * P.Hkv);
   const int h = hk * G + slot % G;
   const int r = (b * P.Hq + h) * P.Lq + qi;
-  att_tile<DT, D, ROW>(P, r, b, h, hk, qi, split, n_split, nullptr, -1, s_m, s_l, s_acc);
+  att_tile<DT, D, ROW, DROP>(P, r, b, h, hk, qi, split, n_split, nullptr, -1, s_m, s_l, s_acc);
 }
 
 template <int DT, int D>
@@ -53,7 +53,8 @@ __global__ __launch_bounds__(D < 64 ? 64 : D) void k_attn_combine(const float* w
 
 template <int DT>
 __global__ __launch_bounds__(256) void k_attn_weights(sah_rows R, const float* logits, int64_t pitch,
-                                                      const float* stats, float unit_inv_w, int dense, void* weights) {
+                                                      const float* stats, float unit_inv_w, int dense, void* weights,
+                                                      sah_dropout drop) {
   const int r = blockIdx.y;
   const float m = stats[2 * (int64_t)r];
   const float den = stats[2 * (int64_t)r + 1];
@@ -68,6 +69,7 @@ __global__ __launch_bounds__(256) void k_attn_weights(sah_rows R, const float* l
     if (R.w) iw = sah_round<DT>(1.0f / sah_round<DT>(R.w[(int64_t)r * R.cap + i] + 1e-6f));
     if (c < 0 || c >= R.n_keys) return;
   }
+  if (drop.thresh) iw *= drop.factor(r, c);
   const float z = logits[(int64_t)r * pitch + i];
   const float p = (z == -INFINITY) ? 0.f : att_exp<DT>(z - m) * iw / den;
   sah_store<DT>(weights, (int64_t)r * R.n_keys + c, p);
@@ -104,7 +106,8 @@ static int att_launch(const sah_attention_args* a, const att_params& P, bool tim
     sah_timed timed("k_sparse_attn", a->stream, timing);
     const int n_tiles = a->rows.n_rows / G;
     const int n_wg = (n_tiles + ATT_XCDS - 1) / ATT_XCDS * ATT_XCDS * G;
-    hipLaunchKernelGGL((k_sparse_attn<DT, D, true>), dim3(n_wg), dim3(ATT_ROW_NT), 0, st, P);
+    if (P.drop.thresh) hipLaunchKernelGGL((k_sparse_attn<DT, D, true, true>), dim3(n_wg), dim3(ATT_ROW_NT), 0, st, P);
+    else hipLaunchKernelGGL((k_sparse_attn<DT, D, true, false>), dim3(n_wg), dim3(ATT_ROW_NT), 0, st, P);
     return sah_launch_status("sah_sparse_attention");
   }
   int rc;
@@ -112,7 +115,8 @@ static int att_launch(const sah_attention_args* a, const att_params& P, bool tim
     sah_timed timed("k_sparse_attn", a->stream, timing);
     const int n_tiles = (a->rows.n_rows / G) * P.n_split;
     const int n_wg = (n_tiles + ATT_XCDS - 1) / ATT_XCDS * ATT_XCDS * G;
-    hipLaunchKernelGGL((k_sparse_attn<DT, D, false>), dim3(n_wg), dim3(ATT_NT), 0, st, P);
+    if (P.drop.thresh) hipLaunchKernelGGL((k_sparse_attn<DT, D, false, true>), dim3(n_wg), dim3(ATT_NT), 0, st, P);
+    else hipLaunchKernelGGL((k_sparse_attn<DT, D, false, false>), dim3(n_wg), dim3(ATT_NT), 0, st, P);
     rc = sah_launch_status("sah_sparse_attention");
   }
   if (rc) return rc;
@@ -185,6 +189,8 @@ int att_prepare(const sah_attention_args* a, att_params& P) {
   P.sinks = a->sinks; P.out = a->out; P.stats = a->stats_out;
   P.logits_out = a->logits_out;
   P.logits_pitch = a->dense ? a->Lk : a->rows.cap;
+  if (!sah_dropout_fill(a->dropout_p, a->dropout_seed, a->dropout_offset, P.drop))
+    return sah_fail(SAH_EINVAL, "sah_sparse_attention: dropout_p %g not in [0, 1)", (double)a->dropout_p);
   const int64_t need = (int64_t)a->rows.n_rows * P.n_split * (a->D + 2);
   if (a->work_floats < need)
     return sah_fail(SAH_ECAPACITY, "sah_sparse_attention: work has %lld floats, need %lld", (long long)a->work_floats,
@@ -265,11 +271,14 @@ extern "C" int sah_attention_weights(const sah_attention_weights_args* a) {
   const int64_t pitch = dense ? a->rows.n_keys : a->rows.cap;
   dim3 g((max_cnt + 255) / 256, a->rows.n_rows), b(256);
   hipStream_t st = (hipStream_t)a->stream;
+  sah_dropout drop;
+  if (!sah_dropout_fill(a->dropout_p, a->dropout_seed, a->dropout_offset, drop))
+    return sah_fail(SAH_EINVAL, "sah_attention_weights: dropout_p %g not in [0, 1)", (double)a->dropout_p);
   sah_timed timed("k_attn_weights", a->stream);
   switch (a->dtype) {
-    case SAH_F32: hipLaunchKernelGGL(k_attn_weights<SAH_F32>, g, b, 0, st, a->rows, a->logits, pitch, a->stats, a->unit_inv_w, dense, a->weights); break;
-    case SAH_BF16: hipLaunchKernelGGL(k_attn_weights<SAH_BF16>, g, b, 0, st, a->rows, a->logits, pitch, a->stats, a->unit_inv_w, dense, a->weights); break;
-    case SAH_F16: hipLaunchKernelGGL(k_attn_weights<SAH_F16>, g, b, 0, st, a->rows, a->logits, pitch, a->stats, a->unit_inv_w, dense, a->weights); break;
+    case SAH_F32: hipLaunchKernelGGL(k_attn_weights<SAH_F32>, g, b, 0, st, a->rows, a->logits, pitch, a->stats, a->unit_inv_w, dense, a->weights, drop); break;
+    case SAH_BF16: hipLaunchKernelGGL(k_attn_weights<SAH_BF16>, g, b, 0, st, a->rows, a->logits, pitch, a->stats, a->unit_inv_w, dense, a->weights, drop); break;
+    case SAH_F16: hipLaunchKernelGGL(k_attn_weights<SAH_F16>, g, b, 0, st, a->rows, a->logits, pitch, a->stats, a->unit_inv_w, dense, a->weights, drop); break;
     default: return sah_fail(SAH_EDTYPE, "sah_attention_weights: dtype %d", a->dtype);
   }
   return sah_launch_status("sah_attention_weights");

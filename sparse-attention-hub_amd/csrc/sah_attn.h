@@ -27,6 +27,7 @@ struct att_params {
   float* work;
   float* logits_out;
   int64_t logits_pitch;
+  sah_dropout drop;
 };
 
 // exact expf for fp32 storage (1e-5 output tolerance), hardware exp2 path otherwise
@@ -242,7 +243,9 @@ struct att_lane {
 // The calling wave attends to the entries first .. first + 63, first + stride .., all below `bound`, of row r:
 // entry i is column col_of(i) (anything outside [0, Lk) is skipped) with inverse weight inv_w_of(i). Batches of UB
 // iterations: the K and V rows of a batch are requested together, so 2 * UB row loads are in flight per lane.
-template <int DT, int D, typename ColOf, typename InvWOf>
+// DROP: training-mode dropout of the exp weights (P.drop) is applied; a variant of its own, so that the decode path
+// carries no trace of it.
+template <int DT, int D, bool DROP = false, typename ColOf, typename InvWOf>
 __device__ __forceinline__ void att_walk(const att_params& P, int r, int b, int h, int hk, int qi, int first, int bound,
                                          int stride, ColOf col_of, InvWOf inv_w_of, att_wave_state& st) {
   typedef att_lane<DT, D> lane_t;
@@ -264,6 +267,7 @@ __device__ __forceinline__ void att_walk(const att_params& P, int r, int b, int 
       idx_l = col_of(my);
       invw_l = inv_w_of(my);
       if (idx_l < 0 || idx_l >= P.Lk) idx_l = -1;
+      if (DROP && idx_l >= 0) invw_l *= P.drop.factor(r, idx_l);
     }
 #pragma unroll
     for (int ib = 0; ib < IT; ib += UB) {
@@ -356,7 +360,7 @@ __device__ __forceinline__ void att_store_row(const att_params& P, int r, int b,
 // ROW = true: a workgroup of 16 waves handles a whole row, every wave an equal share of the row's entries,
 //   and merges the 16 partial results itself: no workspace, no second kernel, every CU gets the same
 //   amount of work when there are at least as many rows as CUs.
-template <int DT, int D, bool ROW>
+template <int DT, int D, bool ROW, bool DROP = false>
 __device__ __forceinline__ void att_tile(const att_params& P, int r, int b, int h, int hk, int qi, int split, int n_split,
                                          const int* cols_known, int cnt_known,
                                          float (&s_m)[(ROW ? ATT_ROW_NT : ATT_NT) / SAH_WAVE],
@@ -401,7 +405,7 @@ __device__ __forceinline__ void att_tile(const att_params& P, int r, int b, int 
   const float* wts = (!P.dense && P.rows.w) ? P.rows.w + (int64_t)r * P.rows.cap : nullptr;
   att_wave_state st;
   st.clear();
-  att_walk<DT, D>(
+  att_walk<DT, D, DROP>(
       P, r, b, h, hk, qi, first, bound, stride,
       [&](int i) { return P.dense == 1 ? i : (P.dense == 2 ? (i < P.closed_sink ? i : P.closed_lo + (i - P.closed_sink)) : cols[i]); },
       // the reference evaluates 1/(w + 1e-6) in the mask dtype (utils/mask.py:737-740)

@@ -89,6 +89,50 @@ __device__ __forceinline__ void sah_touch_kernargs() {
 }
 
 // ---------------------------------------------------------------------------
+// Philox4x32-10 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3")
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ uint32_t sah_mulhi(uint32_t a, uint32_t b) { return (uint32_t)(((uint64_t)a * b) >> 32); }
+
+__device__ __forceinline__ void sah_philox(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1,
+                                           uint32_t (&out)[4]) {
+#pragma unroll
+  for (int round = 0; round < 10; ++round) {
+    const uint32_t hi0 = sah_mulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
+    const uint32_t hi1 = sah_mulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+    const uint32_t n0 = hi1 ^ c1 ^ k0, n2 = hi0 ^ c3 ^ k1;
+    c0 = n0; c1 = lo1; c2 = n2; c3 = lo0;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+// Dropout of the exp weights: what an entry's weight is multiplied by (0, or 1 / (1 - p)). thresh = p * 2^32.
+struct sah_dropout {
+  uint32_t thresh;  // 0: off
+  float scale;
+  uint32_t k0, k1, o0, o1;
+  __device__ __forceinline__ float factor(int row, int col) const {
+    uint32_t u[4];
+    sah_philox((uint32_t)col, (uint32_t)row, o0, o1, k0, k1, u);
+    return u[0] < thresh ? 0.f : scale;
+  }
+};
+// host side: from the entry point's three arguments; false when p is outside [0, 1)
+static inline bool sah_dropout_fill(float p, uint64_t seed, uint64_t offset, sah_dropout& d) {
+  d.thresh = 0; d.scale = 1.f; d.k0 = d.k1 = d.o0 = d.o1 = 0;
+  if (!(p >= 0.f) || !(p < 1.f)) return false;
+  if (p == 0.f) return true;
+  const double t = (double)p * 4294967296.0;
+  d.thresh = t >= 4294967295.0 ? 0xffffffffu : (uint32_t)t;
+  if (d.thresh == 0) d.thresh = 1;
+  d.scale = 1.0f / (1.0f - p);
+  d.k0 = (uint32_t)seed; d.k1 = (uint32_t)(seed >> 32);
+  d.o0 = (uint32_t)offset; d.o1 = (uint32_t)(offset >> 32);
+  return true;
+}
+
+// ---------------------------------------------------------------------------
 // device side: dtype helpers (bf16 / f16 handled as raw bits, fp32 arithmetic)
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ float sah_bits_to_float(uint32_t u) { return __builtin_bit_cast(float, u); }

@@ -341,6 +341,7 @@ extern "C" int sah_hash_decode_attention(const sah_hash_decode_args* a, const sa
   const size_t lds = cols_offset + (size_t)a->rows.cap * 4;
   const bool one_kernel =
       hdec_fusable(a) && A.n_split == 0 && !t->dense && !t->closed_form && !t->amask && !t->logits_out && !t->rows.w && t->Lq == 1 &&
+      t->dropout_p == 0.f &&
       t->rows.cols == a->rows.cols && t->rows.cnt == a->rows.cnt && t->rows.cap == a->rows.cap &&
       t->rows.n_rows == a->rows.n_rows && t->stream == a->stream && t->dtype == a->query_sig->dtype &&
       (t->D == 128 || t->D == 64) && lds <= 150 * 1024;

@@ -284,6 +284,9 @@ class AttentionArgs(C.Structure):
         ("logits_out", C.c_void_p),
         ("stats_out", C.c_void_p),
         ("stream", C.c_void_p),
+        ("dropout_p", C.c_float),
+        ("dropout_seed", C.c_uint64),
+        ("dropout_offset", C.c_uint64),
     ]
 
 
@@ -349,6 +352,9 @@ class AttentionWeightsArgs(C.Structure):
         ("dtype", C.c_int32),
         ("weights", C.c_void_p),
         ("stream", C.c_void_p),
+        ("dropout_p", C.c_float),
+        ("dropout_seed", C.c_uint64),
+        ("dropout_offset", C.c_uint64),
     ]
 
 

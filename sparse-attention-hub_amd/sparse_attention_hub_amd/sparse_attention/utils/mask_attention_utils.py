@@ -12,6 +12,8 @@ from __future__ import annotations
 
 from typing import Any, Dict, Optional, Tuple, Union
 
+import itertools
+
 import numpy as np
 import torch
 from torch import nn
@@ -75,6 +77,7 @@ def _run_attention(
     return_attention_weights: bool,
     out: Optional[torch.Tensor] = None,
     return_stats: bool = False,
+    dropout: Tuple[float, int, int] = (0.0, 0, 0),
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """rows=None => dense attention over all keys. `return_stats`: the second value is the kernel's
     fp32 (n_rows, 2) tensor of (largest logit among the row's entries, softmax denominator relative to it)
@@ -135,6 +138,7 @@ def _run_attention(
         None if logits is None else logits.data_ptr(),
         None if stats is None else stats.data_ptr(),
         N.stream_ptr(dev),
+        dropout[0], dropout[1], dropout[2],
     )
     N.call("sah_sparse_attention", args)
     if return_stats:
@@ -144,17 +148,25 @@ def _run_attention(
         weights = torch.zeros((B, Hq, Lq, Lk), dtype=q.dtype, device=dev)
         wargs = N.AttentionWeightsArgs(
             rows_struct, logits.data_ptr(), stats.data_ptr(), unit, 1 if dense else 0, dt,
-            weights.data_ptr(), N.stream_ptr(dev),
+            weights.data_ptr(), N.stream_ptr(dev), dropout[0], dropout[1], dropout[2],
         )
         N.call("sah_attention_weights", wargs)
     return out, weights
 
 
-def _reject_training_dropout(module: Optional[nn.Module], dropout: float) -> None:
-    if dropout > 0.0 and module is not None and getattr(module, "training", False):
-        raise NotImplementedError(
-            "attention dropout in training mode is not implemented by the MI355X decode kernels"
-        )
+_DROPOUT_CALLS = itertools.count()
+
+
+def _training_dropout(module: Optional[nn.Module], dropout: float) -> Tuple[float, int, int]:
+    """(p, seed, offset) for the attention kernel: dropout of the exp weights applies in training mode only
+    (reference: mask_attention_utils.py:234-238, `module.training`). The kernel draws with Philox4x32-10 keyed by
+    torch's seed and a per-call offset where the reference draws from torch's generator: another stream of the same
+    distribution, reseeded by `torch.manual_seed` as well."""
+    if not (dropout > 0.0 and module is not None and getattr(module, "training", False)):
+        return 0.0, 0, 0
+    if not dropout < 1.0:
+        raise ValueError(f"dropout probability has to be below 1 for the attention kernel, but got {dropout}")
+    return float(dropout), int(torch.initial_seed()) & 0xFFFFFFFFFFFFFFFF, next(_DROPOUT_CALLS)
 
 
 def get_true_attention_output(
@@ -168,8 +180,8 @@ def get_true_attention_output(
     **kwargs: Dict[str, Any],
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """Dense attention output (B, Lq, Hq, D) (reference: mask_attention_utils.py:11-70)."""
-    _reject_training_dropout(module, dropout)
-    out, _ = _run_attention(queries, keys, values, attention_mask, None, scaling, None, False)
+    out, _ = _run_attention(queries, keys, values, attention_mask, None, scaling, None, False,
+                            dropout=_training_dropout(module, dropout))
     return out, None
 
 
@@ -197,14 +209,14 @@ def get_masked_attention_output(
 ) -> Union[torch.Tensor, Tuple[torch.Tensor, torch.Tensor]]:
     """Masked attention output (B, Lq, Hq, D) in the query dtype, optionally with the
     dense probabilities (B, Hq, Lq, Lk)."""
-    _reject_training_dropout(module, dropout)
     mask = sparse_attention_mask
     if mask.is_full or mask.is_empty:
         rows = None
     else:
         rows = mask.to_rows(0)
     out, weights = _run_attention(
-        queries, keys, values, attention_mask, sinks, scaling, rows, return_attention_weights
+        queries, keys, values, attention_mask, sinks, scaling, rows, return_attention_weights,
+        dropout=_training_dropout(module, dropout),
     )
     if return_attention_weights:
         return out, weights
@@ -212,14 +224,15 @@ def get_masked_attention_output(
 
 
 # ------------------------------------------------------------------ numerator / denominator helpers
-def _masked_softmax_parts(queries, keys, values, attention_mask, scaling, mask: Mask):
+def _masked_softmax_parts(queries, keys, values, attention_mask, scaling, mask: Mask, dropout=(0.0, 0, 0)):
     """(out (B, Hq, Lq, D) fp32, den (B, Hq, Lq, 1) fp32, m_all (B, Hq, Lq, 1) fp32) of the masked softmax in the
     reference's scale, i.e. relative to the largest logit over ALL keys of the row
     (mask_attention_utils.py:187-240). Two launches of the attention kernel: one over the mask's rows, one dense
     pass whose statistics give the all-key maximum."""
     B, Hq, Lq, D = queries.shape
     rows = None if (mask.is_full or mask.is_empty) else mask.to_rows(0)
-    out, stats = _run_attention(queries, keys, values, attention_mask, None, scaling, rows, False, return_stats=True)
+    out, stats = _run_attention(queries, keys, values, attention_mask, None, scaling, rows, False, return_stats=True,
+                                dropout=dropout)
     if rows is None:
         all_stats = stats
     else:
@@ -235,8 +248,8 @@ def get_attention_denominator(module: Optional[nn.Module], queries: torch.Tensor
                               sparse_attention_mask: Mask, **kwargs: Dict[str, Any]) -> torch.Tensor:
     """sum_j exp(z_j - max_all z) / (w_j + 1e-6) over the mask's entries, (B, Hq, Lq, 1) fp32
     (reference: mask_attention_utils.py:271-311). The kernel needs a value tensor: the keys stand in."""
-    _reject_training_dropout(module, dropout)
-    _, den, _ = _masked_softmax_parts(queries, keys, keys, attention_mask, scaling, sparse_attention_mask)
+    _, den, _ = _masked_softmax_parts(queries, keys, keys, attention_mask, scaling, sparse_attention_mask,
+                                      _training_dropout(module, dropout))
     return den
 
 
@@ -246,8 +259,8 @@ def get_attention_numerator(module: Optional[nn.Module], queries: torch.Tensor, 
     """sum_j exp(z_j - max_all z) / (w_j + 1e-6) * V_j, (B, Hq, Lq, D) fp32 (reference :314-355). Rebuilt as the
     kernel's normalised output times the denominator, so for bf16 / fp16 inputs it carries the output's rounding
     (one part in 2^8 / 2^11) where the reference's fp32 product does not."""
-    _reject_training_dropout(module, dropout)
-    out, den, _ = _masked_softmax_parts(queries, keys, values, attention_mask, scaling, sparse_attention_mask)
+    out, den, _ = _masked_softmax_parts(queries, keys, values, attention_mask, scaling, sparse_attention_mask,
+                                        _training_dropout(module, dropout))
     return out * den
 
 

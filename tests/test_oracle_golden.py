@@ -605,3 +605,53 @@ def test_hat_weight_loader_runs_no_code_from_the_file(tmp_path):
         pickle.dump([1, 2, 3], f)
     with pytest.raises(ValueError, match="expected Dict"):
         load_hat_weights(str(bad))
+
+
+def test_dropout_keep_follows_the_counter_layout_and_the_rate():
+    """The fate of entry (row r, column j): word 0 of Philox4x32-10 with counter (j, r, offset lo, offset hi) and key
+    (seed lo, seed hi), kept when it is at least p * 2^32. Checked against single calls of the Philox function (which the
+    Random123 vectors pin), so a swapped row / column or a wrong word fails; and the kept share is 1 - p."""
+    import numpy as np
+
+    seed, offset, p = 0x1234_5678_9ABC_DEF0, (5 << 32) | 77, 0.3
+    keep = O.dropout_keep(seed, offset, 6, 40, p)
+    key = (seed & 0xFFFFFFFF, seed >> 32)
+    for r, j in ((0, 0), (1, 0), (0, 1), (5, 39), (3, 17)):
+        u = O.philox4x32_10(np.array([[j, r, offset & 0xFFFFFFFF, offset >> 32]], dtype=np.uint64), key)[0, 0]
+        assert bool(keep[r, j]) == (int(u) >= int(p * 2 ** 32)), (r, j)
+    big = O.dropout_keep(seed, offset, 64, 4096, p)
+    assert abs(float(big.float().mean()) - (1 - p)) < 0.005
+    assert not torch.equal(O.dropout_keep(seed, offset + 1, 6, 40, p), keep)      # another call, another stream
+    assert not torch.equal(O.dropout_keep(seed + 1, offset, 6, 40, p), keep)
+
+
+def test_masked_attention_dropout_has_the_form_of_torch_dropout():
+    """torch.nn.functional.dropout zeroes an element with probability p and scales the others by 1 / (1 - p)
+    (mask_attention_utils.py:234-238 applies it to the exp weights, before numerator and denominator). The oracle's
+    probabilities with dropout, times their denominator, are therefore 0 or the undropped exp weight / (1 - p); the output
+    is the softmax over the kept entries; the sink term is not scaled."""
+    g = torch.Generator().manual_seed(3)
+    B, H, Lq, Lk, D, p = 1, 2, 2, 50, 8, 0.4
+    q, k, v = (torch.randn(B, H, n, D, generator=g) for n in (Lq, Lk, Lk))
+    dense = torch.zeros(B, H, Lq, Lk)
+    dense[..., ::3] = 1.0
+    dense[..., 1] = 0.5
+    m = O.OMask("dense", tuple(dense.shape), dense.dtype, dense)
+    sinks = torch.tensor([0.3, -0.2])
+    drop = (p, 11, 5)
+    out0, w0 = O.masked_attention(q, k, v, None, sinks, 0.5, m)
+    out1, w1 = O.masked_attention(q, k, v, None, sinks, 0.5, m, dropout=drop)
+    keep = O.dropout_keep(11, 5, B * H * Lq, Lk, p).view(B, H, Lq, Lk)
+    assert torch.equal(w1 != 0, (w0 != 0) & keep)
+    # by hand, in fp64: e = exp(z - max) / (w + 1e-6) on the mask, times keep / (1 - p); den += exp(sink - max)
+    z = torch.matmul(q.double(), k.double().transpose(2, 3)) * 0.5
+    mx = z.max(dim=-1, keepdim=True)[0]
+    e = torch.exp(z - mx) * torch.where(dense != 0, 1.0 / (dense.double() + 1e-6), torch.zeros(()).double())
+    e = e * keep.double() / (1.0 - float(torch.tensor(p, dtype=torch.float32)))
+    srow = sinks.double().view(1, H, 1, 1)
+    nm = torch.maximum(mx, srow)
+    sc = torch.exp(mx - nm)
+    den = e.sum(-1, keepdim=True) * sc + torch.exp(srow - nm)
+    want = (torch.matmul(e, v.double()) * sc / den).transpose(1, 2)
+    assert torch.allclose(out1.double(), want, rtol=1e-5, atol=1e-6)
+    assert not torch.allclose(out1, out0, rtol=1e-3)
