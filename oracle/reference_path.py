@@ -33,7 +33,7 @@ check that a dropped term, a wrong sign or index or a transposed operand fails.
 Not reproducible by any restatement, because the reference leaves them to torch's RNG or to an
 unspecified library choice: which samples `torch.randint` draws (adaptive / random sampling, k-means
 initialisation and reseeding; the oracle takes the draws or the start centres as inputs, or draws
-with Philox) and which of several equal scores `torch.topk` keeps (lowest index here).
+with Philox), which elements `torch.nn.functional.dropout` zeroes in training mode (Philox here as well) and which of several equal scores `torch.topk` keeps (lowest index here).
 """
 from __future__ import annotations
 
