@@ -6,7 +6,7 @@
 A step is one `ResearchAttention.custom_attention` call with one query token on a warm
 cache (hash signatures / PQ codes of all earlier keys already built, one new key appended
 per step), on synthetic inputs that are resident in HBM before the timed region. Default
-workload: BASELINE config 3, the one the headline target is quoted on (Sink 128 + Local 512
+workload: headline configuration 3, the one the headline target is quoted on (Sink 128 + Local 512
 + HashAttention top-2048, batch 8, 32 query / 8 KV heads, head_dim 128, 32768 keys, bf16).
 
 Timing. K steps are timed between two synchronisations (host clock and HIP events on the
@@ -19,7 +19,7 @@ reported beside it.
 
 Prints ONE JSON line: whole-step microseconds (`value`), the roofline of the dominant kernel
 from HIP-event timings taken inside this run, the parity of the last timed step against the
-CPU oracle, the oracle timed on the host cores, and short sub-runs of the other BASELINE
+CPU oracle, the oracle timed on the host cores, and short sub-runs of the other headline
 configurations (`other_configs`).
 """
 from __future__ import annotations
@@ -318,7 +318,7 @@ def parity_and_cpu_baseline(run, last, budget_s=25.0):
 
 
 def sub_run(cfg: int, dev) -> dict:
-    """A short run of another BASELINE configuration: cold call, 5 warm-up steps, one bracket of timed steps."""
+    """A short run of another configuration of the headline set: cold call, 5 warm-up steps, one bracket of timed steps."""
     import torch
 
     w = dict(WORKLOADS[cfg])
@@ -342,7 +342,7 @@ def sub_run(cfg: int, dev) -> dict:
 
 
 def cold_probe(dev) -> dict:
-    """The matrix-core kernels of the cold calls at their BASELINE shapes, timed with HIP events: two Lloyd iterations
+    """The matrix-core kernels of the cold calls at the shapes of the headline configurations, timed with HIP events: two Lloyd iterations
     of the config-4 k-means (4 x 8 KV heads x 16 sub-spaces, 32640 keys, 256 centres, sub-vectors of 8) and the
     config-3 bulk signature build (8 x 32 heads x 32768 keys, MLP 128-128-128-32)."""
     import torch

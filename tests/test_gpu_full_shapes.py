@@ -27,7 +27,7 @@ def _unpack_codes(codes, bits=32):
 
 
 def test_config3_step_is_one_kernel_and_matches_the_oracle(cuda):
-    """BASELINE config 3 at its full shape (batch 8, 32 query / 8 KV heads, 32768 keys, bf16, Sink 128 + Local 512 +
+    """headline configuration 3 at its full shape (batch 8, 32 query / 8 KV heads, 32768 keys, bf16, Sink 128 + Local 512 +
     HashAttention top-2048): the warm decode step is ONE launch of k_hash_decode_attn, every row holds
     128 + 512 + 2048 distinct columns, and for batch rows 0 and 7 the selected sets are bit-identical to the
     oracle's (scoring the kernel's own signatures) and the outputs agree within the bf16 bar."""
