@@ -2,10 +2,13 @@
 //
 // One workgroup of 1024 threads per mask row. A lane owns eight consecutive candidates of a
 // 512-candidate chunk: one 16-byte load brings their keys, one byte of the bitmap row tells
-// which of them are already active. The k-th largest key is found by two 256-bin histogram
-// levels (high byte in wave-private LDS histograms, then the low byte of the keys inside the
-// chosen bin), so the pass count is fixed: level 1, level 2, count, write; rows of up to
-// 131072 candidates stay in registers from the first pass on.
+// which of them are already active. The k-th largest key is found byte by byte. Rows of up to 64
+// keys per thread: the high byte from the row's largest key and packed-compare counts of the few
+// bins below it (float scores: the k-th largest key lies within a bin or two of the largest), the
+// low byte from a small histogram that only the keys of that bin touch. Longer rows, or a threshold
+// further down: two 256-bin histogram levels (high byte with one counter per lane and bin, then the
+// low byte of the keys inside the chosen bin). Either way the pass count is fixed: threshold, count,
+// write; rows of up to 131072 candidates stay in registers from the first pass on.
 // Winners above the threshold are written by every wave independently; only the wave that
 // holds the last accepted tie walks its candidates in column order, which keeps the
 // canonical rule "equal keys: lowest column first" at the cost of one ordered wave.
