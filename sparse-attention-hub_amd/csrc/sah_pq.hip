@@ -212,51 +212,71 @@ __global__ __launch_bounds__(PQB_NT) void k_pq_assign_block(pq_assign_params P) 
   const int b = bh / P.Hkv;
   const int g = bh * P.n_sub + s;
   const int d_sub = P.d_sub, n_cent = P.n_cent;
-  for (int i = tid; i < n_cent * d_sub; i += PQB_NT) s_c[i] = P.centres[(int64_t)g * n_cent * d_sub + i];
-  __syncthreads();
-  for (int n = wave; n < P.n_keys; n += PQB_NT / SAH_WAVE) {
-    const int64_t off = (int64_t)b * P.ks_b + (int64_t)hk * P.ks_h + (int64_t)s * d_sub + (int64_t)(P.key_offset + n) * P.ks_l;
-    float x[PQ_MAX_D];
+  // centres transposed, s_c[d][c]: the lanes of a wave (consecutive centres) read consecutive words
+  for (int i = tid; i < n_cent * d_sub; i += PQB_NT) {
+    const int c = i / d_sub, d = i - c * d_sub;
+    s_c[d * n_cent + c] = P.centres[(int64_t)g * n_cent * d_sub + i];
+  }
+  // this wave's keys (every 16th), up to four of them requested before the first is used
+  constexpr int NW = PQB_NT / SAH_WAVE;
+  constexpr int KB = 4;
+  const int64_t key0 = (int64_t)b * P.ks_b + (int64_t)hk * P.ks_h + (int64_t)s * d_sub;
+  auto load_key = [&](int n, float (&x)[PQ_MAX_D]) {
+    const int64_t off = key0 + (int64_t)(P.key_offset + n) * P.ks_l;
 #pragma unroll
     for (int d = 0; d < PQ_MAX_D; ++d) x[d] = d < d_sub ? sah_load<DT>(P.k, off + d) : 0.f;
-    float dist = INFINITY;
-    int best = 0x7fffffff;
-    for (int c = lane; c < n_cent; c += SAH_WAVE) {
-      const float* cc = s_c + c * d_sub;
-      float dd = 0.f;
-      if (P.round_dist) {
+  };
+  __syncthreads();
+  for (int n0 = wave; n0 < P.n_keys; n0 += KB * NW) {
+    float xs[KB][PQ_MAX_D];
 #pragma unroll
-        for (int d = 0; d < PQ_MAX_D; ++d) {
-          if (d < d_sub) {
-            const float df = sah_round_hw<DT>(x[d] - cc[d]);
-            dd += sah_round_hw<DT>(df * df);
-          }
-        }
-        dd = sah_round_hw<DT>(dd);
-      } else {
-#pragma unroll
-        for (int d = 0; d < PQ_MAX_D; ++d) {
-          if (d < d_sub) {
-            const float df = x[d] - cc[d];
-            dd = fmaf(df, df, dd);
-          }
-        }
-      }
-      if (dd < dist) {  // c ascends: the first minimum is kept
-        dist = dd;
-        best = c;
-      }
+    for (int u = 0; u < KB; ++u) {
+      const int n = n0 + u * NW;
+      load_key(n < P.n_keys ? n : n0, xs[u]);
     }
 #pragma unroll
-    for (int o = 1; o < SAH_WAVE; o <<= 1) {
-      const float od = __shfl_xor(dist, o);
-      const int oi = __shfl_xor(best, o);
-      if (od < dist || (od == dist && oi < best)) {
-        dist = od;
-        best = oi;
+    for (int u = 0; u < KB; ++u) {
+      const int n = n0 + u * NW;
+      if (n >= P.n_keys) break;  // uniform across the wave
+      const float (&x)[PQ_MAX_D] = xs[u];
+      float dist = INFINITY;
+      int best = 0x7fffffff;
+      for (int c = lane; c < n_cent; c += SAH_WAVE) {
+        float dd = 0.f;
+        if (P.round_dist) {
+#pragma unroll
+          for (int d = 0; d < PQ_MAX_D; ++d) {
+            if (d < d_sub) {
+              const float df = sah_round_hw<DT>(x[d] - s_c[d * n_cent + c]);
+              dd += sah_round_hw<DT>(df * df);
+            }
+          }
+          dd = sah_round_hw<DT>(dd);
+        } else {
+#pragma unroll
+          for (int d = 0; d < PQ_MAX_D; ++d) {
+            if (d < d_sub) {
+              const float df = x[d] - s_c[d * n_cent + c];
+              dd = fmaf(df, df, dd);
+            }
+          }
+        }
+        if (dd < dist) {  // c ascends: the first minimum is kept
+          dist = dd;
+          best = c;
+        }
       }
+#pragma unroll
+      for (int o = 1; o < SAH_WAVE; o <<= 1) {
+        const float od = __shfl_xor(dist, o);
+        const int oi = __shfl_xor(best, o);
+        if (od < dist || (od == dist && oi < best)) {
+          dist = od;
+          best = oi;
+        }
+      }
+      if (lane == 0) P.codes[(((int64_t)bh * P.code_pitch) + P.code_offset + n) * P.n_sub + s] = (uint8_t)best;
     }
-    if (lane == 0) P.codes[(((int64_t)bh * P.code_pitch) + P.code_offset + n) * P.n_sub + s] = (uint8_t)best;
   }
 }
 
