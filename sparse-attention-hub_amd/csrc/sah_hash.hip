@@ -129,7 +129,7 @@ __global__ __launch_bounds__(GEMV_NT) void k_hash_sig_gemv(sig_pair PP) {
 #define SGM_PAD 8               // elements of padding per LDS row: 16 B
 
 template <int DT>
-__global__ __launch_bounds__(SGM_NT, 1) void k_hash_sig_mfma(sig_params P, int n_chunks, int tiles_per_wg) {
+__global__ __launch_bounds__(SGM_NT, 4) void k_hash_sig_mfma(sig_params P, int n_chunks, int tiles_per_wg) {
   HIP_DYNAMIC_SHARED(unsigned char, sgm_dyn)
   const int tid = threadIdx.x;
   const int lane = tid & (SAH_WAVE - 1);
@@ -206,49 +206,61 @@ __global__ __launch_bounds__(SGM_NT, 1) void k_hash_sig_mfma(sig_params P, int n
       if (l >= P.n_layers) break;
       const bool last = (l == P.n_layers - 1);
       const int mt = (P.d_out[l] + 31) >> 5;
-      sah_f32x16 acc[SGM_MAXM];
-#pragma unroll
-      for (int q = 0; q < SGM_MAXM; ++q) {
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc[q][v] = 0.f;
-      }
       const uint16_t* wl = s_w[l] + i32 * pitch[l] + 8 * g;
+      const float* bl = s_bias + l * SGM_MAXW + 4 * g;
+      // one 32-row tile of the layer's output: 32x32x16 steps over the input, accumulator from zero
+      auto tile = [&](int q) {
+        sah_f32x16 acc;
 #pragma unroll
-      for (int q = 0; q < SGM_MAXM; ++q) {
-        if (q < mt) {
+        for (int v = 0; v < 16; ++v) acc[v] = 0.f;
 #pragma unroll
-          for (int s = 0; s < SGM_MAXK; ++s) {
-            if (s < ksteps) {
-              const uint4 a = *(const uint4*)(wl + q * 32 * pitch[l] + s * 16);
-              acc[q] = sah_mfma_32x32x16<DT>(a, bop[s], acc[q]);
-            }
+        for (int s = 0; s < SGM_MAXK; ++s) {
+          if (s < ksteps) {
+            const uint4 a = *(const uint4*)(wl + q * 32 * pitch[l] + s * 16);
+            acc = sah_mfma_32x32x16<DT>(a, bop[s], acc);
           }
         }
-      }
-      const float* bl = s_bias + l * SGM_MAXW + 4 * g;
+        return acc;
+      };
       if (!last) {
-        // bias, activation, rounding as torch rounds them; the result is the next layer's B operand
+        // bias, activation, rounding as torch rounds them; the result is the next layer's B operand. Two tiles at a
+        // time: their accumulators, this layer's operand and the next one's are all that is live (four waves per SIMD)
+        uint4 nxt[SGM_MAXK];
 #pragma unroll
         for (int q = 0; q < SGM_MAXM; ++q) {
           float y[16];
+          if (q < mt) {
+            const sah_f32x16 acc = tile(q);
 #pragma unroll
-          for (int v = 0; v < 16; ++v) {
-            float z = sah_round_hw<DT>(acc[q][v]);
-            z = sah_round_hw<DT>(z + bl[q * 32 + 8 * (v >> 2) + (v & 3)]);
-            y[v] = q < mt ? sig_act_fast(P.act, z) : 0.f;  // rounded by the packing below
+            for (int v4 = 0; v4 < 4; ++v4) {
+              const float4 b4 = *(const float4*)(bl + q * 32 + 8 * v4);  // four biases in one read
+              const float bb[4] = {b4.x, b4.y, b4.z, b4.w};
+#pragma unroll
+              for (int t = 0; t < 4; ++t) {
+                float z = sah_round_hw<DT>(acc[4 * v4 + t]);
+                z = sah_round_hw<DT>(z + bb[t]);
+                y[4 * v4 + t] = sig_act_fast(P.act, z);  // rounded by the packing below
+              }
+            }
+          } else {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) y[v] = 0.f;
           }
-          bop[2 * q] = make_uint4(sah_pack2_hw<DT>(y[0], y[1]), sah_pack2_hw<DT>(y[2], y[3]), sah_pack2_hw<DT>(y[4], y[5]),
+          nxt[2 * q] = make_uint4(sah_pack2_hw<DT>(y[0], y[1]), sah_pack2_hw<DT>(y[2], y[3]), sah_pack2_hw<DT>(y[4], y[5]),
                                   sah_pack2_hw<DT>(y[6], y[7]));
-          bop[2 * q + 1] = make_uint4(sah_pack2_hw<DT>(y[8], y[9]), sah_pack2_hw<DT>(y[10], y[11]), sah_pack2_hw<DT>(y[12], y[13]),
+          nxt[2 * q + 1] = make_uint4(sah_pack2_hw<DT>(y[8], y[9]), sah_pack2_hw<DT>(y[10], y[11]), sah_pack2_hw<DT>(y[12], y[13]),
                                       sah_pack2_hw<DT>(y[14], y[15]));
         }
+#pragma unroll
+        for (int s = 0; s < SGM_MAXK; ++s) bop[s] = nxt[s];
         ksteps = 2 * mt;
       } else {
         // sign planes: this lane holds 16 of the vector's bits, lane ^ 32 the other 16
+        const sah_f32x16 acc0 = tile(0);
         uint32_t pos = 0u, nz = 0u;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          float z = sah_round_hw<DT>(acc[0][v]);
+          float z = sah_round_hw<DT>(acc0[v]);
           z = sah_round_hw<DT>(z + bl[8 * (v >> 2) + (v & 3)]);
           const int bit = 8 * (v >> 2) + 4 * g + (v & 3);
           pos |= (z > 0.f ? 1u : 0u) << bit;
