@@ -190,7 +190,7 @@ struct att_lane {
     }
   }
   // the batch's logits (scaled, plus the additive mask; -inf for a lane without a key), and their maximum over the wave
-  template <int UB>
+  template <int UB, bool PLAIN = false>
   __device__ __forceinline__ float logits(const att_params& P, int64_t moff, const float (&qv)[8], const att_batch<DT, UB>& B,
                                           float (&z)[UB]) const {
     float mb = -INFINITY;
@@ -203,7 +203,7 @@ struct att_lane {
       for (int e = 0; e < 8; ++e) d = fmaf(qv[e], kf[e], d);
       d = att_group_sum<LPK>(d) * P.scaling;
       if (B.id[u] >= 0) {
-        if (P.amask) d += sah_load<DT>(P.amask, moff + B.id[u]);
+        if (!PLAIN && P.amask) d += sah_load<DT>(P.amask, moff + B.id[u]);
       } else {
         d = -INFINITY;
       }
@@ -244,8 +244,11 @@ struct att_lane {
 // entry i is column col_of(i) (anything outside [0, Lk) is skipped) with inverse weight inv_w_of(i). Batches of UB
 // iterations: the K and V rows of a batch are requested together, so 2 * UB row loads are in flight per lane.
 // DROP: training-mode dropout of the exp weights (P.drop) is applied; a variant of its own, so that the decode path
-// carries no trace of it.
-template <int DT, int D, bool DROP = false, typename ColOf, typename InvWOf>
+// carries no trace of it. PLAIN: the caller knows that there is no additive mask and no logits output (the one-kernel
+// decode step): their tests and code stay out. A caller whose column list lives in LDS hands col_of a pointer the
+// compiler can see to be LDS: through a generic pointer every read of the list would be a flat load, which waits for
+// all of the wave's outstanding row loads as well.
+template <int DT, int D, bool DROP = false, bool PLAIN = false, typename ColOf, typename InvWOf>
 __device__ __forceinline__ void att_walk(const att_params& P, int r, int b, int h, int hk, int qi, int first, int bound,
                                          int stride, ColOf col_of, InvWOf inv_w_of, att_wave_state& st) {
   typedef att_lane<DT, D> lane_t;
@@ -254,7 +257,7 @@ __device__ __forceinline__ void att_walk(const att_params& P, int r, int b, int 
   constexpr int UB = IT < 4 ? IT : 4;   // iterations per batch
   const int lane = threadIdx.x & (SAH_WAVE - 1);
   const lane_t L(P, b, hk);
-  const int64_t moff = P.amask ? ((int64_t)b * P.ms_b + (int64_t)h * P.ms_h + (int64_t)qi * P.ms_l) : 0;
+  const int64_t moff = (!PLAIN && P.amask) ? ((int64_t)b * P.ms_b + (int64_t)h * P.ms_h + (int64_t)qi * P.ms_l) : 0;
   float qv[8];
   L.load_q(P, b, h, qi, qv);
 
@@ -277,8 +280,8 @@ __device__ __forceinline__ void att_walk(const att_params& P, int r, int b, int 
       for (int u = 0; u < UB; ++u) B.id[u] = __shfl(idx_l, (ib + u) * KPI + L.grp);
       L.request(B);
       float z[UB];
-      const float mb = L.logits(P, moff, qv, B, z);
-      if (P.logits_out && L.sub == 0) {
+      const float mb = L.template logits<UB, PLAIN>(P, moff, qv, B, z);
+      if (!PLAIN && P.logits_out && L.sub == 0) {
 #pragma unroll
         for (int u = 0; u < UB; ++u) {
           const int pos = cbase + (ib + u) * KPI + L.grp;

@@ -53,7 +53,8 @@ struct hdec_params {
 // The mask row r of one decode step; returns its entry count. s_cols (optional, LDS, R.cap ints): copy of the
 // row's column list for a caller that continues with it in the same kernel (complete after its next barrier).
 // CP: the codes are read in their compact form (one sign plane per column + exception list).
-template <int DT, bool MF, bool CP>
+// SILU: both MLPs use SiLU (checked by the host): the matrix-core form then carries no other activation's code
+template <int DT, bool MF, bool CP, bool SILU = false>
 __device__ __forceinline__ int hdec_row(const hdec_params& P, int r, hsw_lds& S, unsigned char* hdec_dyn, int* s_cols) {
   typedef typename hdec_sig<MF>::lds hdec_sig_lds;
   const sah_rows& R = P.R;
@@ -121,7 +122,8 @@ __device__ __forceinline__ int hdec_row(const hdec_params& P, int r, hsw_lds& S,
     fixed_part();
   };
   if constexpr (MF) {
-    sig_mfma_block<DT>(P.job[job], active, tid % HDEC_GROUP, r / Hq, r % Hq, 0, 1, P.job[0].n_layers, s_sig[job], prefetch);
+    sig_mfma_block<DT, decltype(prefetch), SILU ? SAH_ACT_SILU : -1>(P.job[job], active, tid % HDEC_GROUP, r / Hq, r % Hq, 0, 1,
+                                                                      P.job[0].n_layers, s_sig[job], prefetch);
   } else {
     sig_gemv_block<DT, 1, HDEC_GROUP, HDEC_ROWS, PF>(P.job[job], active, tid % HDEC_GROUP, r / Hq, r % Hq, 0, 1,
                                                       P.job[0].n_layers, s_sig[job], prefetch);
@@ -136,12 +138,12 @@ __device__ __forceinline__ int hdec_row(const hdec_params& P, int r, hsw_lds& S,
                             s_cols, CP ? &cs : nullptr, s_hi, n_local > 0 ? lo2 : n);
 }
 
-template <int DT, bool MF, bool CP>
+template <int DT, bool MF, bool CP, bool SILU>
 __global__ __launch_bounds__(HSW_NT) void k_hash_decode(hdec_params P) {
   sah_touch_kernargs<sizeof(hdec_params)>();
   __shared__ hsw_lds S;
   HIP_DYNAMIC_SHARED(unsigned char, hdec_dyn)
-  hdec_row<DT, MF, CP>(P, blockIdx.x, S, hdec_dyn, nullptr);
+  hdec_row<DT, MF, CP, SILU>(P, blockIdx.x, S, hdec_dyn, nullptr);
 }
 
 // Selection and attention of a row in one workgroup: as soon as a row's columns are chosen its K / V rows are
@@ -149,7 +151,7 @@ __global__ __launch_bounds__(HSW_NT) void k_hash_decode(hdec_params P) {
 // was selected early starts streaming while others still select, and the attention's start-up latency is paid
 // while the memory system would otherwise idle. Workgroup -> row mapping as in k_sparse_attn (the query heads
 // of a GQA group on one XCD).
-template <int DT, bool MF, bool CP, int D>
+template <int DT, bool MF, bool CP, int D, bool SILU>
 __global__ __launch_bounds__(HSW_NT) void k_hash_decode_attn(hdec_params P, att_params A, int cols_offset) {
   __shared__ hsw_lds S;
   __shared__ float s_m[HSW_NW];
@@ -166,9 +168,26 @@ __global__ __launch_bounds__(HSW_NT) void k_hash_decode_attn(hdec_params P, att_
   const int h = hk * G + slot % G;
   const int r = b * A.Hq + h;
   int* s_cols = (int*)(hdec_dyn + cols_offset);
-  const int cnt = hdec_row<DT, MF, CP>(P, r, S, hdec_dyn, s_cols);
+  const int cnt = hdec_row<DT, MF, CP, SILU>(P, r, S, hdec_dyn, s_cols);
   __syncthreads();  // the column list in LDS is complete
-  att_tile<DT, D, true>(A, r, b, h, hk, 0, 0, 1, s_cols, cnt, s_m, s_l, s_acc);
+  // the whole-row attention over the list in LDS: no additive mask, no weights, no logits output on this path
+  {
+    constexpr int KPI = SAH_WAVE / (D / 8);
+    const int wave = sah_wave_id();
+    const int per = (((cnt + HSW_NW - 1) / HSW_NW) + KPI - 1) / KPI * KPI;  // entries per wave
+    const int first = wave * per;
+    const int bound = first + per < cnt ? first + per : cnt;
+    att_wave_state st;
+    st.clear();
+    const float unit = A.unit_inv_w;
+    att_walk<DT, D, false, true>(
+        A, r, b, h, hk, 0, first, bound, SAH_WAVE, [&](int i) { return s_cols[i]; }, [&](int) { return unit; }, st);
+    att_park<D, HSW_NW>(st, wave, s_m, s_l, s_acc);
+    __syncthreads();
+    float a, M, l;
+    att_gather<DT, D, HSW_NW>(s_m, s_l, s_acc, a, M, l);
+    att_store_row<DT, D>(A, r, b, h, 0, a, M, l);
+  }
 }
 
 static size_t hdec_lds_bytes(int n_keys) {
@@ -178,12 +197,25 @@ static size_t hdec_lds_bytes(int n_keys) {
   return bm + (key > sig ? key : sig);
 }
 
+// both MLPs of the step with SiLU, in the matrix-core form: the kernel variant without the other activations
+static bool hdec_silu(const hdec_params& P) {
+  return P.job[0].act == SAH_ACT_SILU && (!P.has_key || P.job[1].act == SAH_ACT_SILU);
+}
+
+template <int DT, bool MF, bool CP, bool SILU>
+static int hdec_launch_s(const sah_hash_decode_args* a, const hdec_params& P, size_t lds) {
+  if (int rc = sah_allow_lds((const void*)k_hash_decode<DT, MF, CP, SILU>, 150 * 1024, "sah_hash_decode_topk")) return rc;
+  sah_timed timed("k_hash_decode", a->stream);
+  hipLaunchKernelGGL((k_hash_decode<DT, MF, CP, SILU>), dim3(a->rows.n_rows), dim3(HSW_NT), lds, (hipStream_t)a->stream, P);
+  return sah_launch_status("sah_hash_decode_topk");
+}
+
 template <int DT, bool MF, bool CP>
 static int hdec_launch_t(const sah_hash_decode_args* a, const hdec_params& P, size_t lds) {
-  if (int rc = sah_allow_lds((const void*)k_hash_decode<DT, MF, CP>, 150 * 1024, "sah_hash_decode_topk")) return rc;
-  sah_timed timed("k_hash_decode", a->stream);
-  hipLaunchKernelGGL((k_hash_decode<DT, MF, CP>), dim3(a->rows.n_rows), dim3(HSW_NT), lds, (hipStream_t)a->stream, P);
-  return sah_launch_status("sah_hash_decode_topk");
+  if constexpr (MF) {
+    if (hdec_silu(P)) return hdec_launch_s<DT, MF, CP, true>(a, P, lds);
+  }
+  return hdec_launch_s<DT, MF, CP, false>(a, P, lds);
 }
 
 template <int DT, bool MF>
@@ -312,15 +344,23 @@ extern "C" int sah_hash_decode_topk(const sah_hash_decode_args* a) {
   }
 }
 
-template <int DT, bool MF, bool CP, int D>
-static int hdec_attn_launch_t(const sah_hash_decode_args* a, const hdec_params& P, const att_params& A, size_t lds, int cols_offset) {
-  if (int rc = sah_allow_lds((const void*)k_hash_decode_attn<DT, MF, CP, D>, 150 * 1024, "sah_hash_decode_attention")) return rc;
+template <int DT, bool MF, bool CP, int D, bool SILU>
+static int hdec_attn_launch_s(const sah_hash_decode_args* a, const hdec_params& P, const att_params& A, size_t lds, int cols_offset) {
+  if (int rc = sah_allow_lds((const void*)k_hash_decode_attn<DT, MF, CP, D, SILU>, 150 * 1024, "sah_hash_decode_attention")) return rc;
   const int G = A.Hq / A.Hkv;
   const int n_tiles = P.R.n_rows / G;
   const int n_wg = (n_tiles + ATT_XCDS - 1) / ATT_XCDS * ATT_XCDS * G;
   sah_timed timed("k_hash_decode_attn", a->stream);
-  hipLaunchKernelGGL((k_hash_decode_attn<DT, MF, CP, D>), dim3(n_wg), dim3(HSW_NT), lds, (hipStream_t)a->stream, P, A, cols_offset);
+  hipLaunchKernelGGL((k_hash_decode_attn<DT, MF, CP, D, SILU>), dim3(n_wg), dim3(HSW_NT), lds, (hipStream_t)a->stream, P, A, cols_offset);
   return sah_launch_status("sah_hash_decode_attention");
+}
+
+template <int DT, bool MF, bool CP, int D>
+static int hdec_attn_launch_t(const sah_hash_decode_args* a, const hdec_params& P, const att_params& A, size_t lds, int cols_offset) {
+  if constexpr (MF) {
+    if (hdec_silu(P)) return hdec_attn_launch_s<DT, MF, CP, D, true>(a, P, A, lds, cols_offset);
+  }
+  return hdec_attn_launch_s<DT, MF, CP, D, false>(a, P, A, lds, cols_offset);
 }
 
 template <int DT, bool MF, int D>

@@ -128,7 +128,9 @@ __global__ __launch_bounds__(GEMV_NT) void k_hash_sig_gemv(sig_pair PP) {
 #define SGM_MAXM (SGM_MAXW / 32)
 #define SGM_PAD 8               // elements of padding per LDS row: 16 B
 
-template <int DT>
+// ACT: the activation, fixed at compile time (one kernel each: with the choice left to run time the four epilogues,
+// GELU's error function included, end up inside the hot loop and the code outgrows the instruction cache)
+template <int DT, int ACT>
 __global__ __launch_bounds__(SGM_NT, 4) void k_hash_sig_mfma(sig_params P, int n_chunks, int tiles_per_wg) {
   HIP_DYNAMIC_SHARED(unsigned char, sgm_dyn)
   const int tid = threadIdx.x;
@@ -148,13 +150,16 @@ __global__ __launch_bounds__(SGM_NT, 4) void k_hash_sig_mfma(sig_params P, int n
   const int h = hx * P.group + hq;
 
   // ---- stage W^T (and the biases as fp32) in LDS
-  uint16_t* s_w[SAH_MAX_MLP_LAYERS];
+  // (offsets, not pointers: a pointer that has been through an array is a generic one to the compiler, and every read
+  // through it a flat load, which also waits for the wave's outstanding global loads)
+  int w_off[SAH_MAX_MLP_LAYERS];
   int pitch[SAH_MAX_MLP_LAYERS];
   int w_elems = 0;
+  uint16_t* const s_w0 = (uint16_t*)sgm_dyn;
   {
     int din = P.D;
     for (int l = 0; l < P.n_layers; ++l) {
-      s_w[l] = (uint16_t*)sgm_dyn + w_elems;
+      w_off[l] = w_elems;
       pitch[l] = din + SGM_PAD;
       w_elems += ((P.d_out[l] + 31) & ~31) * pitch[l];
       din = P.d_out[l];
@@ -175,7 +180,7 @@ __global__ __launch_bounds__(SGM_NT, 4) void k_hash_sig_mfma(sig_params P, int n
         const int dsub = (l > 0 && (sub == 1 || sub == 2)) ? (sub ^ 3) : sub;
         uint2 val = make_uint2(0u, 0u);
         if (row < dout) val = *(const uint2*)(wt + (int64_t)row * din + c4 * 4);
-        *(uint2*)(s_w[l] + row * pitch[l] + blk * 16 + dsub * 4) = val;
+        *(uint2*)(s_w0 + w_off[l] + row * pitch[l] + blk * 16 + dsub * 4) = val;
       }
       for (int e = tid; e < SGM_MAXW; e += SGM_NT)
         s_bias[l * SGM_MAXW + e] = e < dout ? sah_load<DT>(P.bias[l], (int64_t)h * dout + e) : 0.f;
@@ -206,7 +211,7 @@ __global__ __launch_bounds__(SGM_NT, 4) void k_hash_sig_mfma(sig_params P, int n
       if (l >= P.n_layers) break;
       const bool last = (l == P.n_layers - 1);
       const int mt = (P.d_out[l] + 31) >> 5;
-      const uint16_t* wl = s_w[l] + i32 * pitch[l] + 8 * g;
+      const uint16_t* wl = s_w0 + w_off[l] + i32 * pitch[l] + 8 * g;
       const float* bl = s_bias + l * SGM_MAXW + 4 * g;
       // one 32-row tile of the layer's output: 32x32x16 steps over the input, accumulator from zero
       auto tile = [&](int q) {
@@ -239,7 +244,7 @@ __global__ __launch_bounds__(SGM_NT, 4) void k_hash_sig_mfma(sig_params P, int n
               for (int t = 0; t < 4; ++t) {
                 float z = sah_round_hw<DT>(acc[4 * v4 + t]);
                 z = sah_round_hw<DT>(z + bb[t]);
-                y[4 * v4 + t] = sig_act_fast(P.act, z);  // rounded by the packing below
+                y[4 * v4 + t] = sig_act_fast(ACT, z);  // rounded by the packing below
               }
             }
           } else {
@@ -299,18 +304,28 @@ static bool sig_mfma_ok(const sah_hash_sig_args* a) {
   return sgm_lds_bytes(a) <= 150 * 1024;
 }
 
-template <int DT>
-static int sig_launch_mfma_t(const sah_hash_sig_args* a, const sig_params& P) {
-  if (int rc = sah_allow_lds((const void*)k_hash_sig_mfma<DT>, 150 * 1024, "sah_hash_signatures")) return rc;
+template <int DT, int ACT>
+static int sig_launch_mfma_a(const sah_hash_sig_args* a, const sig_params& P) {
+  if (int rc = sah_allow_lds((const void*)k_hash_sig_mfma<DT, ACT>, 150 * 1024, "sah_hash_signatures")) return rc;
   const int n_tiles = (a->L + SGM_TILE - 1) / SGM_TILE;
   const int tiles_per_wg = n_tiles < 8 ? n_tiles : 8;   // the staged weights serve up to 8 tiles
   const int n_chunks = (n_tiles + tiles_per_wg - 1) / tiles_per_wg;
   const int64_t n_wg = (int64_t)a->B * a->Hq * n_chunks;
   if (n_wg > 0x7fffffff) return sah_fail(SAH_ESHAPE, "sah_hash_signatures: too many workgroups");
   sah_timed timed("k_hash_sig_mfma", a->stream);
-  hipLaunchKernelGGL(k_hash_sig_mfma<DT>, dim3((unsigned)n_wg), dim3(SGM_NT), sgm_lds_bytes(a), (hipStream_t)a->stream, P,
+  hipLaunchKernelGGL((k_hash_sig_mfma<DT, ACT>), dim3((unsigned)n_wg), dim3(SGM_NT), sgm_lds_bytes(a), (hipStream_t)a->stream, P,
                      n_chunks, tiles_per_wg);
   return sah_launch_status("sah_hash_signatures");
+}
+
+template <int DT>
+static int sig_launch_mfma_t(const sah_hash_sig_args* a, const sig_params& P) {
+  switch (a->act) {
+    case SAH_ACT_RELU: return sig_launch_mfma_a<DT, SAH_ACT_RELU>(a, P);
+    case SAH_ACT_SILU: return sig_launch_mfma_a<DT, SAH_ACT_SILU>(a, P);
+    case SAH_ACT_GELU: return sig_launch_mfma_a<DT, SAH_ACT_GELU>(a, P);
+    default: return sig_launch_mfma_a<DT, SAH_ACT_TANH>(a, P);
+  }
 }
 
 // decode-size jobs on the matrix cores: up to 16 vectors of one head per workgroup

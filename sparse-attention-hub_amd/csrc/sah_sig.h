@@ -296,7 +296,9 @@ struct sig_mfma_lds {
 
 // `after_requests` runs once every load of the MLP has been requested: the place for a caller to put loads of
 // its own on their way without delaying the MLP's.
-template <int DT, typename Hook = sig_no_hook>
+// ACT >= 0: the activation is that one, whatever P.act says (the caller has checked): the other three, GELU's error
+// function among them, then stay out of the kernel's code; ACT < 0: P.act decides at run time. Same arithmetic either way.
+template <int DT, typename Hook = sig_no_hook, int ACT = -1>
 __device__ __forceinline__ void sig_mfma_block(const sig_params& P, bool active, int tid, int b, int h, int l0, int nl,
                                                int n_layers, sig_mfma_lds& S, Hook after_requests = Hook()) {
   const int lane = tid & (SAH_WAVE - 1);
@@ -305,7 +307,7 @@ __device__ __forceinline__ void sig_mfma_block(const sig_params& P, bool active,
   const int g = lane >> 4;    // k-group of the operands, row group of C
   const int hx = active ? h / P.group : 0;
   const int D = active ? P.D : 32;
-  const int act = active ? P.act : 0;
+  const int act = ACT >= 0 ? ACT : (active ? P.act : 0);
   const int f0 = 16 * wave + 4 * g;  // this lane's 4 output features of every layer: f0 .. f0 + 3
 
   // ---- first requests, only what the first layer needs, so that it can start as early as possible: the
