@@ -53,7 +53,8 @@ struct hdec_params {
 // The mask row r of one decode step; returns its entry count. s_cols (optional, LDS, R.cap ints): copy of the
 // row's column list for a caller that continues with it in the same kernel (complete after its next barrier).
 // CP: the codes are read in their compact form (one sign plane per column + exception list).
-// SILU: both MLPs use SiLU (checked by the host): the matrix-core form then carries no other activation's code
+// SILU: both MLPs use SiLU and have the usual shape, 128 -> 128 -> 128 -> 32 (checked by the host): the matrix-core form
+// then carries no other activation's code and knows every width at compile time
 template <int DT, bool MF, bool CP, bool SILU = false>
 __device__ __forceinline__ int hdec_row(const hdec_params& P, int r, hsw_lds& S, unsigned char* hdec_dyn, int* s_cols) {
   typedef typename hdec_sig<MF>::lds hdec_sig_lds;
@@ -122,7 +123,7 @@ __device__ __forceinline__ int hdec_row(const hdec_params& P, int r, hsw_lds& S,
     fixed_part();
   };
   if constexpr (MF) {
-    sig_mfma_block<DT, decltype(prefetch), SILU ? SAH_ACT_SILU : -1>(P.job[job], active, tid % HDEC_GROUP, r / Hq, r % Hq, 0, 1,
+    sig_mfma_block<DT, decltype(prefetch), SILU ? SAH_ACT_SILU : -1, SILU>(P.job[job], active, tid % HDEC_GROUP, r / Hq, r % Hq, 0, 1,
                                                                       P.job[0].n_layers, s_sig[job], prefetch);
   } else {
     sig_gemv_block<DT, 1, HDEC_GROUP, HDEC_ROWS, PF>(P.job[job], active, tid % HDEC_GROUP, r / Hq, r % Hq, 0, 1,
@@ -197,9 +198,14 @@ static size_t hdec_lds_bytes(int n_keys) {
   return bm + (key > sig ? key : sig);
 }
 
-// both MLPs of the step with SiLU, in the matrix-core form: the kernel variant without the other activations
+// both MLPs of the step with SiLU and the usual widths, in the matrix-core form: the kernel variant that knows it
 static bool hdec_silu(const hdec_params& P) {
-  return P.job[0].act == SAH_ACT_SILU && (!P.has_key || P.job[1].act == SAH_ACT_SILU);
+  for (int j = 0; j < (P.has_key ? 2 : 1); ++j) {
+    const sig_params& J = P.job[j];
+    if (J.act != SAH_ACT_SILU || J.D != 128 || J.n_layers != 3 || J.d_out[0] != 128 || J.d_out[1] != 128 || J.d_out[2] != 32)
+      return false;
+  }
+  return true;
 }
 
 template <int DT, bool MF, bool CP, bool SILU>

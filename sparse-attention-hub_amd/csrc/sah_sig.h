@@ -297,8 +297,11 @@ struct sig_mfma_lds {
 // `after_requests` runs once every load of the MLP has been requested: the place for a caller to put loads of
 // its own on their way without delaying the MLP's.
 // ACT >= 0: the activation is that one, whatever P.act says (the caller has checked): the other three, GELU's error
-// function among them, then stay out of the kernel's code; ACT < 0: P.act decides at run time. Same arithmetic either way.
-template <int DT, typename Hook = sig_no_hook, int ACT = -1>
+// function among them, then stay out of the kernel's code; ACT < 0: P.act decides at run time. STD: the job has the usual
+// HashAttention shape (inputs of 128, layers of 128, 128 and 32 outputs; the caller has checked): every width is then a
+// compile-time constant, no load hides behind a branch, and the waits before a layer's matrix instructions count exactly
+// the loads that layer needs instead of "everything outstanding". Same arithmetic either way.
+template <int DT, typename Hook = sig_no_hook, int ACT = -1, bool STD = false>
 __device__ __forceinline__ void sig_mfma_block(const sig_params& P, bool active, int tid, int b, int h, int l0, int nl,
                                                int n_layers, sig_mfma_lds& S, Hook after_requests = Hook()) {
   const int lane = tid & (SAH_WAVE - 1);
@@ -306,7 +309,9 @@ __device__ __forceinline__ void sig_mfma_block(const sig_params& P, bool active,
   const int i16 = lane & 15;  // row of A, column (vector) of B and C
   const int g = lane >> 4;    // k-group of the operands, row group of C
   const int hx = active ? h / P.group : 0;
-  const int D = active ? P.D : 32;
+  const int D = STD ? 128 : (active ? P.D : 32);
+  const int NL = STD ? 3 : n_layers;
+  auto dw = [&](int l) -> int { return STD ? (l < 2 ? 128 : 32) : P.d_out[l]; };  // width of layer l
   const int act = ACT >= 0 ? ACT : (active ? P.act : 0);
   const int f0 = 16 * wave + 4 * g;  // this lane's 4 output features of every layer: f0 .. f0 + 3
 
@@ -317,9 +322,9 @@ __device__ __forceinline__ void sig_mfma_block(const sig_params& P, bool active,
   uint2 bias_raw[SAH_MAX_MLP_LAYERS];
   uint4 wr[SAH_MAX_MLP_LAYERS][SMB_MAXK];
   auto request_weights = [&](int l) {
-    if (l < n_layers && 16 * wave < P.d_out[l]) {  // a wave skips the layers it has no rows of
-      const int dout = P.d_out[l];
-      const int din = l == 0 ? D : P.d_out[l - 1];
+    if (l < NL && 16 * wave < dw(l)) {  // a wave skips the layers it has no rows of
+      const int dout = dw(l);
+      const int din = l == 0 ? D : dw(l - 1);
       int row = 16 * wave + i16;
       if (row > dout - 1) row = dout - 1;  // rows beyond the width repeat the last one; their results are dropped
       const uint16_t* wrow = (const uint16_t*)P.Wt[l] + ((int64_t)h * dout + row) * din + 8 * g;
@@ -336,8 +341,8 @@ __device__ __forceinline__ void sig_mfma_block(const sig_params& P, bool active,
       if (32 * s < D) bop0[s] = *(const uint4*)(xrow + 32 * s);
 #pragma unroll
     for (int l = 0; l < SAH_MAX_MLP_LAYERS; ++l) {
-      const int ll = l < n_layers ? l : 0;
-      const int dout = P.d_out[ll];
+      const int ll = l < NL ? l : 0;
+      const int dout = dw(ll);
       bias_raw[l] = *(const uint2*)((const uint16_t*)P.bias[ll] + (int64_t)h * dout + (f0 + 4 <= dout ? f0 : 0));
     }
     request_weights(0);
@@ -346,9 +351,9 @@ __device__ __forceinline__ void sig_mfma_block(const sig_params& P, bool active,
   int din = D;
 #pragma unroll
   for (int l = 0; l < SAH_MAX_MLP_LAYERS; ++l) {
-    if (l >= n_layers) break;
-    const int dout = active ? P.d_out[l] : 16;
-    const bool last = (l == n_layers - 1);
+    if (l >= NL) break;
+    const int dout = STD ? dw(l) : (active ? P.d_out[l] : 16);
+    const bool last = (l == NL - 1);
     sah_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
     const bool mine = active && 16 * wave < dout;
     if (mine) {
