@@ -140,13 +140,9 @@ __device__ __forceinline__ uint32_t sah_float_to_bits(float f) { return __builti
 
 __device__ __forceinline__ float sah_bf16_to_float(uint16_t h) { return sah_bits_to_float(((uint32_t)h) << 16); }
 
-// round-to-nearest-even fp32 -> bf16 (what torch's .to(bfloat16) does)
-__device__ __forceinline__ uint16_t sah_float_to_bf16(float f) {
-  uint32_t u = sah_float_to_bits(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);  // NaN stays NaN
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
-}
+// round-to-nearest-even fp32 -> bf16 (what torch's .to(bfloat16) does): the hardware converter, one instruction
+// and no branch (a NaN stays a NaN)
+__device__ __forceinline__ uint16_t sah_float_to_bf16(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
 
 __device__ __forceinline__ float sah_f16_to_float(uint16_t h) {
   return (float)__builtin_bit_cast(_Float16, h);
@@ -158,19 +154,11 @@ __device__ __forceinline__ uint16_t sah_float_to_f16(float f) {
 // value of `f` after a round trip through storage type DT
 template <int DT>
 __device__ __forceinline__ float sah_round(float f) {
-  if (DT == SAH_BF16) return sah_bf16_to_float(sah_float_to_bf16(f));
-  if (DT == SAH_F16) return sah_f16_to_float(sah_float_to_f16(f));
-  return f;
-}
-
-// The same roundings through the hardware converters (round to nearest even): for code that rounds per element
-// in an inner loop.
-template <int DT>
-__device__ __forceinline__ float sah_round_hw(float f) {
   if (DT == SAH_BF16) return (float)(__bf16)f;
   if (DT == SAH_F16) return (float)(_Float16)f;
   return f;
 }
+
 // two values rounded to the 16-bit storage type DT and packed, lo in the low half
 template <int DT>
 __device__ __forceinline__ uint32_t sah_pack2_hw(float lo, float hi) {

@@ -242,8 +242,8 @@ __global__ __launch_bounds__(SGM_NT, 4) void k_hash_sig_mfma(sig_params P, int n
               const float bb[4] = {b4.x, b4.y, b4.z, b4.w};
 #pragma unroll
               for (int t = 0; t < 4; ++t) {
-                float z = sah_round_hw<DT>(acc[4 * v4 + t]);
-                z = sah_round_hw<DT>(z + bb[t]);
+                float z = sah_round<DT>(acc[4 * v4 + t]);
+                z = sah_round<DT>(z + bb[t]);
                 y[4 * v4 + t] = sig_act_fast(ACT, z);  // rounded by the packing below
               }
             }
@@ -265,8 +265,8 @@ __global__ __launch_bounds__(SGM_NT, 4) void k_hash_sig_mfma(sig_params P, int n
         uint32_t pos = 0u, nz = 0u;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          float z = sah_round_hw<DT>(acc0[v]);
-          z = sah_round_hw<DT>(z + bl[8 * (v >> 2) + (v & 3)]);
+          float z = sah_round<DT>(acc0[v]);
+          z = sah_round<DT>(z + bl[8 * (v >> 2) + (v & 3)]);
           const int bit = 8 * (v >> 2) + 4 * g + (v & 3);
           pos |= (z > 0.f ? 1u : 0u) << bit;
           nz |= (z != 0.f ? 1u : 0u) << bit;

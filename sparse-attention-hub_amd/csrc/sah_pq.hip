@@ -247,11 +247,11 @@ __global__ __launch_bounds__(PQB_NT) void k_pq_assign_block(pq_assign_params P) 
 #pragma unroll
           for (int d = 0; d < PQ_MAX_D; ++d) {
             if (d < d_sub) {
-              const float df = sah_round_hw<DT>(x[d] - s_c[d * n_cent + c]);
-              dd += sah_round_hw<DT>(df * df);
+              const float df = sah_round<DT>(x[d] - s_c[d * n_cent + c]);
+              dd += sah_round<DT>(df * df);
             }
           }
-          dd = sah_round_hw<DT>(dd);
+          dd = sah_round<DT>(dd);
         } else {
 #pragma unroll
           for (int d = 0; d < PQ_MAX_D; ++d) {

@@ -120,7 +120,8 @@ __device__ __forceinline__ float sc_reduce4(float d0, float d1, float d2, float 
   return z;
 }
 
-template <int DT, int D>
+// AM: an additive attention mask is given (P.amask); without one the scoring loop holds no load but the rows'
+template <int DT, int D, bool AM>
 __global__ __launch_bounds__(SC_NT) void k_qk_scores(qk_params P) {
   sah_touch_kernargs<sizeof(qk_params)>();
   constexpr int LPK = D / 8;
@@ -158,13 +159,22 @@ __global__ __launch_bounds__(SC_NT) void k_qk_scores(qk_params P) {
     sc_load<DT>((const char*)P.q + ((int64_t)b * P.qs_b + (int64_t)h * P.qs_h + (int64_t)qi * P.qs_l + sub * 8) * ES, qv[i]);
     if (live) {
       row[i] = (b * P.Hq + h) * P.Lq + qi;
-      if (P.amask) moff[i] = (int64_t)b * P.ms_b + (int64_t)h * P.ms_h + (int64_t)qi * P.ms_l;
+      if (AM) moff[i] = (int64_t)b * P.ms_b + (int64_t)h * P.ms_h + (int64_t)qi * P.ms_l;
     }
   }
   const char* kbase = (const char*)P.k + ((int64_t)b * P.ks_b + (int64_t)hk * P.ks_h + sub * 8) * ES;
   const int64_t krow = P.ks_l * ES;
   // which of the four totals this lane ends up with after sc_reduce4
   const int mine = FAST4 ? (2 * (sub & 1) + ((sub >> 1) & 1)) : 0;
+  int row_mine = row[0];
+  int64_t moff_mine = moff[0];
+#pragma unroll
+  for (int i = 1; i < SC_NQ; ++i) {
+    if (mine == i) {
+      row_mine = row[i];
+      moff_mine = moff[i];
+    }
+  }
 
   // A wave owns 64 consecutive keys of every tile and the matching columns of s_out: no workgroup
   // barrier anywhere. The rows come in half-slices of HB iterations through two register buffers;
@@ -199,18 +209,11 @@ __global__ __launch_bounds__(SC_NT) void k_qk_scores(qk_params P) {
       if constexpr (FAST4) {
         const float d = sc_reduce4<LPK>(sc_dot<DT>(qv[0], buf[it]), sc_dot<DT>(qv[1], buf[it]), sc_dot<DT>(qv[2], buf[it]),
                                          sc_dot<DT>(qv[3], buf[it]), sub);
-        int rr = row[0];
-        int64_t mo = moff[0];
-#pragma unroll
-        for (int i = 1; i < SC_NQ; ++i) {
-          if (mine == i) {
-            rr = row[i];
-            mo = moff[i];
-          }
-        }
-        if (sub < 4 && j < P.Lk && rr >= 0) {
+        // without a mask nothing is read here: keys past the row's end and dead query vectors park a value that
+        // the copy-out below never stores
+        if (sub < 4 && (!AM || (j < P.Lk && row_mine >= 0))) {
           float s = sah_round<DT>(d);
-          if (P.amask) s = sah_round<DT>(s + sah_load<DT>(P.amask, mo + j));
+          if (AM) s = sah_round<DT>(s + sah_load<DT>(P.amask, moff_mine + j));
           s_out[mine][jl] = (key_t)sah_sort_key<DT>(s);
         }
       } else {
@@ -219,7 +222,7 @@ __global__ __launch_bounds__(SC_NT) void k_qk_scores(qk_params P) {
           const float d = sc_group_sum<LPK>(sc_dot<DT>(qv[i], buf[it]));
           if (sub == (i % LPK) && j < P.Lk && row[i] >= 0) {
             float s = sah_round<DT>(d);
-            if (P.amask) s = sah_round<DT>(s + sah_load<DT>(P.amask, moff[i] + j));
+            if (AM) s = sah_round<DT>(s + sah_load<DT>(P.amask, moff[i] + j));
             s_out[i][jl] = (key_t)sah_sort_key<DT>(s);
           }
         }
@@ -236,13 +239,24 @@ __global__ __launch_bounds__(SC_NT) void k_qk_scores(qk_params P) {
       sah_wave_lds_sync();  // the columns are free again for the next tile
     }
   };
+  // No request of the steady state sits behind a condition: where a path with and a path without a request meet,
+  // the compiler's wait for the buffer about to be scored is the stricter of the two, i.e. it also waits for the
+  // loads just issued and the two buffers no longer overlap. The last one or two parts are a copy of their own.
   sc_raw<DT> ka[HB], kb[HB];
   request(ka, 0);
-  for (int hs = 0; hs < n_half; hs += 2) {
-    if (hs + 1 < n_half) request(kb, hs + 1);
+  int hs = 0;
+  for (; hs + 2 < n_half; hs += 2) {
+    request(kb, hs + 1);
     score(ka, hs);
-    if (hs + 2 < n_half) request(ka, hs + 2);
-    if (hs + 1 < n_half) score(kb, hs + 1);
+    request(ka, hs + 2);
+    score(kb, hs + 1);
+  }
+  if (hs + 1 < n_half) {
+    request(kb, hs + 1);
+    score(ka, hs);
+    score(kb, hs + 1);
+  } else {
+    score(ka, hs);
   }
 }
 
@@ -259,7 +273,8 @@ static int qk_launch(const sah_qk_scores_args* a, const qk_params& P) {
   Q.iters = iters;
   dim3 g((unsigned)((tiles + iters - 1) / iters), a->B * a->Hkv, (nvec + SC_NQ - 1) / SC_NQ);
   sah_timed timed("k_qk_scores", a->stream);
-  hipLaunchKernelGGL((k_qk_scores<DT, D>), g, dim3(SC_NT), 0, (hipStream_t)a->stream, Q);
+  if (a->amask) hipLaunchKernelGGL((k_qk_scores<DT, D, true>), g, dim3(SC_NT), 0, (hipStream_t)a->stream, Q);
+  else hipLaunchKernelGGL((k_qk_scores<DT, D, false>), g, dim3(SC_NT), 0, (hipStream_t)a->stream, Q);
   return sah_launch_status("sah_qk_scores");
 }
 

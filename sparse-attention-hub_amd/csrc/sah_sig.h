@@ -384,7 +384,7 @@ __device__ __forceinline__ void sig_mfma_block(const sig_params& P, bool active,
       for (int v = 0; v < 4; ++v) {
         const uint16_t bb = (uint16_t)(braw[v >> 1] >> (16 * (v & 1)));
         const float bv = (f0 + 4 <= dout) ? ((DT == SAH_BF16) ? sah_bf16_to_float(bb) : sah_f16_to_float(bb)) : 0.f;
-        y[v] = sah_round_hw<DT>(sah_round_hw<DT>(acc[v]) + bv);
+        y[v] = sah_round<DT>(sah_round<DT>(acc[v]) + bv);
       }
       if (!last) {
         if (f0 + 4 <= dout) {
