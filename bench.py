@@ -318,12 +318,13 @@ def parity_and_cpu_baseline(run, last, budget_s=25.0):
 
 
 def sub_run(cfg: int, dev) -> dict:
-    """A short run of another configuration of the headline set: cold call, 5 warm-up steps, one bracket of timed steps."""
+    """A short run of another configuration of the headline set: cold call, warm-up steps (about 10 ms of them, so
+    that the clocks have settled), one bracket of timed steps."""
     import torch
 
     w = dict(WORKLOADS[cfg])
     steps = 24 if cfg == 5 else 64
-    run = Run(w, dev, steps, 5, 1, 0, host_rng=False)
+    run = Run(w, dev, steps, 8 if cfg == 5 else 160, 1, 0, host_rng=False)
     cold_ms = run.cold()
     wall, gpu, _, _ = run.timed()
     sampled = 0.0
@@ -389,7 +390,9 @@ def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=256,
+                    help="untimed steps before the first bracket; after an idle GPU the step time settles over the first "
+                         "~200 steps (the clocks ramp up), fewer warm-up steps time that ramp")
     ap.add_argument("--config", type=int, default=3, choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-configs", action="store_true", help="skip the short sub-runs of the other configurations")
