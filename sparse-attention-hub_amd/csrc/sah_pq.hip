@@ -294,8 +294,10 @@ __global__ __launch_bounds__(PQB_NT) void k_pq_assign_block(pq_assign_params P) 
 #define PQM_NW (PQM_NT / SAH_WAVE)
 #define PQM_KEY_TILES 16  // 32-key tiles per wave and workgroup: 2048 keys per workgroup
 
+// (two waves per SIMD at least: with at most 256 registers a wave the compiler keeps the accumulators in ordinary
+// vector registers, which the minimum search reads directly)
 template <int DT, int KS>  // KS = d_sub / 2 k-steps
-__global__ __launch_bounds__(PQM_NT) void k_pq_assign_mfma(pq_assign_params P) {
+__global__ __launch_bounds__(PQM_NT, 2) void k_pq_assign_mfma(pq_assign_params P) {
   constexpr int DS = 2 * KS;
   __shared__ __attribute__((aligned(16))) float s_a[(PQ_MAX_CENT / 32) * 2 * 32 * KS];  // -2 c, [tile][g][i][s]
   __shared__ __attribute__((aligned(16))) float s_cn[(PQ_MAX_CENT / 32) * 2 * 16];      // ||c||^2, [tile][g][v]
@@ -350,8 +352,8 @@ __global__ __launch_bounds__(PQM_NT) void k_pq_assign_mfma(pq_assign_params P) {
     for (int s = 0; s < KS; ++s) xs[s] = sah_load<DT>(P.k, off + 2 * s + g);
     float best = INFINITY;
     int bidx = 0;
-    for (int t = 0; t < n_tiles; ++t) {
-      sah_f32x16 acc;
+    // accumulator of centre tile t: seeded with the norms, then the KS matrix instructions
+    auto product = [&](sah_f32x16& acc, int t) {
       const float4* cn4 = (const float4*)(s_cn + (t * 2 + g) * 16);
 #pragma unroll
       for (int q4 = 0; q4 < 4; ++q4) {
@@ -361,14 +363,43 @@ __global__ __launch_bounds__(PQM_NT) void k_pq_assign_mfma(pq_assign_params P) {
       const float* ap = s_a + ((t * 2 + g) * 32 + j) * KS;
 #pragma unroll
       for (int s = 0; s < KS; ++s) acc = sah_mfma_32x32x2_f32(ap[s], xs[s], acc);
+    };
+    // the tile's first minimum and its accumulator slot (constants), then one comparison with the best so far:
+    // bidx holds 16 t + slot until the end
+    auto take_min = [&](const sah_f32x16& acc, int t) {
+      float m = acc[0];
+      int mv = 0;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {  // ascending centre index: the first minimum is kept
-        if (acc[v] < best) {
-          best = acc[v];
-          bidx = t * 32 + 8 * (v >> 2) + 4 * g + (v & 3);
+      for (int v = 1; v < 16; ++v) {  // ascending centre index: the first minimum is kept
+        if (acc[v] < m) {
+          m = acc[v];
+          mv = v;
         }
       }
+      if (m < best) {
+        best = m;
+        bidx = t * 16 + mv;
+      }
+    };
+    // Two accumulators: while the matrix unit works on one tile, the vector unit takes the minimum of the tile
+    // before (48 vector instructions against 4 matrix instructions of 16 passes: about the same time).
+    sah_f32x16 acc0, acc1;
+    product(acc0, 0);
+    int t = 0;
+    for (; t + 2 < n_tiles; t += 2) {
+      product(acc1, t + 1);
+      take_min(acc0, t);
+      product(acc0, t + 2);
+      take_min(acc1, t + 1);
     }
+    if (t + 1 < n_tiles) {
+      product(acc1, t + 1);
+      take_min(acc0, t);
+      take_min(acc1, t + 1);
+    } else {
+      take_min(acc0, t);
+    }
+    bidx = (bidx >> 4) * 32 + 8 * ((bidx >> 2) & 3) + 4 * g + (bidx & 3);  // tile, slot -> centre
     const float ob = __shfl_xor(best, 32);
     const int oi = __shfl_xor(bidx, 32);
     if (ob < best || (ob == best && oi < bidx)) {
