@@ -15,7 +15,10 @@ one key per step, until the timed steps add up to a multiple of 64 and to at lea
 the HashAttention plan hashes new keys 64 at a time (one extra launch pair every 64 steps),
 so a multiple of 64 steps holds exactly its share of that work whatever K is. `value` is
 the mean over all timed steps; the median and minimum over the K-step brackets are
-reported beside it.
+reported beside it. Before the W warm-up steps bench.py runs untimed steps of its own until
+256 steps have run (`clock_settle_steps` in the output): a GPU that had no work for some
+milliseconds runs its first ~10 ms of work at a lower clock, and W = 5 with K = 20 would time
+nothing else.
 
 Prints ONE JSON line: whole-step microseconds (`value`), the roofline of the dominant kernel
 from HIP-event timings taken inside this run, the parity of the last timed step against the
@@ -53,6 +56,7 @@ WORKLOADS = {
             adaptive=dict(rate=0.01, epsilon=0.05, delta=0.05)),
 }
 HQ, HKV, D = 32, 8, 128
+SETTLE_STEPS = 256   # untimed steps before the first bracket, the W warm-up steps included
 
 
 def algorithmic_bytes(w, sampled_per_row: float = 0.0) -> dict:
@@ -158,15 +162,19 @@ def median(xs):
 class Run:
     """One workload on the GPU: cold call, warm-up, timed brackets; keeps the last step's output and rows."""
 
-    def __init__(self, w, dev, steps, warm, reps, probe, host_rng):
+    def __init__(self, w, dev, steps, warm, reps, probe, host_rng, settle=0):
         import torch
 
         self.torch = torch
         self.w, self.dev, self.steps, self.warm, self.reps, self.probe = w, dev, steps, warm, reps, probe
         self.total = steps * reps
-        self.first = w["Lk"] - (warm + self.total)         # the last timed step runs at exactly Lk keys
+        # Steps run before the W warm-up steps so that the clocks have settled when the first bracket starts: after
+        # some milliseconds without work the GPU runs its first ~10 ms of work at a lower clock (config 3: 64 us per
+        # step falling to 60.5 over the first ~150 steps), which W = 5 warm-up steps and 20-step brackets never leave.
+        self.settle = settle
+        self.first = w["Lk"] - (settle + warm + self.total)  # the last timed step runs at exactly Lk keys
         if self.first <= w["sink"] + w["local"] + w["k"] + 512:
-            raise SystemExit(f"bench.py: {warm} + {self.total} steps do not fit below {w['Lk']} keys")
+            raise SystemExit(f"bench.py: {settle} + {warm} + {self.total} steps do not fit below {w['Lk']} keys")
         self.ra, self.qs, self.k, self.v, self.extra = build_workload(w, dev, w["Lk"] + probe, host_rng)
         self.meta = {}
         self.scaling = D ** -0.5
@@ -188,11 +196,11 @@ class Run:
         each bracket's steps after the first few: by then the host runs ahead of the GPU, so that region holds kernels
         back to back without the start-up gap of a bracket that begins on an idle GPU)."""
         torch = self.torch
-        for i in range(self.warm):
+        for i in range(self.settle + self.warm):
             self.step(i, self.first + 1 + i)
         torch.cuda.synchronize()
         wall, gpu, host, inner = [], [], [], []
-        n = self.first + self.warm
+        n = self.first + self.settle + self.warm
         skip = min(4, self.steps // 2)
         for _ in range(self.reps):
             ev0, ev1, evm = (torch.cuda.Event(enable_timing=True) for _ in range(3))
@@ -390,9 +398,9 @@ def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
-    ap.add_argument("--warmup", type=int, default=256,
-                    help="untimed steps before the first bracket; after an idle GPU the step time settles over the first "
-                         "~200 steps (the clocks ramp up), fewer warm-up steps time that ramp")
+    ap.add_argument("--warmup", type=int, default=20,
+                    help="untimed steps before the first bracket (bench.py runs untimed steps of its own before them "
+                         "until SETTLE_STEPS have run, so that the clocks have settled)")
     ap.add_argument("--config", type=int, default=3, choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-configs", action="store_true", help="skip the short sub-runs of the other configurations")
@@ -429,7 +437,8 @@ def main() -> None:
     steps, warm = args.steps, args.warmup
     reps = repeats_for(steps)
     probe = 2 * HASH_BLOCK                                # instrumented steps for the per-kernel durations
-    run = Run(w, dev, steps, warm, reps, probe, host_rng=True)
+    settle = max(0, SETTLE_STEPS - warm)
+    run = Run(w, dev, steps, warm, reps, probe, host_rng=True, settle=settle)
     cold_ms = run.cold()
 
     if args.pmc_probe:
@@ -493,6 +502,7 @@ def main() -> None:
         "n_gpus": 1,
         "steps": steps,
         "warmup": warm,
+        "clock_settle_steps": settle,
         "ms_per_step": round(ms_per_step, 5),
         "higher_is_better": False,
         "scaling": "weak",
