@@ -495,6 +495,11 @@ typedef struct sah_adaptive_budget_args {
   float* prob;            /* [n_rows] out */
   float* stats;           /* [n_rows, 4] out, or NULL */
   void* stream;
+  int32_t max_in_rows;    /* != 0: the caller's promise that every row's largest key belongs to a column that  */
+                          /* is already in the row (an exact top-k over these very keys has just run, with    */
+                          /* k >= 1): the row maximum of adaptive_sampling.py:195-196 is then taken from the   */
+                          /* row's entries instead of a pass over all n_keys keys. Ignored with an additive    */
+                          /* mask, with prev_empty, and with scaling <= 0                                      */
 } sah_adaptive_budget_args;
 int sah_adaptive_budget(const sah_adaptive_budget_args* a);
 

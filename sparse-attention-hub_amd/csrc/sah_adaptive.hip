@@ -12,6 +12,7 @@
 
 #define AD_NT 1024
 #define AD_NW (AD_NT / SAH_WAVE)
+#define AD_EPT 4          // entries of a row a thread keeps in registers
 #define AD_MAX_LDS_WORDS 36864  // 144 KB bitmap: sampling range up to ~1.17 M keys
 
 // uniform column of [start, start + range) from one 32-bit draw
@@ -35,12 +36,17 @@ struct ad_row {
   int64_t moff;
   float scaling;
   float zmax;
-  __device__ __forceinline__ float z(int j) const {
-    float s = sah_round<DT>(ad_key_score<DT>(keys[j]) * scaling);
+  // z and the numerator of column j whose score key the caller holds
+  __device__ __forceinline__ float z_of(uint32_t key, int j) const {
+    float s = sah_round<DT>(ad_key_score<DT>(key) * scaling);
     if (amask) s = sah_round<DT>(s + sah_load<DT>(amask, moff + j));
     return s;
   }
-  __device__ __forceinline__ float e(int j) const { return sah_round<DT>(expf(sah_round<DT>(z(j) - zmax))); }
+  __device__ __forceinline__ float e_of(uint32_t key, int j) const {
+    return sah_round<DT>(expf(sah_round<DT>(z_of(key, j) - zmax)));
+  }
+  __device__ __forceinline__ float z(int j) const { return z_of(keys[j], j); }
+  __device__ __forceinline__ float e(int j) const { return e_of(keys[j], j); }
 };
 
 __device__ __forceinline__ float ad_block_sum(float v, float* s_red) {
@@ -75,6 +81,7 @@ struct ad_budget_params {
   float eps, ppf;
   uint32_t k0, k1, o0, o1;
   int prev_empty;
+  int max_in_rows;  // the caller's promise: every row's largest key belongs to a column already in the row
   int vec_keys;  // 1: every row of keys starts 16-byte aligned (vector loads in the row-maximum pass)
   int* budget;
   float* prob;
@@ -106,9 +113,43 @@ __global__ __launch_bounds__(AD_NT) void k_adaptive_budget(ad_budget_params P) {
 
   for (int i = tid; i < nw; i += AD_NT) s_bits[i] = 0u;
 
+  // The row's entries, the first AD_EPT of every thread held in registers: they serve the row maximum (when the
+  // caller promises that it is among them) and the static denominator from one fetch.
+  int ent_c[AD_EPT];
+  uint32_t ent_k[AD_EPT];
+  int cnt = 0;
+  const int* cols = P.rows.cols + (int64_t)r * P.rows.cap;
+  if (!P.prev_empty) {
+    cnt = P.rows.cnt[r];
+    if (cnt > P.rows.cap) cnt = P.rows.cap;
+  }
   // ---- row maximum of z over ALL keys (adaptive_sampling.py:195-196)
   float zm = -INFINITY;
-  if (!P.amask && P.vec_keys && P.scaling > 0.f) {
+  const bool from_entries = P.max_in_rows && !P.prev_empty && !P.amask && P.scaling > 0.f;
+  if (from_entries) {
+    // z is a non-decreasing function of the score and the keys keep the scores' order: the maximum is z of the
+    // largest key, and an exact top-k over these keys has put that key's column into the row
+    uint32_t best = 0u;
+#pragma unroll
+    for (int u = 0; u < AD_EPT; ++u) {
+      const int i = tid + u * AD_NT;
+      int c = i < cnt ? cols[i] : -1;
+      if (c >= Lk) c = -1;
+      ent_c[u] = c;
+    }
+#pragma unroll
+    for (int u = 0; u < AD_EPT; ++u) {
+      ent_k[u] = ent_c[u] >= 0 ? (uint32_t)row.keys[ent_c[u]] : 0u;  // key 0 is the smallest key
+      best = ent_k[u] > best ? ent_k[u] : best;
+    }
+    for (int i = tid + AD_EPT * AD_NT; i < cnt; i += AD_NT) {
+      const int c = cols[i];
+      if (c < 0 || c >= Lk) continue;
+      const uint32_t kc = (uint32_t)row.keys[c];
+      best = kc > best ? kc : best;
+    }
+    zm = sah_round<DT>(ad_key_score<DT>(best) * row.scaling);
+  } else if (!P.amask && P.vec_keys && P.scaling > 0.f) {
     // Without an additive mask z is a non-decreasing function of the score, and the keys keep the
     // scores' order: the row maximum is z of the largest key. 16 bytes of keys per load, integer max.
     constexpr int KPV = (DT == SAH_F32) ? 4 : 8;  // keys per 16-byte vector
@@ -153,16 +194,22 @@ __global__ __launch_bounds__(AD_NT) void k_adaptive_budget(ad_budget_params P) {
   if (P.prev_empty) {
     for (int j = tid; j < Lk; j += AD_NT) part += row.e(j);
   } else {
-    int cnt = P.rows.cnt[r];
-    if (cnt > P.rows.cap) cnt = P.rows.cap;
-    const int* cols = P.rows.cols + (int64_t)r * P.rows.cap;
     const float* w = P.rows.w ? P.rows.w + (int64_t)r * P.rows.cap : nullptr;
-    for (int i = tid; i < cnt; i += AD_NT) {
-      const int c = cols[i];
-      if (c < 0 || c >= Lk) continue;
+    auto add = [&](int i, int c, float num) {
       float iw = sah_round<DT>(1.0f / sah_round<DT>(1.0f + 1e-6f));
       if (w) iw = sah_round<DT>(1.0f / sah_round<DT>(w[i] + 1e-6f));
-      part += sah_round<DT>(row.e(c) * iw);
+      part += sah_round<DT>(num * iw);
+    };
+    int i = tid;
+    if (from_entries) {
+#pragma unroll
+      for (int u = 0; u < AD_EPT; ++u, i += AD_NT)
+        if (ent_c[u] >= 0) add(i, ent_c[u], row.e_of(ent_k[u], ent_c[u]));
+    }
+    for (; i < cnt; i += AD_NT) {
+      const int c = cols[i];
+      if (c < 0 || c >= Lk) continue;
+      add(i, c, row.e(c));
     }
   }
   const float static_den = sah_round<DT>(ad_block_sum(part, s_red));
@@ -170,6 +217,7 @@ __global__ __launch_bounds__(AD_NT) void k_adaptive_budget(ad_budget_params P) {
   // ---- base sample: mean, unbiased std, and the set of distinct columns
   const int n_calls = (P.n_base + 3) >> 2;
   part = 0.f;
+  float first_e[4] = {0.f, 0.f, 0.f, 0.f};  // numerators of the thread's first call (all of them up to 4096 draws)
   for (int c = tid; c < n_calls; c += AD_NT) {
     uint32_t u[4];
     sah_philox((uint32_t)c, (uint32_t)r, P.o0, P.o1, P.k0, P.k1, u);
@@ -177,14 +225,25 @@ __global__ __launch_bounds__(AD_NT) void k_adaptive_budget(ad_budget_params P) {
     for (int t = 0; t < 4; ++t) {
       if (4 * c + t < P.n_base) {
         const int j = ad_column(u[t], P.start, P.range);
-        part += row.e(j);
+        const float ej = row.e(j);
+        if (c == tid) first_e[t] = ej;
+        part += ej;
         atomicOr(&s_bits[(j >> 5) - w0], 1u << (j & 31));
       }
     }
   }
   const float mean = ad_block_sum(part, s_red) / (float)P.n_base;
   part = 0.f;
-  for (int c = tid; c < n_calls; c += AD_NT) {
+  if (tid < n_calls) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      if (4 * tid + t < P.n_base) {
+        const float d = first_e[t] - mean;
+        part = fmaf(d, d, part);
+      }
+    }
+  }
+  for (int c = tid + AD_NT; c < n_calls; c += AD_NT) {
     uint32_t u[4];
     sah_philox((uint32_t)c, (uint32_t)r, P.o0, P.o1, P.k0, P.k1, u);
 #pragma unroll
@@ -398,6 +457,7 @@ extern "C" int sah_adaptive_budget(const sah_adaptive_budget_args* a) {
   P.Hq = a->Hq; P.Lq = a->Lq;
   P.scaling = a->scaling;
   P.start = a->start; P.range = a->range; P.n_base = a->n_base;
+  P.max_in_rows = a->max_in_rows;
   P.eps = a->eps; P.ppf = a->delta_ppf;
   P.k0 = (uint32_t)a->seed; P.k1 = (uint32_t)(a->seed >> 32);
   P.o0 = (uint32_t)a->offset; P.o1 = (uint32_t)(a->offset >> 32);

@@ -246,6 +246,7 @@ class AdaptiveBudgetArgs(C.Structure):
         ("prob", C.c_void_p),
         ("stats", C.c_void_p),
         ("stream", C.c_void_p),
+        ("max_in_rows", C.c_int32),
     ]
 
 

@@ -94,6 +94,9 @@ class OracleTopK(TopKMasker):
         shared = kwargs.get("_call_scratch")
         if am_ptr is None and isinstance(shared, dict):
             shared["qk_score_keys"] = keybuf  # later maskers of this call can skip their own scoring pass
+            # ... and know that the largest key of every row now belongs to a column of the row: the k_eff >= 1
+            # largest keys outside the previous mask were just added
+            shared["qk_top_in_rows"] = True
         # active columns rank where `scores[prev != 0] = finfo(mask dtype).min` puts them
         excluded = sortable_key_of(torch.finfo(previous_mask.dtype).min, q.dtype)
         self._select_into_rows(rows, keybuf, 32 if q.dtype == torch.float32 else 16, Lk, 0, k_eff, excluded)

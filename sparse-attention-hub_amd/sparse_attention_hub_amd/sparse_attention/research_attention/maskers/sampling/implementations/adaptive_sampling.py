@@ -172,6 +172,8 @@ class AdaptiveSamplingMasker(SamplingMasker):
         # masker that ran earlier in this call (OracleTopK) when there is one
         shared = kwargs.get("_call_scratch")
         keybuf = shared.get("qk_score_keys") if isinstance(shared, dict) else None
+        # an exact top-k over these keys ran earlier in this call: the row maximum is among the rows' entries
+        max_in_rows = keybuf is not None and bool(shared.get("qk_top_in_rows"))
         if keybuf is None:
             k = _inner_contiguous(keys)
             keybuf = score_key_buffer(n_rows, Lk, q.dtype, q.device)
@@ -208,6 +210,7 @@ class AdaptiveSamplingMasker(SamplingMasker):
             start, n, nb, float(self.epsilon), self.delta_ppf,
             seed, offset, int(prev_empty),
             budget.data_ptr(), prob.data_ptr(), None if stats is None else stats.data_ptr(), stream,
+            int(max_in_rows and not prev_empty and am_ptr is None),
         ))
         if w_fresh:
             rows.w = torch.empty((rows.n_rows, rows.cap), dtype=torch.float32, device=q.device)

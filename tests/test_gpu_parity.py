@@ -1176,6 +1176,58 @@ def test_adaptive_sampling_denominator_guarantee_at_scale(cuda):
     assert bool(((cols >= 0) & (cols < Lk) | ~valid).all())
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", ["small", "beyond_the_register_copies"])
+def test_adaptive_budget_row_maximum_from_the_rows_entries(cuda, dtype, shape, monkeypatch):
+    """After an exact top-k over the score keys the row maximum is among the row's entries: the budget kernel then
+    skips its pass over all keys (`max_in_rows`). Budgets, probabilities and statistics must not change by a bit;
+    the larger shape has more than 4096 entries per row and more than 4096 base draws (the parts of both that a
+    thread does not keep in registers)."""
+    sa = _sa()
+    if shape == "small":
+        B, Hq, Hkv, Lk, D, heavy, rate = 2, 4, 2, 3000, 32, 0.05, 0.05
+    else:
+        B, Hq, Hkv, Lk, D, heavy, rate = 1, 2, 1, 12000, 32, 5000, 0.75
+    q, k, v = make_qkv(B, Hq, Hkv, 1, Lk, D, dtype, seed=23)
+    scaling = D ** -0.5
+
+    def run():
+        cfgs = [sa.SinkMaskerConfig(sink_size=8), sa.LocalMaskerConfig(window_size=16), sa.OracleTopKConfig(heavy_size=heavy),
+                sa.AdaptiveSamplingMaskerConfig(base_rate_sampling=rate, epsilon=0.25, delta=0.25, init_offset=8, local_offset=16)]
+        ra = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=cfgs))
+        m = ra.maskers[-1]
+        m.seed, m.keep_stats = 5, True
+        out, _ = ra.custom_attention(None, q.to(cuda), k.to(cuda), v.to(cuda), None, scaling, 0.0, sparse_meta_data={}, layer_idx=0)
+        return out.cpu(), m.last_budget.cpu(), m.last_probability.cpu(), m.last_stats.cpu(), m.last_rows.cnt.cpu()
+
+    from sparse_attention_hub_amd import _native as N
+
+    seen = []
+    orig_call = N.call
+
+    def spy(name, args):
+        if name == "sah_adaptive_budget":
+            seen.append(int(args.max_in_rows))
+        return orig_call(name, args)
+
+    monkeypatch.setattr(N, "call", spy)
+    with_flag = run()
+    orig_add = sa.OracleTopK.add_mask
+
+    def without_promise(self, *a, **kw):
+        mask = orig_add(self, *a, **kw)
+        kw["_call_scratch"].pop("qk_top_in_rows", None)
+        return mask
+
+    monkeypatch.setattr(sa.OracleTopK, "add_mask", without_promise)
+    without_flag = run()
+    assert seen == [1, 0]
+    for a, b in zip(with_flag, without_flag):
+        assert torch.equal(a, b)
+    if shape != "small":
+        assert int(with_flag[4].min()) > 4096 + 24
+
+
 def test_adaptive_sampling_abi_rejects_bad_arguments(cuda):
     from sparse_attention_hub_amd import _native as N
     from sparse_attention_hub_amd.sparse_attention.utils.native_rows import NativeRows
