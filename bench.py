@@ -394,6 +394,46 @@ def cold_probe(dev) -> dict:
             "note": "HIP events around every launch; flops = 2 x keys x centres x dims (k-means), 2 x MLP multiply-adds (signatures)"}
 
 
+def hw_probe(dev) -> dict:
+    """What the GPU gives to two patterns of the library (`sah_hw_probe`, HIP events around back-to-back launches):
+    a 4 GiB read stream alone and with 1/32 of its volume written back (the exact-score pass over K at config 5), and
+    matrix / vector / interleaved instruction streams (the Lloyd assignment)."""
+    import torch
+
+    from sparse_attention_hub_amd import _native as N
+
+    out = {"hw_probe": True}
+    n = 4 << 30
+    src = torch.empty(n, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty(n // 32 + 4096, dtype=torch.uint8, device=dev)
+    stream = N.stream_ptr(dev)
+
+    def timed(args, reps):
+        for _ in range(3):
+            N.call("sah_hw_probe", args)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(reps):
+            N.call("sah_hw_probe", args)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / reps
+
+    names = {0: "read_4GiB", 1: "read_4GiB_write_4x128B_per_16KB", 2: "read_4GiB_write_512B_per_16KB"}
+    for kind in (0, 1, 2, 0):
+        us = timed(N.HwProbeArgs(kind, src.data_ptr(), n, dst.data_ptr(), dst.numel(), 0, 0, stream), 10)
+        out.setdefault(names[kind], []).append({"us": round(us, 1), "read_TBps": round(n / us / 1e6, 3)})
+    names = {3: "matrix_only", 4: "vector_only", 5: "matrix_and_vector_interleaved"}
+    for wgs in (256, 1024):
+        for kind in (3, 4, 5):
+            us = timed(N.HwProbeArgs(kind, None, 0, dst.data_ptr(), dst.numel(), 2000, wgs, stream), 5)
+            out[f"{names[kind]}_{wgs // 256}_waves_per_simd_us"] = round(us, 1)
+    out["note"] = ("stream kinds: 65536 workgroups x 64 KB, non-temporal 16-byte loads; issue kinds: 2000 iterations of 4 dependent "
+                   "32x32x2 fp32 matrix instructions and / or 48 vector FMAs per wave")
+    return out
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -409,6 +449,9 @@ def main() -> None:
     ap.add_argument("--cold-probe", action="store_true",
                     help="short run for `rocprofv3 --pmc` / `--kernel-trace` of the two matrix-core kernels of the cold calls: "
                          "two Lloyd iterations of the config-4 k-means and the config-3 bulk signature build")
+    ap.add_argument("--hw-probe", action="store_true",
+                    help="times the probe kernels of sah_hw_probe: read-stream ceilings with and without a write stream, "
+                         "matrix / vector instruction overlap")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="short run for `rocprofv3 --pmc`: a few layer-steps plus three 256 MiB copy kernels of known size")
     args = ap.parse_args()
@@ -427,6 +470,9 @@ def main() -> None:
     dev = torch.device("cuda:0")
     if args.cold_probe:
         print(json.dumps(cold_probe(dev)))
+        return
+    if args.hw_probe:
+        print(json.dumps(hw_probe(dev)))
         return
     w = dict(WORKLOADS[args.config])
     study = bool(args.batch or args.keys)

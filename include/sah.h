@@ -592,6 +592,32 @@ int sah_hash_compact_codes(const sah_hash_compact_args* a);
 int sah_hash_decode_attention(const sah_hash_decode_args* a, const sah_attention_args* t);
 
 /* ---------------------------------------------------------------------------
+ * Measurement aid; no counterpart in the reference and no part of the decode path. One launch of a probe kernel
+ * that shows what this GPU gives to two patterns of the library, so that the roofline fractions of the kernels
+ * that have them can be judged against what is attainable (`bench.py --hw-probe` times it):
+ *   kind 0  a read stream of `bytes` bytes (64 KB per workgroup, 1 KB per wave instruction, non-temporal loads):
+ *           the pattern of sah_qk_scores over K;
+ *   kind 1  the same with 1/32 of the volume written to dst, as four 128-byte stores to four rows per 16 KB read
+ *           (the 2-byte score keys of the four query heads of a group);
+ *   kind 2  the same volume written as one 512-byte store per 16 KB;
+ *   kind 3  `workgroups` workgroups of 4 waves, `iters` iterations of four dependent 32x32x2 fp32 matrix
+ *           instructions (one centre tile of sah_pq_kmeans_assign);
+ *   kind 4  the same loop with 48 vector instructions instead (that tile's minimum search);
+ *   kind 5  both, interleaved.
+ * bytes: a multiple of 65536; dst_bytes >= bytes / 32 (kinds 0-2; kind 0 writes nothing), >= 4 (kinds 3-5).   */
+typedef struct sah_hw_probe_args {
+  int32_t kind;
+  const void* src;
+  int64_t bytes;
+  void* dst;
+  int64_t dst_bytes;
+  int32_t iters;
+  int32_t workgroups;
+  void* stream;
+} sah_hw_probe_args;
+int sah_hw_probe(const sah_hw_probe_args* a);
+
+/* ---------------------------------------------------------------------------
  * One decode layer-step as a single call: runs, in this order and on the stream
  * each block names, every stage whose pointer is not NULL -
  *   sink_local -> (sig_a, sig_b as sah_hash_signatures_pair) -> compact -> hamming

@@ -52,6 +52,7 @@ EXPECTED_SYMBOLS = (
     "sah_sparse_attention_static",
     "sah_attention_weights",
     "sah_run_chain",
+    "sah_hw_probe",
 )
 
 
@@ -247,6 +248,16 @@ class AdaptiveBudgetArgs(C.Structure):
         ("stats", C.c_void_p),
         ("stream", C.c_void_p),
         ("max_in_rows", C.c_int32),
+    ]
+
+
+class HwProbeArgs(C.Structure):
+    _fields_ = [
+        ("kind", C.c_int32),
+        ("src", C.c_void_p), ("bytes", C.c_int64),
+        ("dst", C.c_void_p), ("dst_bytes", C.c_int64),
+        ("iters", C.c_int32), ("workgroups", C.c_int32),
+        ("stream", C.c_void_p),
     ]
 
 

@@ -68,7 +68,7 @@ def test_every_entry_point_refuses_null_and_names_itself():
                "sah_hamming_scores", "sah_qk_scores", "sah_select_topk", "sah_pq_keys_absmax", "sah_pq_kmeans_assign",
                "sah_pq_kmeans_update", "sah_pq_adc_scores", "sah_sparse_attention", "sah_sparse_attention_static",
                "sah_attention_weights", "sah_adaptive_budget", "sah_adaptive_sample", "sah_hash_decode_topk",
-               "sah_hash_compact_codes", "sah_run_chain"]
+               "sah_hash_compact_codes", "sah_run_chain", "sah_hw_probe"]
     for fn in one_arg:
         assert getattr(lib, fn)(None) == -2, fn
         assert fn.replace("_static", "").encode() in lib.sah_last_error() or fn.encode() in lib.sah_last_error(), fn
