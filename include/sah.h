@@ -14,6 +14,9 @@
  *   - return value 0 = success, negative = SAH_E* argument error (nothing was
  *     launched), positive = hipError_t from the launch;
  *   - sah_last_error() returns a thread-local description of the last failure;
+ *   - calls may come from several threads; the library's only state of its own is a per-device record of the
+ *     kernels whose dynamic-LDS limit has been raised and the optional timing registry of sah_timing_enable
+ *     (both behind a mutex) and the fixed workspace of sah_sparse_attention_static (see there);
  *   - tensors are addressed by element strides, the innermost (head_dim)
  *     stride must be 1.
  *

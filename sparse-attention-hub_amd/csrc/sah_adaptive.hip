@@ -409,15 +409,6 @@ __global__ __launch_bounds__(AD_NT) void k_adaptive_sample(ad_sample_params P) {
 // ---------------------------------------------------------------------------
 static int ad_lds_words(int start, int range) { return ((start + range + 31) >> 5) - (start >> 5); }
 
-template <typename K>
-static int ad_allow_lds(K kernel, int bytes, bool* done, const char* what) {
-  if (*done) return SAH_OK;
-  hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, AD_MAX_LDS_WORDS * 4);
-  if (e != hipSuccess) return sah_fail((int)e, "%s: cannot raise the LDS limit: %s", what, hipGetErrorString(e));
-  *done = true;
-  return SAH_OK;
-}
-
 static int ad_check_range(const sah_rows& rows, int start, int range, const char* what) {
   if (start < 0 || range < 2 || (int64_t)start + range > rows.n_keys)
     return sah_fail(SAH_EINVAL, "%s: sampling range [%d, %d) must hold >= 2 columns inside [0, %d)", what, start,
@@ -430,8 +421,7 @@ static int ad_check_range(const sah_rows& rows, int start, int range, const char
 
 template <int DT>
 static int ad_budget_launch(const sah_adaptive_budget_args* a, const ad_budget_params& P) {
-  static bool allowed = false;
-  int rc = ad_allow_lds(k_adaptive_budget<DT>, 0, &allowed, "sah_adaptive_budget");
+  int rc = sah_allow_lds((const void*)k_adaptive_budget<DT>, AD_MAX_LDS_WORDS * 4, "sah_adaptive_budget");
   if (rc) return rc;
   const size_t lds = (size_t)ad_lds_words(a->start, a->range) * 4;
   sah_timed timed("k_adaptive_budget", a->stream);
@@ -477,8 +467,7 @@ extern "C" int sah_adaptive_budget(const sah_adaptive_budget_args* a) {
 
 template <int DT>
 static int ad_sample_launch(const sah_adaptive_sample_args* a, const ad_sample_params& P) {
-  static bool allowed = false;
-  int rc = ad_allow_lds(k_adaptive_sample<DT>, 0, &allowed, "sah_adaptive_sample");
+  int rc = sah_allow_lds((const void*)k_adaptive_sample<DT>, AD_MAX_LDS_WORDS * 4, "sah_adaptive_sample");
   if (rc) return rc;
   const size_t lds = (size_t)ad_lds_words(a->start, a->range) * 4;
   sah_timed timed("k_adaptive_sample", a->stream);
