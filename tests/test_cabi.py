@@ -109,3 +109,14 @@ def test_bad_argument_blocks_are_refused_with_the_documented_codes():
     assert lib.sah_select_topk(ctypes.byref(sel)) == -1
     # what the no-allocation attention refuses is more than its built-in buffer holds
     assert N.work_floats(1024, 131072, 128) > 4 * 1024 * 1024 >= N.work_floats(512, 131072, 128)
+    # the measurement aid checks its sizes before it launches anything
+    big = ctypes.create_string_buffer(1 << 16)
+    bptr = (ctypes.addressof(big) + 15) & ~15
+    probe = N.HwProbeArgs(0, bptr, 65536 + 64, bptr, 1 << 12, 0, 0, None)              # not a multiple of 64 KB
+    assert lib.sah_hw_probe(ctypes.byref(probe)) == -1
+    probe = N.HwProbeArgs(1, bptr, 1 << 20, bptr, 1 << 10, 0, 0, None)                 # dst smaller than bytes / 32
+    assert lib.sah_hw_probe(ctypes.byref(probe)) == -1 and b"dst_bytes" in lib.sah_last_error()
+    probe = N.HwProbeArgs(5, None, 0, bptr, 4, 0, 16, None)                            # no iterations
+    assert lib.sah_hw_probe(ctypes.byref(probe)) == -1
+    probe = N.HwProbeArgs(9, None, 0, bptr, 4, 1, 1, None)
+    assert lib.sah_hw_probe(ctypes.byref(probe)) == -1 and b"kind" in lib.sah_last_error()
