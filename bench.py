@@ -139,7 +139,8 @@ def build_workload(w, device, total_keys, host_rng=True):
         a = w["adaptive"]
         cfgs.append(AdaptiveSamplingMaskerConfig(base_rate_sampling=a["rate"], epsilon=a["epsilon"], delta=a["delta"],
                                                  init_offset=w["sink"], local_offset=w["local"]))
-    ra = ResearchAttention.create_from_config(ResearchAttentionConfig(masker_configs=cfgs))
+    extra["config"] = ResearchAttentionConfig(masker_configs=cfgs)
+    ra = ResearchAttention.create_from_config(extra["config"])
     if w.get("adaptive"):
         ra.maskers[-1].seed = 0
     ra.return_attention_weights = False  # HF attention modules drop the dense probabilities in decode
@@ -162,7 +163,7 @@ def median(xs):
 class Run:
     """One workload on the GPU: cold call, warm-up, timed brackets; keeps the last step's output and rows."""
 
-    def __init__(self, w, dev, steps, warm, reps, probe, host_rng, settle=0):
+    def __init__(self, w, dev, steps, warm, reps, probe, host_rng, settle=0, hf_layers=0):
         import torch
 
         self.torch = torch
@@ -178,8 +179,32 @@ class Run:
         self.ra, self.qs, self.k, self.v, self.extra = build_workload(w, dev, w["Lk"] + probe, host_rng)
         self.meta = {}
         self.scaling = D ** -0.5
+        # hf_layers > 0: every step enters through the callable ModelAdapterHF registers in HuggingFace's attention
+        # registry, with what HuggingFace passes it in a decode step of an unpadded batch: the attention module (its
+        # layer_idx), the eager mask - a (B, 1, 1, keys) tensor of zeros, a new one per forward pass, i.e. every
+        # `hf_layers` layer-steps - and sparse_meta_data among the keyword arguments. (Every timed step here has one
+        # key more than the one before, where the layers of one forward pass share a key count: the mask is as wide
+        # as the final key count and every step uses its first n_keys columns, as the reference slices it.)
+        self.hf_layers = hf_layers
+        if hf_layers:
+            from types import SimpleNamespace
+
+            from sparse_attention_hub_amd.adapters import ModelAdapterHF
+
+            adapter = ModelAdapterHF(None, self.extra["config"])        # default arguments
+            self.ra = adapter.sparse_attention
+            self.hf_fn = adapter.get_custom_attention_function(self.ra)
+            self.hf_module = SimpleNamespace(layer_idx=0, training=False)
+            self.hf_mask = None
+            self.hf_calls = 0
 
     def step(self, i, n_keys):
+        if self.hf_layers:
+            if self.hf_calls % self.hf_layers == 0:
+                self.hf_mask = self.torch.zeros((self.w["B"], 1, 1, self.k.shape[2]), dtype=self.qs.dtype, device=self.dev)
+            self.hf_calls += 1
+            return self.hf_fn(self.hf_module, self.qs[i % self.qs.shape[0]], self.k[:, :, :n_keys], self.v[:, :, :n_keys],
+                              self.hf_mask, scaling=self.scaling, dropout=0.0, sparse_meta_data=self.meta)
         return self.ra.custom_attention(None, self.qs[i % self.qs.shape[0]], self.k[:, :, :n_keys], self.v[:, :, :n_keys], None,
                                         self.scaling, 0.0, sparse_meta_data=self.meta, layer_idx=0)
 
@@ -325,6 +350,30 @@ def parity_and_cpu_baseline(run, last, budget_s=25.0):
     return parity, base
 
 
+def hf_callable_run(w, dev, steps, warm, reps, probe, settle, direct_us, direct_out, layers=32) -> dict:
+    """The same workload and the same timed brackets, entered the way HuggingFace enters: through the callable
+    `ModelAdapterHF` (default arguments) registers, with the attention module, the eager mask of an unpadded decode
+    step (zeros, a new tensor every `layers` layer-steps = once per forward pass of a `layers`-layer model) and
+    sparse_meta_data as a keyword argument."""
+    import torch
+
+    run = Run(w, dev, steps, warm, reps, probe, host_rng=True, settle=settle, hf_layers=layers)  # same seeded inputs
+    run.cold()
+    wall, gpu, host, _ = run.timed()
+    total = run.total
+    per_bracket_us = [x / steps * 1e3 for x in wall]
+    us = sum(wall) / total * 1e3
+    same = bool(torch.equal(run.last_out, direct_out))
+    return dict(us=round(us, 2), median_us=round(median(per_bracket_us), 2), min_us=round(min(per_bracket_us), 2),
+                gpu_us=round(sum(gpu) / total * 1e3, 2), host_launch_us=round(sum(host) / total * 1e3, 2),
+                delta_vs_value_us=round(us - direct_us, 2), timed_steps_total=total, forward_pass_layers=layers,
+                last_output_bit_identical_to_direct_call=same,
+                entry="callable of ModelAdapterHF.get_custom_attention_function (default adapter arguments): module with "
+                      "layer_idx, additive mask = zeros of shape (B, 1, 1, keys) in the query dtype re-created once per "
+                      f"{layers} layer-steps, sparse_meta_data in kwargs; the mask is classified on the device once per "
+                      "tensor (one launch and one read-back), then every layer-step of that pass is the one-kernel plan")
+
+
 def sub_run(cfg: int, dev) -> dict:
     """A short run of another configuration of the headline set: cold call, warm-up steps (about 10 ms of them, so
     that the clocks have settled), one bracket of timed steps."""
@@ -395,12 +444,23 @@ def cold_probe(dev) -> dict:
 
 
 def hw_probe(dev) -> dict:
-    """What the GPU gives to two patterns of the library (`sah_hw_probe`, HIP events around back-to-back launches):
-    a 4 GiB read stream alone and with 1/32 of its volume written back (the exact-score pass over K at config 5), and
-    matrix / vector / interleaved instruction streams (the Lloyd assignment)."""
+    """What the GPU gives to two patterns of the library (the bench-only object `bench_hw_probe.so`, built from
+    `bench_hw_probe.hip` beside this file; HIP events around back-to-back launches): a 4 GiB read stream alone and with
+    1/32 of its volume written back (the exact-score pass over K at config 5), and matrix / vector / interleaved
+    instruction streams (the Lloyd assignment)."""
+    import ctypes
+
     import torch
 
     from sparse_attention_hub_amd import _native as N
+
+    path = os.path.join(ROOT, "bench_hw_probe.so")
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} not found: `python __graft_entry__.py` builds it")
+    probe = ctypes.CDLL(path).bench_hw_probe
+    probe.restype = ctypes.c_int
+    probe.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int,
+                      ctypes.c_int, ctypes.c_void_p]
 
     out = {"hw_probe": True}
     n = 4 << 30
@@ -410,24 +470,25 @@ def hw_probe(dev) -> dict:
 
     def timed(args, reps):
         for _ in range(3):
-            N.call("sah_hw_probe", args)
+            if probe(*args) != 0:
+                raise RuntimeError(f"bench_hw_probe refused {args}")
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         e0.record()
         for _ in range(reps):
-            N.call("sah_hw_probe", args)
+            probe(*args)
         e1.record()
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) * 1e3 / reps
 
     names = {0: "read_4GiB", 1: "read_4GiB_write_4x128B_per_16KB", 2: "read_4GiB_write_512B_per_16KB"}
     for kind in (0, 1, 2, 0):
-        us = timed(N.HwProbeArgs(kind, src.data_ptr(), n, dst.data_ptr(), dst.numel(), 0, 0, stream), 10)
+        us = timed((kind, src.data_ptr(), n, dst.data_ptr(), dst.numel(), 0, 0, stream), 10)
         out.setdefault(names[kind], []).append({"us": round(us, 1), "read_TBps": round(n / us / 1e6, 3)})
     names = {3: "matrix_only", 4: "vector_only", 5: "matrix_and_vector_interleaved"}
     for wgs in (256, 1024):
         for kind in (3, 4, 5):
-            us = timed(N.HwProbeArgs(kind, None, 0, dst.data_ptr(), dst.numel(), 2000, wgs, stream), 5)
+            us = timed((kind, None, 0, dst.data_ptr(), dst.numel(), 2000, wgs, stream), 5)
             out[f"{names[kind]}_{wgs // 256}_waves_per_simd_us"] = round(us, 1)
     out["note"] = ("stream kinds: 65536 workgroups x 64 KB, non-temporal 16-byte loads; issue kinds: 2000 iterations of 4 dependent "
                    "32x32x2 fp32 matrix instructions and / or 48 vector FMAs per wave")
@@ -443,6 +504,7 @@ def main() -> None:
                          "until SETTLE_STEPS have run, so that the clocks have settled)")
     ap.add_argument("--config", type=int, default=3, choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-hf-callable", action="store_true", help="skip the sub-run that enters through the HuggingFace callable")
     ap.add_argument("--no-other-configs", action="store_true", help="skip the short sub-runs of the other configurations")
     ap.add_argument("--batch", type=int, default=0, help="study only: override the workload's batch size")
     ap.add_argument("--keys", type=int, default=0, help="study only: override the workload's key count")
@@ -450,7 +512,7 @@ def main() -> None:
                     help="short run for `rocprofv3 --pmc` / `--kernel-trace` of the two matrix-core kernels of the cold calls: "
                          "two Lloyd iterations of the config-4 k-means and the config-3 bulk signature build")
     ap.add_argument("--hw-probe", action="store_true",
-                    help="times the probe kernels of sah_hw_probe: read-stream ceilings with and without a write stream, "
+                    help="times the probe kernels of bench_hw_probe.so: read-stream ceilings with and without a write stream, "
                          "matrix / vector instruction overlap")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="short run for `rocprofv3 --pmc`: a few layer-steps plus three 256 MiB copy kernels of known size")
@@ -576,8 +638,14 @@ def main() -> None:
     }
     if not args.no_cpu_baseline:
         out["parity"], out["cpu_baseline"] = parity_and_cpu_baseline(run, last)
+    if not study and not args.no_hf_callable:
+        del run
+        torch.cuda.empty_cache()
+        out["hf_callable"] = hf_callable_run(w, dev, steps, warm, reps, probe, settle, out["value"], last["out"])
+        run = None
     if not args.no_other_configs and not study:
-        del run, last, rows
+        del last, rows
+        run = None
         torch.cuda.empty_cache()
         others = {}
         for cfg in sorted(WORKLOADS):

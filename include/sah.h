@@ -39,7 +39,11 @@
 extern "C" {
 #endif
 
-#define SAH_VERSION 1
+/* Layout generation of this header. It changes whenever an argument struct gains, loses or reorders a field or an
+ * entry point changes its signature, and never otherwise: a caller compares sah_version() with the SAH_VERSION it was
+ * compiled (or, for a ctypes binding, written) against before its first call and refuses a library that differs,
+ * because a struct of another generation would be read past its end. */
+#define SAH_VERSION 3
 
 enum {
   SAH_OK = 0,
@@ -595,30 +599,25 @@ int sah_hash_compact_codes(const sah_hash_compact_args* a);
 int sah_hash_decode_attention(const sah_hash_decode_args* a, const sah_attention_args* t);
 
 /* ---------------------------------------------------------------------------
- * Measurement aid; no counterpart in the reference and no part of the decode path. One launch of a probe kernel
- * that shows what this GPU gives to two patterns of the library, so that the roofline fractions of the kernels
- * that have them can be judged against what is attainable (`bench.py --hw-probe` times it):
- *   kind 0  a read stream of `bytes` bytes (64 KB per workgroup, 1 KB per wave instruction, non-temporal loads):
- *           the pattern of sah_qk_scores over K;
- *   kind 1  the same with 1/32 of the volume written to dst, as four 128-byte stores to four rows per 16 KB read
- *           (the 2-byte score keys of the four query heads of a group);
- *   kind 2  the same volume written as one 512-byte store per 16 KB;
- *   kind 3  `workgroups` workgroups of 4 waves, `iters` iterations of four dependent 32x32x2 fp32 matrix
- *           instructions (one centre tile of sah_pq_kmeans_assign);
- *   kind 4  the same loop with 48 vector instructions instead (that tile's minimum search);
- *   kind 5  both, interleaved.
- * bytes: a multiple of 65536; dst_bytes >= bytes / 32 (kinds 0-2; kind 0 writes nothing), >= 4 (kinds 3-5).   */
-typedef struct sah_hw_probe_args {
-  int32_t kind;
-  const void* src;
-  int64_t bytes;
-  void* dst;
-  int64_t dst_bytes;
-  int32_t iters;
-  int32_t workgroups;
+ * What an additive attention mask holds. The reference adds the mask it is given to every score row
+ * (hashattention_top_k.py:365-368, oracle_top_k.py:70-72) and to the attention logits
+ * (utils/mask_attention_utils.py:221-225) whatever it contains; through HuggingFace it is the eager mask
+ * (adapters/huggingface.py:311-319), which for a single decode query of an unpadded batch is all zeros. Adding
+ * zeros changes nothing, so a caller that knows the mask is all zeros may pass NULL instead and skip its reads.
+ * ORs into *flags (an int32 the caller has zeroed): SAH_AMASK_NONZERO if any of the first Lk columns of any row is not
+ * 0, SAH_AMASK_GENERAL if any such value lies above the lowest finite value of `dtype` (i.e. is neither 0 nor a
+ * "hidden column" marker such as finfo.min or -inf). Asynchronous like every call: read *flags after the stream has
+ * reached this point. Mask shape (B, Hm, Lq, >= Lk), element strides ms_*, innermost stride 1. */
+enum { SAH_AMASK_NONZERO = 1, SAH_AMASK_GENERAL = 2 };
+typedef struct sah_amask_classify_args {
+  const void* amask;
+  int64_t ms_b, ms_h, ms_l;
+  int32_t dtype;
+  int32_t B, Hm, Lq, Lk;
+  int32_t* flags;
   void* stream;
-} sah_hw_probe_args;
-int sah_hw_probe(const sah_hw_probe_args* a);
+} sah_amask_classify_args;
+int sah_amask_classify(const sah_amask_classify_args* a);
 
 /* ---------------------------------------------------------------------------
  * One decode layer-step as a single call: runs, in this order and on the stream

@@ -77,6 +77,7 @@ __device__ __forceinline__ int sah_wave_id() { return __builtin_amdgcn_readfirst
 template <int BYTES>
 __device__ __forceinline__ void sah_touch_kernargs() {
   static_assert(BYTES <= 1024, "at most 16 lines");
+#if defined(__HIP_DEVICE_COMPILE__)
   typedef const int __attribute__((address_space(4))) karg_int;
   karg_int* p = (karg_int*)__builtin_amdgcn_kernarg_segment_ptr();
   // word o of line i, or of line 0 again when the block is shorter; one sink for all of them, so that every
@@ -86,6 +87,7 @@ __device__ __forceinline__ void sah_touch_kernargs() {
                "s"(SAH_KARG(6)), "s"(SAH_KARG(7)), "s"(SAH_KARG(8)), "s"(SAH_KARG(9)), "s"(SAH_KARG(10)), "s"(SAH_KARG(11)),
                "s"(SAH_KARG(12)), "s"(SAH_KARG(13)), "s"(SAH_KARG(14)), "s"(SAH_KARG(15)));
 #undef SAH_KARG
+#endif
 }
 
 // ---------------------------------------------------------------------------

@@ -235,7 +235,7 @@ __global__ __launch_bounds__(SGM_NT, 4) void k_hash_sig_mfma(sig_params P, int n
         for (int q = 0; q < SGM_MAXM; ++q) {
           float y[16];
           if (q < mt) {
-            const sah_f32x16 acc = tile(q);
+            sah_f32x16 acc = tile(q);
 #pragma unroll
             for (int v4 = 0; v4 < 4; ++v4) {
               const float4 b4 = *(const float4*)(bl + q * 32 + 8 * v4);  // four biases in one read
@@ -261,7 +261,7 @@ __global__ __launch_bounds__(SGM_NT, 4) void k_hash_sig_mfma(sig_params P, int n
         ksteps = 2 * mt;
       } else {
         // sign planes: this lane holds 16 of the vector's bits, lane ^ 32 the other 16
-        const sah_f32x16 acc0 = tile(0);
+        sah_f32x16 acc0 = tile(0);
         uint32_t pos = 0u, nz = 0u;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {

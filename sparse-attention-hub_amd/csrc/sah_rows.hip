@@ -345,3 +345,61 @@ extern "C" int sah_rows_to_dense(const sah_dense_rows_args* a) {
   }
   return sah_launch_status("sah_rows_to_dense");
 }
+
+// ---------------------------------------------------------------------------
+// What an additive attention mask holds, so that the host can tell once per forward pass whether the mask of a
+// decode step is all zeros (HuggingFace's eager mask of an unpadded single-token step) and drop it for every layer.
+// ---------------------------------------------------------------------------
+#define AMC_NT 256
+#define AMC_PER_THREAD 8
+
+template <int DT>
+__global__ __launch_bounds__(AMC_NT) void k_amask_classify(const void* amask, int64_t ms_b, int64_t ms_h, int64_t ms_l, int Hm,
+                                                           int Lq, int Lk, float lowest, int* flags) {
+  const int row = blockIdx.y;  // (b * Hm + h) * Lq + q
+  const int q = row % Lq, h = (row / Lq) % Hm, b = row / (Lq * Hm);
+  const int64_t base = b * ms_b + h * ms_h + q * ms_l;
+  const int c0 = (blockIdx.x * AMC_NT + threadIdx.x) * AMC_PER_THREAD;
+  int f = 0;
+#pragma unroll
+  for (int i = 0; i < AMC_PER_THREAD; ++i) {
+    const int c = c0 + i;
+    if (c < Lk) {
+      const float x = sah_load<DT>(amask, base + c);
+      if (x != 0.f) f |= (x <= lowest) ? SAH_AMASK_NONZERO : (SAH_AMASK_NONZERO | SAH_AMASK_GENERAL);  // NaN: general
+    }
+  }
+  if (__ballot(f != 0)) {
+    // one atomic per wave that saw anything
+    for (int m = 32; m >= 1; m >>= 1) f |= __shfl_xor(f, m);
+    if ((threadIdx.x & (SAH_WAVE - 1)) == 0) atomicOr(flags, f);
+  }
+}
+
+extern "C" int sah_amask_classify(const sah_amask_classify_args* a) {
+  if (!a) return sah_fail(SAH_ENULL, "sah_amask_classify: args is NULL");
+  if (!a->amask || !a->flags) return sah_fail(SAH_ENULL, "sah_amask_classify: amask / flags is NULL");
+  if (a->B <= 0 || a->Hm <= 0 || a->Lq <= 0 || a->Lk <= 0) return sah_fail(SAH_EINVAL, "sah_amask_classify: B, Hm, Lq, Lk must be > 0");
+  const int64_t rows = (int64_t)a->B * a->Hm * a->Lq;
+  if (rows > 65535) return sah_fail(SAH_ESHAPE, "sah_amask_classify: %lld mask rows exceed 65535", (long long)rows);
+  const dim3 g((unsigned)((a->Lk + AMC_NT * AMC_PER_THREAD - 1) / (AMC_NT * AMC_PER_THREAD)), (unsigned)rows), blk(AMC_NT);
+  hipStream_t st = (hipStream_t)a->stream;
+  sah_timed timed("k_amask_classify", a->stream);
+  // "as low as the lowest finite value of the dtype" (what HuggingFace's masks put on a hidden column) or -inf
+  switch (a->dtype) {
+    case SAH_F32:
+      hipLaunchKernelGGL(k_amask_classify<SAH_F32>, g, blk, 0, st, a->amask, a->ms_b, a->ms_h, a->ms_l, a->Hm, a->Lq, a->Lk,
+                         -3.4028234663852886e38f, a->flags);
+      break;
+    case SAH_BF16:
+      hipLaunchKernelGGL(k_amask_classify<SAH_BF16>, g, blk, 0, st, a->amask, a->ms_b, a->ms_h, a->ms_l, a->Hm, a->Lq, a->Lk,
+                         -3.3895313892515355e38f, a->flags);
+      break;
+    case SAH_F16:
+      hipLaunchKernelGGL(k_amask_classify<SAH_F16>, g, blk, 0, st, a->amask, a->ms_b, a->ms_h, a->ms_l, a->Hm, a->Lq, a->Lk, -65504.0f,
+                         a->flags);
+      break;
+    default: return sah_fail(SAH_EDTYPE, "sah_amask_classify: dtype %d", a->dtype);
+  }
+  return sah_launch_status("sah_amask_classify");
+}

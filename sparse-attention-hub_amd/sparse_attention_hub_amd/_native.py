@@ -17,6 +17,9 @@ import torch
 _PKG_ROOT = Path(__file__).resolve().parent.parent  # sparse-attention-hub_amd/
 _DEFAULT_LIB = _PKG_ROOT / "lib" / "libsah_mi355.so"
 
+# SAH_VERSION of the include/sah.h the structures below were written against
+ABI_VERSION = 3
+
 SAH_F32, SAH_BF16, SAH_F16 = 0, 1, 2
 SAH_ACT = {"relu": 0, "silu": 1, "gelu": 2, "tanh": 3}
 SAH_MAX_MLP_LAYERS = 4
@@ -52,7 +55,7 @@ EXPECTED_SYMBOLS = (
     "sah_sparse_attention_static",
     "sah_attention_weights",
     "sah_run_chain",
-    "sah_hw_probe",
+    "sah_amask_classify",
 )
 
 
@@ -251,16 +254,6 @@ class AdaptiveBudgetArgs(C.Structure):
     ]
 
 
-class HwProbeArgs(C.Structure):
-    _fields_ = [
-        ("kind", C.c_int32),
-        ("src", C.c_void_p), ("bytes", C.c_int64),
-        ("dst", C.c_void_p), ("dst_bytes", C.c_int64),
-        ("iters", C.c_int32), ("workgroups", C.c_int32),
-        ("stream", C.c_void_p),
-    ]
-
-
 class AdaptiveSampleArgs(C.Structure):
     _fields_ = [
         ("rows", Rows),
@@ -354,6 +347,19 @@ class ChainArgs(C.Structure):
     ]
 
 
+class AmaskClassifyArgs(C.Structure):
+    _fields_ = [
+        ("amask", C.c_void_p), ("ms_b", C.c_int64), ("ms_h", C.c_int64), ("ms_l", C.c_int64),
+        ("dtype", C.c_int32),
+        ("B", C.c_int32), ("Hm", C.c_int32), ("Lq", C.c_int32), ("Lk", C.c_int32),
+        ("flags", C.c_void_p),
+        ("stream", C.c_void_p),
+    ]
+
+
+AMASK_NONZERO, AMASK_GENERAL = 1, 2
+
+
 class AttentionWeightsArgs(C.Structure):
     _fields_ = [
         ("rows", Rows),
@@ -371,9 +377,6 @@ class AttentionWeightsArgs(C.Structure):
 
 
 _lib: Optional[C.CDLL] = None
-# Tests that drive the kernels through a host-memory build of the library set
-# this to False; product code never does.
-REQUIRE_DEVICE_TENSORS = True
 
 
 def library_path() -> Path:
@@ -400,6 +403,11 @@ def lib() -> C.CDLL:
     if missing:
         raise NativeLibraryError(f"{path} lacks symbols {missing}; rebuild it")
     handle.sah_version.restype = C.c_int
+    found = int(handle.sah_version())
+    if found != ABI_VERSION:
+        raise NativeLibraryError(
+            f"{path} is layout generation {found} of include/sah.h, this binding is generation {ABI_VERSION}: "
+            "the argument structures would not match; rebuild the library from this tree")
     handle.sah_last_error.restype = C.c_char_p
     handle.sah_sparse_attention_work_floats.restype = C.c_int64
     handle.sah_sparse_attention_work_floats.argtypes = [C.c_int32, C.c_int32, C.c_int32]
@@ -463,7 +471,7 @@ def work_floats(n_rows: int, max_cnt: int, head_dim: int) -> int:
 
 
 def require_device(t: torch.Tensor, what: str) -> None:
-    if REQUIRE_DEVICE_TENSORS and not t.is_cuda:
+    if not t.is_cuda:
         raise NativeLibraryError(
             f"{what} is on {t.device}: the MI355X kernels need GPU tensors and there is no CPU fallback"
         )

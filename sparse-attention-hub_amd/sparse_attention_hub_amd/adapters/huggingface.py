@@ -32,7 +32,7 @@ class ModelAdapterHF:
     """Wraps a HuggingFace causal LM whose attention layers go through the attention-function registry."""
 
     def __init__(self, model: torch.nn.Module, sparse_attention_config: Optional[SparseAttentionConfig],
-                 hybrid: bool = False, drop_unpadded_decode_mask: bool = False) -> None:
+                 hybrid: bool = False) -> None:
         self.model = model
         self.sparse_attention_config = sparse_attention_config
         self._sparse_attention_available: bool = sparse_attention_config is not None
@@ -44,9 +44,6 @@ class ModelAdapterHF:
             self.sparse_attention.return_attention_weights = False
         # feed the question one token at a time (the reference does so for hybrid linear-attention models)
         self.hybrid = hybrid
-        # With unpadded sequences the additive mask of a single decode query is all zeros. Passing None
-        # instead lets the decode step take the one-call plan; only valid when no sequence is padded.
-        self.drop_unpadded_decode_mask = drop_unpadded_decode_mask
         self._registered_attention_name: Optional[str] = None
         self._custom_attention_fn: Optional[Callable] = None
 
@@ -58,8 +55,6 @@ class ModelAdapterHF:
 
     # ------------------------------------------------------------------ the attention callable
     def get_custom_attention_function(self, sparse_attention: SparseAttention) -> Callable:
-        drop_mask = self.drop_unpadded_decode_mask
-
         def custom_attention_callable(module: torch.nn.Module, queries: torch.Tensor, keys: torch.Tensor,
                                       values: torch.Tensor, attention_mask: Optional[torch.Tensor],
                                       scaling: float = 1.0, dropout: float = 0.0,
@@ -72,8 +67,6 @@ class ModelAdapterHF:
                 sparse_meta_data: Dict[Any, Any] = kwargs.pop("sparse_meta_data")
             else:
                 raise ValueError("sparse_meta_data must be provided while calling model.forward()")
-            if drop_mask and queries.shape[2] == 1:
-                attention_mask = None
             return sparse_attention.custom_attention(
                 module=module, queries=queries, keys=keys, values=values, attention_mask=attention_mask,
                 scaling=scaling, dropout=dropout, sparse_meta_data=sparse_meta_data, **kwargs,

@@ -18,7 +18,7 @@ from ... import _native
 from ...metric_logging import MicroMetricLogger
 from ..base import SparseAttention, SparseAttentionConfig
 from ..utils.mask import Mask
-from ..utils.mask_attention_utils import get_masked_attention_output, get_true_attention_output
+from ..utils.mask_attention_utils import AdditiveMaskFacts, get_masked_attention_output, get_true_attention_output
 from ..utils.native_rows import NativeRows
 from .decode_plan import DecodePlan, plan_kind
 from .maskers.base import MaskerConfig, ResearchMasker
@@ -54,6 +54,7 @@ class ResearchAttention(SparseAttention):
         self.maskers = maskers
         self._plan_kind = plan_kind(maskers)
         self._plans: Dict[Any, DecodePlan] = {}
+        self._mask_facts = AdditiveMaskFacts()
 
     def _planned_capacity(self, dims) -> Optional[int]:
         """Entries per row the whole chain can add, if every masker can tell without the device."""
@@ -81,6 +82,13 @@ class ResearchAttention(SparseAttention):
             raise ValueError("sparse_meta_data must be provided in kwargs while calling custom_attention()")
         sparse_meta_data: Dict[Any, Any] = kwargs.pop("sparse_meta_data")
 
+        if (attention_mask is not None and attention_mask.is_cuda and attention_mask.dim() == 4
+                and attention_mask.shape[-1] >= keys.shape[2] and attention_mask.dtype in (torch.float32, torch.bfloat16, torch.float16)
+                and self._mask_facts.all_zero(attention_mask)):
+            # an additive mask of zeros (HuggingFace's eager mask of an unpadded decode step) adds nothing anywhere:
+            # established once per mask tensor, i.e. once per forward pass, not per layer
+            attention_mask = None
+
         metrics = MicroMetricLogger()
         want_density = metrics.is_metric_enabled("research_attention_density")
         want_error = metrics.is_metric_enabled("research_attention_output_error")
@@ -88,9 +96,9 @@ class ResearchAttention(SparseAttention):
         if (not (want_density or want_error)  # the metrics read the finished mask: masker-by-masker path
                 and not self.return_attention_weights and attention_mask is None and self._plan_kind is not None
                 and not isinstance(kwargs.get("s_aux"), torch.Tensor) and queries.dim() == 4
-                and (queries.is_cuda or not _native.REQUIRE_DEVICE_TENSORS)
                 and not (dropout > 0.0 and module is not None and getattr(module, "training", False))):
             # decode fast path: the whole chain as one native call over cached argument blocks
+            _native.require_device(queries, "queries")
             key = (queries.device, queries.dtype, tuple(queries.shape), keys.shape[1])
             plan = self._plans.get(key)
             if plan is None:

@@ -66,6 +66,40 @@ def additive_mask_args(attention_mask: Optional[torch.Tensor], queries: torch.Te
     return am, am.data_ptr(), sb, sh, am.stride(2)
 
 
+class AdditiveMaskFacts:
+    """What the additive mask of the current forward pass holds, established once per mask tensor.
+
+    HuggingFace builds one mask per forward pass and hands the same tensor to every layer; for a single decode
+    query of an unpadded batch its eager mask is all zeros, and adding zeros to scores and logits changes nothing
+    (reference: hashattention_top_k.py:367-368, oracle_top_k.py:71-72, utils/mask_attention_utils.py:221-225).
+    `all_zero` asks the device once per tensor (one small launch and one read-back, over the mask's whole width: a
+    mask that is zero everywhere is zero on the columns of any key count) and remembers the answer for as long as
+    the same, unmodified tensor keeps arriving; the tensor is kept referenced meanwhile, so its memory cannot be
+    handed to another tensor that would then be mistaken for it."""
+
+    def __init__(self) -> None:
+        self._tensor: Optional[torch.Tensor] = None
+        self._version = -1
+        self._flags = 0
+
+    def flags(self, attention_mask: torch.Tensor) -> int:
+        am = attention_mask
+        if am is self._tensor and am._version == self._version:
+            return self._flags
+        if am.dim() != 4 or am.stride(-1) != 1 or not am.is_cuda or am.numel() == 0:
+            return N.AMASK_NONZERO | N.AMASK_GENERAL  # nothing established: every consumer reads the mask itself
+        out = torch.zeros(1, dtype=torch.int32, device=am.device)
+        N.call("sah_amask_classify", N.AmaskClassifyArgs(
+            am.data_ptr(), am.stride(0), am.stride(1), am.stride(2), N.dtype_code(am.dtype),
+            am.shape[0], am.shape[1], am.shape[2], am.shape[3], out.data_ptr(), N.stream_ptr(am.device)))
+        self._flags = int(out.item())
+        self._tensor, self._version = am, am._version
+        return self._flags
+
+    def all_zero(self, attention_mask: torch.Tensor) -> bool:
+        return self.flags(attention_mask) == 0
+
+
 def _run_attention(
     queries: torch.Tensor,
     keys: torch.Tensor,

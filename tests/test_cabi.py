@@ -3,6 +3,8 @@ import ctypes
 import os
 import re
 
+import pytest
+
 from sparse_attention_hub_amd import _native as N
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -17,7 +19,17 @@ def _declared_functions():
 def test_library_is_built_and_loads():
     assert N.library_path().exists(), "build it with python sparse-attention-hub_amd/build.py"
     lib = N.lib()
-    assert lib.sah_version() == 1
+    assert lib.sah_version() == N.ABI_VERSION == 3
+
+
+def test_a_library_of_another_layout_generation_is_refused(monkeypatch):
+    """The argument structures of another SAH_VERSION would be read past their end: the binding refuses to load."""
+    monkeypatch.setattr(N, "_lib", None)
+    monkeypatch.setattr(N, "ABI_VERSION", N.ABI_VERSION + 1)
+    with pytest.raises(N.NativeLibraryError, match="layout generation"):
+        N.lib()
+    monkeypatch.undo()
+    assert N.lib().sah_version() == N.ABI_VERSION
 
 
 def test_every_declared_symbol_is_exported_and_bound():
@@ -68,7 +80,7 @@ def test_every_entry_point_refuses_null_and_names_itself():
                "sah_hamming_scores", "sah_qk_scores", "sah_select_topk", "sah_pq_keys_absmax", "sah_pq_kmeans_assign",
                "sah_pq_kmeans_update", "sah_pq_adc_scores", "sah_sparse_attention", "sah_sparse_attention_static",
                "sah_attention_weights", "sah_adaptive_budget", "sah_adaptive_sample", "sah_hash_decode_topk",
-               "sah_hash_compact_codes", "sah_run_chain", "sah_hw_probe"]
+               "sah_hash_compact_codes", "sah_run_chain", "sah_amask_classify"]
     for fn in one_arg:
         assert getattr(lib, fn)(None) == -2, fn
         assert fn.replace("_static", "").encode() in lib.sah_last_error() or fn.encode() in lib.sah_last_error(), fn
@@ -109,14 +121,10 @@ def test_bad_argument_blocks_are_refused_with_the_documented_codes():
     assert lib.sah_select_topk(ctypes.byref(sel)) == -1
     # what the no-allocation attention refuses is more than its built-in buffer holds
     assert N.work_floats(1024, 131072, 128) > 4 * 1024 * 1024 >= N.work_floats(512, 131072, 128)
-    # the measurement aid checks its sizes before it launches anything
-    big = ctypes.create_string_buffer(1 << 16)
-    bptr = (ctypes.addressof(big) + 15) & ~15
-    probe = N.HwProbeArgs(0, bptr, 65536 + 64, bptr, 1 << 12, 0, 0, None)              # not a multiple of 64 KB
-    assert lib.sah_hw_probe(ctypes.byref(probe)) == -1
-    probe = N.HwProbeArgs(1, bptr, 1 << 20, bptr, 1 << 10, 0, 0, None)                 # dst smaller than bytes / 32
-    assert lib.sah_hw_probe(ctypes.byref(probe)) == -1 and b"dst_bytes" in lib.sah_last_error()
-    probe = N.HwProbeArgs(5, None, 0, bptr, 4, 0, 16, None)                            # no iterations
-    assert lib.sah_hw_probe(ctypes.byref(probe)) == -1
-    probe = N.HwProbeArgs(9, None, 0, bptr, 4, 1, 1, None)
-    assert lib.sah_hw_probe(ctypes.byref(probe)) == -1 and b"kind" in lib.sah_last_error()
+    # additive-mask classification: empty shape, too many rows, unknown dtype
+    amc = N.AmaskClassifyArgs(ptr, 0, 0, 0, 1, 2, 1, 1, 0, ptr, None)
+    assert lib.sah_amask_classify(ctypes.byref(amc)) == -1
+    amc = N.AmaskClassifyArgs(ptr, 0, 0, 0, 1, 70000, 1, 1, 8, ptr, None)
+    assert lib.sah_amask_classify(ctypes.byref(amc)) == -3
+    amc = N.AmaskClassifyArgs(ptr, 0, 0, 0, 1, 2, 1, 1, 8, None, None)
+    assert lib.sah_amask_classify(ctypes.byref(amc)) == -2

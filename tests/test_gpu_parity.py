@@ -1317,34 +1317,3 @@ def test_composite_sampling_stacks(cuda, base):
     oo, ow, om = O.research_attention(specs, q, k, v, None, scaling, None, state)
     assert torch.equal(w.cpu() != 0, ow != 0)
     assert rel_err(out, oo) < TOL[dtype]
-
-
-def test_hw_probe_kernels_read_what_they_are_given_and_write_where_they_say(cuda):
-    """The measurement aid `sah_hw_probe`: every kind launches; the stream kinds write exactly the 1/32 of the read
-    volume they describe (a source of equal words folds to zero: row r of kind 1 holds r, kind 2 zeros) and nothing
-    beyond it."""
-    from sparse_attention_hub_amd import _native as N
-
-    n = 1 << 20
-    src = torch.full((n,), 1, dtype=torch.uint8, device=cuda)
-    stream = N.stream_ptr(cuda)
-    for kind in (0, 1, 2):
-        dst = torch.full((n // 32 + 256,), 0xEE, dtype=torch.uint8, device=cuda)
-        N.call("sah_hw_probe", N.HwProbeArgs(kind, src.data_ptr(), n, dst.data_ptr(), n // 32, 0, 0, stream))
-        torch.cuda.synchronize()
-        out = dst.cpu()
-        assert bool((out[n // 32:] == 0xEE).all())
-        body = out[: n // 32]
-        if kind == 0:
-            assert bool((body == 0xEE).all())
-        elif kind == 1:
-            rows = body.view(torch.int16).reshape(4, -1)
-            for r in range(4):
-                assert bool((rows[r] == r).all())
-        else:
-            assert bool((body == 0).all())
-    sink = torch.zeros(4, dtype=torch.float32, device=cuda)
-    for kind in (3, 4, 5):
-        N.call("sah_hw_probe", N.HwProbeArgs(kind, None, 0, sink.data_ptr(), 16, 8, 4, stream))
-    torch.cuda.synchronize()
-    assert float(sink.abs().sum()) == 0.0

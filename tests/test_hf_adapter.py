@@ -142,10 +142,15 @@ def test_generation_loop_with_a_dense_stand_in_reproduces_the_plain_model(hybrid
 
 # --------------------------------------------------------------------------------------- GPU
 class _OracleAttention:
-    """The CPU oracle as a SparseAttention stand-in (test infrastructure): same masker chain, reference semantics."""
+    """The CPU oracle as a SparseAttention stand-in (test infrastructure): same masker chain, reference semantics.
+    `key_sig_for(layer)` seeds the layer's signature cache and `query_sig_for(layer, queries)` replaces the query MLP,
+    so that a model-level comparison can score the kernels' own signature bits (a float MLP on the host may round a
+    borderline output to the other side of zero; the MLP itself is compared bit by bit elsewhere)."""
 
-    def __init__(self, specs_for_layer):
+    def __init__(self, specs_for_layer, key_sig_for=None, query_sig_for=None):
         self.specs_for_layer = specs_for_layer
+        self.key_sig_for = key_sig_for
+        self.query_sig_for = query_sig_for
         self.state = {}
 
     def custom_attention(self, module, queries, keys, values, attention_mask, scaling, dropout, **kwargs):
@@ -154,6 +159,10 @@ class _OracleAttention:
         layer = kwargs.get("layer_idx")
         st = self.state.setdefault(layer, {})
         st.pop("query_sig", None)
+        if self.key_sig_for is not None and "key_sig" not in st:
+            st["key_sig"] = self.key_sig_for(layer)
+        if self.query_sig_for is not None:
+            st["query_sig"] = self.query_sig_for(layer, queries)
         out, _, _ = O.research_attention(self.specs_for_layer(layer), queries.cpu(), keys.cpu(), values.cpu(),
                                          None if attention_mask is None else attention_mask.cpu(), scaling, None, st)
         return out.to(queries.device), None
@@ -204,4 +213,182 @@ def test_tiny_llama_through_the_adapter_matches_the_oracle(cuda, chain):
     want = run(_adapter_with(model, _OracleAttention(specs_for)))
     for a, b in zip(ours, want):
         assert a.shape == b.shape
+        assert ((a - b).norm() / b.norm()).item() < 1e-4
+
+
+def _llama_shaped(cuda, layers=2, seed=0):
+    """A random-weight Llama with Llama-3.1-8B's attention geometry (32 query / 8 KV heads of 128) and a narrow MLP."""
+    from transformers import LlamaConfig, LlamaForCausalLM
+
+    torch.manual_seed(seed)
+    cfg = LlamaConfig(vocab_size=128, hidden_size=4096, intermediate_size=512, num_hidden_layers=layers,
+                      num_attention_heads=32, num_key_value_heads=8, head_dim=128, max_position_embeddings=16384)
+    return LlamaForCausalLM(cfg).to(torch.bfloat16).to(cuda).eval()
+
+
+def _unpack_codes(codes):
+    c = codes.cpu().long() & 0xFFFFFFFF
+    shifts = torch.arange(32)
+    pos = (c[..., 0].unsqueeze(-1) >> shifts) & 1
+    nonzero = (c[..., 1].unsqueeze(-1) >> shifts) & 1
+    return ((pos * 2 - 1) * nonzero).float()
+
+
+@pytest.mark.gpu
+def test_llama_shaped_decode_through_the_default_adapter_is_one_kernel_per_layer(cuda):
+    """What HuggingFace hands the registered callable in a decode step is the eager mask, a (B, 1, 1, Lk) tensor that
+    is all zeros when no sequence is padded (reference adapters/huggingface.py:227-275, :311-319). Through
+    ModelAdapterHF with its default arguments a bf16 Llama-shaped stack (B = 8, 32 query / 8 KV heads of 128, 8192
+    context keys, Sink + Local + HashAttention top-k) must run every decode layer-step as ONE launch of
+    k_hash_decode_attn (plus one mask classification per forward pass), give the oracle's logits when the oracle is
+    plugged into the same model, and select exactly the oracle's columns given the kernel's signatures."""
+    from oracle import reference_path as O
+    from sparse_attention_hub_amd import _native as N
+    from sparse_attention_hub_amd.adapters import ModelAdapterHF
+    from sparse_attention_hub_amd.sparse_attention import (
+        HashAttentionTopKMaskerConfig, LocalMaskerConfig, ResearchAttentionConfig, SinkMaskerConfig)
+    from sparse_attention_hub_amd.sparse_attention.utils.hashattention_utils import random_hat_weights
+
+    B, Hq, D, n_ctx, layers = 8, 32, 128, 8192, 2
+    sink, window, heavy = 128, 512, 1024
+    model = _llama_shaped(cuda, layers)
+    wts = random_hat_weights(layers, Hq, D, 32, 3, 128, dtype=torch.bfloat16, seed=5)
+    cfgs = [SinkMaskerConfig(sink_size=sink), LocalMaskerConfig(window_size=window),
+            HashAttentionTopKMaskerConfig(heavy_size=heavy, hat_bits=32, hat_mlp_layers=3, hat_mlp_hidden_size=128,
+                                          hat_mlp_activation="silu", hat_weights=wts)]
+    specs_for = lambda layer: [("sink", sink), ("local", window), ("hash_topk", heavy, wts[layer], "silu")]
+    g = torch.Generator().manual_seed(4)
+    context = torch.randint(0, 128, (B, n_ctx), generator=g).to(cuda)
+    question = torch.randint(0, 128, (B, 4), generator=g).to(cuda)
+    steps = torch.randint(0, 128, (5, B), generator=g).to(cuda)
+    n_timed = 3
+
+    def prefill(meta):
+        past = None
+        with torch.no_grad():
+            for at in range(0, n_ctx, 2048):      # the model's own attention, in pieces
+                out = model(context[:, at:at + 2048], past_key_values=past, use_cache=True, sparse_meta_data=meta)
+                past = out.past_key_values
+        return past
+
+    def run(adapter, timed):
+        meta, logits, launches = {}, [], None
+        past = prefill(meta)
+        with torch.no_grad(), adapter.enable_sparse_mode():
+            out = model(input_ids=question, past_key_values=past, use_cache=True, sparse_meta_data=meta)
+            logits.append(out.logits[:, -1].float().cpu())
+            past = out.past_key_values
+            for i, t in enumerate(steps):
+                if timed and i == len(steps) - n_timed:
+                    torch.cuda.synchronize()
+                    N.timing_enable(True)
+                out = model(input_ids=t.view(B, 1), past_key_values=past, use_cache=True, sparse_meta_data=meta)
+                logits.append(out.logits[:, -1].float().cpu())
+                past = out.past_key_values
+            if timed:
+                torch.cuda.synchronize()
+                launches = N.timing_collect()
+                N.timing_enable(False)
+        adapter._cleanup_attention_registration()
+        return logits, launches, meta
+
+    adapter = ModelAdapterHF(model, ResearchAttentionConfig(masker_configs=cfgs))      # default arguments
+    seen = {}
+    inner = adapter.sparse_attention.custom_attention
+
+    def recording(module, queries, keys, values, attention_mask, scaling, dropout, **kw):
+        seen["last"] = (kw.get("layer_idx"), queries, keys, values, attention_mask, scaling)
+        return inner(module, queries, keys, values, attention_mask, scaling, dropout, **kw)
+
+    adapter.sparse_attention.custom_attention = recording
+    ours, launches, meta = run(adapter, True)
+    assert set(launches) == {"k_hash_decode_attn", "k_amask_classify"}, launches
+    assert launches["k_hash_decode_attn"][0] == n_timed * layers and launches["k_amask_classify"][0] == n_timed, launches
+
+    # the last layer-step: what HuggingFace passed, and the columns the kernel selected for it
+    layer, q, k, v, amask, scaling = seen["last"]
+    assert layer == layers - 1 and tuple(amask.shape) == (B, 1, 1, k.shape[2]) and not bool(amask.any())
+    Lk = k.shape[2]
+    plan = next(iter(adapter.sparse_attention._plans.values()))
+    total = sink + window + heavy
+    assert bool((plan.cnt.cpu() == total).all())
+    member = torch.zeros((B * Hq, Lk), dtype=torch.bool, device=cuda)
+    member.scatter_(1, plan.cols[:, :total].long(), True)
+    member = member.cpu().view(B, Hq, Lk)
+    cache = meta["key"][layer]
+    masker = adapter.sparse_attention.maskers[2]
+    qcodes = torch.empty((B * Hq, 2), dtype=torch.int32, device=cuda)
+    masker._hash(q, Hq, Hq, 0, 1, layer, "query", qcodes, 1, 0)
+    qsig = _unpack_codes(qcodes).view(B, Hq, 1, 32)
+    for b in (0, B - 1):
+        state = {"key_sig": _unpack_codes(cache.codes[b:b + 1, :, :cache.n]), "query_sig": qsig[b:b + 1]}
+        _, _, om = O.research_attention(specs_for(layer), q[b:b + 1].cpu(), k[b:b + 1].cpu(), v[b:b + 1].cpu(),
+                                        amask[b:b + 1].cpu(), scaling, state=state)
+        assert torch.equal(member[b], om.to_dense()[0, :, 0] != 0), f"batch row {b}: selected sets differ"
+
+    # The oracle plugged into the same model, scoring the kernels' signature bits: the context keys' from the run above
+    # (the context was prefilled by the model's own attention, so its keys are the same in both runs; later keys are
+    # hashed by the oracle itself and sit inside the local window whenever they matter), the queries' from the
+    # stand-alone signature kernel.
+    ctx_sig = {l: _unpack_codes(meta["key"][l].codes[:, :, :n_ctx]) for l in range(layers)}
+
+    def query_sig(layer, queries):
+        Lq = queries.shape[2]
+        codes = torch.empty((B * Hq * Lq, 2), dtype=torch.int32, device=cuda)
+        masker._hash(queries, Hq, Hq, 0, Lq, layer, "query", codes, Lq, 0)
+        return _unpack_codes(codes).view(B, Hq, Lq, 32)
+
+    want, _, _ = run(_adapter_with(model, _OracleAttention(specs_for, ctx_sig.get, query_sig)), False)
+    for a, b in zip(ours, want):
+        assert a.shape == b.shape
+        assert ((a - b).norm() / b.norm()).item() < 2e-2
+
+
+@pytest.mark.gpu
+def test_padded_batch_decode_through_the_default_adapter_matches_the_oracle(cuda):
+    """A left-padded batch: the eager mask hides the padding columns with finfo.min, so it is not all zeros and must
+    be honoured by the top-k scores and by the attention logits (hashattention_top_k.py:367-368,
+    utils/mask_attention_utils.py:221-225)."""
+    from sparse_attention_hub_amd.adapters import ModelAdapterHF
+    from sparse_attention_hub_amd.sparse_attention import (
+        LocalMaskerConfig, OracleTopKConfig, ResearchAttentionConfig, SinkMaskerConfig)
+
+    model = _tiny_llama(torch.float32).to(cuda)
+    cfgs = [SinkMaskerConfig(sink_size=4), LocalMaskerConfig(window_size=8), OracleTopKConfig(heavy_size=12)]
+    specs_for = lambda layer: [("sink", 4), ("local", 8), ("oracle_topk", 12)]
+    g = torch.Generator().manual_seed(6)
+    B, n_ctx, pad = 2, 60, 9
+    context = torch.randint(0, 96, (B, n_ctx), generator=g).to(cuda)
+    amask = torch.ones(B, n_ctx, dtype=torch.long, device=cuda)
+    amask[1, :pad] = 0                                                 # row 1 starts with 9 padding tokens
+    steps = torch.randint(0, 96, (3, B), generator=g).to(cuda)
+    seen = []
+
+    def run(adapter, record):
+        meta, logits, am = {}, [], amask
+        with torch.no_grad():
+            ctx = model(context, attention_mask=am, past_key_values=None, use_cache=True, sparse_meta_data=meta)
+            past = ctx.past_key_values
+            with adapter.enable_sparse_mode():
+                for t in steps:
+                    am = torch.cat([am, torch.ones(B, 1, dtype=torch.long, device=cuda)], dim=1)
+                    out = model(input_ids=t.view(B, 1), attention_mask=am, past_key_values=past, use_cache=True,
+                                sparse_meta_data=meta)
+                    logits.append(out.logits[:, -1].float().cpu())
+                    past = out.past_key_values
+        adapter._cleanup_attention_registration()
+        return logits
+
+    adapter = ModelAdapterHF(model, ResearchAttentionConfig(masker_configs=cfgs))
+    inner = adapter.sparse_attention.custom_attention
+
+    def recording(module, queries, keys, values, attention_mask, scaling, dropout, **kw):
+        seen.append(attention_mask)
+        return inner(module, queries, keys, values, attention_mask, scaling, dropout, **kw)
+
+    adapter.sparse_attention.custom_attention = recording
+    ours = run(adapter, True)
+    assert all(m is not None and float(m[1, 0, 0, :pad].max()) < -1e30 and not bool(m[0].any()) for m in seen)
+    want = run(_adapter_with(model, _OracleAttention(specs_for)), False)
+    for a, b in zip(ours, want):
         assert ((a - b).norm() / b.norm()).item() < 1e-4
