@@ -12,7 +12,9 @@
 #include "sah_common.h"
 
 #define PQ_NT 256
-#define PQ_MAX_D 17  // 16 plus the extra coordinate of inner-product search done as L2 search
+#define PQ_MAX_D 17  // widest sub-vector of the kernels that keep a key in registers: 16 plus the extra coordinate of
+                     // inner-product search done as L2 search; wider sub-vectors (up to PQM_MAX_D) take the matrix-core
+                     // assignment and the one-centre-per-thread quantisation
 #define PQ_MAX_CENT 256
 #define PQ_TILES 8  // key tiles of PQ_NT per workgroup
 
@@ -293,18 +295,25 @@ __global__ __launch_bounds__(PQB_NT) void k_pq_assign_block(pq_assign_params P) 
 #define PQM_NT 256
 #define PQM_NW (PQM_NT / SAH_WAVE)
 #define PQM_KEY_TILES 16  // 32-key tiles per wave and workgroup: 2048 keys per workgroup
+#define PQM_MAX_D 128     // widest sub-vector of the matrix-core assignment (64 k-steps)
+#define PQM_FUSED_LDS (80 * 1024)  // operands + sums up to this much LDS: sums in the same kernel, two workgroups a CU
+
+// LDS of the assignment kernel: A operands, centre norms and, when the sums are fused, the fixed-point sums and counts
+static size_t pqm_lds_bytes(int n_cent, int d_sub, int ks, bool sums) {
+  const size_t n_tiles = (size_t)(n_cent + 31) / 32;
+  size_t bytes = n_tiles * 64 * ks * 4 + n_tiles * 32 * 4;
+  if (sums) bytes += (size_t)n_cent * d_sub * 8 + (size_t)n_cent * 4;
+  return bytes;
+}
 
 // (two waves per SIMD at least: with at most 256 registers a wave the compiler keeps the accumulators in ordinary
 // vector registers, which the minimum search reads directly)
-template <int DT, int KS>  // KS = d_sub / 2 k-steps
+// KS k-steps of two dimensions each: sub-vectors of up to 2 KS dimensions (the operands beyond d_sub are zero).
+// SUMS: the per-centre sums of the update step are accumulated here (P.sums given and the LDS holds them).
+template <int DT, int KS, bool SUMS>
 __global__ __launch_bounds__(PQM_NT, 2) void k_pq_assign_mfma(pq_assign_params P) {
-  constexpr int DS = 2 * KS;
-  __shared__ __attribute__((aligned(16))) float s_a[(PQ_MAX_CENT / 32) * 2 * 32 * KS];  // -2 c, [tile][g][i][s]
-  __shared__ __attribute__((aligned(16))) float s_cn[(PQ_MAX_CENT / 32) * 2 * 16];      // ||c||^2, [tile][g][v]
-  __shared__ long long s_sum[PQ_MAX_CENT * DS];
-  __shared__ int s_cnt[PQ_MAX_CENT];
+  HIP_DYNAMIC_SHARED(unsigned char, pqm_dyn)
   if (P.skip_flag && *P.skip_flag) return;
-  const float sum_scale = P.sums ? pq_sum_scale(*P.absmax_bits) : 1.f;
   const int tid = threadIdx.x;
   const int lane = tid & (SAH_WAVE - 1);
   const int wave = sah_wave_id();
@@ -315,14 +324,23 @@ __global__ __launch_bounds__(PQM_NT, 2) void k_pq_assign_mfma(pq_assign_params P
   const int hk = bh % P.Hkv;
   const int b = bh / P.Hkv;
   const int grp = bh * P.n_sub + s_idx;
-  const int n_cent = P.n_cent;
+  const int n_cent = P.n_cent, d_sub = P.d_sub;
   const int n_tiles = (n_cent + 31) >> 5;
-  const float* cbase = P.centres + (int64_t)grp * n_cent * DS;
+  const float* cbase = P.centres + (int64_t)grp * n_cent * d_sub;
+  // -2 c as the A operand: element (k-step s, half g, centre row i of tile t). Four k-steps of a row sit together
+  // and consecutive rows follow each other, so that a wave's 16-byte reads are conflict-free whatever KS is.
+  float* s_a = (float*)pqm_dyn;                                    // [tile][g][s / 4][i][s % 4]   (KS = 2: [tile][g][i][s])
+  float* s_cn = s_a + (size_t)n_tiles * 64 * KS;                   // ||c||^2, [tile][g][v]
+  long long* s_sum = (long long*)(s_cn + (size_t)n_tiles * 32);    // [centre][d]      (SUMS only; 8-byte aligned: both
+  int* s_cnt = (int*)(s_sum + (size_t)n_cent * d_sub);             // [centre]          sizes above are multiples of 8)
+  const float sum_scale = SUMS ? pq_sum_scale(*P.absmax_bits) : 1.f;
+  constexpr int SQ = KS >= 4 ? 4 : KS;  // k-steps per 16-byte (8-byte) group
 
-  for (int idx = tid; idx < n_tiles * 2 * 32 * KS; idx += PQM_NT) {
-    const int s = idx % KS, i = (idx / KS) & 31, gg = (idx / (KS * 32)) & 1, t = idx / (KS * 64);
-    const int c = t * 32 + i;
-    s_a[idx] = c < n_cent ? -2.0f * cbase[c * DS + 2 * s + gg] : 0.f;
+  for (int idx = tid; idx < n_tiles * 64 * KS; idx += PQM_NT) {
+    const int s4 = idx % SQ, i = (idx / SQ) & 31, q = (idx / (SQ * 32)) % (KS / SQ), gg = (idx / (SQ * 32 * (KS / SQ))) & 1,
+              t = idx / (64 * KS);
+    const int c = t * 32 + i, d = 2 * (q * SQ + s4) + gg;
+    s_a[idx] = (c < n_cent && d < d_sub) ? -2.0f * cbase[c * d_sub + d] : 0.f;
   }
   for (int idx = tid; idx < n_tiles * 32; idx += PQM_NT) {
     const int v = idx & 15, gg = (idx >> 4) & 1, t = idx >> 5;
@@ -330,17 +348,17 @@ __global__ __launch_bounds__(PQM_NT, 2) void k_pq_assign_mfma(pq_assign_params P
     float nn = INFINITY;  // centres beyond n_cent never win
     if (c < n_cent) {
       nn = 0.f;
-      for (int d = 0; d < DS; ++d) nn = fmaf(cbase[c * DS + d], cbase[c * DS + d], nn);
+      for (int d = 0; d < d_sub; ++d) nn = fmaf(cbase[c * d_sub + d], cbase[c * d_sub + d], nn);
     }
     s_cn[idx] = nn;
   }
-  if (P.sums) {
-    for (int i = tid; i < n_cent * DS; i += PQM_NT) s_sum[i] = 0;
+  if (SUMS) {
+    for (int i = tid; i < n_cent * d_sub; i += PQM_NT) s_sum[i] = 0;
     for (int i = tid; i < n_cent; i += PQM_NT) s_cnt[i] = 0;
   }
   __syncthreads();
 
-  const int64_t kbase = (int64_t)b * P.ks_b + (int64_t)hk * P.ks_h + (int64_t)s_idx * DS;
+  const int64_t kbase = (int64_t)b * P.ks_b + (int64_t)hk * P.ks_h + (int64_t)s_idx * d_sub;
   for (int kt = 0; kt < PQM_KEY_TILES; ++kt) {
     const int n0 = ((tg * PQM_KEY_TILES + kt) * PQM_NW + wave) * 32;
     if (n0 >= P.n_keys) break;  // uniform across the wave
@@ -349,7 +367,7 @@ __global__ __launch_bounds__(PQM_NT, 2) void k_pq_assign_mfma(pq_assign_params P
     const int64_t off = kbase + (int64_t)(P.key_offset + (valid ? n : P.n_keys - 1)) * P.ks_l;
     float xs[KS];  // this lane's dims 2 s + g of its key
 #pragma unroll
-    for (int s = 0; s < KS; ++s) xs[s] = sah_load<DT>(P.k, off + 2 * s + g);
+    for (int s = 0; s < KS; ++s) xs[s] = (2 * s + g < d_sub) ? sah_load<DT>(P.k, off + 2 * s + g) : 0.f;
     float best = INFINITY;
     int bidx = 0;
     // accumulator of centre tile t: seeded with the norms, then the KS matrix instructions
@@ -360,9 +378,21 @@ __global__ __launch_bounds__(PQM_NT, 2) void k_pq_assign_mfma(pq_assign_params P
         const float4 c4 = cn4[q4];
         acc[4 * q4] = c4.x; acc[4 * q4 + 1] = c4.y; acc[4 * q4 + 2] = c4.z; acc[4 * q4 + 3] = c4.w;
       }
-      const float* ap = s_a + ((t * 2 + g) * 32 + j) * KS;
+      if constexpr (KS >= 4) {
+        const float4* ap = (const float4*)(s_a + (size_t)(t * 2 + g) * 32 * KS) + j;
 #pragma unroll
-      for (int s = 0; s < KS; ++s) acc = sah_mfma_32x32x2_f32(ap[s], xs[s], acc);
+        for (int q = 0; q < KS / 4; ++q) {
+          const float4 a4 = ap[q * 32];
+          acc = sah_mfma_32x32x2_f32(a4.x, xs[4 * q], acc);
+          acc = sah_mfma_32x32x2_f32(a4.y, xs[4 * q + 1], acc);
+          acc = sah_mfma_32x32x2_f32(a4.z, xs[4 * q + 2], acc);
+          acc = sah_mfma_32x32x2_f32(a4.w, xs[4 * q + 3], acc);
+        }
+      } else {
+        const float* ap = s_a + ((t * 2 + g) * 32 + j) * KS;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) acc = sah_mfma_32x32x2_f32(ap[s], xs[s], acc);
+      }
     };
     // the tile's first minimum and its accumulator slot (constants), then one comparison with the best so far:
     // bidx holds 16 t + slot until the end
@@ -408,37 +438,107 @@ __global__ __launch_bounds__(PQM_NT, 2) void k_pq_assign_mfma(pq_assign_params P
     }
     if (valid) {
       if (g == 0) P.codes[(((int64_t)bh * P.code_pitch) + P.code_offset + n) * P.n_sub + s_idx] = (uint8_t)bidx;
-      if (P.sums) {
+      if (SUMS) {
 #pragma unroll
-        for (int s = 0; s < KS; ++s) pq_sum_add(&s_sum[bidx * DS + 2 * s + g], xs[s], sum_scale);
+        for (int s = 0; s < KS; ++s)
+          if (2 * s + g < d_sub) pq_sum_add(&s_sum[bidx * d_sub + 2 * s + g], xs[s], sum_scale);
         if (g == 0) atomicAdd(&s_cnt[bidx], 1);
       }
     }
   }
-  if (!P.sums) return;
+  if (!SUMS) return;
   __syncthreads();
   for (int c = tid; c < n_cent; c += PQM_NT) {
     const int cn = s_cnt[c];
     if (cn) {
       atomicAdd(&P.counts[(int64_t)grp * n_cent + c], cn);
-      for (int d = 0; d < DS; ++d)
-        atomicAdd((unsigned long long*)&P.sums[(int64_t)grp * n_cent * DS + c * DS + d], (unsigned long long)s_sum[c * DS + d]);
+      for (int d = 0; d < d_sub; ++d)
+        atomicAdd((unsigned long long*)&P.sums[(int64_t)grp * n_cent * d_sub + c * d_sub + d], (unsigned long long)s_sum[c * d_sub + d]);
     }
   }
 }
 
+// Per-centre sums and counts from the codes an assignment wrote, for shapes whose sums do not fit beside the
+// assignment's operands in LDS. One workgroup takes 2048 keys of a group; consecutive threads take consecutive
+// dimensions of a key, so their LDS atomics fall into consecutive words of one centre's row.
+#define PQS_NT 1024
+#define PQS_KEYS 2048
 template <int DT>
-static int pq_launch_mfma(const sah_pq_assign_args* a, const pq_assign_params& P) {
+__global__ __launch_bounds__(PQS_NT) void k_pq_sums(pq_assign_params P) {
+  HIP_DYNAMIC_SHARED(unsigned char, pqs_dyn)
+  if (P.skip_flag && *P.skip_flag) return;
+  const int tid = threadIdx.x;
+  const int s_idx = blockIdx.x % P.n_sub;
+  const int tg = blockIdx.x / P.n_sub;
+  const int bh = blockIdx.y;
+  const int hk = bh % P.Hkv;
+  const int b = bh / P.Hkv;
+  const int grp = bh * P.n_sub + s_idx;
+  const int n_cent = P.n_cent, d_sub = P.d_sub;
+  long long* s_sum = (long long*)pqs_dyn;
+  int* s_cnt = (int*)(s_sum + (size_t)n_cent * d_sub);
+  const float sum_scale = pq_sum_scale(*P.absmax_bits);
+  for (int i = tid; i < n_cent * d_sub; i += PQS_NT) s_sum[i] = 0;
+  for (int i = tid; i < n_cent; i += PQS_NT) s_cnt[i] = 0;
+  __syncthreads();
+  const int first = tg * PQS_KEYS;
+  const int count = P.n_keys - first < PQS_KEYS ? P.n_keys - first : PQS_KEYS;
+  const int64_t kbase = (int64_t)b * P.ks_b + (int64_t)hk * P.ks_h + (int64_t)s_idx * d_sub;
+  for (int idx = tid; idx < count * d_sub; idx += PQS_NT) {
+    const int n = first + idx / d_sub, d = idx % d_sub;
+    const int code = P.codes[(((int64_t)bh * P.code_pitch) + P.code_offset + n) * P.n_sub + s_idx];
+    pq_sum_add(&s_sum[code * d_sub + d], sah_load<DT>(P.k, kbase + (int64_t)(P.key_offset + n) * P.ks_l + d), sum_scale);
+    if (d == 0) atomicAdd(&s_cnt[code], 1);
+  }
+  __syncthreads();
+  for (int i = tid; i < n_cent * d_sub; i += PQS_NT) {
+    const int c = i / d_sub;
+    if (s_cnt[c]) atomicAdd((unsigned long long*)&P.sums[(int64_t)grp * n_cent * d_sub + i], (unsigned long long)s_sum[i]);
+  }
+  for (int c = tid; c < n_cent; c += PQS_NT)
+    if (s_cnt[c]) atomicAdd(&P.counts[(int64_t)grp * n_cent + c], s_cnt[c]);
+}
+
+template <int DT, int KS>
+static int pq_launch_mfma_ks(const sah_pq_assign_args* a, const pq_assign_params& P, bool fused, size_t lds) {
   const int per_wg = PQM_NW * 32 * PQM_KEY_TILES;
   dim3 g(((a->n_keys + per_wg - 1) / per_wg) * a->n_sub, a->B * a->Hkv), blk(PQM_NT);
   hipStream_t st = (hipStream_t)a->stream;
   sah_timed timed("k_pq_assign_mfma", a->stream);
-  switch (a->d_sub) {
-    case 4: hipLaunchKernelGGL((k_pq_assign_mfma<DT, 2>), g, blk, 0, st, P); break;
-    case 8: hipLaunchKernelGGL((k_pq_assign_mfma<DT, 4>), g, blk, 0, st, P); break;
-    default: hipLaunchKernelGGL((k_pq_assign_mfma<DT, 8>), g, blk, 0, st, P); break;
+  if (fused) {
+    if (int rc = sah_allow_lds((const void*)k_pq_assign_mfma<DT, KS, true>, 160 * 1024, "sah_pq_kmeans_assign")) return rc;
+    hipLaunchKernelGGL((k_pq_assign_mfma<DT, KS, true>), g, blk, lds, st, P);
+  } else {
+    if (int rc = sah_allow_lds((const void*)k_pq_assign_mfma<DT, KS, false>, 160 * 1024, "sah_pq_kmeans_assign")) return rc;
+    hipLaunchKernelGGL((k_pq_assign_mfma<DT, KS, false>), g, blk, lds, st, P);
   }
   return sah_launch_status("sah_pq_kmeans_assign");
+}
+
+template <int DT>
+static int pq_launch_mfma(const sah_pq_assign_args* a, const pq_assign_params& P) {
+  int ks = 2;
+  while (2 * ks < a->d_sub) ks *= 2;  // 2, 4, 8, 16, 32, 64 k-steps: sub-vectors of up to 4 ... 128 dimensions
+  const bool want_sums = a->sums != nullptr;
+  const bool fused = want_sums && pqm_lds_bytes(a->n_cent, a->d_sub, ks, true) <= PQM_FUSED_LDS;
+  const size_t lds = pqm_lds_bytes(a->n_cent, a->d_sub, ks, fused);
+  int rc;
+  switch (ks) {
+    case 2: rc = pq_launch_mfma_ks<DT, 2>(a, P, fused, lds); break;
+    case 4: rc = pq_launch_mfma_ks<DT, 4>(a, P, fused, lds); break;
+    case 8: rc = pq_launch_mfma_ks<DT, 8>(a, P, fused, lds); break;
+    case 16: rc = pq_launch_mfma_ks<DT, 16>(a, P, fused, lds); break;
+    case 32: rc = pq_launch_mfma_ks<DT, 32>(a, P, fused, lds); break;
+    default: rc = pq_launch_mfma_ks<DT, 64>(a, P, fused, lds); break;
+  }
+  if (rc || !want_sums || fused) return rc;
+  // the sums from the codes just written, in a launch of their own
+  const size_t lds_s = (size_t)a->n_cent * a->d_sub * 8 + (size_t)a->n_cent * 4;
+  if ((rc = sah_allow_lds((const void*)k_pq_sums<DT>, 160 * 1024, "sah_pq_kmeans_assign"))) return rc;
+  dim3 g(((a->n_keys + PQS_KEYS - 1) / PQS_KEYS) * a->n_sub, a->B * a->Hkv), blk(PQS_NT);
+  sah_timed timed("k_pq_sums", a->stream);
+  hipLaunchKernelGGL(k_pq_sums<DT>, g, blk, lds_s, (hipStream_t)a->stream, P);
+  return sah_launch_status("sah_pq_kmeans_assign(sums)");
 }
 
 struct pq_update_params {
@@ -850,7 +950,7 @@ static int adc_launch(const pq_adc_params& P, const void* lut, dim3 g, hipStream
 
 static int pq_check_common(const char* what, int B, int Hkv, int n_sub, int d_sub, int n_cent) {
   if (B <= 0 || Hkv <= 0 || n_sub <= 0) return sah_fail(SAH_EINVAL, "%s: bad B/Hkv/n_sub", what);
-  if (d_sub <= 0 || d_sub > PQ_MAX_D) return sah_fail(SAH_ESHAPE, "%s: d_sub %d not in [1, %d]", what, d_sub, PQ_MAX_D);
+  if (d_sub <= 0 || d_sub > PQM_MAX_D) return sah_fail(SAH_ESHAPE, "%s: d_sub %d not in [1, %d]", what, d_sub, PQM_MAX_D);
   if (n_cent <= 0 || n_cent > PQ_MAX_CENT) return sah_fail(SAH_ESHAPE, "%s: n_cent %d not in [1, %d]", what, n_cent, PQ_MAX_CENT);
   if ((int64_t)B * Hkv > 65535) return sah_fail(SAH_ESHAPE, "%s: B*Hkv > 65535", what);
   return SAH_OK;
@@ -921,18 +1021,28 @@ extern "C" int sah_pq_kmeans_assign(const sah_pq_assign_args* a) {
   P.round_dist = a->round_dist;
   P.skip_flag = a->skip_flag;
   hipStream_t st = (hipStream_t)a->stream;
-  if (!a->sums && !a->skip_flag && a->n_keys <= 32) {  // new keys of a decode step
-    dim3 gf(a->n_sub, a->B * a->Hkv, a->n_keys), blk(PQ_NT);
-    sah_timed timed("k_pq_assign_few", a->stream);
-    switch (a->dtype) {
-      case SAH_F32: hipLaunchKernelGGL(k_pq_assign_few<SAH_F32>, gf, blk, 0, st, P); break;
-      case SAH_BF16: hipLaunchKernelGGL(k_pq_assign_few<SAH_BF16>, gf, blk, 0, st, P); break;
-      case SAH_F16: hipLaunchKernelGGL(k_pq_assign_few<SAH_F16>, gf, blk, 0, st, P); break;
-      default: return sah_fail(SAH_EDTYPE, "sah_pq_kmeans_assign: dtype %d", a->dtype);
+  const bool wide = a->d_sub > PQ_MAX_D;  // no kernel keeps such a key in registers
+  if (wide && a->round_dist && a->sums)
+    return sah_fail(SAH_ESHAPE, "sah_pq_kmeans_assign: rounded distances with sums need d_sub <= %d", PQ_MAX_D);
+  if ((!a->sums && !a->skip_flag && a->n_keys <= 32) || (wide && a->round_dist)) {
+    // new keys of a decode step (or, for wide sub-vectors, any number of keys against frozen centres)
+    for (int first = 0; first < a->n_keys; first += 32768) {
+      pq_assign_params Q = P;
+      Q.key_offset += first; Q.code_offset += first;
+      Q.n_keys = a->n_keys - first < 32768 ? a->n_keys - first : 32768;
+      dim3 gf(a->n_sub, a->B * a->Hkv, Q.n_keys), blk(PQ_NT);
+      sah_timed timed("k_pq_assign_few", a->stream);
+      switch (a->dtype) {
+        case SAH_F32: hipLaunchKernelGGL(k_pq_assign_few<SAH_F32>, gf, blk, 0, st, Q); break;
+        case SAH_BF16: hipLaunchKernelGGL(k_pq_assign_few<SAH_BF16>, gf, blk, 0, st, Q); break;
+        case SAH_F16: hipLaunchKernelGGL(k_pq_assign_few<SAH_F16>, gf, blk, 0, st, Q); break;
+        default: return sah_fail(SAH_EDTYPE, "sah_pq_kmeans_assign: dtype %d", a->dtype);
+      }
+      if (int rc2 = sah_launch_status("sah_pq_kmeans_assign")) return rc2;
     }
-    return sah_launch_status("sah_pq_kmeans_assign");
+    return SAH_OK;
   }
-  if (!a->sums && !a->skip_flag && a->n_keys <= 512) {  // a block of new keys of a decode plan
+  if (!wide && !a->sums && !a->skip_flag && a->n_keys <= 512) {  // a block of new keys of a decode plan
     dim3 gb(a->n_sub, a->B * a->Hkv), blk(PQB_NT);
     sah_timed timed("k_pq_assign_block", a->stream);
     switch (a->dtype) {
@@ -943,7 +1053,7 @@ extern "C" int sah_pq_kmeans_assign(const sah_pq_assign_args* a) {
     }
     return sah_launch_status("sah_pq_kmeans_assign");
   }
-  if (!a->round_dist && a->n_keys >= 1024 && (a->d_sub == 4 || a->d_sub == 8 || a->d_sub == 16)) {
+  if (!a->round_dist && (wide || (a->n_keys >= 1024 && (a->d_sub == 4 || a->d_sub == 8 || a->d_sub == 16)))) {
     // Lloyd iterations over a whole context: the contraction goes to the matrix cores
     switch (a->dtype) {
       case SAH_F32: return pq_launch_mfma<SAH_F32>(a, P);

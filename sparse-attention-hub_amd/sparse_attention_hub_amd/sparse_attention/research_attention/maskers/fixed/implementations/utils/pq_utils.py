@@ -146,8 +146,8 @@ def kmeans_batched(
     if not 1 <= num_clusters <= 256:
         raise ValueError(f"num_clusters must be in [1, 256] (one-byte codes), got {num_clusters}")
     b, n, d = X.shape
-    if d > 17 or b > 65535:
-        raise ValueError(f"the Lloyd kernels cluster up to 65535 groups of vectors of at most 17 dimensions, got b={b}, d={d}")
+    if d > 128 or b > 65535:
+        raise ValueError(f"the Lloyd kernels cluster up to 65535 groups of vectors of at most 128 dimensions, got b={b}, d={d}")
     if cluster_centers is not None and tuple(cluster_centers.shape) != (b, num_clusters, d):
         raise ValueError(
             f"cluster_centers shape mismatch. Expected ({b}, {num_clusters}, {d}), got {tuple(cluster_centers.shape)}")

@@ -303,3 +303,40 @@ def test_adaptive_chain_at_131072_keys_keeps_the_denominator_guarantee(cuda, Lk,
     oo, _ = O.masked_attention(q.cpu(), k.cpu(), v.cpu(), None, None, scaling,
                                O.OMask("dense", tuple(dense.shape), torch.bfloat16, dense))
     assert rel_err(out, oo) < 2e-2
+
+
+@pytest.mark.parametrize("d,k", [(24, 64), (64, 64), (100, 16), (128, 256)])
+def test_kmeans_batched_on_wide_vectors_matches_the_oracle(cuda, d, k):
+    """`kmeans_batched` (pq_utils.py:260-438) on vectors wider than the 16 dimensions of the headline geometry: the
+    matrix-core assignment pads the contraction to the next of 32 / 64 / 128 dimensions, and 256 centres of 128
+    dimensions take their sums in a launch of their own. Three Lloyd steps from shared start centres against the
+    oracle; keys whose two nearest centres are (nearly) equally far may take the other one."""
+    from sparse_attention_hub_amd.sparse_attention.research_attention.maskers.fixed.implementations.utils.pq_utils import (
+        kmeans_batched,
+    )
+
+    b, n = 3, 3000
+    g = torch.Generator().manual_seed(60 + d)
+    X = torch.randn(b, n, d, generator=g) + 2.0 * torch.randn(b, 1, d, generator=g)
+    start = torch.stack([X[i, torch.randperm(n, generator=g)[:k]] for i in range(b)])
+    centres_in = start
+    for _ in range(3):                      # every step starts from the ORACLE's centres, so a disagreement cannot compound
+        codes_o, cent_o = O.kmeans_lloyd(X, centres_in, 1)
+        choice, centres = kmeans_batched(X.to(cuda), k, cluster_centers=centres_in.to(cuda), iter_limit=1)
+        assert choice.shape == (b, n) and choice.dtype == torch.int64 and centres.shape == (b, k, d)
+        got = choice.cpu()
+        same = got == codes_o
+        assert same.float().mean().item() >= 0.995, same.float().mean().item()
+        g_i, n_i = torch.nonzero(~same, as_tuple=True)
+        if g_i.numel():                      # where they differ, the two centres are (nearly) equally far from the vector
+            x = X[g_i, n_i]
+            da = ((x - centres_in[g_i, got[g_i, n_i]]) ** 2).sum(-1)
+            db = ((x - centres_in[g_i, codes_o[g_i, n_i]]) ** 2).sum(-1)
+            assert bool(((da - db).abs() <= 1e-3 * torch.maximum(da, db) + 1e-5).all())
+        agree = torch.ones(b, k, dtype=torch.bool)
+        for gi in range(b):
+            bad = torch.cat([got[gi][~same[gi]], codes_o[gi][~same[gi]]])
+            agree[gi, bad] = False
+        assert agree.float().mean().item() > 0.9
+        assert torch.allclose(centres.cpu()[agree], cent_o.float()[agree], rtol=1e-4, atol=1e-4)
+        centres_in = cent_o.float()

@@ -291,7 +291,10 @@ def test_hash_signatures_bits_and_cache_growth(cuda):
             masker._update_key_signatures(kc[:, :, :100].contiguous(), Hq, meta, 0)
 
 
-@pytest.mark.parametrize("geometry", [(64, 8), (128, 16)])   # (head_dim, sub-spaces); 16 one-byte codes = one 16-byte load
+# (head_dim, sub-spaces, bits). 16 one-byte codes = one 16-byte load; (128, 2 | 4) with 4 / 6 / 8 bits are the geometries
+# the reference's own PQCache configurations use (sub-vectors of 64 and 32: docs/baselines/pqcache.md:17-25,
+# benchmark/raytune/config_builders/pqcache.py:51-67); 256 centres of 64 dimensions take their sums in a launch of their own
+@pytest.mark.parametrize("geometry", [(64, 8, 4), (128, 16, 4), (128, 2, 6), (128, 4, 6), (128, 4, 4), (128, 2, 8)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_pq_chain_cold_and_warm(cuda, dtype, geometry):
     sa = _sa()
@@ -299,9 +302,9 @@ def test_pq_chain_cold_and_warm(cuda, dtype, geometry):
         gather_sub_vectors, seeded_initial_centres,
     )
 
-    D, n_sub = geometry
+    D, n_sub, bits = geometry
     B, Hq, Hkv, Lk = 2, 8, 2, 1200
-    bits, off, iters, heavy = 4, 16, 5, 64
+    off, iters, heavy = 16, 5, 64
     n_cent = 2 ** bits
     q, k, v = make_qkv(B, Hq, Hkv, 1, Lk, D, dtype, outliers=True)
     cfg = sa.PQCacheConfig(heavy_size=heavy, pq_group_factor=n_sub, pq_bits=bits, kmeans_iter=iters, init_offset=off,
@@ -438,7 +441,7 @@ def test_missing_sparse_meta_data_and_layer_idx_raise(cuda):
         ra.custom_attention(None, q.to(cuda), k.to(cuda), v.to(cuda), None, 1.0, 0.0, sparse_meta_data={})
 
 
-@pytest.mark.parametrize("kind", ["fixed", "hash", "oracle", "pq"])
+@pytest.mark.parametrize("kind", ["fixed", "hash", "oracle", "pq", "pq_wide"])
 def test_decode_plan_matches_masker_by_masker_path(cuda, kind):
     """The one-call decode plan (weights not requested) gives bit-identical outputs to the general
     masker-by-masker path over several appended-key steps, and really is the path taken."""
@@ -454,6 +457,8 @@ def test_decode_plan_matches_masker_by_masker_path(cuda, kind):
         cfgs.append(sa.OracleTopKConfig(heavy_size=0.05))
     elif kind == "pq":
         cfgs.append(sa.PQCacheConfig(heavy_size=64, pq_group_factor=16, pq_bits=6, kmeans_iter=4, init_offset=16, metric="euclidean"))
+    elif kind == "pq_wide":      # the reference's own geometry: two sub-vectors of 64
+        cfgs.append(sa.PQCacheConfig(heavy_size=64, pq_group_factor=2, pq_bits=6, kmeans_iter=4, init_offset=16, metric="euclidean"))
     fast = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=cfgs))
     fast.return_attention_weights = False
     ref = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=cfgs))
@@ -466,7 +471,7 @@ def test_decode_plan_matches_masker_by_masker_path(cuda, kind):
         n = Lk + step
         qq = make_qkv(B, Hq, Hkv, 1, 1, D, dtype, seed=50 + step)[0].to(cuda)
         o1, w1 = fast.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m1, layer_idx=0)
-        if kind == "pq" and step == 0:
+        if kind.startswith("pq") and step == 0:
             # Both instances would take the general path here and cluster the keys; the Lloyd sums use floating-point
             # atomics, so two clusterings may differ in a last bit. The comparison is about the steps after it: the
             # second instance starts from a copy of the first one's codebook.
@@ -512,7 +517,8 @@ def test_decode_plan_hashes_new_keys_in_blocks(cuda):
     assert torch.equal(c1.codes[:, :, : c1.n], c2.codes[:, :, : c1.n])
 
 
-def test_decode_plan_quantises_new_keys_in_blocks(cuda):
+@pytest.mark.parametrize("n_sub", [16, 4])
+def test_decode_plan_quantises_new_keys_in_blocks(cuda, n_sub):
     """PQCache decode through the plan: keys still inside the local window are quantised a block at a time (one
     launch every `window` steps here), and the scoring pass covers the quantised keys only. Over enough steps for
     such keys to leave the window and compete, every output equals the masker-by-masker path's, which quantises one
@@ -523,7 +529,7 @@ def test_decode_plan_quantises_new_keys_in_blocks(cuda):
     steps, window, off = 40, 16, 8
     q, k, v = make_qkv(B, Hq, Hkv, 1, Lk + steps, D, dtype, outliers=True, seed=13)
     cfgs = [sa.SinkMaskerConfig(sink_size=off), sa.LocalMaskerConfig(window_size=window),
-            sa.PQCacheConfig(heavy_size=100, pq_group_factor=16, pq_bits=6, kmeans_iter=3, init_offset=off, metric="euclidean")]
+            sa.PQCacheConfig(heavy_size=100, pq_group_factor=n_sub, pq_bits=6, kmeans_iter=3, init_offset=off, metric="euclidean")]
     fast = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=cfgs))
     fast.return_attention_weights = False
     ref = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=cfgs))
