@@ -463,8 +463,10 @@ __global__ __launch_bounds__(PQM_NT, 2) void k_pq_assign_mfma(pq_assign_params P
 // dimensions of a key, so their LDS atomics fall into consecutive words of one centre's row.
 #define PQS_NT 1024
 #define PQS_KEYS 2048
+#define PQS_MAX_SUMS 16384  // fixed-point sums a workgroup keeps in LDS (128 KB): wider groups are split by dimension
+// grid.z splits the dimensions into slices of d_chunk; slice 0 also counts the members
 template <int DT>
-__global__ __launch_bounds__(PQS_NT) void k_pq_sums(pq_assign_params P) {
+__global__ __launch_bounds__(PQS_NT) void k_pq_sums(pq_assign_params P, int d_chunk) {
   HIP_DYNAMIC_SHARED(unsigned char, pqs_dyn)
   if (P.skip_flag && *P.skip_flag) return;
   const int tid = threadIdx.x;
@@ -475,28 +477,32 @@ __global__ __launch_bounds__(PQS_NT) void k_pq_sums(pq_assign_params P) {
   const int b = bh / P.Hkv;
   const int grp = bh * P.n_sub + s_idx;
   const int n_cent = P.n_cent, d_sub = P.d_sub;
-  long long* s_sum = (long long*)pqs_dyn;
-  int* s_cnt = (int*)(s_sum + (size_t)n_cent * d_sub);
+  const int d0 = blockIdx.z * d_chunk;
+  const int dn = d_sub - d0 < d_chunk ? d_sub - d0 : d_chunk;
+  long long* s_sum = (long long*)pqs_dyn;                  // [centre][dn]
+  int* s_cnt = (int*)(s_sum + (size_t)n_cent * d_chunk);
   const float sum_scale = pq_sum_scale(*P.absmax_bits);
-  for (int i = tid; i < n_cent * d_sub; i += PQS_NT) s_sum[i] = 0;
+  for (int i = tid; i < n_cent * dn; i += PQS_NT) s_sum[i] = 0;
   for (int i = tid; i < n_cent; i += PQS_NT) s_cnt[i] = 0;
   __syncthreads();
   const int first = tg * PQS_KEYS;
   const int count = P.n_keys - first < PQS_KEYS ? P.n_keys - first : PQS_KEYS;
-  const int64_t kbase = (int64_t)b * P.ks_b + (int64_t)hk * P.ks_h + (int64_t)s_idx * d_sub;
-  for (int idx = tid; idx < count * d_sub; idx += PQS_NT) {
-    const int n = first + idx / d_sub, d = idx % d_sub;
+  const int64_t kbase = (int64_t)b * P.ks_b + (int64_t)hk * P.ks_h + (int64_t)s_idx * d_sub + d0;
+  for (int idx = tid; idx < count * dn; idx += PQS_NT) {
+    const int n = first + idx / dn, d = idx % dn;
     const int code = P.codes[(((int64_t)bh * P.code_pitch) + P.code_offset + n) * P.n_sub + s_idx];
-    pq_sum_add(&s_sum[code * d_sub + d], sah_load<DT>(P.k, kbase + (int64_t)(P.key_offset + n) * P.ks_l + d), sum_scale);
+    pq_sum_add(&s_sum[code * dn + d], sah_load<DT>(P.k, kbase + (int64_t)(P.key_offset + n) * P.ks_l + d), sum_scale);
     if (d == 0) atomicAdd(&s_cnt[code], 1);
   }
   __syncthreads();
-  for (int i = tid; i < n_cent * d_sub; i += PQS_NT) {
-    const int c = i / d_sub;
-    if (s_cnt[c]) atomicAdd((unsigned long long*)&P.sums[(int64_t)grp * n_cent * d_sub + i], (unsigned long long)s_sum[i]);
+  for (int i = tid; i < n_cent * dn; i += PQS_NT) {
+    const int c = i / dn, d = i % dn;
+    if (s_cnt[c])
+      atomicAdd((unsigned long long*)&P.sums[(int64_t)grp * n_cent * d_sub + c * d_sub + d0 + d], (unsigned long long)s_sum[i]);
   }
-  for (int c = tid; c < n_cent; c += PQS_NT)
-    if (s_cnt[c]) atomicAdd(&P.counts[(int64_t)grp * n_cent + c], s_cnt[c]);
+  if (blockIdx.z == 0)
+    for (int c = tid; c < n_cent; c += PQS_NT)
+      if (s_cnt[c]) atomicAdd(&P.counts[(int64_t)grp * n_cent + c], s_cnt[c]);
 }
 
 template <int DT, int KS>
@@ -533,11 +539,13 @@ static int pq_launch_mfma(const sah_pq_assign_args* a, const pq_assign_params& P
   }
   if (rc || !want_sums || fused) return rc;
   // the sums from the codes just written, in a launch of their own
-  const size_t lds_s = (size_t)a->n_cent * a->d_sub * 8 + (size_t)a->n_cent * 4;
+  int d_chunk = a->d_sub;
+  while (a->n_cent * d_chunk > PQS_MAX_SUMS) d_chunk = (d_chunk + 1) / 2;
+  const size_t lds_s = (size_t)a->n_cent * d_chunk * 8 + (size_t)a->n_cent * 4;
   if ((rc = sah_allow_lds((const void*)k_pq_sums<DT>, 160 * 1024, "sah_pq_kmeans_assign"))) return rc;
-  dim3 g(((a->n_keys + PQS_KEYS - 1) / PQS_KEYS) * a->n_sub, a->B * a->Hkv), blk(PQS_NT);
+  dim3 g(((a->n_keys + PQS_KEYS - 1) / PQS_KEYS) * a->n_sub, a->B * a->Hkv, (a->d_sub + d_chunk - 1) / d_chunk), blk(PQS_NT);
   sah_timed timed("k_pq_sums", a->stream);
-  hipLaunchKernelGGL(k_pq_sums<DT>, g, blk, lds_s, (hipStream_t)a->stream, P);
+  hipLaunchKernelGGL(k_pq_sums<DT>, g, blk, lds_s, (hipStream_t)a->stream, P, d_chunk);
   return sah_launch_status("sah_pq_kmeans_assign(sums)");
 }
 

@@ -142,15 +142,10 @@ def test_generation_loop_with_a_dense_stand_in_reproduces_the_plain_model(hybrid
 
 # --------------------------------------------------------------------------------------- GPU
 class _OracleAttention:
-    """The CPU oracle as a SparseAttention stand-in (test infrastructure): same masker chain, reference semantics.
-    `key_sig_for(layer)` seeds the layer's signature cache and `query_sig_for(layer, queries)` replaces the query MLP,
-    so that a model-level comparison can score the kernels' own signature bits (a float MLP on the host may round a
-    borderline output to the other side of zero; the MLP itself is compared bit by bit elsewhere)."""
+    """The CPU oracle as a SparseAttention stand-in (test infrastructure): same masker chain, reference semantics."""
 
-    def __init__(self, specs_for_layer, key_sig_for=None, query_sig_for=None):
+    def __init__(self, specs_for_layer):
         self.specs_for_layer = specs_for_layer
-        self.key_sig_for = key_sig_for
-        self.query_sig_for = query_sig_for
         self.state = {}
 
     def custom_attention(self, module, queries, keys, values, attention_mask, scaling, dropout, **kwargs):
@@ -159,10 +154,6 @@ class _OracleAttention:
         layer = kwargs.get("layer_idx")
         st = self.state.setdefault(layer, {})
         st.pop("query_sig", None)
-        if self.key_sig_for is not None and "key_sig" not in st:
-            st["key_sig"] = self.key_sig_for(layer)
-        if self.query_sig_for is not None:
-            st["query_sig"] = self.query_sig_for(layer, queries)
         out, _, _ = O.research_attention(self.specs_for_layer(layer), queries.cpu(), keys.cpu(), values.cpu(),
                                          None if attention_mask is None else attention_mask.cpu(), scaling, None, st)
         return out.to(queries.device), None
@@ -240,8 +231,10 @@ def test_llama_shaped_decode_through_the_default_adapter_is_one_kernel_per_layer
     is all zeros when no sequence is padded (reference adapters/huggingface.py:227-275, :311-319). Through
     ModelAdapterHF with its default arguments a bf16 Llama-shaped stack (B = 8, 32 query / 8 KV heads of 128, 8192
     context keys, Sink + Local + HashAttention top-k) must run every decode layer-step as ONE launch of
-    k_hash_decode_attn (plus one mask classification per forward pass), give the oracle's logits when the oracle is
-    plugged into the same model, and select exactly the oracle's columns given the kernel's signatures."""
+    k_hash_decode_attn (plus one mask classification per forward pass), give the oracle's attention output on the
+    tensors of every call HuggingFace makes, and select exactly the oracle's columns given the kernel's signatures.
+    (Whole-model logits of two runs are not compared: with a random model a last-bit difference in one layer's output
+    flips signature bits of the next layer's query, i.e. the comparison would be of two different selections.)"""
     from oracle import reference_path as O
     from sparse_attention_hub_amd import _native as N
     from sparse_attention_hub_amd.adapters import ModelAdapterHF
@@ -293,55 +286,50 @@ def test_llama_shaped_decode_through_the_default_adapter_is_one_kernel_per_layer
         return logits, launches, meta
 
     adapter = ModelAdapterHF(model, ResearchAttentionConfig(masker_configs=cfgs))      # default arguments
-    seen = {}
+    masker = adapter.sparse_attention.maskers[2]
+    seen = {"calls": 0, "worst": 0.0}
     inner = adapter.sparse_attention.custom_attention
 
-    def recording(module, queries, keys, values, attention_mask, scaling, dropout, **kw):
-        seen["last"] = (kw.get("layer_idx"), queries, keys, values, attention_mask, scaling)
-        return inner(module, queries, keys, values, attention_mask, scaling, dropout, **kw)
+    def checked(module, queries, keys, values, attention_mask, scaling, dropout, **kw):
+        """Every call HuggingFace makes (question pass and decode steps, both layers) against the oracle on the very
+        tensors it was given, batch rows 0 and B - 1, scoring the kernels' own signature bits (a float MLP on the host
+        may round a borderline output to the other side of zero; the MLP is compared bit by bit elsewhere)."""
+        out = inner(module, queries, keys, values, attention_mask, scaling, dropout, **kw)
+        layer, Lq = kw["layer_idx"], queries.shape[2]
+        cache = kw["sparse_meta_data"]["key"][layer]
+        qcodes = torch.empty((B * Hq * Lq, 2), dtype=torch.int32, device=cuda)
+        masker._hash(queries, Hq, Hq, 0, Lq, layer, "query", qcodes, Lq, 0)
+        qsig = _unpack_codes(qcodes).view(B, Hq, Lq, 32)
+        n = min(cache.n, keys.shape[2])       # keys hashed so far; the rest sit inside the local window
+        for b in (0, B - 1):
+            state = {"key_sig": _unpack_codes(cache.codes[b:b + 1, :, :n]), "query_sig": qsig[b:b + 1]}
+            oo, _, om = O.research_attention(specs_for(layer), queries[b:b + 1].cpu(), keys[b:b + 1].cpu(), values[b:b + 1].cpu(),
+                                             attention_mask[b:b + 1].cpu(), scaling, state=state)
+            got = out[0][b:b + 1].float().cpu()
+            seen["worst"] = max(seen["worst"], ((got - oo.float()).norm() / oo.float().norm()).item())
+            seen["last"] = (layer, b, om, attention_mask, keys.shape[2])
+        seen["calls"] += 1
+        return out
 
-    adapter.sparse_attention.custom_attention = recording
+    adapter.sparse_attention.custom_attention = checked
     ours, launches, meta = run(adapter, True)
-    assert set(launches) == {"k_hash_decode_attn", "k_amask_classify"}, launches
+    assert seen["calls"] == layers * (1 + len(steps)) and len(ours) == 1 + len(steps)
+    assert seen["worst"] < 2e-2, seen["worst"]
+    assert set(launches) - {"k_hash_sig_small_mfma", "k_hash_sig_gemv"} == {"k_hash_decode_attn", "k_amask_classify"}, launches
     assert launches["k_hash_decode_attn"][0] == n_timed * layers and launches["k_amask_classify"][0] == n_timed, launches
+    # the stand-alone signature kernel above is the check's own (the query signatures it hands the oracle)
+    assert all(launches[n][0] == n_timed * layers for n in launches if n.startswith("k_hash_sig")), launches
 
     # the last layer-step: what HuggingFace passed, and the columns the kernel selected for it
-    layer, q, k, v, amask, scaling = seen["last"]
-    assert layer == layers - 1 and tuple(amask.shape) == (B, 1, 1, k.shape[2]) and not bool(amask.any())
-    Lk = k.shape[2]
+    layer, b, om, amask, Lk = seen["last"]
+    assert layer == layers - 1 and b == B - 1 and tuple(amask.shape) == (B, 1, 1, Lk) and not bool(amask.any())
     plan = next(iter(adapter.sparse_attention._plans.values()))
     total = sink + window + heavy
     assert bool((plan.cnt.cpu() == total).all())
     member = torch.zeros((B * Hq, Lk), dtype=torch.bool, device=cuda)
     member.scatter_(1, plan.cols[:, :total].long(), True)
     member = member.cpu().view(B, Hq, Lk)
-    cache = meta["key"][layer]
-    masker = adapter.sparse_attention.maskers[2]
-    qcodes = torch.empty((B * Hq, 2), dtype=torch.int32, device=cuda)
-    masker._hash(q, Hq, Hq, 0, 1, layer, "query", qcodes, 1, 0)
-    qsig = _unpack_codes(qcodes).view(B, Hq, 1, 32)
-    for b in (0, B - 1):
-        state = {"key_sig": _unpack_codes(cache.codes[b:b + 1, :, :cache.n]), "query_sig": qsig[b:b + 1]}
-        _, _, om = O.research_attention(specs_for(layer), q[b:b + 1].cpu(), k[b:b + 1].cpu(), v[b:b + 1].cpu(),
-                                        amask[b:b + 1].cpu(), scaling, state=state)
-        assert torch.equal(member[b], om.to_dense()[0, :, 0] != 0), f"batch row {b}: selected sets differ"
-
-    # The oracle plugged into the same model, scoring the kernels' signature bits: the context keys' from the run above
-    # (the context was prefilled by the model's own attention, so its keys are the same in both runs; later keys are
-    # hashed by the oracle itself and sit inside the local window whenever they matter), the queries' from the
-    # stand-alone signature kernel.
-    ctx_sig = {l: _unpack_codes(meta["key"][l].codes[:, :, :n_ctx]) for l in range(layers)}
-
-    def query_sig(layer, queries):
-        Lq = queries.shape[2]
-        codes = torch.empty((B * Hq * Lq, 2), dtype=torch.int32, device=cuda)
-        masker._hash(queries, Hq, Hq, 0, Lq, layer, "query", codes, Lq, 0)
-        return _unpack_codes(codes).view(B, Hq, Lq, 32)
-
-    want, _, _ = run(_adapter_with(model, _OracleAttention(specs_for, ctx_sig.get, query_sig)), False)
-    for a, b in zip(ours, want):
-        assert a.shape == b.shape
-        assert ((a - b).norm() / b.norm()).item() < 2e-2
+    assert torch.equal(member[b], om.to_dense()[0, :, 0] != 0), "selected sets differ"
 
 
 @pytest.mark.gpu
