@@ -54,6 +54,11 @@ WORKLOADS = {
     5: dict(name="cfg5 Sink128+Local1024+OracleTopK2%+AdaptiveSampling(1%, eps=delta=0.05) bf16 B16 Lk131072", B=16,
             Lk=131072, dtype="bf16", sink=128, local=1024, kind="oracle", k=2621, outliers=True,
             adaptive=dict(rate=0.01, epsilon=0.05, delta=0.05)),
+    # the reference's own PQCache example (docs/baselines/pqcache.md:10-27: Sink 128 + Local 128 + PQCache 10 %, two
+    # sub-vectors of 64, 6 bits, 10 Lloyd iterations, 32K context, one query); its published 0.867 ms (unnamed CUDA GPU,
+    # docs/baselines/pqcache.md:50-61) is context, not a baseline for this hardware
+    6: dict(name="ref-docs PQCache: Sink128+Local128+PQCache(10%, group factor 2, 6 bits) bf16 B1 Lk32768", B=1, Lk=32768,
+            dtype="bf16", sink=128, local=128, kind="pq", k=3276, outliers=True, pq_group_factor=2, pq_bits=6),
 }
 HQ, HKV, D = 32, 8, 128
 SETTLE_STEPS = 256   # untimed steps before the first bracket, the W warm-up steps included
@@ -75,7 +80,7 @@ def algorithmic_bytes(w, sampled_per_row: float = 0.0) -> dict:
     qo = 2 * R * D * es
     # one 4-byte signature per (query head, key): the sign plane the decode kernel scans (the non-zero plane of the
     # two-plane cache is read only for the few keys that have a zero component)
-    scan = {"none": 0, "oracle": B * HKV * Lk * row, "hash": R * Lk * 4, "pq": B * HKV * (Lk - w["sink"]) * 16}[w["kind"]]
+    scan = {"none": 0, "oracle": B * HKV * Lk * row, "hash": R * Lk * 4, "pq": B * HKV * (Lk - w["sink"]) * w.get("pq_group_factor", 16)}[w["kind"]]
     attn = gather_topk + gather_fixed + int(R * (fixed + w["k"] + 2 * sampled_per_row) * 4) + qo
     return dict(step=gather_topk + gather_fixed + idx + qo + scan, attention_kernel=attn, scan=scan)
 
@@ -133,8 +138,8 @@ def build_workload(w, device, total_keys, host_rng=True):
         cfgs.append(HashAttentionTopKMaskerConfig(heavy_size=w["k"], hat_bits=32, hat_mlp_layers=3, hat_mlp_hidden_size=128,
                                                   hat_mlp_activation="silu", hat_weights=wts))
     elif w["kind"] == "pq":
-        cfgs.append(PQCacheConfig(heavy_size=w["k"], pq_group_factor=16, pq_bits=8, kmeans_iter=10, init_offset=w["sink"],
-                                  metric="euclidean"))
+        cfgs.append(PQCacheConfig(heavy_size=w["k"], pq_group_factor=w.get("pq_group_factor", 16), pq_bits=w.get("pq_bits", 8),
+                                  kmeans_iter=10, init_offset=w["sink"], metric="euclidean"))
     if w.get("adaptive"):
         a = w["adaptive"]
         cfgs.append(AdaptiveSamplingMaskerConfig(base_rate_sampling=a["rate"], epsilon=a["epsilon"], delta=a["delta"],

@@ -340,3 +340,147 @@ def test_kmeans_batched_on_wide_vectors_matches_the_oracle(cuda, d, k):
         assert agree.float().mean().item() > 0.9
         assert torch.allclose(centres.cpu()[agree], cent_o.float()[agree], rtol=1e-4, atol=1e-4)
         centres_in = cent_o.float()
+
+
+def _rows_membership(plan, n_keys, device):
+    member = torch.zeros((plan.n_rows, n_keys), dtype=torch.bool, device=device)
+    cnt = plan.cnt.long()
+    cols = plan.cols.long()
+    valid = torch.arange(cols.shape[1], device=device).unsqueeze(0) < cnt.unsqueeze(1)
+    member.scatter_(1, torch.where(valid, cols, cols[:, :1]), True)   # a row's first entry stands in for its unused slots
+    return member.cpu()
+
+
+def test_config1_closed_form_plan_matches_the_oracle(cuda):
+    """Headline configuration 1 at its full shape (batch 1, 32 query / 8 KV heads, 4096 keys, fp32, Sink 128 + Local 256)
+    through the decode plan: ONE launch of the attention kernel with the sink + local columns in closed form,
+    against the oracle directly, 1e-5."""
+    from sparse_attention_hub_amd import _native as N
+
+    sa = _sa()
+    B, Hq, Hkv, Lk, D = 1, 32, 8, 4096, 128
+    q, k, v = make_qkv(B, Hq, Hkv, 1, Lk, D, torch.float32, seed=0)
+    ra = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(
+        masker_configs=[sa.SinkMaskerConfig(sink_size=128), sa.LocalMaskerConfig(window_size=256)]))
+    ra.return_attention_weights = False
+    N.timing_enable(True)
+    out, w = ra.custom_attention(None, q.to(cuda), k.to(cuda), v.to(cuda), None, D ** -0.5, 0.0, sparse_meta_data={}, layer_idx=0)
+    torch.cuda.synchronize()
+    launches = N.timing_collect()
+    N.timing_enable(False)
+    assert w is None and set(launches) == {"k_sparse_attn"} and launches["k_sparse_attn"][0] == 1, launches
+    plan = next(iter(ra._plans.values()))
+    assert plan.att.closed_form == 1 and plan.att.closed_sink == 128 and plan.att.closed_window == 256
+    oo, _, _ = O.research_attention([("sink", 128), ("local", 256)], q, k, v, None, D ** -0.5)
+    assert rel_err(out, oo) < 1e-5
+
+
+def test_config2_oracle_plan_at_full_shape_matches_the_oracle(cuda):
+    """Headline configuration 2 at its full shape (batch 4, 32768 keys, bf16 with outlier channels, Sink 128 + Local 512 +
+    OracleTopK 5 %) through the decode plan (scoring pass, selection that also writes the sink / local columns,
+    attention), batch rows 0 and 3 against the oracle directly."""
+    sa = _sa()
+    B, Hq, Hkv, Lk, D = 4, 32, 8, 32768, 128
+    sink, window, heavy = 128, 512, 1638
+    dtype = torch.bfloat16
+    q, k, v = make_qkv(B, Hq, Hkv, 1, Lk, D, dtype, outliers=True, seed=71)
+    ra = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=[
+        sa.SinkMaskerConfig(sink_size=sink), sa.LocalMaskerConfig(window_size=window), sa.OracleTopKConfig(heavy_size=heavy)]))
+    ra.return_attention_weights = False
+    out, _ = ra.custom_attention(None, q.to(cuda), k.to(cuda), v.to(cuda), None, D ** -0.5, 0.0, sparse_meta_data={}, layer_idx=0)
+    torch.cuda.synchronize()
+    plan = next(iter(ra._plans.values()))
+    assert plan.kind == "oracle" and plan.att.Lk == Lk
+    total = sink + window + heavy
+    assert bool((plan.cnt.cpu() == total).all())
+    member = _rows_membership(plan, Lk, cuda).view(B, Hq, Lk)
+    specs = [("sink", sink), ("local", window), ("oracle_topk", heavy)]
+    for b in (0, B - 1):
+        oo, _, om = O.research_attention(specs, q[b:b + 1], k[b:b + 1], v[b:b + 1], None, D ** -0.5)
+        want = om.to_dense()[0, :, 0] != 0
+        # bf16 rounding of an fp32 accumulation: torch's CPU matmul may round a score on a rounding boundary the other
+        # way, which can swap two neighbours at the threshold
+        overlap = (member[b] & want).sum().item() / want.sum().item()
+        assert overlap >= 0.999, (b, overlap)
+        assert rel_err(out[b], oo[0]) < 2e-2
+
+
+def test_config4_pq_plan_at_full_shape_matches_the_oracle(cuda):
+    """Headline configuration 4 at its full shape (batch 4, 32768 keys, bf16 with outlier channels, Sink 128 + Local 256 +
+    PQCache top-1024 with 16 sub-vectors of 8 and 256 centres; 3 Lloyd iterations here): the warm step through the
+    decode plan (ADC scoring, selection that also writes the sink / local columns, attention), batch rows 0 and 3
+    against the oracle given the kernel's codebook: selected sets bit-exact."""
+    sa = _sa()
+    B, Hq, Hkv, Lk, D = 4, 32, 8, 32768, 128
+    sink, window, heavy = 128, 256, 1024
+    dtype = torch.bfloat16
+    q, k, v = make_qkv(B, Hq, Hkv, 1, Lk, D, dtype, outliers=True, seed=73)
+    q0 = make_qkv(B, Hq, Hkv, 1, 1, D, dtype, seed=74)[0]
+    ra = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=[
+        sa.SinkMaskerConfig(sink_size=sink), sa.LocalMaskerConfig(window_size=window),
+        sa.PQCacheConfig(heavy_size=heavy, pq_group_factor=16, pq_bits=8, kmeans_iter=3, init_offset=sink, metric="euclidean")]))
+    ra.return_attention_weights = False
+    meta = {}
+    kc, vc = k.to(cuda), v.to(cuda)
+    ra.custom_attention(None, q0.to(cuda), kc[:, :, :Lk - 1], vc[:, :, :Lk - 1], None, D ** -0.5, 0.0, sparse_meta_data=meta, layer_idx=0)
+    out, _ = ra.custom_attention(None, q.to(cuda), kc, vc, None, D ** -0.5, 0.0, sparse_meta_data=meta, layer_idx=0)
+    torch.cuda.synchronize()
+    plan = next(iter(ra._plans.values()))
+    assert plan.kind == "pq" and plan.att.Lk == Lk
+    total = sink + window + heavy
+    assert bool((plan.cnt.cpu() == total).all())
+    member = _rows_membership(plan, Lk, cuda).view(B, Hq, Lk)
+    book = meta["pq_codebook"][0]
+    assert book.n == Lk - 1 - sink               # the newest key sits inside the local window: quantised with the next block
+    for b in (0, B - 1):
+        cent = meta["pq_centroids"][0][b:b + 1].cpu()
+        codes = book.to_reference()[b:b + 1].cpu()
+        # the oracle scores every quantised key; the newest one is not quantised yet and lies inside the local window
+        kb, vb = k[b:b + 1], v[b:b + 1]
+        codes_full = torch.cat([codes, codes[:, -1:]], dim=1)        # a stand-in code for the window key (already active)
+        oo, _, om = O.research_attention([("sink", sink), ("local", window), ("pq_topk", heavy, sink, cent, codes_full)],
+                                         q[b:b + 1], kb, vb, None, D ** -0.5)
+        assert torch.equal(member[b], om.to_dense()[0, :, 0] != 0), f"batch row {b}: selected sets differ"
+        assert rel_err(out[b], oo[0]) < 2e-2
+
+
+@pytest.mark.parametrize("B", [4, 16])
+def test_config3_chain_at_other_batch_sizes_matches_the_oracle(cuda, B):
+    """The HashAttention decode step of configuration 3 at batch 4 (128 mask rows: fewer rows than CUs) and batch 16
+    (512 rows: two rounds of one workgroup per CU), 32768 keys: first and last batch row against the oracle given the
+    kernel's signatures, selected sets bit-exact."""
+    from sparse_attention_hub_amd.sparse_attention.utils.hashattention_utils import random_hat_weights
+
+    sa = _sa()
+    Hq, Hkv, Lk, D = 32, 8, 32768, 128
+    sink, window, heavy = 128, 512, 2048
+    dtype = torch.bfloat16
+    q, k, v = make_qkv(B, Hq, Hkv, 1, Lk, D, dtype, seed=81)
+    q0 = make_qkv(B, Hq, Hkv, 1, 1, D, dtype, seed=82)[0]
+    wts = random_hat_weights(1, Hq, D, 32, 3, 128, dtype=dtype, seed=1)
+    cfg = sa.HashAttentionTopKMaskerConfig(heavy_size=heavy, hat_bits=32, hat_mlp_layers=3, hat_mlp_hidden_size=128,
+                                           hat_mlp_activation="silu", hat_weights=wts)
+    ra = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(
+        masker_configs=[sa.SinkMaskerConfig(sink_size=sink), sa.LocalMaskerConfig(window_size=window), cfg]))
+    ra.return_attention_weights = False
+    meta = {}
+    kc, vc = k.to(cuda), v.to(cuda)
+    scaling = D ** -0.5
+    for n in (Lk - 2, Lk - 1):
+        ra.custom_attention(None, q0.to(cuda), kc[:, :, :n], vc[:, :, :n], None, scaling, 0.0, sparse_meta_data=meta, layer_idx=0)
+    out, _ = ra.custom_attention(None, q.to(cuda), kc, vc, None, scaling, 0.0, sparse_meta_data=meta, layer_idx=0)
+    torch.cuda.synchronize()
+    plan = next(iter(ra._plans.values()))
+    total = sink + window + heavy
+    assert plan.kind == "hash" and bool((plan.cnt.cpu() == total).all())
+    member = _rows_membership(plan, Lk, cuda).view(B, Hq, Lk)
+    cache = meta["key"][0]
+    qcodes = torch.empty((B * Hq, 2), dtype=torch.int32, device=cuda)
+    ra.maskers[2]._hash(q.to(cuda), Hq, Hq, 0, 1, 0, "query", qcodes, 1, 0)
+    qsig = _unpack_codes(qcodes).view(B, Hq, 1, 32)
+    specs = [("sink", sink), ("local", window), ("hash_topk", heavy, wts[0], "silu")]
+    for b in (0, B - 1):
+        state = {"key_sig": _unpack_codes(cache.codes[b:b + 1, :, :cache.n]), "query_sig": qsig[b:b + 1]}
+        oo, _, om = O.research_attention(specs, q[b:b + 1], k[b:b + 1], v[b:b + 1], None, scaling, state=state)
+        assert torch.equal(member[b], om.to_dense()[0, :, 0] != 0), f"batch row {b}: selected sets differ"
+        assert rel_err(out[b], oo[0]) < 2e-2
