@@ -133,7 +133,7 @@ def build_workload(w, device, total_keys, host_rng=True):
     if w["kind"] == "oracle":
         cfgs.append(OracleTopKConfig(heavy_size=w["k"]))
     elif w["kind"] == "hash":
-        wts = random_hat_weights(1, HQ, D, 32, 3, 128, dtype=dtype, seed=1)
+        wts = random_hat_weights(2, HQ, D, 32, 3, 128, dtype=dtype, seed=1)   # layer 1: the second cold call only
         extra["hat_weights"] = wts
         cfgs.append(HashAttentionTopKMaskerConfig(heavy_size=w["k"], hat_bits=32, hat_mlp_layers=3, hat_mlp_hidden_size=128,
                                                   hat_mlp_activation="silu", hat_weights=wts))
@@ -203,7 +203,7 @@ class Run:
             self.hf_mask = None
             self.hf_calls = 0
 
-    def step(self, i, n_keys):
+    def step(self, i, n_keys, layer=0):
         if self.hf_layers:
             if self.hf_calls % self.hf_layers == 0:
                 self.hf_mask = self.torch.zeros((self.w["B"], 1, 1, self.k.shape[2]), dtype=self.qs.dtype, device=self.dev)
@@ -211,15 +211,33 @@ class Run:
             return self.hf_fn(self.hf_module, self.qs[i % self.qs.shape[0]], self.k[:, :, :n_keys], self.v[:, :, :n_keys],
                               self.hf_mask, scaling=self.scaling, dropout=0.0, sparse_meta_data=self.meta)
         return self.ra.custom_attention(None, self.qs[i % self.qs.shape[0]], self.k[:, :, :n_keys], self.v[:, :, :n_keys], None,
-                                        self.scaling, 0.0, sparse_meta_data=self.meta, layer_idx=0)
+                                        self.scaling, 0.0, sparse_meta_data=self.meta, layer_idx=layer)
 
-    def cold(self):
+    def cold(self, second_layer=True):
+        """The first call of a layer (it hashes / clusters every key), timed on the host clock with the library's
+        per-kernel HIP events on: once for layer 0 - the process's first call, which also loads the code object,
+        creates the plan and its buffers - and once more for a second layer index on the same keys, which pays only
+        what every further layer of a model pays. Returns the two wall times and the kernel time inside each."""
+        from sparse_attention_hub_amd import _native as N
+
         torch = self.torch
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        self.step(0, self.first)
-        torch.cuda.synchronize()
-        return (time.perf_counter() - t0) * 1e3
+        out = {}
+        for name, layer in (("first_call", 0), ("next_layer_cold", 1)):
+            if layer and (not second_layer or self.hf_layers):
+                break
+            torch.cuda.synchronize()
+            N.timing_enable(True)
+            t0 = time.perf_counter()
+            self.step(0, self.first, layer)
+            torch.cuda.synchronize()
+            out[name + "_ms"] = round((time.perf_counter() - t0) * 1e3, 2)
+            kt = N.timing_collect()
+            N.timing_enable(False)
+            out[name + "_kernels_ms"] = round(sum(ms for _, ms in kt.values()), 2)
+        for per_layer in self.meta.values():       # the second layer's caches are not needed again
+            if isinstance(per_layer, dict):
+                per_layer.pop(1, None)
+        return out
 
     def timed(self):
         """(wall ms per bracket, HIP-event ms per bracket, host launch-loop ms per bracket, HIP-event ms per step over
@@ -252,7 +270,20 @@ class Run:
             gpu.append(ev0.elapsed_time(ev1))
             inner.append(evm.elapsed_time(ev1) / (self.steps - skip))
         assert n == self.w["Lk"]
+        self.last = self.last_state()
         return wall, gpu, host, inner
+
+    def last_state(self):
+        """What the parity check needs of the last timed step: output, query set, selected columns, warm-cache extent."""
+        rows = self.last_rows()
+        cache = self.meta.get("key", {}).get(0) if self.w["kind"] == "hash" else None
+        last = dict(out=self.last_out, q=self.last_q, n_hashed=getattr(cache, "n", 0),
+                    cols=None if rows is None else rows[0].clone(), cnt=None if rows is None else rows[1].clone())
+        if self.w.get("adaptive"):
+            masker = self.ra.maskers[-1]
+            last["budget"] = masker.last_budget.clone()
+            last["adaptive_call"] = masker.call_index - 1
+        return last
 
     def last_rows(self):
         """(cols int32 [R, cap], cnt int32 [R]) of the last step's mask, or None when no row list was written."""
@@ -277,8 +308,8 @@ class Run:
         return {name: dict(launches=c, avg_us=1e3 * ms / c) for name, (c, ms) in kt.items()}
 
 
-def oracle_specs(run, n_keys, n_hashed):
-    """Masker specs and warm state (one batch row) for `oracle.reference_path.research_attention`."""
+def oracle_specs(run, n_keys, n_hashed, b=0, adaptive_call=0):
+    """Masker specs and warm state (batch row `b`) for `oracle.reference_path.research_attention`."""
     w, extra, meta = run.w, run.extra, run.meta
     specs = [("sink", w["sink"]), ("local", w["local"])]
     state = {}
@@ -288,70 +319,109 @@ def oracle_specs(run, n_keys, n_hashed):
         specs.append(("hash_topk", w["k"], extra["hat_weights"][0], "silu"))
         cache = meta["key"][0]
         sub = type(cache).__new__(type(cache))            # one batch row, the keys hashed when the step ran
-        sub.bits, sub.n, sub.codes = cache.bits, n_hashed, cache.codes[:1]
+        sub.bits, sub.n, sub.codes = cache.bits, n_hashed, cache.codes[b:b + 1]
         state["key_sig"] = sub.unpack(run.qs.dtype).cpu()
     elif w["kind"] == "pq":
-        cent = meta["pq_centroids"][0][:1].cpu()
-        book = meta["pq_codebook"][0].to_reference()[:1, : n_keys - w["sink"]].cpu()
+        cent = meta["pq_centroids"][0][b:b + 1].cpu()
+        book = meta["pq_codebook"][0].to_reference()[b:b + 1, : n_keys - w["sink"]].cpu()
+        if book.shape[1] < n_keys - w["sink"]:
+            # keys not quantised yet sit inside the local window (the plan quantises them a block at a time): the
+            # oracle scores every key beyond init_offset, so they get a stand-in code; they are active already
+            pad = book[:, -1:].expand(-1, n_keys - w["sink"] - book.shape[1], -1, -1)
+            book = __import__("torch").cat([book, pad], dim=1)
         specs.append(("pq_topk", w["k"], w["sink"], cent, book))
     if w.get("adaptive"):
         a = w["adaptive"]
-        specs.append(("adaptive", a["rate"], a["epsilon"], a["delta"], w["sink"], w["local"], 0, 0))
+        # the Philox stream of the masker's call (seed 0, offset 2 x its index)
+        specs.append(("adaptive", a["rate"], a["epsilon"], a["delta"], w["sink"], w["local"], 0, 2 * adaptive_call))
     return specs, state
 
 
 def parity_and_cpu_baseline(run, last, budget_s=25.0):
-    """The reference algorithm (dense masks, repeat_kv, full-key fp32 softmax) as restated by the oracle, on ONE
-    batch row of the last timed step: first as the checker of that step's output and selected columns, then timed
-    on the host cores and scaled by the batch size (batch rows are independent). Warm caches (key signatures / PQ
+    """The reference algorithm (dense masks, repeat_kv, full-key fp32 softmax) as restated by the oracle, on single
+    batch rows of the last timed step: first as the checker of that step's output and selected columns (batch rows 0
+    and B - 1; the adaptive chain: row 0, whose mask rows carry the Philox row indices the oracle uses), then timed on
+    the host cores on row 0 and scaled by the batch size (batch rows are independent). Warm caches (key signatures / PQ
     codes) are the GPU run's, so only the layer-step is restated."""
     import torch
 
     from oracle import reference_path as O
 
     w = run.w
+    B = w["B"]
     n_keys = w["Lk"]
     cores = os.cpu_count() or 1
     torch.set_num_threads(cores)
-    q = run.qs[last["q"]][:1].cpu()
-    k = run.k[:1, :, :n_keys].cpu()
-    v = run.v[:1, :, :n_keys].cpu()
-    specs, state = oracle_specs(run, n_keys, last["n_hashed"])
-    if w["kind"] == "hash":
-        # the query's signature bits as the kernels compute them (a float MLP on the host may round a borderline
-        # output to the other side of zero)
-        qcodes = torch.empty((HQ, 2), dtype=torch.int32, device=run.dev)
-        run.ra.maskers[2]._hash(run.qs[last["q"]][:1], HQ, HQ, 0, 1, 0, "query", qcodes, 1, 0)
-        c = qcodes.cpu().to(torch.int64) & 0xFFFFFFFF
-        shifts = torch.arange(32)
-        state["query_sig"] = ((((c[:, 0:1] >> shifts) & 1) * 2 - 1) * ((c[:, 1:2] >> shifts) & 1)).to(q.dtype).view(1, HQ, 1, 32)
-    parity = None
+    adaptive = bool(w.get("adaptive"))
+    tol = 1e-5 if w["dtype"] == "f32" else 2e-2
+
+    def inputs(b):
+        q = run.qs[last["q"]][b:b + 1].cpu()
+        k = run.k[b:b + 1, :, :n_keys].cpu()
+        v = run.v[b:b + 1, :, :n_keys].cpu()
+        specs, state = oracle_specs(run, n_keys, last["n_hashed"], b, last.get("adaptive_call", 0))
+        if w["kind"] == "hash":
+            # the query's signature bits as the kernels compute them (a float MLP on the host may round a borderline
+            # output to the other side of zero)
+            qcodes = torch.empty((HQ, 2), dtype=torch.int32, device=run.dev)
+            run.ra.maskers[2]._hash(run.qs[last["q"]][b:b + 1], HQ, HQ, 0, 1, 0, "query", qcodes, 1, 0)
+            c = qcodes.cpu().to(torch.int64) & 0xFFFFFFFF
+            shifts = torch.arange(32)
+            state["query_sig"] = ((((c[:, 0:1] >> shifts) & 1) * 2 - 1) * ((c[:, 1:2] >> shifts) & 1)).to(q.dtype).view(1, HQ, 1, 32)
+        if adaptive:
+            state["budget"] = last["budget"][b * HQ:(b + 1) * HQ].long().cpu()     # the kernels' budgets: sets given the budget
+        return q, k, v, specs, state
+
+    def membership(b):
+        cols = last["cols"][b * HQ:(b + 1) * HQ].long().cpu()
+        cnt = last["cnt"][b * HQ:(b + 1) * HQ].long().cpu()
+        member = torch.zeros((HQ, n_keys), dtype=torch.bool)
+        for r in range(HQ):
+            member[r, cols[r, : cnt[r]]] = True
+        return member
+
+    rows_checked = [0] if adaptive or B == 1 else [0, B - 1]
+    worst_err, sets_equal, overlap = 0.0, True, 1.0
     times = []
-    t_all = time.perf_counter()
-    for it in range(12):
-        st = dict(state)
+    for b in rows_checked:
+        q, k, v, specs, state = inputs(b)
         t0 = time.perf_counter()
-        oo, _, om = O.research_attention(specs, q, k, v, None, D ** -0.5, state=st)
+        oo, _, om = O.research_attention(specs, q, k, v, None, D ** -0.5, state=dict(state))
+        if b == 0:
+            times.append(time.perf_counter() - t0)
+        got = last["out"][b:b + 1].float().cpu()
+        worst_err = max(worst_err, ((got - oo.float()).norm() / oo.float().norm()).item())
+        if last["cols"] is not None:
+            want = om.to_dense()[0, :, 0] != 0
+            member = membership(b)
+            sets_equal = sets_equal and bool(torch.equal(member, want))
+            overlap = min(overlap, float((member & want).sum()) / float(want.sum()))
+    parity = dict(rel_err=float(f"{worst_err:.3e}"), tolerance=tol,
+                  rows_checked=f"batch rows {rows_checked} ({HQ} mask rows each, of {B * HQ}) of the last timed step; worst row reported")
+    if last["cols"] is not None:
+        parity["index_sets_equal"] = sets_equal
+        parity["index_set_overlap"] = round(overlap, 6)
+    if adaptive:
+        parity["note"] = ("sampled sets compared given the kernels' budgets (the budget itself is a float formula truncated to an "
+                          "integer, compared with the oracle's to one unit of precision in the tests)")
+        b_or = None
+        q, k, v, specs, state = inputs(0)
+        st = {kk: vv for kk, vv in state.items() if kk != "budget"}
+        O.research_attention(specs, q, k, v, None, D ** -0.5, state=st)
+        b_or = st["budget_oracle"].reshape(-1).double()
+        b_k = state["budget"].double()
+        parity["budget_max_rel_diff_vs_oracle"] = float(f"{((b_k - b_or).abs() / b_or.clamp_min(1)).max().item():.3e}")
+    # CPU baseline: more timed passes over batch row 0 within the budget
+    q, k, v, specs, state = inputs(0)
+    t_all = time.perf_counter()
+    while len(times) < 12 and (len(times) < 2 or time.perf_counter() - t_all < budget_s):
+        t0 = time.perf_counter()
+        O.research_attention(specs, q, k, v, None, D ** -0.5, state=dict(state))
         times.append(time.perf_counter() - t0)
-        if parity is None and not w.get("adaptive"):
-            got = last["out"][:1].float().cpu()
-            err = ((got - oo.float()).norm() / oo.float().norm()).item()
-            parity = dict(rel_err=float(f"{err:.3e}"), tolerance=1e-5 if w["dtype"] == "f32" else 2e-2,
-                          rows_checked=f"batch row 0 ({HQ} of {w['B'] * HQ} mask rows) of the last timed step")
-            if last["cols"] is not None:
-                want = om.to_dense()[0, :, 0] != 0
-                member = torch.zeros_like(want)
-                cols, cnt = last["cols"][:HQ].long().cpu(), last["cnt"][:HQ].long().cpu()
-                for r in range(HQ):
-                    member[r, cols[r, : cnt[r]]] = True
-                parity["index_sets_equal"] = bool(torch.equal(member, want))
-                parity["index_set_overlap"] = round(float((member & want).sum()) / float(want.sum()), 6)
-        if time.perf_counter() - t_all > budget_s and it >= 1:
-            break
     per_row = median(times[1:] or times)
-    base = dict(value=per_row * w["B"] * 1e6, unit="us/layer-step", cores=cores, kind="port",
-                sample=f"oracle (torch-CPU restatement of the reference path) on 1 of {w['B']} batch rows, "
-                       f"median of {max(1, len(times) - 1)} warm steps x {w['B']}; torch threads={cores}")
+    base = dict(value=round(per_row * B * 1e6, 1), unit="us/layer-step", cores=cores, kind="port",
+                sample=f"oracle (torch-CPU restatement of the reference path) on 1 of {B} batch rows, "
+                       f"median of {max(1, len(times) - 1)} warm steps x {B}; torch threads={cores}")
     return parity, base
 
 
@@ -363,7 +433,7 @@ def hf_callable_run(w, dev, steps, warm, reps, probe, settle, direct_us, direct_
     import torch
 
     run = Run(w, dev, steps, warm, reps, probe, host_rng=True, settle=settle, hf_layers=layers)  # same seeded inputs
-    run.cold()
+    run.cold(second_layer=False)
     wall, gpu, host, _ = run.timed()
     total = run.total
     per_bracket_us = [x / steps * 1e3 for x in wall]
@@ -379,26 +449,32 @@ def hf_callable_run(w, dev, steps, warm, reps, probe, settle, direct_us, direct_
                       "tensor (one launch and one read-back), then every layer-step of that pass is the one-kernel plan")
 
 
-def sub_run(cfg: int, dev) -> dict:
-    """A short run of another configuration of the headline set: cold call, warm-up steps (about 10 ms of them, so
-    that the clocks have settled), one bracket of timed steps."""
+def sub_run(cfg: int, dev, cpu_budget_s: float) -> dict:
+    """A run of another configuration of the headline set: the two cold calls, warm-up steps (about 10 ms of them, so
+    that the clocks have settled), two brackets of 64 timed steps, parity of the last step against the oracle and the
+    oracle timed on the host cores (bounded by `cpu_budget_s`)."""
     import torch
 
     w = dict(WORKLOADS[cfg])
-    steps = 24 if cfg == 5 else 64
-    run = Run(w, dev, steps, 8 if cfg == 5 else 160, 1, 0, host_rng=False)
-    cold_ms = run.cold()
+    steps, reps = 64, 2
+    run = Run(w, dev, steps, 8 if cfg == 5 else 160, reps, 0, host_rng=False)
+    cold = run.cold()
     wall, gpu, _, _ = run.timed()
+    total = steps * reps
     sampled = 0.0
     if w.get("adaptive"):
         sampled = float(run.ra.maskers[-1].last_rows.cnt.float().mean().item()) - (w["sink"] + w["local"] + w["k"])
     ab = algorithmic_bytes(w, sampled)["step"]
-    us, gpu_us = wall[0] / steps * 1e3, gpu[0] / steps * 1e3
-    out = dict(workload=w["name"], us=round(us, 2), gpu_us=round(gpu_us, 2), steps=steps, algorithmic_bytes=ab,
+    per_bracket_us = [x / steps * 1e3 for x in wall]
+    us, gpu_us = sum(wall) / total * 1e3, sum(gpu) / total * 1e3
+    out = dict(workload=w["name"], us=round(us, 2), median_us=round(median(per_bracket_us), 2), min_us=round(min(per_bracket_us), 2),
+               gpu_us=round(gpu_us, 2), timed_steps_total=total, brackets=reps, algorithmic_bytes=ab,
                achieved_GBps=round(ab / (gpu_us * 1e-6) / 1e9, 1), frac=round(ab / (gpu_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
-               cold_call_ms=round(cold_ms, 2), data="synthetic, drawn on the device")
+               data="synthetic, drawn on the device", **cold)
     if w.get("adaptive"):
         out["keys_per_row"] = round(w["sink"] + w["local"] + w["k"] + sampled, 1)
+    if cpu_budget_s > 0:
+        out["parity"], out["cpu_baseline"] = parity_and_cpu_baseline(run, run.last, cpu_budget_s)
     del run
     torch.cuda.empty_cache()
     return out
@@ -552,7 +628,7 @@ def main() -> None:
     probe = 2 * HASH_BLOCK                                # instrumented steps for the per-kernel durations
     settle = max(0, SETTLE_STEPS - warm)
     run = Run(w, dev, steps, warm, reps, probe, host_rng=True, settle=settle)
-    cold_ms = run.cold()
+    cold = run.cold()
 
     if args.pmc_probe:
         for i in range(5):
@@ -569,10 +645,7 @@ def main() -> None:
     total = run.total
     ms_per_step = sum(wall) / total
     gpu_ms_per_step = sum(gpu) / total
-    rows = run.last_rows()
-    cache = run.meta.get("key", {}).get(0) if w["kind"] == "hash" else None
-    last = dict(out=run.last_out, q=run.last_q, n_hashed=getattr(cache, "n", 0),
-                cols=None if rows is None else rows[0].clone(), cnt=None if rows is None else rows[1].clone())
+    last = run.last
 
     kernels = run.instrumented()
     sampled = 0.0
@@ -635,7 +708,7 @@ def main() -> None:
         "step_algorithmic_bytes": ab["step"],
         "step_achieved_GBps": round(step_gbs, 1),
         "step_frac_of_hbm_peak": round(step_gbs / HBM_PEAK_GBS, 4),
-        "cold_call_ms": round(cold_ms, 2),
+        **cold,
         "amortised_hash_us": round(amortised_hash_us, 3),
         "kernels_avg_us": {n: round(d["avg_us"], 2) for n, d in sorted(kernels.items())},
         "kernels_avg_us_note": "HIP events around every single launch (they include the event markers' own gaps)",
@@ -649,13 +722,13 @@ def main() -> None:
         out["hf_callable"] = hf_callable_run(w, dev, steps, warm, reps, probe, settle, out["value"], last["out"])
         run = None
     if not args.no_other_configs and not study:
-        del last, rows
+        del last
         run = None
         torch.cuda.empty_cache()
         others = {}
         for cfg in sorted(WORKLOADS):
             if cfg != args.config:
-                others[f"cfg{cfg}"] = sub_run(cfg, dev)
+                others[f"cfg{cfg}"] = sub_run(cfg, dev, 0.0 if args.no_cpu_baseline else 4.0)
         out["other_configs"] = others
     print(json.dumps(out))
 
