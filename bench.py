@@ -667,6 +667,11 @@ def main() -> None:
                   "then run back to back; a bracket starts on an idle GPU and its first launch waits for the host), divided by "
                   "their number, mean over all brackets; one launch per step, the periodic new-key hashing launches included")
         del kernels[dom]                                  # per-launch event pairs measure launch gaps for this one
+    elif "k_select16_attn" in kernels:
+        # selection and attention of a row in one kernel: the attention's bytes plus the row's 2-byte score keys, read once
+        dom, dom_bytes = "k_select16_attn", ab["attention_kernel"] + w["B"] * HQ * w["Lk"] * 2
+        dom_us = kernels[dom]["avg_us"]
+        timing = "HIP events around every launch"
     else:
         dom, dom_bytes = "k_sparse_attn", ab["attention_kernel"]
         dom_us = kernels[dom]["avg_us"]

@@ -599,6 +599,20 @@ int sah_hash_compact_codes(const sah_hash_compact_args* a);
 int sah_hash_decode_attention(const sah_hash_decode_args* a, const sah_attention_args* t);
 
 /* ---------------------------------------------------------------------------
+ * sah_select_topk followed by sah_sparse_attention over the same rows, with the same results up to the order of
+ * the attention's sums. Replaces the tail of a chain with a scoring pass of its own - `topk; scatter_` and
+ * get_masked_attention_output (oracle_top_k.py:73-79, pq_top_k.py:513-537, utils/mask_attention_utils.py:406-491).
+ * When the selection is the 16-bit form with at most 65536 candidates and the attention is the plain decode case
+ * (no additive mask, unit weights, no logits output, no dropout, head_dim 64 or 128, 2-byte dtype, same rows and
+ * stream) both run in ONE kernel: every row is given several workgroups when there are fewer rows than compute
+ * units; each finds the row's columns by itself, attends to its share of them, and the one that finishes last
+ * merges the partial results, which meet in t->work (sah_sparse_attention_work_floats covers them).
+ * tickets: rows.n_rows 32-bit words in which the workgroups of a row count their arrivals; zero before the first
+ * call, left zero by every call (calls that share them must not overlap). NULL: rows are never given more than one
+ * workgroup. rows.cols / rows.cnt / rows.bitmap are still written. Otherwise the two calls are made. */
+int sah_select_topk_attention(const sah_select_topk_args* s, const sah_attention_args* t, uint32_t* tickets);
+
+/* ---------------------------------------------------------------------------
  * What an additive attention mask holds. The reference adds the mask it is given to every score row
  * (hashattention_top_k.py:365-368, oracle_top_k.py:70-72) and to the attention logits
  * (utils/mask_attention_utils.py:221-225) whatever it contains; through HuggingFace it is the eager mask
@@ -629,7 +643,8 @@ int sah_amask_classify(const sah_amask_classify_args* a);
  * (tensor pointers, key count). Replaces the per-masker Python dispatch of
  * ResearchAttention.custom_attention (research_attention/base.py:108-148) on the
  * decode path; stops at the first stage that fails and returns its code.
- * hash_decode directly followed by attention runs as sah_hash_decode_attention.
+ * hash_decode directly followed by attention runs as sah_hash_decode_attention,
+ * select directly followed by attention as sah_select_topk_attention.
  * ------------------------------------------------------------------------- */
 typedef struct sah_chain_args {
   const sah_sink_local_args* sink_local;
@@ -643,6 +658,7 @@ typedef struct sah_chain_args {
   const sah_select_topk_args* select;
   const sah_attention_args* attention;
   const sah_hash_compact_args* compact;
+  uint32_t* tickets;   /* for select + attention as one kernel (sah_select_topk_attention), or NULL */
 } sah_chain_args;
 int sah_run_chain(const sah_chain_args* a);
 

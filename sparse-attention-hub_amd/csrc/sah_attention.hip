@@ -91,11 +91,16 @@ static int att_pick_split(int n_rows, int max_cnt) {
   return (chunks + cps - 1) / cps;
 }
 
+// with the selection in the same kernel (sah_select_topk_attention): partial results of a row's parts and their tickets
+int64_t selattn_work_floats(int n_rows, int D);
+
 extern "C" int64_t sah_sparse_attention_work_floats(int32_t n_rows, int32_t max_cnt, int32_t D) {
   if (n_rows <= 0 || max_cnt < 0 || D <= 0) return 0;
-  if (att_use_row_form(n_rows, max_cnt)) return 0;
+  const int64_t fused = selattn_work_floats(n_rows, D);
+  if (att_use_row_form(n_rows, max_cnt)) return fused;
   int n_split = att_pick_split(n_rows, max_cnt);
-  return (int64_t)n_rows * n_split * (D + 2);
+  const int64_t split = (int64_t)n_rows * n_split * (D + 2);
+  return split > fused ? split : fused;
 }
 
 template <int DT, int D>
@@ -303,6 +308,7 @@ extern "C" int sah_run_chain(const sah_chain_args* a) {
   if (a->qk && (rc = sah_qk_scores(a->qk))) return rc;
   if (a->pq_assign && (rc = sah_pq_kmeans_assign(a->pq_assign))) return rc;
   if (a->pq_adc && (rc = sah_pq_adc_scores(a->pq_adc))) return rc;
+  if (a->select && a->attention) return sah_select_topk_attention(a->select, a->attention, a->tickets);  // one kernel when shapes allow
   if (a->select && (rc = sah_select_topk(a->select))) return rc;
   if (a->attention && (rc = sah_sparse_attention(a->attention))) return rc;
   return SAH_OK;

@@ -330,6 +330,54 @@ __device__ __forceinline__ uint32_t sah_pk_ne01_u16(uint32_t a, uint32_t b) {
 #endif
 }
 
+// ---------------------------------------------------------------------------
+// Hand-over between workgroups of one kernel, without a cache write-back.
+// An MI355X has eight L2 caches (one per die). A device-scope release fence makes a workgroup's ordinary stores
+// visible to the other dies by writing the whole L2 back, which costs more than the kernels here run for. The
+// accesses below are device-scope *atomic* loads / stores / read-modify-writes (relaxed): they bypass the
+// non-coherent cache levels by themselves, so data handed over with them needs no fence, only the wait that orders
+// a workgroup's stores before its arrival ticket:
+//   producer: sah_agent_store_* the data; sah_stores_done(); __syncthreads(); one thread calls sah_last_arrival
+//   consumer: (the workgroup that arrived last) __syncthreads(); sah_agent_load_* the data
+// Nobody ever waits for another workgroup: the last one to arrive does the common work.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ void sah_agent_store_f32(float* p, float v) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#else
+  *(volatile float*)p = v;
+#endif
+}
+__device__ __forceinline__ float sah_agent_load_f32(const float* p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#else
+  return *(const volatile float*)p;
+#endif
+}
+// every store this thread has issued has reached its point of coherence
+__device__ __forceinline__ void sah_stores_done() {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#endif
+}
+// Arrival ticket of one of `n` workgroups that share `word` (zero before the first of them arrives): returns true for
+// the one that arrives last, which also puts the word back to zero for the next kernel that uses it. One atomic
+// read-modify-write per workgroup, no retry loop: eight workgroups arriving together do not queue behind each other.
+__device__ __forceinline__ bool sah_last_arrival(uint32_t* word, uint32_t n) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const uint32_t before = __hip_atomic_fetch_add(word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (before + 1u != n) return false;
+  __hip_atomic_store(word, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return true;
+#else
+  const uint32_t before = __atomic_fetch_add(word, 1u, __ATOMIC_RELAXED);
+  if (before + 1u != n) return false;
+  __atomic_store_n(word, 0u, __ATOMIC_RELAXED);
+  return true;
+#endif
+}
+
 // Orders the LDS traffic of ONE wave: what its lanes wrote before is visible to its lanes after.
 // For LDS regions that a single wave owns; costs a wait on the wave's own LDS queue, no workgroup barrier.
 __device__ __forceinline__ void sah_wave_lds_sync() {

@@ -183,10 +183,17 @@ __device__ __forceinline__ uint32_t sf_lowest(uint32_t m, int allowed) {
 
 // CPW > 0: a wave keeps the effective keys of its (at most CPW) chunks in registers through
 // all passes; CPW == 0: rows too long for that re-read their keys from memory in every pass.
+// s_cols (optional, LDS, R.cap ints; may lie over the histograms, which are dead by then): the columns this call
+// appends are also written there, at the positions they take in the row's list, for a caller that goes on with the
+// list in the same kernel; the entries before them (the row's earlier ones) are the caller's to fill in.
+// to_memory = false: the row's list, count and bitmap in memory are left alone (another workgroup writes them).
+// Returns the row's entry count after the call; *first_new = the count before it.
 template <int CPW>
-__device__ __forceinline__ void sf_select_row(sf_lds& S, unsigned char* dyn, const sah_rows& R, int r,
-                                              const uint16_t* keys, int n_cand, int col_offset, int k,
-                                              uint32_t excluded_key, int fresh, int sink, int window) {
+__device__ __forceinline__ int sf_select_row(sf_lds& S, unsigned char* dyn, const sah_rows& R, int r,
+                                             const uint16_t* keys, int n_cand, int col_offset, int k,
+                                             uint32_t excluded_key, int fresh, int sink, int window,
+                                             int* s_cols = nullptr, bool to_memory = true, bool write_bitmap = true,
+                                             int* first_new = nullptr) {
   constexpr bool REG = CPW > 0;
   constexpr int NREG = REG ? CPW : 1;
   // The short way to the threshold (below) costs four packed compares per key word and pays up to 64 keys per
@@ -257,9 +264,11 @@ __device__ __forceinline__ void sf_select_row(sf_lds& S, unsigned char* dyn, con
     const int lo2 = lo > s_hi ? lo : s_hi;
     const int fixed = s_hi + (hi > lo2 ? hi - lo2 : 0);
     int* cols0 = R.cols + (int64_t)r * R.cap;
-    for (int i = tid; i < fixed && i < R.cap; i += SF_NT) {
-      cols0[i] = i < s_hi ? i : lo2 + (i - s_hi);
-      if (R.w) R.w[(int64_t)r * R.cap + i] = 1.0f;
+    if (to_memory) {
+      for (int i = tid; i < fixed && i < R.cap; i += SF_NT) {
+        cols0[i] = i < s_hi ? i : lo2 + (i - s_hi);
+        if (R.w) R.w[(int64_t)r * R.cap + i] = 1.0f;
+      }
     }
     cnt0 = fixed < R.cap ? fixed : R.cap;
     clear_counters();
@@ -522,23 +531,33 @@ __device__ __forceinline__ void sf_select_row(sf_lds& S, unsigned char* dyn, con
     uint32_t em = emit_mask(c, kk, u);
     if (em) {
       const int col0 = c * SF_CHUNK + lane * 8 + col_offset;
-      atomicOr(&s_bm[col0 >> 5], em << (col0 & 31));
-      if ((col0 & 31) > 24) atomicOr(&s_bm[(col0 >> 5) + 1], em >> (32 - (col0 & 31)));
+      if (to_memory && write_bitmap) {
+        atomicOr(&s_bm[col0 >> 5], em << (col0 & 31));
+        if ((col0 & 31) > 24) atomicOr(&s_bm[(col0 >> 5) + 1], em >> (32 - (col0 & 31)));
+      }
       while (em) {
         const int t = __builtin_ctz(em);
         em &= em - 1;
         if (pos < R.cap) {
-          cols[pos] = col0 + t;
-          if (wgt) wgt[pos] = 1.0f;
+          if (to_memory) {
+            cols[pos] = col0 + t;
+            if (wgt) wgt[pos] = 1.0f;
+          }
+          if (s_cols) s_cols[pos] = col0 + t;
         }
         ++pos;
       }
     }
   });
   __syncthreads();
-  if (total > 0 || fresh)
-    for (int i = tid; i < R.n_words; i += SF_NT) bm[i] = s_bm[i];
-  if (tid == 0) R.cnt[r] = cnt0 + total;
+  if (to_memory) {
+    if (write_bitmap && (total > 0 || fresh))
+      for (int i = tid; i < R.n_words; i += SF_NT) bm[i] = s_bm[i];
+    if (tid == 0) R.cnt[r] = cnt0 + total;
+  }
+  if (first_new) *first_new = cnt0;
+  const int after = cnt0 + total;
+  return after < R.cap ? after : R.cap;
 }
 
 // dynamic LDS bytes of one launch
@@ -549,4 +568,16 @@ static inline size_t sf_lds_bytes(int n_words) {
 static inline int sf_chunks_per_wave(int n_cand) {
   const int n_chunks = (n_cand + SF_CHUNK - 1) / SF_CHUNK;
   return (n_chunks + SF_NW - 1) / SF_NW;
+}
+
+// byte offset, inside the dynamic LDS of sf_select_row, of the region its histograms occupy (dead once the threshold
+// is known): where a caller may keep the row's column list
+static inline size_t sf_hist_offset(int n_words) { return (size_t)((n_words + 2 + 3) & ~3) * 4; }
+static inline size_t sf_hist_bytes() { return (size_t)2 * 256 * SF_COPIES * 4; }
+
+// argument checks of sah_select_topk (defined with it), for entry points that run the same selection
+int sel_validate(const sah_select_topk_args* a, const char* who);
+// may this call take the eight-keys-per-lane kernel? (16-bit keys, aligned rows, the LDS fits)
+static inline bool sel16_ok(const sah_select_topk_args* a) {
+  return a->key_bits == 16 && a->key_pitch % 8 == 0 && ((uintptr_t)a->keys % 16) == 0 && sf_lds_bytes(a->rows.n_words) <= 150 * 1024;
 }

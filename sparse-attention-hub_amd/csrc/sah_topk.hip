@@ -450,28 +450,33 @@ extern "C" int sah_hamming_scores(const sah_hamming_scores_args* a) {
   return sah_launch_status("sah_hamming_scores");
 }
 
-extern "C" int sah_select_topk(const sah_select_topk_args* a) {
-  if (!a) return sah_fail(SAH_ENULL, "sah_select_topk: args is NULL");
-  int rc = sah_check_rows(a->rows, "sah_select_topk");
+int sel_validate(const sah_select_topk_args* a, const char* who) {
+  if (!a) return sah_fail(SAH_ENULL, "%s: args is NULL", who);
+  int rc = sah_check_rows(a->rows, who);
   if (rc) return rc;
-  if (!a->keys) return sah_fail(SAH_ENULL, "sah_select_topk: keys is NULL");
-  if (a->key_bits != 16 && a->key_bits != 32) return sah_fail(SAH_EINVAL, "sah_select_topk: key_bits must be 16 or 32");
+  if (!a->keys) return sah_fail(SAH_ENULL, "%s: keys is NULL", who);
+  if (a->key_bits != 16 && a->key_bits != 32) return sah_fail(SAH_EINVAL, "%s: key_bits must be 16 or 32", who);
   if (a->n_cand <= 0 || a->col_offset < 0 || (int64_t)a->col_offset + a->n_cand > a->rows.n_keys)
-    return sah_fail(SAH_EINVAL, "sah_select_topk: candidate range [%d, %d) outside [0, %d)", a->col_offset,
+    return sah_fail(SAH_EINVAL, "%s: candidate range [%d, %d) outside [0, %d)", who, a->col_offset,
                     a->col_offset + a->n_cand, a->rows.n_keys);
-  if (a->k <= 0) return sah_fail(SAH_EINVAL, "sah_select_topk: k must be > 0");
-  if (a->key_pitch < a->n_cand) return sah_fail(SAH_EINVAL, "sah_select_topk: key_pitch < n_cand");
+  if (a->k <= 0) return sah_fail(SAH_EINVAL, "%s: k must be > 0", who);
+  if (a->key_pitch < a->n_cand) return sah_fail(SAH_EINVAL, "%s: key_pitch < n_cand", who);
   if (a->fresh && (a->fresh_sink < 0 || a->fresh_window < 0))
-    return sah_fail(SAH_EINVAL, "sah_select_topk: fresh_sink / fresh_window must be >= 0");
+    return sah_fail(SAH_EINVAL, "%s: fresh_sink / fresh_window must be >= 0", who);
   if (a->fresh) {
     int64_t worst = (int64_t)a->fresh_sink + a->fresh_window;
     if (worst > a->rows.n_keys) worst = a->rows.n_keys;
     if (worst > a->rows.cap)
-      return sah_fail(SAH_ECAPACITY, "sah_select_topk: cap %d < sink+window %lld", a->rows.cap, (long long)worst);
+      return sah_fail(SAH_ECAPACITY, "%s: cap %d < sink+window %lld", who, a->rows.cap, (long long)worst);
   }
+  return SAH_OK;
+}
+
+extern "C" int sah_select_topk(const sah_select_topk_args* a) {
+  int rc = sel_validate(a, "sah_select_topk");
+  if (rc) return rc;
   hipStream_t st = (hipStream_t)a->stream;
-  if (a->key_bits == 16 && a->key_pitch % 8 == 0 && ((uintptr_t)a->keys % 16) == 0 &&
-      sf_lds_bytes(a->rows.n_words) <= 150 * 1024) {
+  if (sel16_ok(a)) {
     // eight keys per lane: needs 16-byte aligned key rows
     const size_t lds = sf_lds_bytes(a->rows.n_words);
     const int cpw = sf_chunks_per_wave(a->n_cand);

@@ -56,6 +56,7 @@ EXPECTED_SYMBOLS = (
     "sah_attention_weights",
     "sah_run_chain",
     "sah_amask_classify",
+    "sah_select_topk_attention",
 )
 
 
@@ -344,6 +345,7 @@ class ChainArgs(C.Structure):
         ("select", C.c_void_p),
         ("attention", C.c_void_p),
         ("compact", C.c_void_p),
+        ("tickets", C.c_void_p),
     ]
 
 
@@ -420,6 +422,10 @@ def lib() -> C.CDLL:
         if name in ("sah_hash_signatures_pair", "sah_hash_decode_attention"):
             getattr(handle, name).restype = C.c_int
             getattr(handle, name).argtypes = [C.c_void_p, C.c_void_p]
+            continue
+        if name == "sah_select_topk_attention":
+            getattr(handle, name).restype = C.c_int
+            getattr(handle, name).argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
             continue
         fn = getattr(handle, name)
         fn.restype = C.c_int

@@ -96,6 +96,8 @@ class DecodePlan:
         self.att = N.AttentionArgs()
         self.chain = N.ChainArgs()
         self.unit = unit_inverse_weight(q.dtype)
+        # arrival counters of the one-kernel selection + attention (zero between calls: the kernel puts them back)
+        self.tickets = torch.zeros((self.n_rows,), dtype=torch.int32, device=self.device)
         self._excluded_min = sortable_key_of(torch.finfo(q.dtype).min, q.dtype)
 
     def signature(self, q: torch.Tensor, k: torch.Tensor) -> Tuple:
@@ -326,6 +328,7 @@ class DecodePlan:
             chain.sink_local = None
         at.stream = stream
         chain.attention = C.addressof(at)
+        chain.tickets = self.tickets.data_ptr()
         N.call("sah_run_chain", chain)
         for obj, name, value in commit:
             setattr(obj, name, value)

@@ -54,13 +54,20 @@ def test_argument_errors_are_reported_without_a_gpu():
     # workgroups to cover the chip while the row still has chunks to hand out
     for n_rows, max_cnt, D in ((128, 2278, 128), (512, 131072, 128), (64, 2688, 64), (32, 1500, 128), (1, 70000, 128)):
         floats = N.work_floats(n_rows, max_cnt, D)
+        # fewer rows than compute units: also room for the one-kernel selection + attention, which gives a row
+        # min(8, 256 // rows) workgroups - their partial results
+        parts = min(8, 256 // n_rows) if n_rows < 192 else 1
+        fused = n_rows * parts * (D + 2) if parts > 1 else 0
+        assert floats >= fused
+        if floats == fused:
+            continue
         assert floats > 0 and floats % (n_rows * (D + 2)) == 0
         n_split = floats // (n_rows * (D + 2))
         chunks = -(-max_cnt // 256)
         assert 1 <= n_split <= min(64, chunks)
         assert -(-chunks // n_split) <= 11 or n_split == 64
         assert n_rows * n_split >= 2048 or 2 * n_split > min(64, chunks)
-    assert N.work_floats(32, 300, 128) == 0  # short rows: whole-row form
+    assert N.work_floats(32, 300, 128) == 32 * 8 * 130  # short rows: whole-row form, or the one-kernel form
     assert N.work_floats(0, 100, 128) == 0 and N.work_floats(16, 100, 0) == 0
     for fn in ("sah_hash_decode_topk", "sah_adaptive_budget", "sah_adaptive_sample", "sah_pq_adc_scores"):
         assert getattr(lib, fn)(None) == -2 and fn.encode() in lib.sah_last_error()
@@ -86,10 +93,11 @@ def test_every_entry_point_refuses_null_and_names_itself():
         assert fn.replace("_static", "").encode() in lib.sah_last_error() or fn.encode() in lib.sah_last_error(), fn
     assert lib.sah_hash_signatures_pair(None, None) == -2
     assert lib.sah_hash_decode_attention(None, None) == -2
+    assert lib.sah_select_topk_attention(None, None, None) == -2
     # whatever takes an argument block is in one of the two lists above
     plain = {"sah_version", "sah_last_error", "sah_timing_enable", "sah_timing_collect", "sah_pq_adc_lut_bytes",
              "sah_sparse_attention_work_floats"}
-    assert set(one_arg) | {"sah_hash_signatures_pair", "sah_hash_decode_attention"} | plain == set(_declared_functions())
+    assert set(one_arg) | {"sah_hash_signatures_pair", "sah_hash_decode_attention", "sah_select_topk_attention"} | plain == set(_declared_functions())
 
 
 def test_bad_argument_blocks_are_refused_with_the_documented_codes():

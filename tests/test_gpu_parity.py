@@ -479,7 +479,16 @@ def test_decode_plan_matches_masker_by_masker_path(cuda, kind):
             continue
         o2, w2 = ref.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m2, layer_idx=0)
         assert w1 is None and w2 is not None
-        assert torch.equal(o1, o2), f"step {step}"
+        if kind in ("fixed", "hash"):
+            assert torch.equal(o1, o2), f"step {step}"
+        else:
+            # selection and attention of these chains run as one kernel that deals a row's entries to its workgroups
+            # in another order than the stand-alone attention: same columns, sums that may differ in a last bit
+            plan = next(iter(fast._plans.values()))
+            member = torch.zeros((B * Hq, n), dtype=torch.bool, device=cuda)
+            member.scatter_(1, plan.cols[:, :int(plan.cnt[0])].long(), True)
+            assert bool((plan.cnt == plan.cnt[0]).all()) and torch.equal(member.view(B, Hq, n), w2[:, :, 0] != 0), f"step {step}"
+            assert rel_err(o1, o2) < 4e-3, f"step {step}"
     plan = next(iter(fast._plans.values()))
     assert plan.att.out is not None and plan.att.Lk == Lk + 3     # the last step went through the plan
 
@@ -543,7 +552,7 @@ def test_decode_plan_quantises_new_keys_in_blocks(cuda, n_sub):
         qq = make_qkv(B, Hq, Hkv, 1, 1, D, dtype, seed=250 + step)[0].to(cuda)
         o1, _ = fast.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m1, layer_idx=0)
         o2, _ = ref.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m2, layer_idx=0)
-        assert torch.equal(o1, o2), f"step {step}"
+        assert rel_err(o1, o2) < 4e-3, f"step {step}"      # same columns; the one-kernel form sums in another order
         b1, b2 = m1["pq_codebook"][0], m2["pq_codebook"][0]
         assert b2.n == n - off and n - off - window < b1.n <= n - off
         quantised.append(b1.n)
