@@ -30,6 +30,7 @@ static_assert(SF_TOP_BINS % 2 == 0, "the short path counts its bins in pairs");
 struct sf_lds {
   int part[SF_NW];
   int eq[SF_NW];
+  int gt[SF_NW];  // FUSED: keys above the threshold per wave
   int out[SF_NW];
   int top[SF_TOP_BINS];  // short path: candidates at or above each of the top high-byte bins
   int sel_bin, sel_need;
@@ -183,19 +184,24 @@ __device__ __forceinline__ uint32_t sf_lowest(uint32_t m, int allowed) {
 
 // CPW > 0: a wave keeps the effective keys of its (at most CPW) chunks in registers through
 // all passes; CPW == 0: rows too long for that re-read their keys from memory in every pass.
-// s_cols (optional, LDS, R.cap ints; may lie over the histograms, which are dead by then): the columns this call
-// appends are also written there, at the positions they take in the row's list, for a caller that goes on with the
-// list in the same kernel; the entries before them (the row's earlier ones) are the caller's to fill in.
 // to_memory = false: the row's list, count and bitmap in memory are left alone (another workgroup writes them).
 // Returns the row's entry count after the call; *first_new = the count before it.
-template <int CPW>
-__device__ __forceinline__ int sf_select_row(sf_lds& S, unsigned char* dyn, const sah_rows& R, int r,
-                                             const uint16_t* keys, int n_cand, int col_offset, int k,
-                                             uint32_t excluded_key, int fresh, int sink, int window,
-                                             int* s_cols = nullptr, bool to_memory = true, bool write_bitmap = true,
-                                             int* first_new = nullptr) {
+//
+// FUSED: the caller attends to the chosen columns in the same kernel, as one of `parts` workgroups that each run this
+// selection for the row. The winners are written to the list s_cols (LDS; it may lie over the histograms, which are
+// dead by then) at the positions they take in the row's list - complete after the caller's next barrier, entries
+// [*first_new, return value); the entries before are the caller's to fill in or to derive. The row in memory: every
+// part writes the columns of its own candidate chunks (chunk c belongs to part c % parts), part 0 (to_memory) also
+// the count; the bitmap row is left complete in LDS (at the start of dyn) for part 0 to copy out after that barrier.
+template <int CPW, bool FUSED = false>
+__device__ __forceinline__ int sf_select_impl(sf_lds& S, unsigned char* dyn, const sah_rows& R, int r,
+                                              const uint16_t* keys, int n_cand, int col_offset, int k,
+                                              uint32_t excluded_key, int fresh, int sink, int window,
+                                              bool to_memory, bool write_bitmap, int* first_new, int* s_cols, int part,
+                                              int parts) {
   constexpr bool REG = CPW > 0;
   constexpr int NREG = REG ? CPW : 1;
+  static_assert(!FUSED || (REG && CPW <= 8), "the fused form keeps a row's keys and its emission masks in registers");
   // The short way to the threshold (below) costs four packed compares per key word and pays up to 64 keys per
   // thread; longer rows amortise the histograms' fixed cost better (512 x 131072: 134 us against 107)
   constexpr bool SHORT = REG && CPW <= 8;
@@ -476,6 +482,10 @@ __device__ __forceinline__ int sf_select_row(sf_lds& S, unsigned char* dyn, cons
   });
   const int wave_eq = sah_wave_sum_i(n_eq);
   if (lane == 0) S.eq[wave] = wave_eq;
+  if constexpr (FUSED) {
+    const int wave_gt = sah_wave_sum_i(n_gt);
+    if (lane == 0) S.gt[wave] = wave_gt;
+  }
   __syncthreads();
   int tie_base = 0;
 #pragma unroll
@@ -506,6 +516,72 @@ __device__ __forceinline__ int sf_select_row(sf_lds& S, unsigned char* dyn, cons
     return gt | (take & ~ex);
   };
 
+  if constexpr (FUSED) {
+    // ---- the winners into the LDS list (all of them, at the positions they take in the row's list) and, for the
+    // chunks of this part, into the row in memory. Every wave's number of winners follows from the counts exchanged
+    // at the tie barrier (its keys above the threshold plus the ties it may take), so the positions need no second
+    // barrier - unless active candidates may rank (`slow`), whose ties cannot be counted ahead.
+    uint32_t em_all[(NREG + 3) / 4];  // emission masks of the wave's chunks, 8 bits each
+#pragma unroll
+    for (int i = 0; i < (NREG + 3) / 4; ++i) em_all[i] = 0;
+    int mine_all = 0;
+    for_chunks_slot([&](int c, const uint32_t (&kk)[4], int u) {
+      const uint32_t em = emit_mask(c, kk, u);
+      em_all[u >> 2] |= em << (8 * (u & 3));
+      mine_all += __popc(em);
+    });
+    const int incl_a = sah_wave_incl_scan(mine_all);
+    int out_base = 0, total = 0;
+    if (!slow) {
+      int ties_before = 0;
+#pragma unroll
+      for (int w = 0; w < SF_NW; ++w) {
+        int take = need - ties_before;
+        take = take < 0 ? 0 : (take > S.eq[w] ? S.eq[w] : take);
+        const int v = S.gt[w] + take;
+        out_base += w < wave ? v : 0;
+        total += v;
+        ties_before += S.eq[w];
+      }
+    } else {
+      if (lane == SAH_WAVE - 1) S.out[wave] = incl_a;
+      __syncthreads();
+      for (int w = 0; w < SF_NW; ++w) {
+        const int v = S.out[w];
+        out_base += w < wave ? v : 0;
+        total += v;
+      }
+    }
+    int* cols = R.cols + (int64_t)r * R.cap;
+    int pos = cnt0 + out_base + incl_a - mine_all;
+#pragma unroll
+    for (int u = 0; u < NREG; ++u) {
+      const int c = c0 + u;
+      if (c < c1) {
+        uint32_t em = (em_all[u >> 2] >> (8 * (u & 3))) & 0xffu;
+        const int col0 = c * SF_CHUNK + lane * 8 + col_offset;
+        if (em && to_memory && write_bitmap) {
+          atomicOr(&s_bm[col0 >> 5], em << (col0 & 31));
+          if ((col0 & 31) > 24) atomicOr(&s_bm[(col0 >> 5) + 1], em >> (32 - (col0 & 31)));
+        }
+        const bool my_chunk = c % parts == part;
+        while (em) {
+          const int t = __builtin_ctz(em);
+          em &= em - 1;
+          if (pos < R.cap) {
+            s_cols[pos] = col0 + t;
+            if (my_chunk) cols[pos] = col0 + t;
+          }
+          ++pos;
+        }
+      }
+    }
+    if (to_memory && tid == 0) R.cnt[r] = cnt0 + total;
+    // (part 0 writes the bitmap row, complete in LDS after the caller's next barrier, back to memory)
+    if (first_new) *first_new = cnt0;
+    const int after = cnt0 + total;
+    return after < R.cap ? after : R.cap;
+  }
   // what each lane emits: known from the counts, except where ties are cut or may be active
   int mine = n_gt + (mode == 1 ? n_eq : 0);
   if (mode == 2 || slow) {
@@ -543,7 +619,6 @@ __device__ __forceinline__ int sf_select_row(sf_lds& S, unsigned char* dyn, cons
             cols[pos] = col0 + t;
             if (wgt) wgt[pos] = 1.0f;
           }
-          if (s_cols) s_cols[pos] = col0 + t;
         }
         ++pos;
       }
@@ -558,6 +633,15 @@ __device__ __forceinline__ int sf_select_row(sf_lds& S, unsigned char* dyn, cons
   if (first_new) *first_new = cnt0;
   const int after = cnt0 + total;
   return after < R.cap ? after : R.cap;
+}
+
+// The stand-alone form: the row's list, count and bitmap in memory are extended.
+template <int CPW>
+__device__ __forceinline__ int sf_select_row(sf_lds& S, unsigned char* dyn, const sah_rows& R, int r,
+                                             const uint16_t* keys, int n_cand, int col_offset, int k,
+                                             uint32_t excluded_key, int fresh, int sink, int window) {
+  return sf_select_impl<CPW>(S, dyn, R, r, keys, n_cand, col_offset, k, excluded_key, fresh, sink, window, true, true, nullptr,
+                             nullptr, 0, 1);
 }
 
 // dynamic LDS bytes of one launch

@@ -5,9 +5,9 @@
 // with one workgroup per mask row, a gather in split form and a merge kernel; with the 128 rows of a batch of 4
 // half of the CUs idle through the selection, and a CU gathers K / V rows at a fixed rate however few of them work.
 // Here every row is given `parts` workgroups (rows x parts ~ the number of CUs). Each of them finds the row's
-// threshold and builds the row's column list by itself, in LDS (the same arithmetic in every part, so the lists are
-// identical; the score keys of a row are read `parts` times, from L2 after the first: the parts of a KV group share
-// a die), then attends to its share of the list. The parts' partial results meet in the workspace; the part that
+// threshold by itself (the same arithmetic in every part; the score keys of a row are read `parts` times, from L2
+// after the first: the parts of a KV group share a die) and builds the row's column list in LDS, then attends to its
+// share of the list. The parts' partial results meet in the workspace; the part that
 // arrives last merges them and writes the row. No part ever waits for another, so the grid cannot stall, and the
 // hand-over uses device-scope atomic accesses, which need no cache write-back (sah_common.h).
 #include "sah_common.h"
@@ -58,27 +58,23 @@ __global__ __launch_bounds__(SF_NT) void k_select16_attn(selattn_params P, att_p
   const int r = (b * A.Hq + h) * A.Lq + qi;
 
   int* s_cols = (int*)(sa_dyn + P.cols_offset);
-  int first_new = 0;
-  const int cnt = sf_select_row<CPW>(S, sa_dyn, P.R, r, P.keys + (int64_t)r * P.pitch, P.n_cand, P.col_offset,
-                                     P.k < P.n_cand ? P.k : P.n_cand, P.excluded_key, P.fresh, P.sink, P.window, s_cols,
-                                     part == 0, true, &first_new);
-  // the entries the row held before: the sink and local columns in closed form (fresh rows), or its list in memory
-  if (P.fresh) {
-    const int n = P.R.n_keys;
-    const int s_hi = P.sink < n ? P.sink : n;
-    int lo = P.window > 0 ? n - P.window : n;
-    if (lo < 0) lo = 0;
-    const int lo2 = lo > s_hi ? lo : s_hi;
-    for (int i = tid; i < first_new; i += SF_NT) s_cols[i] = i < s_hi ? i : lo2 + (i - s_hi);
-  } else {
-    const int* cols = P.R.cols + (int64_t)r * P.R.cap;
-    for (int i = tid; i < first_new; i += SF_NT) s_cols[i] = cols[i];
-  }
-  __syncthreads();  // the column list in LDS is complete
+  int earlier = 0;
+  const int cnt = sf_select_impl<CPW, true>(S, sa_dyn, P.R, r, P.keys + (int64_t)r * P.pitch, P.n_cand, P.col_offset,
+                                            P.k < P.n_cand ? P.k : P.n_cand, P.excluded_key, P.fresh, P.sink, P.window,
+                                            part == 0, true, &earlier, s_cols, part, P.parts);
+  __syncthreads();  // the winners' part of the list is complete in LDS, and so is the bitmap row
 
-  // this part's share: the row's entries dealt to parts x 16 waves, a wave of part p taking every parts-th run
+  // This part's share of the row: its entries dealt to parts x 16 waves, a wave of part p taking every parts-th run.
+  // The entries the row held before come first: the sink and local columns of one query in closed form (fresh rows),
+  // or the row's list in memory.
   constexpr int KPI = SAH_WAVE / (D / 8);
   const int wave = sah_wave_id();
+  const int n = P.R.n_keys;
+  const int s_hi = P.sink < n ? P.sink : n;
+  int lo = P.window > 0 ? n - P.window : n;
+  if (lo < 0) lo = 0;
+  const int lo2 = lo > s_hi ? lo : s_hi;
+  const int* cols_mem = P.R.cols + (int64_t)r * P.R.cap;
   const int n_runs = NW * P.parts;
   const int per = (((cnt + n_runs - 1) / n_runs) + KPI - 1) / KPI * KPI;  // entries per run
   const int first = (wave * P.parts + part) * per;
@@ -86,10 +82,21 @@ __global__ __launch_bounds__(SF_NT) void k_select16_attn(selattn_params P, att_p
   att_wave_state st;
   st.clear();
   const float unit = A.unit_inv_w;
-  att_walk<DT, D, false, true>(
-      A, r, b, h, hk, qi, first, bound, SAH_WAVE, [&](int i) { return s_cols[i]; }, [&](int) { return unit; }, st);
+  if (P.fresh)
+    att_walk<DT, D, false, true>(
+        A, r, b, h, hk, qi, first, bound, SAH_WAVE,
+        [&](int i) { return i >= earlier ? s_cols[i] : (i < s_hi ? i : lo2 + (i - s_hi)); }, [&](int) { return unit; }, st);
+  else
+    att_walk<DT, D, false, true>(
+        A, r, b, h, hk, qi, first, bound, SAH_WAVE, [&](int i) { return i >= earlier ? s_cols[i] : cols_mem[i]; },
+        [&](int) { return unit; }, st);
   att_park<D, NW>(st, wave, s_m, s_l, s_acc);
   __syncthreads();
+  if (part == 0) {  // the row's bitmap, complete in LDS since the barrier
+    const uint32_t* s_bm = (const uint32_t*)sa_dyn;
+    uint32_t* bm = P.R.bitmap + (int64_t)r * P.R.n_words;
+    for (int i = tid; i < P.R.n_words; i += SF_NT) bm[i] = s_bm[i];
+  }
   float a, M, l;
   att_gather<DT, D, NW>(s_m, s_l, s_acc, a, M, l);
   if (P.parts == 1) {
@@ -182,7 +189,8 @@ extern "C" int sah_select_topk_attention(const sah_select_topk_args* s, const sa
       t->rows.cols == s->rows.cols && t->rows.cnt == s->rows.cnt && t->rows.cap == s->rows.cap && t->rows.n_rows == n_rows &&
       t->stream == s->stream && (t->dtype == SAH_BF16 || t->dtype == SAH_F16) && (t->D == 128 || t->D == 64) &&
       // one workgroup per row pays when the rows are short enough for the whole-row form; several per row always
-      (parts > 1 ? (tickets && t->work && t->work_floats >= need) : worst <= 8192);
+      // several workgroups per row read the row's count while one of them rewrites it: fresh rows only
+      (parts > 1 ? (tickets && t->work && t->work_floats >= need && s->fresh) : worst <= 8192);
   if (!one_kernel) {
     if ((rc = sah_select_topk(s))) return rc;
     return sah_sparse_attention(t);
