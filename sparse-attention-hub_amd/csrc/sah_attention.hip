@@ -14,7 +14,7 @@
 
 #include <mutex>
 
-template <int DT, int D, bool ROW, bool DROP>
+template <int DT, int D, bool ROW, bool DROP, bool FULL>
 __global__ __launch_bounds__(ROW ? ATT_ROW_NT : ATT_NT, ROW ? 1 : 5) void k_sparse_attn(att_params P) {
   sah_touch_kernargs<sizeof(att_params)>();
   constexpr int NW = (ROW ? ATT_ROW_NT : ATT_NT) / SAH_WAVE;
@@ -40,15 +40,15 @@ __global__ __launch_bounds__(ROW ? ATT_ROW_NT : ATT_NT, ROW ? 1 : 5) void k_spar
   const int b = gidx / (P.Lq * P.Hkv);
   const int h = hk * G + slot % G;
   const int r = (b * P.Hq + h) * P.Lq + qi;
-  att_tile<DT, D, ROW, DROP>(P, r, b, h, hk, qi, split, n_split, nullptr, -1, s_m, s_l, s_acc);
+  att_tile<DT, D, ROW, DROP, FULL>(P, r, b, h, hk, qi, split, n_split, nullptr, -1, s_m, s_l, s_acc);
 }
 
 template <int DT, int D>
-__global__ __launch_bounds__(D < 64 ? 64 : D) void k_attn_combine(const float* work, int n_split, int Hq, int Lq,
+__global__ __launch_bounds__(D < 64 ? 64 : D) void k_attn_combine(const float* work, int n_split, int Hq, int Lq, int d_real,
                                                                   const float* sinks, void* out, float* stats) {
   __shared__ float s_m[ATT_MAX_SPLIT];
   __shared__ float s_l[ATT_MAX_SPLIT];
-  att_combine_row<DT, D>(work, n_split, blockIdx.x, Hq, Lq, sinks, out, stats, s_m, s_l);
+  att_combine_row<DT, D>(work, n_split, blockIdx.x, Hq, Lq, d_real, sinks, out, stats, s_m, s_l);
 }
 
 template <int DT>
@@ -91,11 +91,20 @@ static int att_pick_split(int n_rows, int max_cnt) {
   return (chunks + cps - 1) / cps;
 }
 
+// head_dim as the kernels see it: itself if it is 16, 32, 64 or 128, otherwise the next power of two (0: not supported)
+static int att_pad_dim(int D) {
+  if (D <= 0 || D % 8 || D > 256) return 0;
+  int dp = 16;
+  while (dp < D) dp *= 2;
+  return dp;
+}
+
 // with the selection in the same kernel (sah_select_topk_attention): partial results of a row's parts and their tickets
 int64_t selattn_work_floats(int n_rows, int D);
 
 extern "C" int64_t sah_sparse_attention_work_floats(int32_t n_rows, int32_t max_cnt, int32_t D) {
   if (n_rows <= 0 || max_cnt < 0 || D <= 0) return 0;
+  D = att_pad_dim(D) ? att_pad_dim(D) : D;
   const int64_t fused = selattn_work_floats(n_rows, D);
   if (att_use_row_form(n_rows, max_cnt)) return fused;
   int n_split = att_pick_split(n_rows, max_cnt);
@@ -103,7 +112,7 @@ extern "C" int64_t sah_sparse_attention_work_floats(int32_t n_rows, int32_t max_
   return split > fused ? split : fused;
 }
 
-template <int DT, int D>
+template <int DT, int D, bool FULL>
 static int att_launch(const sah_attention_args* a, const att_params& P, bool timing) {
   hipStream_t st = (hipStream_t)a->stream;
   const int G = a->Hq / a->Hkv;
@@ -111,8 +120,8 @@ static int att_launch(const sah_attention_args* a, const att_params& P, bool tim
     sah_timed timed("k_sparse_attn", a->stream, timing);
     const int n_tiles = a->rows.n_rows / G;
     const int n_wg = (n_tiles + ATT_XCDS - 1) / ATT_XCDS * ATT_XCDS * G;
-    if (P.drop.thresh) hipLaunchKernelGGL((k_sparse_attn<DT, D, true, true>), dim3(n_wg), dim3(ATT_ROW_NT), 0, st, P);
-    else hipLaunchKernelGGL((k_sparse_attn<DT, D, true, false>), dim3(n_wg), dim3(ATT_ROW_NT), 0, st, P);
+    if (P.drop.thresh) hipLaunchKernelGGL((k_sparse_attn<DT, D, true, true, FULL>), dim3(n_wg), dim3(ATT_ROW_NT), 0, st, P);
+    else hipLaunchKernelGGL((k_sparse_attn<DT, D, true, false, FULL>), dim3(n_wg), dim3(ATT_ROW_NT), 0, st, P);
     return sah_launch_status("sah_sparse_attention");
   }
   int rc;
@@ -120,25 +129,34 @@ static int att_launch(const sah_attention_args* a, const att_params& P, bool tim
     sah_timed timed("k_sparse_attn", a->stream, timing);
     const int n_tiles = (a->rows.n_rows / G) * P.n_split;
     const int n_wg = (n_tiles + ATT_XCDS - 1) / ATT_XCDS * ATT_XCDS * G;
-    if (P.drop.thresh) hipLaunchKernelGGL((k_sparse_attn<DT, D, false, true>), dim3(n_wg), dim3(ATT_NT), 0, st, P);
-    else hipLaunchKernelGGL((k_sparse_attn<DT, D, false, false>), dim3(n_wg), dim3(ATT_NT), 0, st, P);
+    if (P.drop.thresh) hipLaunchKernelGGL((k_sparse_attn<DT, D, false, true, FULL>), dim3(n_wg), dim3(ATT_NT), 0, st, P);
+    else hipLaunchKernelGGL((k_sparse_attn<DT, D, false, false, FULL>), dim3(n_wg), dim3(ATT_NT), 0, st, P);
     rc = sah_launch_status("sah_sparse_attention");
   }
   if (rc) return rc;
   sah_timed timed("k_attn_combine", a->stream, timing);
   hipLaunchKernelGGL((k_attn_combine<DT, D>), dim3(a->rows.n_rows), dim3(D < 64 ? 64 : D), 0, st,
-                     (const float*)a->work, P.n_split, a->Hq, a->Lq, a->sinks, a->out, a->stats_out);
+                     (const float*)a->work, P.n_split, a->Hq, a->Lq, a->D, a->sinks, a->out, a->stats_out);
   return sah_launch_status("sah_sparse_attention(combine)");
 }
 
 template <int DT>
 static int att_dispatch_d(const sah_attention_args* a, const att_params& P, bool timing) {
   switch (a->D) {
-    case 16: return att_launch<DT, 16>(a, P, timing);
-    case 32: return att_launch<DT, 32>(a, P, timing);
-    case 64: return att_launch<DT, 64>(a, P, timing);
-    case 128: return att_launch<DT, 128>(a, P, timing);
-    default: return sah_fail(SAH_ESHAPE, "sah_sparse_attention: head_dim %d not in {16,32,64,128}", a->D);
+    case 16: return att_launch<DT, 16, true>(a, P, timing);
+    case 32: return att_launch<DT, 32, true>(a, P, timing);
+    case 64: return att_launch<DT, 64, true>(a, P, timing);
+    case 128: return att_launch<DT, 128, true>(a, P, timing);
+    default: break;
+  }
+  // any other multiple of 8 up to 256: the next power of two, the lanes beyond head_dim idle
+  switch (att_pad_dim(a->D)) {
+    case 16: return att_launch<DT, 16, false>(a, P, timing);
+    case 32: return att_launch<DT, 32, false>(a, P, timing);
+    case 64: return att_launch<DT, 64, false>(a, P, timing);
+    case 128: return att_launch<DT, 128, false>(a, P, timing);
+    case 256: return att_launch<DT, 256, false>(a, P, timing);
+    default: return sah_fail(SAH_ESHAPE, "sah_sparse_attention: head_dim %d is not a multiple of 8 in [8, 256]", a->D);
   }
 }
 
@@ -187,6 +205,7 @@ int att_prepare(const sah_attention_args* a, att_params& P) {
   P.v = a->v; P.vs_b = a->vs_b; P.vs_h = a->vs_h; P.vs_l = a->vs_l;
   P.amask = a->amask; P.ms_b = a->ms_b; P.ms_h = a->ms_h; P.ms_l = a->ms_l;
   P.Hq = a->Hq; P.Hkv = a->Hkv; P.Lq = a->Lq; P.Lk = a->Lk;
+  P.d_real = a->D;
   P.scaling = a->scaling; P.unit_inv_w = a->unit_inv_w;
   P.dense = a->dense ? 1 : (a->closed_form ? 2 : 0);
   P.n_split = att_use_row_form(a->rows.n_rows, max_cnt) ? 0 : att_pick_split(a->rows.n_rows, max_cnt);  // 0: whole rows
@@ -196,7 +215,8 @@ int att_prepare(const sah_attention_args* a, att_params& P) {
   P.logits_pitch = a->dense ? a->Lk : a->rows.cap;
   if (!sah_dropout_fill(a->dropout_p, a->dropout_seed, a->dropout_offset, P.drop))
     return sah_fail(SAH_EINVAL, "sah_sparse_attention: dropout_p %g not in [0, 1)", (double)a->dropout_p);
-  const int64_t need = (int64_t)a->rows.n_rows * P.n_split * (a->D + 2);
+  if (!att_pad_dim(a->D)) return sah_fail(SAH_ESHAPE, "sah_sparse_attention: head_dim %d is not a multiple of 8 in [8, 256]", a->D);
+  const int64_t need = (int64_t)a->rows.n_rows * P.n_split * (att_pad_dim(a->D) + 2);
   if (a->work_floats < need)
     return sah_fail(SAH_ECAPACITY, "sah_sparse_attention: work has %lld floats, need %lld", (long long)a->work_floats,
                     (long long)need);

@@ -17,6 +17,7 @@ struct att_params {
   const void* v; int64_t vs_b, vs_h, vs_l;
   const void* amask; int64_t ms_b, ms_h, ms_l;
   int Hq, Hkv, Lq, Lk;
+  int d_real;  // head_dim; the kernels' D is d_real padded to a power of two (lanes beyond d_real carry zeros)
   float scaling, unit_inv_w;
   int dense;
   int closed_sink, closed_lo, closed_cnt;  // dense == 2: entries [0, closed_sink) are columns [0, closed_sink), the rest start at closed_lo
@@ -38,11 +39,12 @@ __device__ __forceinline__ float att_exp(float x) {
 
 template <int LPK>
 __device__ __forceinline__ float att_group_sum(float v) {
-  // sum over each aligned group of LPK lanes (LPK in {2,4,8,16})
+  // sum over each aligned group of LPK lanes (LPK in {2,4,8,16,32})
   v += sah_dpp<0xB1>(v);
   if (LPK >= 4) v += sah_dpp<0x4E>(v);
   if (LPK >= 8) v += sah_dpp<0x141>(v);
   if (LPK >= 16) v += sah_dpp<0x140>(v);
+  if (LPK >= 32) v += __shfl_xor(v, 16);
   return v;
 }
 
@@ -88,7 +90,7 @@ __device__ __forceinline__ void att_unpack(const att_raw<DT>& r, float (&o)[8]) 
 // so the merge costs about two memory round trips whatever the number of splits. Every thread of the
 // workgroup calls it (one barrier inside); thread d < D produces output element d.
 template <int DT, int D>
-__device__ __forceinline__ void att_combine_row(const float* work, int n_split, int r, int Hq, int Lq, const float* sinks,
+__device__ __forceinline__ void att_combine_row(const float* work, int n_split, int r, int Hq, int Lq, int d_real, const float* sinks,
                                                 void* out, float* stats, float* s_m, float* s_l) {
   const int d = threadIdx.x;
   const float* w = work + (int64_t)r * n_split * (D + 2);
@@ -128,7 +130,7 @@ __device__ __forceinline__ void att_combine_row(const float* work, int n_split, 
     a *= sc;
     den = L * sc + att_exp<DT>(sk - Mf);
   }
-  if (d < D) sah_store<DT>(out, (((int64_t)b * Lq + qi) * Hq + h) * D + d, a / den);
+  if (d < d_real) sah_store<DT>(out, (((int64_t)b * Lq + qi) * Hq + h) * d_real + d, a / den);
   if (stats && d == 0) {
     stats[2 * (int64_t)r] = Mf;
     stats[2 * (int64_t)r + 1] = den;
@@ -158,7 +160,9 @@ struct att_batch {
 };
 
 // the calling lane's slice (8 elements) of the rows of head (b, hk): addresses, and the query's elements
-template <int DT, int D>
+// FULL: head_dim is D itself; otherwise D is head_dim padded to a power of two and the lanes of a key beyond head_dim
+// load nothing and carry zeros
+template <int DT, int D, bool FULL = true>
 struct att_lane {
   static constexpr int LPK = D / 8;            // lanes per key
   static constexpr int KPI = SAH_WAVE / LPK;   // keys per wave iteration
@@ -167,17 +171,24 @@ struct att_lane {
   const char* vbase;
   int64_t krow, vrow;
   int sub, grp;  // which 8-element slice of the row, which key of the iteration
+  bool live;     // this lane's slice lies inside head_dim
   __device__ __forceinline__ att_lane(const att_params& P, int b, int hk) {
     const int lane = threadIdx.x & (SAH_WAVE - 1);
     sub = lane % LPK;
     grp = lane / LPK;
+    live = FULL || sub * 8 < P.d_real;
     kbase = (const char*)P.k + ((int64_t)b * P.ks_b + (int64_t)hk * P.ks_h + sub * 8) * ES;
     vbase = (const char*)P.v + ((int64_t)b * P.vs_b + (int64_t)hk * P.vs_h + sub * 8) * ES;
     krow = P.ks_l * ES;
     vrow = P.vs_l * ES;
   }
   __device__ __forceinline__ void load_q(const att_params& P, int b, int h, int qi, float (&qv)[8]) const {
-    sah_load8<DT>(P.q, (int64_t)b * P.qs_b + (int64_t)h * P.qs_h + (int64_t)qi * P.qs_l + sub * 8, qv);
+    if (FULL || live) {
+      sah_load8<DT>(P.q, (int64_t)b * P.qs_b + (int64_t)h * P.qs_h + (int64_t)qi * P.qs_l + sub * 8, qv);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) qv[e] = 0.f;
+    }
   }
   // puts the batch's 2 * UB row loads on their way
   template <int UB>
@@ -185,8 +196,12 @@ struct att_lane {
 #pragma unroll
     for (int u = 0; u < UB; ++u) {
       const int safe = B.id[u] >= 0 ? B.id[u] : 0;
-      att_load_raw<DT>(kbase + (int64_t)safe * krow, B.kr[u]);
-      att_load_raw<DT>(vbase + (int64_t)safe * vrow, B.vr[u]);
+      if (FULL || live) {
+        att_load_raw<DT>(kbase + (int64_t)safe * krow, B.kr[u]);
+        att_load_raw<DT>(vbase + (int64_t)safe * vrow, B.vr[u]);
+      } else {
+        B.kr[u].lo = B.kr[u].hi = B.vr[u].lo = B.vr[u].hi = make_uint4(0u, 0u, 0u, 0u);
+      }
     }
   }
   // the batch's logits (scaled, plus the additive mask; -inf for a lane without a key), and their maximum over the wave
@@ -248,10 +263,10 @@ struct att_lane {
 // decode step): their tests and code stay out. A caller whose column list lives in LDS hands col_of a pointer the
 // compiler can see to be LDS: through a generic pointer every read of the list would be a flat load, which waits for
 // all of the wave's outstanding row loads as well.
-template <int DT, int D, bool DROP = false, bool PLAIN = false, typename ColOf, typename InvWOf>
+template <int DT, int D, bool DROP = false, bool PLAIN = false, bool FULL = true, typename ColOf, typename InvWOf>
 __device__ __forceinline__ void att_walk(const att_params& P, int r, int b, int h, int hk, int qi, int first, int bound,
                                          int stride, ColOf col_of, InvWOf inv_w_of, att_wave_state& st) {
-  typedef att_lane<DT, D> lane_t;
+  typedef att_lane<DT, D, FULL> lane_t;
   constexpr int KPI = lane_t::KPI;
   constexpr int IT = SAH_WAVE / KPI;    // iterations per 64-key wave slice
   constexpr int UB = IT < 4 ? IT : 4;   // iterations per batch
@@ -351,7 +366,7 @@ __device__ __forceinline__ void att_store_row(const att_params& P, int r, int b,
     a *= rs;
     den = l * rs + att_exp<DT>(sk - Mf);
   }
-  if (tid < D) sah_store<DT>(P.out, (((int64_t)b * P.Lq + qi) * P.Hq + h) * D + tid, a / den);
+  if (tid < P.d_real) sah_store<DT>(P.out, (((int64_t)b * P.Lq + qi) * P.Hq + h) * P.d_real + tid, a / den);
   if (P.stats && tid == 0) {
     P.stats[2 * (int64_t)r] = Mf;
     P.stats[2 * (int64_t)r + 1] = den;
@@ -363,7 +378,7 @@ __device__ __forceinline__ void att_store_row(const att_params& P, int r, int b,
 // ROW = true: a workgroup of 16 waves handles a whole row, every wave an equal share of the row's entries,
 //   and merges the 16 partial results itself: no workspace, no second kernel, every CU gets the same
 //   amount of work when there are at least as many rows as CUs.
-template <int DT, int D, bool ROW, bool DROP = false>
+template <int DT, int D, bool ROW, bool DROP = false, bool FULL = true>
 __device__ __forceinline__ void att_tile(const att_params& P, int r, int b, int h, int hk, int qi, int split, int n_split,
                                          const int* cols_known, int cnt_known,
                                          float (&s_m)[(ROW ? ATT_ROW_NT : ATT_NT) / SAH_WAVE],
@@ -408,7 +423,7 @@ __device__ __forceinline__ void att_tile(const att_params& P, int r, int b, int 
   const float* wts = (!P.dense && P.rows.w) ? P.rows.w + (int64_t)r * P.rows.cap : nullptr;
   att_wave_state st;
   st.clear();
-  att_walk<DT, D, DROP>(
+  att_walk<DT, D, DROP, false, FULL>(
       P, r, b, h, hk, qi, first, bound, stride,
       [&](int i) { return P.dense == 1 ? i : (P.dense == 2 ? (i < P.closed_sink ? i : P.closed_lo + (i - P.closed_sink)) : cols[i]); },
       // the reference evaluates 1/(w + 1e-6) in the mask dtype (utils/mask.py:737-740)

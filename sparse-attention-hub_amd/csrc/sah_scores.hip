@@ -23,6 +23,7 @@ struct qk_params {
   const void* k; int64_t ks_b, ks_h, ks_l;
   const void* amask; int64_t ms_b, ms_h, ms_l;
   int B, Hq, Hkv, Lq, Lk;
+  int d_real;  // head_dim; the kernel's D is d_real padded to a power of two
   void* keys_out; int64_t key_pitch;
   int iters;  // tiles of SC_TILE keys per workgroup
 };
@@ -121,7 +122,9 @@ __device__ __forceinline__ float sc_reduce4(float d0, float d1, float d2, float 
 }
 
 // AM: an additive attention mask is given (P.amask); without one the scoring loop holds no load but the rows'
-template <int DT, int D, bool AM>
+// FULL: head_dim is D itself; otherwise D is head_dim padded to a power of two: the lanes of a key beyond head_dim
+// carry a zero query slice (and re-read the row's first slice, so that no load sits behind a condition)
+template <int DT, int D, bool AM, bool FULL>
 __global__ __launch_bounds__(SC_NT) void k_qk_scores(qk_params P) {
   sah_touch_kernargs<sizeof(qk_params)>();
   constexpr int LPK = D / 8;
@@ -143,6 +146,8 @@ __global__ __launch_bounds__(SC_NT) void k_qk_scores(qk_params P) {
   const int b = bhk / P.Hkv;
   const int v0 = blockIdx.z * SC_NQ;  // first query vector (of G*Lq) handled here
   const int nvec = G * P.Lq;
+  const bool in_dim = FULL || sub * 8 < P.d_real;
+  const int sub_k = in_dim ? sub : 0;
 
   sc_raw<DT> qv[SC_NQ];
   int row[SC_NQ];
@@ -156,13 +161,21 @@ __global__ __launch_bounds__(SC_NT) void k_qk_scores(qk_params P) {
     if (!live) v = nvec - 1;  // computed and dropped
     const int h = hk * G + v / P.Lq;
     const int qi = v % P.Lq;
-    sc_load<DT>((const char*)P.q + ((int64_t)b * P.qs_b + (int64_t)h * P.qs_h + (int64_t)qi * P.qs_l + sub * 8) * ES, qv[i]);
+    sc_load<DT>((const char*)P.q + ((int64_t)b * P.qs_b + (int64_t)h * P.qs_h + (int64_t)qi * P.qs_l + sub_k * 8) * ES, qv[i]);
+    if (!FULL && !in_dim) {
+      if constexpr (DT == SAH_F32) {
+        qv[i].a = make_float4(0.f, 0.f, 0.f, 0.f);
+        qv[i].b = make_float4(0.f, 0.f, 0.f, 0.f);
+      } else {
+        qv[i].a = make_uint4(0u, 0u, 0u, 0u);
+      }
+    }
     if (live) {
       row[i] = (b * P.Hq + h) * P.Lq + qi;
       if (AM) moff[i] = (int64_t)b * P.ms_b + (int64_t)h * P.ms_h + (int64_t)qi * P.ms_l;
     }
   }
-  const char* kbase = (const char*)P.k + ((int64_t)b * P.ks_b + (int64_t)hk * P.ks_h + sub * 8) * ES;
+  const char* kbase = (const char*)P.k + ((int64_t)b * P.ks_b + (int64_t)hk * P.ks_h + sub_k * 8) * ES;
   const int64_t krow = P.ks_l * ES;
   // which of the four totals this lane ends up with after sc_reduce4
   const int mine = FAST4 ? (2 * (sub & 1) + ((sub >> 1) & 1)) : 0;
@@ -260,7 +273,7 @@ __global__ __launch_bounds__(SC_NT) void k_qk_scores(qk_params P) {
   }
 }
 
-template <int DT, int D>
+template <int DT, int D, bool FULL>
 static int qk_launch(const sah_qk_scores_args* a, const qk_params& P) {
   const int G = a->Hq / a->Hkv;
   const int nvec = G * a->Lq;
@@ -273,20 +286,27 @@ static int qk_launch(const sah_qk_scores_args* a, const qk_params& P) {
   Q.iters = iters;
   dim3 g((unsigned)((tiles + iters - 1) / iters), a->B * a->Hkv, (nvec + SC_NQ - 1) / SC_NQ);
   sah_timed timed("k_qk_scores", a->stream);
-  if (a->amask) hipLaunchKernelGGL((k_qk_scores<DT, D, true>), g, dim3(SC_NT), 0, (hipStream_t)a->stream, Q);
-  else hipLaunchKernelGGL((k_qk_scores<DT, D, false>), g, dim3(SC_NT), 0, (hipStream_t)a->stream, Q);
+  if (a->amask) hipLaunchKernelGGL((k_qk_scores<DT, D, true, FULL>), g, dim3(SC_NT), 0, (hipStream_t)a->stream, Q);
+  else hipLaunchKernelGGL((k_qk_scores<DT, D, false, FULL>), g, dim3(SC_NT), 0, (hipStream_t)a->stream, Q);
   return sah_launch_status("sah_qk_scores");
 }
 
 template <int DT>
 static int qk_dispatch_d(const sah_qk_scores_args* a, const qk_params& P) {
   switch (a->D) {
-    case 16: return qk_launch<DT, 16>(a, P);
-    case 32: return qk_launch<DT, 32>(a, P);
-    case 64: return qk_launch<DT, 64>(a, P);
-    case 128: return qk_launch<DT, 128>(a, P);
-    default: return sah_fail(SAH_ESHAPE, "sah_qk_scores: head_dim %d not in {16,32,64,128}", a->D);
+    case 16: return qk_launch<DT, 16, true>(a, P);
+    case 32: return qk_launch<DT, 32, true>(a, P);
+    case 64: return qk_launch<DT, 64, true>(a, P);
+    case 128: return qk_launch<DT, 128, true>(a, P);
+    default: break;
   }
+  // any other multiple of 8 below 128: the next power of two, the lanes beyond head_dim multiply zeros
+  if (a->D <= 0 || a->D % 8 || a->D > 128)
+    return sah_fail(SAH_ESHAPE, "sah_qk_scores: head_dim %d is not a multiple of 8 in [8, 128]", a->D);
+  if (a->D < 16) return qk_launch<DT, 16, false>(a, P);
+  if (a->D < 32) return qk_launch<DT, 32, false>(a, P);
+  if (a->D < 64) return qk_launch<DT, 64, false>(a, P);
+  return qk_launch<DT, 128, false>(a, P);
 }
 
 extern "C" int sah_qk_scores(const sah_qk_scores_args* a) {
@@ -306,6 +326,7 @@ extern "C" int sah_qk_scores(const sah_qk_scores_args* a) {
   P.k = a->k; P.ks_b = a->ks_b; P.ks_h = a->ks_h; P.ks_l = a->ks_l;
   P.amask = a->amask; P.ms_b = a->ms_b; P.ms_h = a->ms_h; P.ms_l = a->ms_l;
   P.B = a->B; P.Hq = a->Hq; P.Hkv = a->Hkv; P.Lq = a->Lq; P.Lk = a->Lk;
+  P.d_real = a->D;
   P.keys_out = a->keys_out; P.key_pitch = a->key_pitch;
   switch (a->dtype) {
     case SAH_F32: return qk_dispatch_d<SAH_F32>(a, P);

@@ -54,6 +54,24 @@ def test_sink_local_chain(cuda, dtype, D):
                [("sink", 4), ("local", 8)], 2, 4, 2, 1, 333, D, dtype)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("D", [8, 24, 80, 96, 112, 160, 256])
+def test_head_dims_that_are_not_16_32_64_128(cuda, dtype, D):
+    """The reference's masked attention takes any head_dim (utils/mask_attention_utils.py:406-491); the kernels pad a
+    head_dim that is a multiple of 8 up to 256 to the next power of two: Sink + Local rows (whole-row form), dense
+    attention with sink logits (split form and merge kernel), and - up to 128 - the OracleTopK scoring pass."""
+    sa = _sa()
+    _run_chain(cuda, [sa.SinkMaskerConfig(sink_size=4), sa.LocalMaskerConfig(window_size=8)],
+               [("sink", 4), ("local", 8)], 2, 4, 2, 1, 333, D, dtype)
+    _run_chain(cuda, [], [], 1, 4, 2, 2, 1500, D, dtype, sinks=torch.tensor([0.1, -0.3, 0.5, 1.0]))
+    if D <= 128:
+        _run_chain(cuda, [sa.SinkMaskerConfig(sink_size=16), sa.LocalMaskerConfig(window_size=32), sa.OracleTopKConfig(heavy_size=40)],
+                   [("sink", 16), ("local", 32), ("oracle_topk", 40)], 2, 8, 2, 1, 900, D, dtype)
+    else:
+        with pytest.raises(ValueError, match="head_dim"):
+            _run_chain(cuda, [sa.OracleTopKConfig(heavy_size=40)], [("oracle_topk", 40)], 1, 4, 2, 1, 300, D, dtype)
+
+
 def test_sink_local_index_form_is_bit_exact(cuda):
     sa = _sa()
     B, Hq, Lq, Lk = 2, 4, 3, 70
