@@ -408,6 +408,9 @@ typedef struct sah_attention_args {
   float dropout_p;
   uint64_t dropout_seed;
   uint64_t dropout_offset;
+  int32_t dropout_numerator_only; /* != 0: dropped entries leave the denominator as it is, i.e. dropout of the
+                                     normalised probabilities, what the reference's dense path does
+                                     (scaled_dot_product_attention with dropout_p, mask_attention_utils.py:40-52) */
 } sah_attention_args;
 int64_t sah_sparse_attention_work_floats(int32_t n_rows, int32_t max_cnt, int32_t D);
 int sah_sparse_attention(const sah_attention_args* a);

@@ -548,13 +548,16 @@ def dropout_keep(seed: int, offset: int, n_rows: int, n_keys: int, p: float) -> 
 def masked_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, attention_mask: Optional[torch.Tensor],
                      sinks: Optional[torch.Tensor], scaling: float, mask: OMask,
                      accumulate: torch.dtype = torch.float32,
-                     dropout: Optional[Tuple[float, int, int]] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+                     dropout: Optional[Tuple[float, int, int]] = None,
+                     dropout_numerator_only: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
     """(out (B, Lq, Hq, D), weights (B, Hq, Lq, Lk)) in the query dtype —
     mask_attention_utils.py:187-240 (exp weights), :357-402 (sink logit), :406-491 (num/den).
     `accumulate=torch.float64` gives a high-precision variant for tolerance studies.
     `dropout` = (p, seed, offset): training-mode dropout of the exp weights (:234-238, torch.nn.functional.dropout:
     an element is zeroed with probability p, the others are scaled by 1 / (1 - p)), with the element's fate drawn
-    from Philox (dropout_keep) instead of torch's generator."""
+    from Philox (dropout_keep) instead of torch's generator. `dropout_numerator_only`: the dropped entries stay in the
+    denominator - dropout of the normalised probabilities, what scaled_dot_product_attention(dropout_p=...) does on the
+    reference's dense path (:40-52)."""
     G = q.shape[1] // k.shape[1]
     kk = repeat_kv(k, G).to(accumulate)
     vv = repeat_kv(v, G).to(accumulate)
@@ -569,9 +572,14 @@ def masked_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, attentio
         p, seed, offset = dropout
         B, H, Q, Lk = e.shape
         keep = dropout_keep(seed, offset, B * H * Q, Lk, p).view(B, H, Q, Lk)
+        den_e = e
         e = e * keep.to(accumulate) * (1.0 / (1.0 - float(torch.tensor(p, dtype=torch.float32))))
+        if not dropout_numerator_only:
+            den_e = e
+    else:
+        den_e = e
     num = torch.matmul(e, vv)
-    den = e.sum(dim=-1, keepdim=True)
+    den = den_e.sum(dim=-1, keepdim=True)
     if sinks is not None:
         B, H, Q = q.shape[0], q.shape[1], q.shape[2]
         srow = sinks.view(1, H, 1, 1).expand(B, H, Q, 1).to(accumulate)

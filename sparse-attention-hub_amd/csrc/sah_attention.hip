@@ -213,6 +213,7 @@ int att_prepare(const sah_attention_args* a, att_params& P) {
   P.sinks = a->sinks; P.out = a->out; P.stats = a->stats_out;
   P.logits_out = a->logits_out;
   P.logits_pitch = a->dense ? a->Lk : a->rows.cap;
+  P.drop_num_only = a->dropout_numerator_only ? 1 : 0;
   if (!sah_dropout_fill(a->dropout_p, a->dropout_seed, a->dropout_offset, P.drop))
     return sah_fail(SAH_EINVAL, "sah_sparse_attention: dropout_p %g not in [0, 1)", (double)a->dropout_p);
   if (!att_pad_dim(a->D)) return sah_fail(SAH_ESHAPE, "sah_sparse_attention: head_dim %d is not a multiple of 8 in [8, 256]", a->D);

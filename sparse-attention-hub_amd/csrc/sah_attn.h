@@ -29,6 +29,7 @@ struct att_params {
   float* logits_out;
   int64_t logits_pitch;
   sah_dropout drop;
+  int drop_num_only;  // dropout leaves the softmax denominator alone (dropout of the normalised probabilities)
 };
 
 // exact expf for fp32 storage (1e-5 output tolerance), hardware exp2 path otherwise
@@ -231,9 +232,10 @@ struct att_lane {
     return mb;
   }
   // the online-softmax step of a batch: iw[u] is the inverse weight of the lane's key in iteration u
+  // (iw_den: the inverse weights that enter the denominator - the same unless dropout spares it)
   template <int UB>
   __device__ __forceinline__ void accumulate(const att_batch<DT, UB>& B, const float (&z)[UB], float mb, const float (&iw)[UB],
-                                             att_wave_state& st) const {
+                                             const float (&iw_den)[UB], att_wave_state& st) const {
     const float m_new = fmaxf(st.m_run, mb);
     if (m_new != -INFINITY) {
       const float rescale = (st.m_run == -INFINITY) ? 0.f : att_exp<DT>(st.m_run - m_new);
@@ -243,9 +245,13 @@ struct att_lane {
       st.m_run = m_new;
 #pragma unroll
       for (int u = 0; u < UB; ++u) {
-        float p = 0.f;
-        if (z[u] != -INFINITY) p = att_exp<DT>(z[u] - m_new) * iw[u];
-        st.l_run += p;
+        float p = 0.f, pd = 0.f;
+        if (z[u] != -INFINITY) {
+          const float e = att_exp<DT>(z[u] - m_new);
+          p = e * iw[u];
+          pd = e * iw_den[u];
+        }
+        st.l_run += pd;
         float vf[8];
         att_unpack<DT>(B.vr[u], vf);
 #pragma unroll
@@ -280,12 +286,16 @@ __device__ __forceinline__ void att_walk(const att_params& P, int r, int b, int 
     // one column (and its inverse weight) per lane: this wave's next 64 keys
     const int my = cbase + lane;
     int idx_l = -1;
-    float invw_l = P.unit_inv_w;
+    float invw_l = P.unit_inv_w, invw_den_l = P.unit_inv_w;
     if (my < bound) {
       idx_l = col_of(my);
       invw_l = inv_w_of(my);
       if (idx_l < 0 || idx_l >= P.Lk) idx_l = -1;
-      if (DROP && idx_l >= 0) invw_l *= P.drop.factor(r, idx_l);
+      invw_den_l = invw_l;
+      if (DROP && idx_l >= 0) {
+        invw_l *= P.drop.factor(r, idx_l);
+        if (!P.drop_num_only) invw_den_l = invw_l;
+      }
     }
 #pragma unroll
     for (int ib = 0; ib < IT; ib += UB) {
@@ -303,10 +313,13 @@ __device__ __forceinline__ void att_walk(const att_params& P, int r, int b, int 
           if (pos < bound) P.logits_out[(int64_t)r * P.logits_pitch + pos] = z[u];
         }
       }
-      float iw[UB];
+      float iw[UB], iw_den[UB];
 #pragma unroll
-      for (int u = 0; u < UB; ++u) iw[u] = __shfl(invw_l, (ib + u) * KPI + L.grp);
-      L.accumulate(B, z, mb, iw, st);
+      for (int u = 0; u < UB; ++u) {
+        iw[u] = __shfl(invw_l, (ib + u) * KPI + L.grp);
+        iw_den[u] = DROP ? __shfl(invw_den_l, (ib + u) * KPI + L.grp) : iw[u];
+      }
+      L.accumulate(B, z, mb, iw, iw_den, st);
     }
   }
 }

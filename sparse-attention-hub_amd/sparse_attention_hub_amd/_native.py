@@ -293,6 +293,7 @@ class AttentionArgs(C.Structure):
         ("dropout_p", C.c_float),
         ("dropout_seed", C.c_uint64),
         ("dropout_offset", C.c_uint64),
+        ("dropout_numerator_only", C.c_int32),
     ]
 
 

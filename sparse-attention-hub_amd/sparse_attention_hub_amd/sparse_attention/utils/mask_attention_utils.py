@@ -12,7 +12,6 @@ from __future__ import annotations
 
 from typing import Any, Dict, Optional, Tuple, Union
 
-import itertools
 
 import numpy as np
 import torch
@@ -112,6 +111,7 @@ def _run_attention(
     out: Optional[torch.Tensor] = None,
     return_stats: bool = False,
     dropout: Tuple[float, int, int] = (0.0, 0, 0),
+    dropout_numerator_only: bool = False,
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """rows=None => dense attention over all keys. `return_stats`: the second value is the kernel's
     fp32 (n_rows, 2) tensor of (largest logit among the row's entries, softmax denominator relative to it)
@@ -172,7 +172,7 @@ def _run_attention(
         None if logits is None else logits.data_ptr(),
         None if stats is None else stats.data_ptr(),
         N.stream_ptr(dev),
-        dropout[0], dropout[1], dropout[2],
+        dropout[0], dropout[1], dropout[2], int(dropout_numerator_only),
     )
     N.call("sah_sparse_attention", args)
     if return_stats:
@@ -188,19 +188,18 @@ def _run_attention(
     return out, weights
 
 
-_DROPOUT_CALLS = itertools.count()
-
-
 def _training_dropout(module: Optional[nn.Module], dropout: float) -> Tuple[float, int, int]:
     """(p, seed, offset) for the attention kernel: dropout of the exp weights applies in training mode only
     (reference: mask_attention_utils.py:234-238, `module.training`). The kernel draws with Philox4x32-10 keyed by
     torch's seed and a per-call offset where the reference draws from torch's generator: another stream of the same
-    distribution, reseeded by `torch.manual_seed` as well."""
+    distribution. The offset is itself a draw from torch's default generator, so `torch.manual_seed(s)` followed by the
+    same calls gives the same dropout masks again, as it does in the reference."""
     if not (dropout > 0.0 and module is not None and getattr(module, "training", False)):
         return 0.0, 0, 0
     if not dropout < 1.0:
         raise ValueError(f"dropout probability has to be below 1 for the attention kernel, but got {dropout}")
-    return float(dropout), int(torch.initial_seed()) & 0xFFFFFFFFFFFFFFFF, next(_DROPOUT_CALLS)
+    offset = int(torch.randint(0, 2 ** 62, (1,), dtype=torch.int64).item())
+    return float(dropout), int(torch.initial_seed()) & 0xFFFFFFFFFFFFFFFF, offset
 
 
 def get_true_attention_output(
@@ -213,9 +212,11 @@ def get_true_attention_output(
     dropout: float,
     **kwargs: Dict[str, Any],
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
-    """Dense attention output (B, Lq, Hq, D) (reference: mask_attention_utils.py:11-70)."""
+    """Dense attention output (B, Lq, Hq, D) (reference: mask_attention_utils.py:11-70). In training mode the
+    reference's dense path is scaled_dot_product_attention with dropout_p (:40-52): dropout of the normalised
+    probabilities, i.e. a dropped entry leaves the softmax denominator as it is."""
     out, _ = _run_attention(queries, keys, values, attention_mask, None, scaling, None, False,
-                            dropout=_training_dropout(module, dropout))
+                            dropout=_training_dropout(module, dropout), dropout_numerator_only=True)
     return out, None
 
 

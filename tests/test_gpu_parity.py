@@ -140,8 +140,6 @@ def test_training_mode_dropout_follows_the_oracle_stream(cuda, dtype):
     weights): the kernels draw an entry's fate from Philox keyed by torch's seed and a per-call offset, the oracle
     draws the same stream, so outputs and dense probabilities agree entry by entry, with a sparse mask, a sink logit
     and the dense path; eval mode and p = 0 leave everything as it was; p >= 1 is refused."""
-    import itertools
-
     from sparse_attention_hub_amd.sparse_attention.utils import mask_attention_utils as mau
 
     sa = _sa()
@@ -155,18 +153,37 @@ def test_training_mode_dropout_follows_the_oracle_stream(cuda, dtype):
     evalm.eval()
     torch.manual_seed(1234)
     seed = torch.initial_seed()
+    # the per-call offsets are draws from torch's default generator: the same numbers a generator seeded alike gives
+    expect = torch.Generator().manual_seed(1234)
     tol_w = 1e-6 if dtype == torch.float32 else 1e-2
     outs = []
     for call, (c, sp) in enumerate(((cfgs, specs), (cfgs, specs), ([], []))):    # the third: dense attention
-        mau._DROPOUT_CALLS = itertools.count(40 + call)
+        offset = int(torch.randint(0, 2 ** 62, (1,), dtype=torch.int64, generator=expect).item())
         ra = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=c))
         out, w = ra.custom_attention(train, q.to(cuda), k.to(cuda), v.to(cuda), None, D ** -0.5, p, sparse_meta_data={},
                                      layer_idx=0, s_aux=sinks.to(cuda))
-        oo, ow, _ = O.research_attention(sp, q, k, v, None, D ** -0.5, sinks, dropout=(p, seed, 40 + call))
+        oo, ow, _ = O.research_attention(sp, q, k, v, None, D ** -0.5, sinks, dropout=(p, seed, offset))
         assert rel_err(out, oo) < TOL[dtype], call
         assert torch.equal(w.cpu() != 0, ow != 0), call                        # the same entries survive
         assert (w.float().cpu() - ow.float()).abs().max().item() < tol_w
         outs.append(out)
+    # re-seeding reproduces the dropout masks (as torch's generator does for the reference)
+    torch.manual_seed(1234)
+    ra = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(masker_configs=cfgs))
+    again, _ = ra.custom_attention(train, q.to(cuda), k.to(cuda), v.to(cuda), None, D ** -0.5, p, sparse_meta_data={},
+                                   layer_idx=0, s_aux=sinks.to(cuda))
+    assert torch.equal(again, outs[0])
+    expect = torch.Generator().manual_seed(1234)
+    torch.randint(0, 2 ** 62, (1,), dtype=torch.int64, generator=expect)         # the draw of the call above
+    # the "true" dense attention of the error metric: dropout of the normalised probabilities (SDPA with dropout_p on
+    # the reference's dense path, mask_attention_utils.py:40-52): the denominator keeps the dropped entries
+    offset = int(torch.randint(0, 2 ** 62, (1,), dtype=torch.int64, generator=expect).item())
+    true_out, _ = mau.get_true_attention_output(train, q.to(cuda), k.to(cuda), v.to(cuda), None, D ** -0.5, p)
+    empty = O.OMask.empty((B, Hq, Lq, Lk), dtype)
+    want, _ = O.masked_attention(q, k, v, None, None, D ** -0.5, empty, dropout=(p, seed, offset), dropout_numerator_only=True)
+    assert rel_err(true_out, want) < TOL[dtype]
+    both, _ = O.masked_attention(q, k, v, None, None, D ** -0.5, empty, dropout=(p, seed, offset))
+    assert rel_err(true_out, both) > 10 * TOL[dtype] or dtype == torch.bfloat16   # and it is not the other form
     assert not torch.equal(outs[0], outs[1])                                     # every call draws anew
     # about a quarter of the entries of a row are gone
     kept = float((w != 0).float().mean())

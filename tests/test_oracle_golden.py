@@ -655,3 +655,24 @@ def test_masked_attention_dropout_has_the_form_of_torch_dropout():
     want = (torch.matmul(e, v.double()) * sc / den).transpose(1, 2)
     assert torch.allclose(out1.double(), want, rtol=1e-5, atol=1e-6)
     assert not torch.allclose(out1, out0, rtol=1e-3)
+
+
+def test_masked_attention_dropout_of_the_normalised_probabilities():
+    """The reference's dense path is scaled_dot_product_attention(dropout_p=...) (mask_attention_utils.py:40-52):
+    softmax first, then dropout of the probabilities, then the product with V. `dropout_numerator_only` must be exactly
+    that: torch.softmax in fp64, the oracle's own keep mask scaled by 1 / (1 - p), times V - and differ from the form that
+    drops before the denominator."""
+    g = torch.Generator().manual_seed(4)
+    B, H, Lq, Lk, D, p = 1, 2, 2, 40, 8, 0.3
+    q, k, v = (torch.randn(B, H, n, D, generator=g) for n in (Lq, Lk, Lk))
+    empty = O.OMask.empty((B, H, Lq, Lk), torch.float32)
+    drop = (p, 21, 9)
+    out, w = O.masked_attention(q, k, v, None, None, 0.5, empty, dropout=drop, dropout_numerator_only=True)
+    keep = O.dropout_keep(21, 9, B * H * Lq, Lk, p).view(B, H, Lq, Lk)
+    probs = torch.softmax(torch.matmul(q.double(), k.double().transpose(2, 3)) * 0.5, dim=-1)
+    dropped = probs * keep.double() / (1.0 - float(torch.tensor(p, dtype=torch.float32)))
+    want = torch.matmul(dropped, v.double()).transpose(1, 2)
+    assert torch.allclose(out.double(), want, rtol=1e-5, atol=1e-6)
+    assert torch.allclose(w.double(), dropped, rtol=1e-5, atol=1e-7)
+    other, _ = O.masked_attention(q, k, v, None, None, 0.5, empty, dropout=drop)
+    assert not torch.allclose(out, other, rtol=1e-3)

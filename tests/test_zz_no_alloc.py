@@ -11,7 +11,7 @@ from _util import make_qkv
 pytestmark = pytest.mark.gpu
 
 
-def _rows_and_args(N, cuda, B, Hq, Hkv, Lk, D, n_sel, dtype, seed, work):
+def _rows_and_args(N, cuda, B, Hq, Hkv, Lk, D, n_sel, dtype, seed, work, sinks=None, stats=None):
     """A mask of `n_sel` random distinct columns per row in the kernels' layout, and the argument block of an
     attention call over it (out buffer included). `work` = None leaves the workspace fields empty."""
     from sparse_attention_hub_amd.sparse_attention.utils.mask_attention_utils import unit_inverse_weight
@@ -30,12 +30,12 @@ def _rows_and_args(N, cuda, B, Hq, Hkv, Lk, D, n_sel, dtype, seed, work):
         q.data_ptr(), q.stride(0), q.stride(1), q.stride(2),
         k.data_ptr(), k.stride(0), k.stride(1), k.stride(2),
         v.data_ptr(), v.stride(0), v.stride(1), v.stride(2),
-        None, 0, 0, 0, None,
+        None, 0, 0, 0, None if sinks is None else sinks.data_ptr(),
         N.dtype_code(dtype), B, Hq, Hkv, 1, Lk, D,
         float(D ** -0.5), unit_inverse_weight(dtype), 0, 0, 0, 0, n_sel,
         out.data_ptr(),
         None if work is None else work.data_ptr(), 0 if work is None else work.numel(),
-        None, None, N.stream_ptr(cuda),
+        None, None if stats is None else stats.data_ptr(), N.stream_ptr(cuda),
     )
     return args, out, (q, k, v, cols, cnt, bitmap)
 
@@ -55,13 +55,29 @@ def test_static_workspace_entry_point_matches_the_allocating_one(cuda):
         assert floats <= limit
         assert (floats > 0) == (i < 2)
         work = torch.full((max(floats, 1),), float("nan"), dtype=torch.float32, device=cuda)
-        a1, out1, keep1 = _rows_and_args(N, cuda, B, Hq, Hkv, Lk, D, n_sel, dtype, 7 + i, work)
-        a2, out2, keep2 = _rows_and_args(N, cuda, B, Hq, Hkv, Lk, D, n_sel, dtype, 7 + i, None)
+        # the second shape also carries sink logits and asks for the (max, denominator) pairs
+        sinks = torch.linspace(-0.5, 0.5, Hq, device=cuda) if i == 1 else None
+        st1 = torch.zeros((B * Hq, 2), dtype=torch.float32, device=cuda) if i == 1 else None
+        st2 = torch.zeros((B * Hq, 2), dtype=torch.float32, device=cuda) if i == 1 else None
+        a1, out1, keep1 = _rows_and_args(N, cuda, B, Hq, Hkv, Lk, D, n_sel, dtype, 7 + i, work, sinks, st1)
+        a2, out2, keep2 = _rows_and_args(N, cuda, B, Hq, Hkv, Lk, D, n_sel, dtype, 7 + i, None, sinks, st2)
         N.call("sah_sparse_attention", a1)
+        if i == 0:
+            # the first call on a device looks the built-in buffer's address up; a caller that must not even do that
+            # (stream capture) makes one warm-up call first, as here
+            N.call("sah_sparse_attention_static", a2)
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]
+        allocs_before = torch.cuda.memory_stats()["allocation.all.allocated"]
         N.call("sah_sparse_attention_static", a2)
         torch.cuda.synchronize()
+        # what the entry point exists for: no device memory is allocated around the call
+        assert torch.cuda.mem_get_info()[0] == free_before
+        assert torch.cuda.memory_stats()["allocation.all.allocated"] == allocs_before
         assert bool(torch.isfinite(out1.float()).all()) and float(out1.float().abs().max()) > 0
         assert torch.equal(out1, out2), f"call {i}: outputs differ"
+        if i == 1:
+            assert torch.equal(st1, st2) and bool((st1[:, 1] > 0).all())
     # a call that needs more than the built-in buffer is refused before anything is launched
     B, Hq, Hkv, Lk, D, n_sel = 32, 32, 8, 131072, 128, 131072
     assert N.work_floats(B * Hq, n_sel, D) > limit
