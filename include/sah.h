@@ -598,8 +598,10 @@ int sah_hash_compact_codes(const sah_hash_compact_args* a);
  * decode case (one workgroup per row, Lq = 1, no additive mask, unit weights, no logits
  * output, head_dim 64 or 128, same stream and dtype) both run in ONE kernel: the workgroup
  * that selected a row goes straight on to gather that row's K / V, from a column list kept in
- * LDS (rows.cols / rows.cnt are still written). Otherwise the two calls are made. */
-int sah_hash_decode_attention(const sah_hash_decode_args* a, const sah_attention_args* t);
+ * LDS (rows.cols / rows.cnt are still written). With fewer rows than compute units a row is given several
+ * workgroups, as in sah_select_topk_attention (same `tickets`, same use of t->work; NULL tickets: one workgroup per
+ * row or the separate calls). Otherwise the two calls are made. */
+int sah_hash_decode_attention(const sah_hash_decode_args* a, const sah_attention_args* t, uint32_t* tickets);
 
 /* ---------------------------------------------------------------------------
  * sah_select_topk followed by sah_sparse_attention over the same rows, with the same results up to the order of
@@ -661,7 +663,7 @@ typedef struct sah_chain_args {
   const sah_select_topk_args* select;
   const sah_attention_args* attention;
   const sah_hash_compact_args* compact;
-  uint32_t* tickets;   /* for select + attention as one kernel (sah_select_topk_attention), or NULL */
+  uint32_t* tickets;   /* of sah_select_topk_attention / sah_hash_decode_attention, or NULL */
 } sah_chain_args;
 int sah_run_chain(const sah_chain_args* a);
 

@@ -324,7 +324,7 @@ extern "C" int sah_run_chain(const sah_chain_args* a) {
   if (a->compact && (rc = sah_hash_compact_codes(a->compact))) return rc;
   if (a->hamming && (rc = sah_hamming_topk(a->hamming))) return rc;
   if (a->hash_decode && a->attention && !a->qk && !a->pq_assign && !a->pq_adc && !a->select)
-    return sah_hash_decode_attention(a->hash_decode, a->attention);  // one kernel when shapes allow
+    return sah_hash_decode_attention(a->hash_decode, a->attention, a->tickets);  // one kernel when shapes allow
   if (a->hash_decode && (rc = sah_hash_decode_topk(a->hash_decode))) return rc;
   if (a->qk && (rc = sah_qk_scores(a->qk))) return rc;
   if (a->pq_assign && (rc = sah_pq_kmeans_assign(a->pq_assign))) return rc;

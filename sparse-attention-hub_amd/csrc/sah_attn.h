@@ -386,6 +386,58 @@ __device__ __forceinline__ void att_store_row(const att_params& P, int r, int b,
   }
 }
 
+// A row attended to by `parts` workgroups, each holding the partial result (a for thread d < D, M, l) of its share:
+// the partial results meet in `work` ([row][part][D + 2] floats) and the workgroup that arrives last (`ticket`: the
+// row's arrival counter, zero between kernels) merges them, in part order whoever arrived last, and writes the row.
+// Every thread of the workgroup calls it (two barriers inside); nobody waits for another workgroup. The hand-over
+// uses device-scope atomic accesses, which need no cache write-back (sah_common.h).
+#define ATT_MAX_PARTS 8
+template <int DT, int D>
+__device__ __forceinline__ void att_merge_parts(const att_params& P, int r, int b, int h, int qi, float a, float M, float l,
+                                                float* work, uint32_t* ticket, int part, int parts, int& s_last) {
+  const int tid = threadIdx.x;
+  float* wrow = work + (int64_t)r * parts * (D + 2);
+  float* mine = wrow + part * (D + 2);
+  if (tid < D) sah_agent_store_f32(mine + 2 + tid, a);
+  if (tid == 0) {
+    sah_agent_store_f32(mine, M);
+    sah_agent_store_f32(mine + 1, l);
+  }
+  sah_stores_done();
+  __syncthreads();
+  if (tid == 0) s_last = sah_last_arrival(ticket, (uint32_t)parts) ? 1 : 0;
+  __syncthreads();
+  if (!s_last) return;
+  float pm[ATT_MAX_PARTS], pl[ATT_MAX_PARTS], pa[ATT_MAX_PARTS];
+#pragma unroll
+  for (int p = 0; p < ATT_MAX_PARTS; ++p) {
+    const bool have = p < parts;
+    pm[p] = have ? sah_agent_load_f32(wrow + p * (D + 2)) : -INFINITY;
+    pl[p] = have ? sah_agent_load_f32(wrow + p * (D + 2) + 1) : 0.f;
+    pa[p] = (have && tid < D) ? sah_agent_load_f32(wrow + p * (D + 2) + 2 + tid) : 0.f;
+  }
+  M = pm[0];
+#pragma unroll
+  for (int p = 1; p < ATT_MAX_PARTS; ++p) M = fmaxf(M, pm[p]);
+  a = 0.f;
+  l = 0.f;
+#pragma unroll
+  for (int p = 0; p < ATT_MAX_PARTS; ++p) {
+    const float sc = (pm[p] == -INFINITY) ? 0.f : att_exp<DT>(pm[p] - M);
+    a = fmaf(pa[p], sc, a);
+    l = fmaf(pl[p], sc, l);
+  }
+  att_store_row<DT, D>(P, r, b, h, qi, a, M, l);
+}
+
+// workgroups per row of the kernels that select and attend in one launch: as many as it takes to give every CU a
+// workgroup when there are fewer rows than CUs
+static inline int att_row_parts(int n_rows) {
+  int parts = 256 / n_rows;
+  if (n_rows >= 192 || parts < 1) parts = 1;
+  return parts > ATT_MAX_PARTS ? ATT_MAX_PARTS : parts;
+}
+
 // One tile of work of a workgroup. ROW = false: a workgroup of 4 waves handles one (row, split) tile and leaves (m, l, acc) in the workspace
 //   for the merge kernel - the form for few or very uneven rows.
 // ROW = true: a workgroup of 16 waves handles a whole row, every wave an equal share of the row's entries,

@@ -152,21 +152,29 @@ __global__ __launch_bounds__(HSW_NT) void k_hash_decode(hdec_params P) {
 // was selected early starts streaming while others still select, and the attention's start-up latency is paid
 // while the memory system would otherwise idle. Workgroup -> row mapping as in k_sparse_attn (the query heads
 // of a GQA group on one XCD).
+// parts > 1 (fewer rows than CUs): every row is given `parts` workgroups. Each builds the whole row by itself (the
+// same arithmetic, so the lists are identical and both write the same values to the row in memory), attends to its
+// share of the list, and the one that arrives last merges the partial results (att_merge_parts).
 template <int DT, bool MF, bool CP, int D, bool SILU>
-__global__ __launch_bounds__(HSW_NT) void k_hash_decode_attn(hdec_params P, att_params A, int cols_offset) {
+__global__ __launch_bounds__(HSW_NT) void k_hash_decode_attn(hdec_params P, att_params A, int cols_offset, int parts, float* work,
+                                                             uint32_t* tickets) {
   __shared__ hsw_lds S;
   __shared__ float s_m[HSW_NW];
   __shared__ float s_l[HSW_NW];
   __shared__ float s_acc[HSW_NW][D];
+  __shared__ int s_last;
   HIP_DYNAMIC_SHARED(unsigned char, hdec_dyn)
-  sah_touch_kernargs<sizeof(hdec_params) + sizeof(att_params) + 8>();
+  sah_touch_kernargs<sizeof(hdec_params) + sizeof(att_params) + 32>();
   const int G = A.Hq / A.Hkv;
+  const int GP = G * parts;
   const int slot = blockIdx.x / ATT_XCDS;
-  const int tile = (slot / G) * ATT_XCDS + (int)(blockIdx.x % ATT_XCDS);  // b * Hkv + hk
+  const int tile = (slot / GP) * ATT_XCDS + (int)(blockIdx.x % ATT_XCDS);  // b * Hkv + hk
   if (tile >= P.R.n_rows / G) return;  // padding to a multiple of 8 tiles
+  const int within = slot % GP;
+  const int part = within / G;
   const int hk = tile % A.Hkv;
   const int b = tile / A.Hkv;
-  const int h = hk * G + slot % G;
+  const int h = hk * G + within % G;
   const int r = b * A.Hq + h;
   int* s_cols = (int*)(hdec_dyn + cols_offset);
   const int cnt = hdec_row<DT, MF, CP, SILU>(P, r, S, hdec_dyn, s_cols);
@@ -175,8 +183,9 @@ __global__ __launch_bounds__(HSW_NT) void k_hash_decode_attn(hdec_params P, att_
   {
     constexpr int KPI = SAH_WAVE / (D / 8);
     const int wave = sah_wave_id();
-    const int per = (((cnt + HSW_NW - 1) / HSW_NW) + KPI - 1) / KPI * KPI;  // entries per wave
-    const int first = wave * per;
+    const int n_runs = HSW_NW * parts;
+    const int per = (((cnt + n_runs - 1) / n_runs) + KPI - 1) / KPI * KPI;  // entries per wave
+    const int first = (wave * parts + part) * per;
     const int bound = first + per < cnt ? first + per : cnt;
     att_wave_state st;
     st.clear();
@@ -187,7 +196,8 @@ __global__ __launch_bounds__(HSW_NT) void k_hash_decode_attn(hdec_params P, att_
     __syncthreads();
     float a, M, l;
     att_gather<DT, D, HSW_NW>(s_m, s_l, s_acc, a, M, l);
-    att_store_row<DT, D>(A, r, b, h, 0, a, M, l);
+    if (parts == 1) att_store_row<DT, D>(A, r, b, h, 0, a, M, l);
+    else att_merge_parts<DT, D>(A, r, b, h, 0, a, M, l, work, tickets + r, part, parts, s_last);
   }
 }
 
@@ -351,31 +361,35 @@ extern "C" int sah_hash_decode_topk(const sah_hash_decode_args* a) {
 }
 
 template <int DT, bool MF, bool CP, int D, bool SILU>
-static int hdec_attn_launch_s(const sah_hash_decode_args* a, const hdec_params& P, const att_params& A, size_t lds, int cols_offset) {
+static int hdec_attn_launch_s(const sah_hash_decode_args* a, const hdec_params& P, const att_params& A, size_t lds, int cols_offset,
+                              int parts, float* work, uint32_t* tickets) {
   if (int rc = sah_allow_lds((const void*)k_hash_decode_attn<DT, MF, CP, D, SILU>, 150 * 1024, "sah_hash_decode_attention")) return rc;
   const int G = A.Hq / A.Hkv;
   const int n_tiles = P.R.n_rows / G;
-  const int n_wg = (n_tiles + ATT_XCDS - 1) / ATT_XCDS * ATT_XCDS * G;
+  const int n_wg = (n_tiles + ATT_XCDS - 1) / ATT_XCDS * ATT_XCDS * G * parts;
   sah_timed timed("k_hash_decode_attn", a->stream);
-  hipLaunchKernelGGL((k_hash_decode_attn<DT, MF, CP, D, SILU>), dim3(n_wg), dim3(HSW_NT), lds, (hipStream_t)a->stream, P, A, cols_offset);
+  hipLaunchKernelGGL((k_hash_decode_attn<DT, MF, CP, D, SILU>), dim3(n_wg), dim3(HSW_NT), lds, (hipStream_t)a->stream, P, A, cols_offset,
+                     parts, work, tickets);
   return sah_launch_status("sah_hash_decode_attention");
 }
 
 template <int DT, bool MF, bool CP, int D>
-static int hdec_attn_launch_t(const sah_hash_decode_args* a, const hdec_params& P, const att_params& A, size_t lds, int cols_offset) {
+static int hdec_attn_launch_t(const sah_hash_decode_args* a, const hdec_params& P, const att_params& A, size_t lds, int cols_offset,
+                              int parts, float* work, uint32_t* tickets) {
   if constexpr (MF) {
-    if (hdec_silu(P)) return hdec_attn_launch_s<DT, MF, CP, D, true>(a, P, A, lds, cols_offset);
+    if (hdec_silu(P)) return hdec_attn_launch_s<DT, MF, CP, D, true>(a, P, A, lds, cols_offset, parts, work, tickets);
   }
-  return hdec_attn_launch_s<DT, MF, CP, D, false>(a, P, A, lds, cols_offset);
+  return hdec_attn_launch_s<DT, MF, CP, D, false>(a, P, A, lds, cols_offset, parts, work, tickets);
 }
 
 template <int DT, bool MF, int D>
-static int hdec_attn_launch(const sah_hash_decode_args* a, const hdec_params& P, const att_params& A, size_t lds, int cols_offset) {
-  return P.pos ? hdec_attn_launch_t<DT, MF, true, D>(a, P, A, lds, cols_offset)
-               : hdec_attn_launch_t<DT, MF, false, D>(a, P, A, lds, cols_offset);
+static int hdec_attn_launch(const sah_hash_decode_args* a, const hdec_params& P, const att_params& A, size_t lds, int cols_offset,
+                            int parts, float* work, uint32_t* tickets) {
+  return P.pos ? hdec_attn_launch_t<DT, MF, true, D>(a, P, A, lds, cols_offset, parts, work, tickets)
+               : hdec_attn_launch_t<DT, MF, false, D>(a, P, A, lds, cols_offset, parts, work, tickets);
 }
 
-extern "C" int sah_hash_decode_attention(const sah_hash_decode_args* a, const sah_attention_args* t) {
+extern "C" int sah_hash_decode_attention(const sah_hash_decode_args* a, const sah_attention_args* t, uint32_t* tickets) {
   if (!a || !t) return sah_fail(SAH_ENULL, "sah_hash_decode_attention: args is NULL");
   int rc = hdec_validate(a);
   if (rc) return rc;
@@ -385,8 +399,11 @@ extern "C" int sah_hash_decode_attention(const sah_hash_decode_args* a, const sa
   const bool has_key = a->key_sig && a->key_sig->L > 0;
   const size_t cols_offset = (hdec_lds_bytes(a->rows.n_keys) + 15) & ~(size_t)15;
   const size_t lds = cols_offset + (size_t)a->rows.cap * 4;
+  // rows fewer than CUs: several workgroups per row, if the caller brought the tickets and the workspace for it
+  const int parts = att_row_parts(a->rows.n_rows);
+  const bool shared_rows = parts > 1 && tickets && t->work && t->work_floats >= (int64_t)a->rows.n_rows * parts * (t->D + 2);
   const bool one_kernel =
-      hdec_fusable(a) && A.n_split == 0 && !t->dense && !t->closed_form && !t->amask && !t->logits_out && !t->rows.w && t->Lq == 1 &&
+      hdec_fusable(a) && (shared_rows || A.n_split == 0) && !t->dense && !t->closed_form && !t->amask && !t->logits_out && !t->rows.w && t->Lq == 1 &&
       t->dropout_p == 0.f &&
       t->rows.cols == a->rows.cols && t->rows.cnt == a->rows.cnt && t->rows.cap == a->rows.cap &&
       t->rows.n_rows == a->rows.n_rows && t->stream == a->stream && t->dtype == a->query_sig->dtype &&
@@ -399,8 +416,8 @@ extern "C" int sah_hash_decode_attention(const sah_hash_decode_args* a, const sa
   hdec_fill(a, P);
   const bool mf = hdec_sig_kind(a, has_key) == 2;
 #define SAH_HDA(DTC, MFC)                                                                    \
-  (t->D == 128 ? hdec_attn_launch<DTC, MFC, 128>(a, P, A, lds, (int)cols_offset)             \
-               : hdec_attn_launch<DTC, MFC, 64>(a, P, A, lds, (int)cols_offset))
+  (t->D == 128 ? hdec_attn_launch<DTC, MFC, 128>(a, P, A, lds, (int)cols_offset, shared_rows ? parts : 1, t->work, tickets)  \
+               : hdec_attn_launch<DTC, MFC, 64>(a, P, A, lds, (int)cols_offset, shared_rows ? parts : 1, t->work, tickets))
   switch (t->dtype) {
     case SAH_F32: return SAH_HDA(SAH_F32, false);
     case SAH_BF16: return mf ? SAH_HDA(SAH_BF16, true) : SAH_HDA(SAH_BF16, false);

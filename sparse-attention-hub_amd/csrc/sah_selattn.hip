@@ -15,7 +15,6 @@
 #include "sah_sel16.h"
 
 static_assert(ATT_ROW_NT == SF_NT, "selection and whole-row attention share one workgroup");
-#define SELATT_MAX_PARTS 8
 
 struct selattn_params {
   sah_rows R;
@@ -104,50 +103,12 @@ __global__ __launch_bounds__(SF_NT) void k_select16_attn(selattn_params P, att_p
     return;
   }
   // hand the partial result over; the part that arrives last merges
-  float* wrow = P.work + (int64_t)r * P.parts * (D + 2);
-  float* mine = wrow + part * (D + 2);
-  if (tid < D) sah_agent_store_f32(mine + 2 + tid, a);
-  if (tid == 0) {
-    sah_agent_store_f32(mine, M);
-    sah_agent_store_f32(mine + 1, l);
-  }
-  sah_stores_done();
-  __syncthreads();
-  if (tid == 0) s_last = sah_last_arrival(P.tickets + r, (uint32_t)P.parts) ? 1 : 0;
-  __syncthreads();
-  if (!s_last) return;
-  float pm[SELATT_MAX_PARTS], pl[SELATT_MAX_PARTS], pa[SELATT_MAX_PARTS];
-#pragma unroll
-  for (int p = 0; p < SELATT_MAX_PARTS; ++p) {
-    const bool have = p < P.parts;
-    pm[p] = have ? sah_agent_load_f32(wrow + p * (D + 2)) : -INFINITY;
-    pl[p] = have ? sah_agent_load_f32(wrow + p * (D + 2) + 1) : 0.f;
-    pa[p] = (have && tid < D) ? sah_agent_load_f32(wrow + p * (D + 2) + 2 + tid) : 0.f;
-  }
-  M = pm[0];
-#pragma unroll
-  for (int p = 1; p < SELATT_MAX_PARTS; ++p) M = fmaxf(M, pm[p]);
-  a = 0.f;
-  l = 0.f;
-#pragma unroll
-  for (int p = 0; p < SELATT_MAX_PARTS; ++p) {  // in part order, whoever arrived last: the sums do not depend on timing
-    const float sc = (pm[p] == -INFINITY) ? 0.f : att_exp<DT>(pm[p] - M);
-    a = fmaf(pa[p], sc, a);
-    l = fmaf(pl[p], sc, l);
-  }
-  att_store_row<DT, D>(A, r, b, h, qi, a, M, l);
-}
-
-// workgroups per row: as many as it takes to give every CU a workgroup, when there are fewer rows than CUs
-static int selattn_parts(int n_rows) {
-  int parts = 256 / n_rows;
-  if (n_rows >= 192 || parts < 1) parts = 1;
-  return parts > SELATT_MAX_PARTS ? SELATT_MAX_PARTS : parts;
+  att_merge_parts<DT, D>(A, r, b, h, qi, a, M, l, P.work, P.tickets + r, part, P.parts, s_last);
 }
 
 // floats of workspace the fused form needs for n_rows rows: the parts' partial results
 int64_t selattn_work_floats(int n_rows, int D) {
-  const int parts = selattn_parts(n_rows);
+  const int parts = att_row_parts(n_rows);
   if (parts == 1) return 0;
   return (int64_t)n_rows * parts * (D + 2);
 }
@@ -179,7 +140,7 @@ extern "C" int sah_select_topk_attention(const sah_select_topk_args* s, const sa
   const int cpw = sf_chunks_per_wave(s->n_cand);
   const size_t cols_offset = sf_hist_offset(s->rows.n_words);
   const size_t lds = sf_lds_bytes(s->rows.n_words);
-  const int parts = selattn_parts(n_rows);
+  const int parts = att_row_parts(n_rows);
   const int64_t need = selattn_work_floats(n_rows, t->D);
   int64_t worst = (int64_t)s->k + (s->fresh ? (int64_t)s->fresh_sink + s->fresh_window : (int64_t)s->rows.cap);
   if (worst > s->rows.cap) worst = s->rows.cap;

@@ -420,11 +420,11 @@ def lib() -> C.CDLL:
         if name in ("sah_version", "sah_last_error", "sah_sparse_attention_work_floats", "sah_pq_adc_lut_bytes",
                     "sah_timing_enable", "sah_timing_collect"):
             continue
-        if name in ("sah_hash_signatures_pair", "sah_hash_decode_attention"):
+        if name == "sah_hash_signatures_pair":
             getattr(handle, name).restype = C.c_int
             getattr(handle, name).argtypes = [C.c_void_p, C.c_void_p]
             continue
-        if name == "sah_select_topk_attention":
+        if name in ("sah_select_topk_attention", "sah_hash_decode_attention"):
             getattr(handle, name).restype = C.c_int
             getattr(handle, name).argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
             continue

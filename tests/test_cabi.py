@@ -92,7 +92,7 @@ def test_every_entry_point_refuses_null_and_names_itself():
         assert getattr(lib, fn)(None) == -2, fn
         assert fn.replace("_static", "").encode() in lib.sah_last_error() or fn.encode() in lib.sah_last_error(), fn
     assert lib.sah_hash_signatures_pair(None, None) == -2
-    assert lib.sah_hash_decode_attention(None, None) == -2
+    assert lib.sah_hash_decode_attention(None, None, None) == -2
     assert lib.sah_select_topk_attention(None, None, None) == -2
     # whatever takes an argument block is in one of the two lists above
     plain = {"sah_version", "sah_last_error", "sah_timing_enable", "sah_timing_collect", "sah_pq_adc_lut_bytes",

@@ -21,6 +21,15 @@ def _sa():
     return sa
 
 
+def _same_output(o_plan, o_ref, n_rows):
+    """Plan against masker-by-masker path. With at least as many rows as the one-workgroup-per-row forms need, both sum in
+    the same order: bit-identical. With fewer rows the one-kernel forms give a row several workgroups, which deal the
+    row's entries out differently: the same columns, sums that may differ in a last bit."""
+    if n_rows >= 192:
+        return torch.equal(o_plan, o_ref)
+    return rel_err(o_plan, o_ref) < 4e-3
+
+
 def _run_chain(cuda, cfgs, specs, B, Hq, Hkv, Lq, Lk, D, dtype, amask=None, sinks=None, outliers=False, seed=0,
                meta=None, check_weights=True):
     sa = _sa()
@@ -514,8 +523,10 @@ def test_decode_plan_matches_masker_by_masker_path(cuda, kind):
             continue
         o2, w2 = ref.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m2, layer_idx=0)
         assert w1 is None and w2 is not None
-        if kind in ("fixed", "hash"):
+        if kind == "fixed":
             assert torch.equal(o1, o2), f"step {step}"
+        elif kind == "hash":
+            assert _same_output(o1, o2, B * Hq), f"step {step}"
         else:
             # selection and attention of these chains run as one kernel that deals a row's entries to its workgroups
             # in another order than the stand-alone attention: same columns, sums that may differ in a last bit
@@ -553,7 +564,7 @@ def test_decode_plan_hashes_new_keys_in_blocks(cuda):
         qq = make_qkv(B, Hq, Hkv, 1, 1, D, dtype, seed=150 + step)[0].to(cuda)
         o1, _ = fast.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m1, layer_idx=0)
         o2, _ = ref.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m2, layer_idx=0)
-        assert torch.equal(o1, o2), f"step {step}"
+        assert _same_output(o1, o2, B * Hq), f"step {step}"
         c1, c2 = m1["key"][0], m2["key"][0]
         assert c2.n == n and n - window < c1.n <= n
         hashed.append(c1.n)
@@ -656,7 +667,7 @@ def test_compact_codes_with_many_zero_components(cuda, Lk, zero_key_bits, B):
         qq = make_qkv(B, Hq, Hkv, 1, 1, D, dtype, seed=350 + step)[0].to(cuda)
         o1, _ = fast.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m1, layer_idx=0)
         o2, _ = ref.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m2, layer_idx=0)
-        assert torch.equal(o1, o2), f"step {step}"
+        assert _same_output(o1, o2, B * Hq), f"step {step}"
     cache = m1["key"][0]
     assert cache.n_compact == Lk and cache.exc.shape[2] == 1024
     listed = cache.exc_cnt.cpu()
@@ -694,7 +705,7 @@ def test_hash_decode_plan_state_transitions(cuda):
             qq = make_qkv(B, Hq, Hkv, 1, 1, D, dtype, seed=450 + 2 * step + layer)[0].to(cuda)
             o1, w1 = fast.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m1, layer_idx=layer)
             o2, w2 = ref.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m2, layer_idx=layer)
-            assert torch.equal(o1, o2), f"step {step} layer {layer}"
+            assert _same_output(o1, o2, B * Hq), f"step {step} layer {layer}"
             assert (w1 is not None) == general
             if general:
                 assert torch.equal(w1, w2)
@@ -856,8 +867,7 @@ def test_fused_hash_decode_kernel_matches_separate_launches(cuda, monkeypatch, d
 
     sa = _sa()
     _set_hash_block(monkeypatch, block, compact)
-    # 256 rows at the ragged size: enough for the one-workgroup-per-row attention, so that selection and
-    # attention run as ONE kernel; 64 rows at the headline length: attention in its split form, two more launches
+    # 256 rows at the ragged size: one workgroup per row; 64 and 32 rows at the longer ones: four and eight per row
     B, Hq, Hkv, D = (8 if Lk <= 8192 else 2 if Lk <= 32768 else 1), 32, 8, 128   # 70001 keys: 18 chunks per wave
     heavy = 2048 if Lk > 8192 else 300
     q, k, v = make_qkv(B, Hq, Hkv, 1, Lk + 3, D, dtype, seed=3)
@@ -881,12 +891,11 @@ def test_fused_hash_decode_kernel_matches_separate_launches(cuda, monkeypatch, d
             N.timing_enable(False)
             if block == 1 and compact:   # the new key is hashed and added to the compact stream by launches of their own
                 names -= {"k_hash_compact", "k_hash_sig_small_mfma", "k_hash_sig_gemv"}
-            if B * Hq >= 192:
-                assert names == {"k_hash_decode_attn"}, names   # the whole step, attention included, is one kernel
-            else:
-                assert names == {"k_hash_decode", "k_sparse_attn", "k_attn_combine"}, names
+            # the whole step, attention included, is one kernel: one workgroup per row, or - with fewer rows than
+            # compute units - several per row whose partial results the last one to finish merges
+            assert names == {"k_hash_decode_attn"}, names
         o2, _ = ref.custom_attention(None, qq, kc[:, :, :n], vc[:, :, :n], None, D ** -0.5, 0.0, sparse_meta_data=m2, layer_idx=0)
-        assert torch.equal(o1, o2), f"step {step}"
+        assert _same_output(o1, o2, B * Hq), f"step {step}"
         hashed = m1["key"][0].n                                       # block > 1: the newest keys are not hashed yet
         assert hashed == (n if block == 1 else Lk)
         assert torch.equal(m1["key"][0].codes[:, :, :hashed], m2["key"][0].codes[:, :, :hashed]), f"cache, step {step}"
