@@ -257,6 +257,9 @@ typedef struct sah_select_topk_args {
   int32_t fresh_sink;     /* columns of one query per row - what sah_sink_local_indices(lq = 1, fresh = 1) */
   int32_t fresh_window;   /* writes - in the same launch when the keys are 16-bit and 16-byte aligned      */
   void* stream;
+  int32_t skip_bitmap;    /* != 0: rows.bitmap need not be brought up to date (a caller that hands the rows */
+                          /* to the attention only, which reads the column lists); honoured where it saves  */
+                          /* work: by sah_select_topk_attention's one-kernel form                           */
 } sah_select_topk_args;
 int sah_select_topk(const sah_select_topk_args* a);
 

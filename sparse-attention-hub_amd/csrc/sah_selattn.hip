@@ -23,6 +23,7 @@ struct selattn_params {
   int n_cand, col_offset, k;
   uint32_t excluded_key;
   int fresh, sink, window;
+  int write_bitmap;
   int parts;
   int cols_offset;  // of the column list inside the dynamic LDS
   float* work;        // [row][part][D + 2]
@@ -60,7 +61,7 @@ __global__ __launch_bounds__(SF_NT) void k_select16_attn(selattn_params P, att_p
   int earlier = 0;
   const int cnt = sf_select_impl<CPW, true>(S, sa_dyn, P.R, r, P.keys + (int64_t)r * P.pitch, P.n_cand, P.col_offset,
                                             P.k < P.n_cand ? P.k : P.n_cand, P.excluded_key, P.fresh, P.sink, P.window,
-                                            part == 0, true, &earlier, s_cols, part, P.parts);
+                                            part == 0, P.write_bitmap != 0, &earlier, s_cols, part, P.parts);
   __syncthreads();  // the winners' part of the list is complete in LDS, and so is the bitmap row
 
   // This part's share of the row: its entries dealt to parts x 16 waves, a wave of part p taking every parts-th run.
@@ -91,7 +92,7 @@ __global__ __launch_bounds__(SF_NT) void k_select16_attn(selattn_params P, att_p
         [&](int) { return unit; }, st);
   att_park<D, NW>(st, wave, s_m, s_l, s_acc);
   __syncthreads();
-  if (part == 0) {  // the row's bitmap, complete in LDS since the barrier
+  if (part == 0 && P.write_bitmap) {  // the row's bitmap, complete in LDS since the barrier
     const uint32_t* s_bm = (const uint32_t*)sa_dyn;
     uint32_t* bm = P.R.bitmap + (int64_t)r * P.R.n_words;
     for (int i = tid; i < P.R.n_words; i += SF_NT) bm[i] = s_bm[i];
@@ -163,6 +164,7 @@ extern "C" int sah_select_topk_attention(const sah_select_topk_args* s, const sa
   P.n_cand = s->n_cand; P.col_offset = s->col_offset; P.k = s->k;
   P.excluded_key = s->excluded_key;
   P.fresh = s->fresh ? 1 : 0; P.sink = s->fresh_sink; P.window = s->fresh_window;
+  P.write_bitmap = s->skip_bitmap ? 0 : 1;
   P.parts = parts;
   P.cols_offset = (int)cols_offset;
   P.work = t->work;

@@ -172,6 +172,7 @@ class SelectTopkArgs(C.Structure):
         ("fresh_sink", C.c_int32),
         ("fresh_window", C.c_int32),
         ("stream", C.c_void_p),
+        ("skip_bitmap", C.c_int32),
     ]
 
 

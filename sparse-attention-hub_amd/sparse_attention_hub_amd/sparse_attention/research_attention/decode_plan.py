@@ -246,6 +246,7 @@ class DecodePlan:
             se = self.select
             se.rows, se.keys, se.key_pitch, se.key_bits = rows, self.keybuf.data_ptr(), self.keybuf_pitch, self.key_bits
             se.n_cand, se.col_offset, se.k, se.excluded_key, se.stream = Lk, 0, k_eff, self._excluded_min, stream
+            se.skip_bitmap = 1  # only the attention reads these rows, and it reads the column lists
             chain.select = C.addressof(se)
             if Lq == 1:
                 # one query per row: the selection kernel writes the sink + local rows itself
@@ -300,6 +301,7 @@ class DecodePlan:
             se = self.select
             se.rows, se.keys, se.key_pitch, se.key_bits = rows, self.keybuf.data_ptr(), self.keybuf_pitch, self.key_bits
             se.n_cand, se.col_offset, se.k, se.excluded_key, se.stream = current, off, k_eff, self._excluded_min, stream
+            se.skip_bitmap = 1  # only the attention reads these rows, and it reads the column lists
             chain.select = C.addressof(se)
             if Lq == 1:
                 # one query per row: the selection kernel writes the sink + local rows itself
