@@ -232,6 +232,11 @@ typedef struct sah_qk_scores_args {
   void* keys_out;
   int64_t key_pitch;
   void* stream;
+  /* Optional, 16-bit dtypes without amask only: [B*Hq*Lq][key_pitch] 16-bit words, what rounding the fp32 dot product
+   * to `dtype` took away (fp32 dot - rounded score, itself rounded to `dtype`). The key orders the scores exactly as
+   * torch's matmul output orders them; key and remainder together give the dot product to about 16 mantissa bits,
+   * which lets the attention that follows skip K (sah_attention_args.score_keys / score_resid). NULL: not written. */
+  void* resid_out;
 } sah_qk_scores_args;
 int sah_qk_scores(const sah_qk_scores_args* a);
 
@@ -414,6 +419,15 @@ typedef struct sah_attention_args {
   int32_t dropout_numerator_only; /* != 0: dropped entries leave the denominator as it is, i.e. dropout of the
                                      normalised probabilities, what the reference's dense path does
                                      (scaled_dot_product_attention with dropout_p, mask_attention_utils.py:40-52) */
+  /* Optional: q.k of EVERY column of every mask row, [n_rows][score_pitch] each: the 16-bit score keys and the
+   * remainders sah_qk_scores wrote for these q and k (keys_out / resid_out, no additive mask) - a chain whose selection
+   * scored all keys exactly (OracleTopK, oracle_top_k.py:49-60) has them already. The kernels may then take a logit
+   * from there ((score + remainder) * scaling: the fp32 dot product to about 16 mantissa bits) instead of reading the
+   * K row again: half of the gather's bytes. amask, where given, is added as ever. Used when both are given, for
+   * 16-bit tensors, head_dim 64 / 128 and no dropout; otherwise K is read. NULL: none. */
+  const void* score_keys;
+  const void* score_resid;
+  int64_t score_pitch;
 } sah_attention_args;
 int64_t sah_sparse_attention_work_floats(int32_t n_rows, int32_t max_cnt, int32_t D);
 int sah_sparse_attention(const sah_attention_args* a);

@@ -14,7 +14,8 @@
 
 #include <mutex>
 
-template <int DT, int D, bool ROW, bool DROP, bool FULL>
+// KEYED: the logits come from the score keys of an exact q.k scoring pass (P.score_keys); K is not read
+template <int DT, int D, bool ROW, bool DROP, bool FULL, bool KEYED = false>
 __global__ __launch_bounds__(ROW ? ATT_ROW_NT : ATT_NT, ROW ? 1 : 5) void k_sparse_attn(att_params P) {
   sah_touch_kernargs<sizeof(att_params)>();
   constexpr int NW = (ROW ? ATT_ROW_NT : ATT_NT) / SAH_WAVE;
@@ -40,7 +41,7 @@ __global__ __launch_bounds__(ROW ? ATT_ROW_NT : ATT_NT, ROW ? 1 : 5) void k_spar
   const int b = gidx / (P.Lq * P.Hkv);
   const int h = hk * G + slot % G;
   const int r = (b * P.Hq + h) * P.Lq + qi;
-  att_tile<DT, D, ROW, DROP, FULL>(P, r, b, h, hk, qi, split, n_split, nullptr, -1, s_m, s_l, s_acc);
+  att_tile<DT, D, ROW, DROP, FULL, KEYED>(P, r, b, h, hk, qi, split, n_split, nullptr, -1, s_m, s_l, s_acc);
 }
 
 template <int DT, int D>
@@ -116,11 +117,15 @@ template <int DT, int D, bool FULL>
 static int att_launch(const sah_attention_args* a, const att_params& P, bool timing) {
   hipStream_t st = (hipStream_t)a->stream;
   const int G = a->Hq / a->Hkv;
+  // the variant that takes the logits from score keys: 16-bit types, head_dim 64 / 128, no dropout
+  constexpr bool CAN_KEY = DT != SAH_F32 && FULL && (D == 64 || D == 128);
+  const bool keyed = CAN_KEY && P.score_keys && !P.drop.thresh;
   if (P.n_split == 0) {  // whole-row form
     sah_timed timed("k_sparse_attn", a->stream, timing);
     const int n_tiles = a->rows.n_rows / G;
     const int n_wg = (n_tiles + ATT_XCDS - 1) / ATT_XCDS * ATT_XCDS * G;
     if (P.drop.thresh) hipLaunchKernelGGL((k_sparse_attn<DT, D, true, true, FULL>), dim3(n_wg), dim3(ATT_ROW_NT), 0, st, P);
+    else if (keyed) hipLaunchKernelGGL((k_sparse_attn<DT, D, true, false, FULL, CAN_KEY>), dim3(n_wg), dim3(ATT_ROW_NT), 0, st, P);
     else hipLaunchKernelGGL((k_sparse_attn<DT, D, true, false, FULL>), dim3(n_wg), dim3(ATT_ROW_NT), 0, st, P);
     return sah_launch_status("sah_sparse_attention");
   }
@@ -130,6 +135,7 @@ static int att_launch(const sah_attention_args* a, const att_params& P, bool tim
     const int n_tiles = (a->rows.n_rows / G) * P.n_split;
     const int n_wg = (n_tiles + ATT_XCDS - 1) / ATT_XCDS * ATT_XCDS * G;
     if (P.drop.thresh) hipLaunchKernelGGL((k_sparse_attn<DT, D, false, true, FULL>), dim3(n_wg), dim3(ATT_NT), 0, st, P);
+    else if (keyed) hipLaunchKernelGGL((k_sparse_attn<DT, D, false, false, FULL, CAN_KEY>), dim3(n_wg), dim3(ATT_NT), 0, st, P);
     else hipLaunchKernelGGL((k_sparse_attn<DT, D, false, false, FULL>), dim3(n_wg), dim3(ATT_NT), 0, st, P);
     rc = sah_launch_status("sah_sparse_attention");
   }
@@ -214,6 +220,16 @@ int att_prepare(const sah_attention_args* a, att_params& P) {
   P.logits_out = a->logits_out;
   P.logits_pitch = a->dense ? a->Lk : a->rows.cap;
   P.drop_num_only = a->dropout_numerator_only ? 1 : 0;
+  P.score_keys = P.score_resid = nullptr;
+  P.score_pitch = 0;
+  if (a->score_keys && a->score_resid) {
+    if (a->score_pitch < a->Lk) return sah_fail(SAH_EINVAL, "sah_sparse_attention: score_pitch < Lk");
+    if (a->dtype != SAH_F32) {  // fp32 scores do not fit 16-bit keys: K is read as ever
+      P.score_keys = (const uint16_t*)a->score_keys;
+      P.score_resid = (const uint16_t*)a->score_resid;
+      P.score_pitch = a->score_pitch;
+    }
+  }
   if (!sah_dropout_fill(a->dropout_p, a->dropout_seed, a->dropout_offset, P.drop))
     return sah_fail(SAH_EINVAL, "sah_sparse_attention: dropout_p %g not in [0, 1)", (double)a->dropout_p);
   if (!att_pad_dim(a->D)) return sah_fail(SAH_ESHAPE, "sah_sparse_attention: head_dim %d is not a multiple of 8 in [8, 256]", a->D);

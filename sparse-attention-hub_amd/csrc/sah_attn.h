@@ -30,7 +30,26 @@ struct att_params {
   int64_t logits_pitch;
   sah_dropout drop;
   int drop_num_only;  // dropout leaves the softmax denominator alone (dropout of the normalised probabilities)
+  const uint16_t* score_keys;   // [row][score_pitch]: q.k of every column as 16-bit score keys, or NULL
+  const uint16_t* score_resid;  // ... and what the keys' rounding took away
+  int64_t score_pitch;
 };
+
+// The logit source of a walk that reads K itself.
+struct att_no_key {
+  __device__ __forceinline__ uint32_t operator()(int, int) const { return 0u; }
+};
+
+// The dot product a (score key, remainder) pair stands for: the key is sah_sort_key of the dot product rounded to DT
+// (low half of `kr`), the remainder what that rounding took away, in DT's bits (high half).
+template <int DT>
+__device__ __forceinline__ float att_key_score(uint32_t kr) {
+  static_assert(DT != SAH_F32, "16-bit keys hold scores of 16-bit types");
+  const uint32_t key = kr & 0xffffu;
+  const uint32_t u = (key & 0x8000u) ? (key & 0x7fffu) : (~key & 0xffffu);
+  if (DT == SAH_BF16) return sah_bits_to_float(u << 16) + sah_bits_to_float(kr & 0xffff0000u);
+  return sah_f16_to_float((uint16_t)u) + sah_f16_to_float((uint16_t)(kr >> 16));
+}
 
 // exact expf for fp32 storage (1e-5 output tolerance), hardware exp2 path otherwise
 template <int DT>
@@ -191,14 +210,14 @@ struct att_lane {
       for (int e = 0; e < 8; ++e) qv[e] = 0.f;
     }
   }
-  // puts the batch's 2 * UB row loads on their way
-  template <int UB>
+  // puts the batch's 2 * UB row loads on their way (KEYED: the logits are known, only the V rows are read)
+  template <int UB, bool KEYED = false>
   __device__ __forceinline__ void request(att_batch<DT, UB>& B) const {
 #pragma unroll
     for (int u = 0; u < UB; ++u) {
       const int safe = B.id[u] >= 0 ? B.id[u] : 0;
       if (FULL || live) {
-        att_load_raw<DT>(kbase + (int64_t)safe * krow, B.kr[u]);
+        if (!KEYED) att_load_raw<DT>(kbase + (int64_t)safe * krow, B.kr[u]);
         att_load_raw<DT>(vbase + (int64_t)safe * vrow, B.vr[u]);
       } else {
         B.kr[u].lo = B.kr[u].hi = B.vr[u].lo = B.vr[u].hi = make_uint4(0u, 0u, 0u, 0u);
@@ -227,6 +246,28 @@ struct att_lane {
       mb = fmaxf(mb, d);
     }
     // over the lane groups of the wave: m stays uniform across the wave
+#pragma unroll
+    for (int o = LPK; o < SAH_WAVE; o <<= 1) mb = fmaxf(mb, __shfl_xor(mb, o));
+    return mb;
+  }
+  // the same from score keys: key[u] holds q.k of the lane's key in iteration u as (key, remainder)
+  template <int UB, bool PLAIN = false>
+  __device__ __forceinline__ float logits_of_keys(const att_params& P, int64_t moff, const uint32_t (&key)[UB],
+                                                  const att_batch<DT, UB>& B, float (&z)[UB]) const {
+    float mb = -INFINITY;
+    if constexpr (DT != SAH_F32) {
+#pragma unroll
+      for (int u = 0; u < UB; ++u) {
+        float d = att_key_score<DT>(key[u]) * P.scaling;
+        if (B.id[u] >= 0) {
+          if (!PLAIN && P.amask) d += sah_load<DT>(P.amask, moff + B.id[u]);
+        } else {
+          d = -INFINITY;
+        }
+        z[u] = d;
+        mb = fmaxf(mb, d);
+      }
+    }
 #pragma unroll
     for (int o = LPK; o < SAH_WAVE; o <<= 1) mb = fmaxf(mb, __shfl_xor(mb, o));
     return mb;
@@ -269,13 +310,18 @@ struct att_lane {
 // decode step): their tests and code stay out. A caller whose column list lives in LDS hands col_of a pointer the
 // compiler can see to be LDS: through a generic pointer every read of the list would be a flat load, which waits for
 // all of the wave's outstanding row loads as well.
-template <int DT, int D, bool DROP = false, bool PLAIN = false, bool FULL = true, typename ColOf, typename InvWOf>
+// key_of (anything but att_no_key): key_of(i, column) is q.k for entry i as score key (low half) and remainder (high
+// half) - the caller has scored every column already (an exact-score top-k came before); K is then not read at all,
+// and a batch holds twice as many V rows.
+template <int DT, int D, bool DROP = false, bool PLAIN = false, bool FULL = true, typename ColOf, typename InvWOf,
+          typename KeyOf = att_no_key>
 __device__ __forceinline__ void att_walk(const att_params& P, int r, int b, int h, int hk, int qi, int first, int bound,
-                                         int stride, ColOf col_of, InvWOf inv_w_of, att_wave_state& st) {
+                                         int stride, ColOf col_of, InvWOf inv_w_of, att_wave_state& st, KeyOf key_of = KeyOf()) {
   typedef att_lane<DT, D, FULL> lane_t;
+  constexpr bool KEYED = !std::is_same<KeyOf, att_no_key>::value;
   constexpr int KPI = lane_t::KPI;
   constexpr int IT = SAH_WAVE / KPI;    // iterations per 64-key wave slice
-  constexpr int UB = IT < 4 ? IT : 4;   // iterations per batch
+  constexpr int UB = IT < 4 ? IT : ((KEYED && IT >= 8) ? 8 : 4);   // iterations per batch
   const int lane = threadIdx.x & (SAH_WAVE - 1);
   const lane_t L(P, b, hk);
   const int64_t moff = (!PLAIN && P.amask) ? ((int64_t)b * P.ms_b + (int64_t)h * P.ms_h + (int64_t)qi * P.ms_l) : 0;
@@ -286,11 +332,13 @@ __device__ __forceinline__ void att_walk(const att_params& P, int r, int b, int 
     // one column (and its inverse weight) per lane: this wave's next 64 keys
     const int my = cbase + lane;
     int idx_l = -1;
+    uint32_t key_l = 0;
     float invw_l = P.unit_inv_w, invw_den_l = P.unit_inv_w;
     if (my < bound) {
       idx_l = col_of(my);
       invw_l = inv_w_of(my);
       if (idx_l < 0 || idx_l >= P.Lk) idx_l = -1;
+      if (KEYED && idx_l >= 0) key_l = key_of(my, idx_l);
       invw_den_l = invw_l;
       if (DROP && idx_l >= 0) {
         invw_l *= P.drop.factor(r, idx_l);
@@ -303,9 +351,17 @@ __device__ __forceinline__ void att_walk(const att_params& P, int r, int b, int 
       att_batch<DT, UB> B;
 #pragma unroll
       for (int u = 0; u < UB; ++u) B.id[u] = __shfl(idx_l, (ib + u) * KPI + L.grp);
-      L.request(B);
+      L.template request<UB, KEYED>(B);
       float z[UB];
-      const float mb = L.template logits<UB, PLAIN>(P, moff, qv, B, z);
+      float mb;
+      if constexpr (KEYED) {
+        uint32_t kz[UB];
+#pragma unroll
+        for (int u = 0; u < UB; ++u) kz[u] = (uint32_t)__shfl((int)key_l, (ib + u) * KPI + L.grp);
+        mb = L.template logits_of_keys<UB, PLAIN>(P, moff, kz, B, z);
+      } else {
+        mb = L.template logits<UB, PLAIN>(P, moff, qv, B, z);
+      }
       if (!PLAIN && P.logits_out && L.sub == 0) {
 #pragma unroll
         for (int u = 0; u < UB; ++u) {
@@ -443,7 +499,7 @@ static inline int att_row_parts(int n_rows) {
 // ROW = true: a workgroup of 16 waves handles a whole row, every wave an equal share of the row's entries,
 //   and merges the 16 partial results itself: no workspace, no second kernel, every CU gets the same
 //   amount of work when there are at least as many rows as CUs.
-template <int DT, int D, bool ROW, bool DROP = false, bool FULL = true>
+template <int DT, int D, bool ROW, bool DROP = false, bool FULL = true, bool KEYED = false>
 __device__ __forceinline__ void att_tile(const att_params& P, int r, int b, int h, int hk, int qi, int split, int n_split,
                                          const int* cols_known, int cnt_known,
                                          float (&s_m)[(ROW ? ATT_ROW_NT : ATT_NT) / SAH_WAVE],
@@ -488,11 +544,19 @@ __device__ __forceinline__ void att_tile(const att_params& P, int r, int b, int 
   const float* wts = (!P.dense && P.rows.w) ? P.rows.w + (int64_t)r * P.rows.cap : nullptr;
   att_wave_state st;
   st.clear();
-  att_walk<DT, D, DROP, false, FULL>(
-      P, r, b, h, hk, qi, first, bound, stride,
-      [&](int i) { return P.dense == 1 ? i : (P.dense == 2 ? (i < P.closed_sink ? i : P.closed_lo + (i - P.closed_sink)) : cols[i]); },
-      // the reference evaluates 1/(w + 1e-6) in the mask dtype (utils/mask.py:737-740)
-      [&](int i) { return wts ? sah_round<DT>(1.0f / sah_round<DT>(wts[i] + 1e-6f)) : P.unit_inv_w; }, st);
+  auto col_of = [&](int i) {
+    return P.dense == 1 ? i : (P.dense == 2 ? (i < P.closed_sink ? i : P.closed_lo + (i - P.closed_sink)) : cols[i]);
+  };
+  // the reference evaluates 1/(w + 1e-6) in the mask dtype (utils/mask.py:737-740)
+  auto inv_w_of = [&](int i) { return wts ? sah_round<DT>(1.0f / sah_round<DT>(wts[i] + 1e-6f)) : P.unit_inv_w; };
+  if constexpr (KEYED) {
+    const uint16_t* krow = P.score_keys + (int64_t)r * P.score_pitch;
+    const uint16_t* rrow = P.score_resid + (int64_t)r * P.score_pitch;
+    att_walk<DT, D, DROP, false, FULL>(P, r, b, h, hk, qi, first, bound, stride, col_of, inv_w_of, st,
+                                       [&](int, int col) { return (uint32_t)krow[col] | ((uint32_t)rrow[col] << 16); });
+  } else {
+    att_walk<DT, D, DROP, false, FULL>(P, r, b, h, hk, qi, first, bound, stride, col_of, inv_w_of, st);
+  }
 
   // ---- reduce the lane groups of the wave, then the waves (rescaled to a common max)
   att_park<D, NW>(st, wave, s_m, s_l, s_acc);

@@ -4,9 +4,9 @@
 //
 // Layout as in the attention kernel: LPK = D/8 lanes per key row, 8 elements
 // (one 16 B / 32 B vector load) per lane, DPP reduction inside the lane group.
-// Scores are rounded to the storage type exactly where torch rounds them and
-// emitted as order-preserving unsigned keys through an LDS tile so that the
-// global writes are coalesced.
+// The dot products go through an LDS tile; at the copy-out they are rounded to the
+// storage type exactly where torch rounds them and leave as order-preserving
+// unsigned keys, in coalesced writes.
 #include "sah_common.h"
 
 #define SC_NT 256
@@ -25,6 +25,7 @@ struct qk_params {
   int B, Hq, Hkv, Lq, Lk;
   int d_real;  // head_dim; the kernel's D is d_real padded to a power of two
   void* keys_out; int64_t key_pitch;
+  void* resid_out;  // RES: what the rounding of each score took away, same layout as keys_out
   int iters;  // tiles of SC_TILE keys per workgroup
 };
 
@@ -124,7 +125,8 @@ __device__ __forceinline__ float sc_reduce4(float d0, float d1, float d2, float 
 // AM: an additive attention mask is given (P.amask); without one the scoring loop holds no load but the rows'
 // FULL: head_dim is D itself; otherwise D is head_dim padded to a power of two: the lanes of a key beyond head_dim
 // carry a zero query slice (and re-read the row's first slice, so that no load sits behind a condition)
-template <int DT, int D, bool AM, bool FULL>
+// RES: the remainder of every score's rounding goes out beside its key (16-bit types, no mask)
+template <int DT, int D, bool AM, bool FULL, bool RES = false>
 __global__ __launch_bounds__(SC_NT) void k_qk_scores(qk_params P) {
   sah_touch_kernargs<sizeof(qk_params)>();
   constexpr int LPK = D / 8;
@@ -133,8 +135,10 @@ __global__ __launch_bounds__(SC_NT) void k_qk_scores(qk_params P) {
   constexpr int ES = (DT == SAH_F32) ? 4 : 2;
   constexpr bool FAST4 = LPK >= 4;  // transposing reduction of all four query vectors at once
   typedef typename std::conditional<DT == SAH_F32, uint32_t, uint16_t>::type key_t;
-  __shared__ key_t s_out[SC_NQ][SC_TILE];
-
+  // The tile holds the dot products as they come out of the reduction (fp32); rounding, key and remainder are made
+  // at the copy-out, where every lane has one score per query vector - in the scoring loop only the few lanes that
+  // end up with a total would work on them.
+  __shared__ float s_out[SC_NQ][SC_TILE];
   const int tid = threadIdx.x;
   const int lane = tid & (SAH_WAVE - 1);
   const int wave = sah_wave_id();
@@ -155,10 +159,9 @@ __global__ __launch_bounds__(SC_NT) void k_qk_scores(qk_params P) {
 #pragma unroll
   for (int i = 0; i < SC_NQ; ++i) {
     int v = v0 + i;
-    row[i] = -1;
     moff[i] = 0;
-    const bool live = v < nvec;
-    if (!live) v = nvec - 1;  // computed and dropped
+    // a slot beyond the group's query vectors repeats the last one: it computes and writes the same keys again
+    if (v >= nvec) v = nvec - 1;
     const int h = hk * G + v / P.Lq;
     const int qi = v % P.Lq;
     sc_load<DT>((const char*)P.q + ((int64_t)b * P.qs_b + (int64_t)h * P.qs_h + (int64_t)qi * P.qs_l + sub_k * 8) * ES, qv[i]);
@@ -170,24 +173,13 @@ __global__ __launch_bounds__(SC_NT) void k_qk_scores(qk_params P) {
         qv[i].a = make_uint4(0u, 0u, 0u, 0u);
       }
     }
-    if (live) {
-      row[i] = (b * P.Hq + h) * P.Lq + qi;
-      if (AM) moff[i] = (int64_t)b * P.ms_b + (int64_t)h * P.ms_h + (int64_t)qi * P.ms_l;
-    }
+    row[i] = (b * P.Hq + h) * P.Lq + qi;
+    if (AM) moff[i] = (int64_t)b * P.ms_b + (int64_t)h * P.ms_h + (int64_t)qi * P.ms_l;
   }
   const char* kbase = (const char*)P.k + ((int64_t)b * P.ks_b + (int64_t)hk * P.ks_h + sub_k * 8) * ES;
   const int64_t krow = P.ks_l * ES;
   // which of the four totals this lane ends up with after sc_reduce4
   const int mine = FAST4 ? (2 * (sub & 1) + ((sub >> 1) & 1)) : 0;
-  int row_mine = row[0];
-  int64_t moff_mine = moff[0];
-#pragma unroll
-  for (int i = 1; i < SC_NQ; ++i) {
-    if (mine == i) {
-      row_mine = row[i];
-      moff_mine = moff[i];
-    }
-  }
 
   // A wave owns 64 consecutive keys of every tile and the matching columns of s_out: no workgroup
   // barrier anywhere. The rows come in half-slices of HB iterations through two register buffers;
@@ -218,36 +210,42 @@ __global__ __launch_bounds__(SC_NT) void k_qk_scores(qk_params P) {
 #pragma unroll
     for (int it = 0; it < HB; ++it) {
       const int jl = jl0 + it * KPI + grp;
-      const int j = tile * SC_TILE + jl;
       if constexpr (FAST4) {
         const float d = sc_reduce4<LPK>(sc_dot<DT>(qv[0], buf[it]), sc_dot<DT>(qv[1], buf[it]), sc_dot<DT>(qv[2], buf[it]),
                                          sc_dot<DT>(qv[3], buf[it]), sub);
-        // without a mask nothing is read here: keys past the row's end and dead query vectors park a value that
-        // the copy-out below never stores
-        if (sub < 4 && (!AM || (j < P.Lk && row_mine >= 0))) {
-          float s = sah_round<DT>(d);
-          if (AM) s = sah_round<DT>(s + sah_load<DT>(P.amask, moff_mine + j));
-          s_out[mine][jl] = (key_t)sah_sort_key<DT>(s);
-        }
+        // keys past the row's end and dead query vectors park a value that the copy-out below never stores
+        if (sub < 4) s_out[mine][jl] = d;
       } else {
 #pragma unroll
         for (int i = 0; i < SC_NQ; ++i) {
           const float d = sc_group_sum<LPK>(sc_dot<DT>(qv[i], buf[it]));
-          if (sub == (i % LPK) && j < P.Lk && row[i] >= 0) {
-            float s = sah_round<DT>(d);
-            if (AM) s = sah_round<DT>(s + sah_load<DT>(P.amask, moff[i] + j));
-            s_out[i][jl] = (key_t)sah_sort_key<DT>(s);
-          }
+          if (sub == (i % LPK)) s_out[i][jl] = d;
         }
       }
     }
     if (hs % NH == NH - 1) {
-      // the wave's 64 keys of this tile are scored: write them out, one key per lane and query vector
+      // The wave's 64 keys of this tile are scored: write them out, one key per lane and query vector. No store
+      // sits behind a condition (a lane past the row's end has scored the last key again, and writes it again): after
+      // a store that may or may not have been issued, the compiler's waits for the row loads in flight are the
+      // stricter of the two cases, and the two register buffers no longer overlap.
       sah_wave_lds_sync();
-      const int j = tile * SC_TILE + wave * SAH_WAVE + lane;
+      int j = tile * SC_TILE + wave * SAH_WAVE + lane;
+      if (j > P.Lk - 1) j = P.Lk - 1;
 #pragma unroll
       for (int i = 0; i < SC_NQ; ++i) {
-        if (row[i] >= 0 && j < P.Lk) ((key_t*)P.keys_out)[(int64_t)row[i] * P.key_pitch + j] = s_out[i][wave * SAH_WAVE + lane];
+        const float d = s_out[i][wave * SAH_WAVE + lane];
+        float s = sah_round<DT>(d);
+        if (AM) s = sah_round<DT>(s + sah_load<DT>(P.amask, moff[i] + j));
+        ((key_t*)P.keys_out)[(int64_t)row[i] * P.key_pitch + j] = (key_t)sah_sort_key<DT>(s);
+        if constexpr (RES) {
+          // the remainder of the rounding in DT's own bits (bf16: cut off, not rounded - it is a correction of a
+          // correction; a score that rounds to infinity leaves none)
+          const float rem = d - s;
+          uint16_t rb;
+          if (DT == SAH_BF16) rb = (uint16_t)(sah_float_to_bits(rem) >> 16);
+          else rb = fabsf(s) < INFINITY ? (uint16_t)sah_float_to_f16(rem) : (uint16_t)0;
+          ((uint16_t*)P.resid_out)[(int64_t)row[i] * P.key_pitch + j] = rb;
+        }
       }
       sah_wave_lds_sync();  // the columns are free again for the next tile
     }
@@ -286,7 +284,9 @@ static int qk_launch(const sah_qk_scores_args* a, const qk_params& P) {
   Q.iters = iters;
   dim3 g((unsigned)((tiles + iters - 1) / iters), a->B * a->Hkv, (nvec + SC_NQ - 1) / SC_NQ);
   sah_timed timed("k_qk_scores", a->stream);
+  constexpr bool CAN_RES = DT != SAH_F32 && FULL && (D == 64 || D == 128);
   if (a->amask) hipLaunchKernelGGL((k_qk_scores<DT, D, true, FULL>), g, dim3(SC_NT), 0, (hipStream_t)a->stream, Q);
+  else if (CAN_RES && a->resid_out) hipLaunchKernelGGL((k_qk_scores<DT, D, false, FULL, CAN_RES>), g, dim3(SC_NT), 0, (hipStream_t)a->stream, Q);
   else hipLaunchKernelGGL((k_qk_scores<DT, D, false, FULL>), g, dim3(SC_NT), 0, (hipStream_t)a->stream, Q);
   return sah_launch_status("sah_qk_scores");
 }
@@ -328,6 +328,9 @@ extern "C" int sah_qk_scores(const sah_qk_scores_args* a) {
   P.B = a->B; P.Hq = a->Hq; P.Hkv = a->Hkv; P.Lq = a->Lq; P.Lk = a->Lk;
   P.d_real = a->D;
   P.keys_out = a->keys_out; P.key_pitch = a->key_pitch;
+  P.resid_out = a->resid_out;
+  if (a->resid_out && (a->amask || a->dtype == SAH_F32 || (a->D != 64 && a->D != 128)))
+    return sah_fail(SAH_EINVAL, "sah_qk_scores: resid_out needs a 16-bit dtype, head_dim 64 or 128 and no additive mask");
   switch (a->dtype) {
     case SAH_F32: return qk_dispatch_d<SAH_F32>(a, P);
     case SAH_BF16: return qk_dispatch_d<SAH_BF16>(a, P);

@@ -26,11 +26,15 @@ struct selattn_params {
   int write_bitmap;
   int parts;
   int cols_offset;  // of the column list inside the dynamic LDS
+  const uint16_t* resid;  // KEYED: what the keys' rounding took away, laid out like `keys`
   float* work;        // [row][part][D + 2]
   uint32_t* tickets;  // [row], zero between kernels
 };
 
-template <int DT, int D, int CPW>
+// KEYED: the score keys are q.k itself, rounded as torch's matmul rounds it, and come with the remainders of that
+// rounding (the exact scoring pass of OracleTopK): the walk takes its logits from there (two 2-byte reads per entry,
+// of lines the selection has just pulled through the L2) and reads V rows only.
+template <int DT, int D, int CPW, bool KEYED>
 __global__ __launch_bounds__(SF_NT) void k_select16_attn(selattn_params P, att_params A) {
   sah_touch_kernargs<sizeof(selattn_params) + sizeof(att_params)>();
   constexpr int NW = SF_NT / SAH_WAVE;
@@ -82,7 +86,18 @@ __global__ __launch_bounds__(SF_NT) void k_select16_attn(selattn_params P, att_p
   att_wave_state st;
   st.clear();
   const float unit = A.unit_inv_w;
-  if (P.fresh)
+  const uint16_t* krow = P.keys + (int64_t)r * P.pitch;
+  const uint16_t* rrow = KEYED ? P.resid + (int64_t)r * P.pitch : nullptr;
+  auto key_of = [&](int, int col) { return (uint32_t)krow[col] | ((uint32_t)rrow[col] << 16); };  // col_offset is 0
+  if (KEYED && P.fresh)
+    att_walk<DT, D, false, true>(
+        A, r, b, h, hk, qi, first, bound, SAH_WAVE,
+        [&](int i) { return i >= earlier ? s_cols[i] : (i < s_hi ? i : lo2 + (i - s_hi)); }, [&](int) { return unit; }, st, key_of);
+  else if (KEYED)
+    att_walk<DT, D, false, true>(
+        A, r, b, h, hk, qi, first, bound, SAH_WAVE, [&](int i) { return i >= earlier ? s_cols[i] : cols_mem[i]; },
+        [&](int) { return unit; }, st, key_of);
+  else if (P.fresh)
     att_walk<DT, D, false, true>(
         A, r, b, h, hk, qi, first, bound, SAH_WAVE,
         [&](int i) { return i >= earlier ? s_cols[i] : (i < s_hi ? i : lo2 + (i - s_hi)); }, [&](int) { return unit; }, st);
@@ -114,20 +129,22 @@ int64_t selattn_work_floats(int n_rows, int D) {
   return (int64_t)n_rows * parts * (D + 2);
 }
 
-template <int DT, int D, int CPW>
+template <int DT, int D, int CPW, bool KEYED>
 static int selattn_launch(const sah_select_topk_args* s, const selattn_params& P, const att_params& A, size_t lds) {
-  if (int rc = sah_allow_lds((const void*)k_select16_attn<DT, D, CPW>, 150 * 1024, "sah_select_topk_attention")) return rc;
+  if (int rc = sah_allow_lds((const void*)k_select16_attn<DT, D, CPW, KEYED>, 150 * 1024, "sah_select_topk_attention")) return rc;
   const int G = A.Hq / A.Hkv;
   const int n_tiles = P.R.n_rows / G;
   const int n_wg = (n_tiles + ATT_XCDS - 1) / ATT_XCDS * ATT_XCDS * G * P.parts;
   sah_timed timed("k_select16_attn", s->stream);
-  hipLaunchKernelGGL((k_select16_attn<DT, D, CPW>), dim3(n_wg), dim3(SF_NT), lds, (hipStream_t)s->stream, P, A);
+  hipLaunchKernelGGL((k_select16_attn<DT, D, CPW, KEYED>), dim3(n_wg), dim3(SF_NT), lds, (hipStream_t)s->stream, P, A);
   return sah_launch_status("sah_select_topk_attention");
 }
 
 template <int DT, int D>
-static int selattn_launch_c(const sah_select_topk_args* s, const selattn_params& P, const att_params& A, size_t lds, int cpw) {
-  return cpw <= 4 ? selattn_launch<DT, D, 4>(s, P, A, lds) : selattn_launch<DT, D, 8>(s, P, A, lds);
+static int selattn_launch_c(const sah_select_topk_args* s, const selattn_params& P, const att_params& A, size_t lds, int cpw,
+                            bool keyed) {
+  if (keyed) return cpw <= 4 ? selattn_launch<DT, D, 4, true>(s, P, A, lds) : selattn_launch<DT, D, 8, true>(s, P, A, lds);
+  return cpw <= 4 ? selattn_launch<DT, D, 4, false>(s, P, A, lds) : selattn_launch<DT, D, 8, false>(s, P, A, lds);
 }
 
 extern "C" int sah_select_topk_attention(const sah_select_topk_args* s, const sah_attention_args* t, uint32_t* tickets) {
@@ -140,6 +157,9 @@ extern "C" int sah_select_topk_attention(const sah_select_topk_args* s, const sa
   const int n_rows = s->rows.n_rows;
   const int cpw = sf_chunks_per_wave(s->n_cand);
   const size_t cols_offset = sf_hist_offset(s->rows.n_words);
+  // the selection's keys are the attention's logits: the caller names the same array as the attention's score keys
+  const bool keyed = t->score_keys && t->score_resid && t->score_keys == s->keys && t->score_pitch == s->key_pitch &&
+                     s->col_offset == 0 && s->n_cand == s->rows.n_keys;
   const size_t lds = sf_lds_bytes(s->rows.n_words);
   const int parts = att_row_parts(n_rows);
   const int64_t need = selattn_work_floats(n_rows, t->D);
@@ -167,9 +187,11 @@ extern "C" int sah_select_topk_attention(const sah_select_topk_args* s, const sa
   P.write_bitmap = s->skip_bitmap ? 0 : 1;
   P.parts = parts;
   P.cols_offset = (int)cols_offset;
+  P.resid = (const uint16_t*)t->score_resid;
   P.work = t->work;
   P.tickets = tickets;
-#define SAH_SA(DTC) (t->D == 128 ? selattn_launch_c<DTC, 128>(s, P, A, lds, cpw) : selattn_launch_c<DTC, 64>(s, P, A, lds, cpw))
+#define SAH_SA(DTC) \
+  (t->D == 128 ? selattn_launch_c<DTC, 128>(s, P, A, lds, cpw, keyed) : selattn_launch_c<DTC, 64>(s, P, A, lds, cpw, keyed))
   return t->dtype == SAH_BF16 ? SAH_SA(SAH_BF16) : SAH_SA(SAH_F16);
 #undef SAH_SA
 }

@@ -155,6 +155,7 @@ class QkScoresArgs(C.Structure):
         ("keys_out", C.c_void_p),
         ("key_pitch", C.c_int64),
         ("stream", C.c_void_p),
+        ("resid_out", C.c_void_p),
     ]
 
 
@@ -295,6 +296,9 @@ class AttentionArgs(C.Structure):
         ("dropout_seed", C.c_uint64),
         ("dropout_offset", C.c_uint64),
         ("dropout_numerator_only", C.c_int32),
+        ("score_keys", C.c_void_p),
+        ("score_resid", C.c_void_p),
+        ("score_pitch", C.c_int64),
     ]
 
 

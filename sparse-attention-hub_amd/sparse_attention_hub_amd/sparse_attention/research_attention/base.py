@@ -147,6 +147,9 @@ class ResearchAttention(SparseAttention):
         s_aux_raw: Any = kwargs.pop("s_aux", None)
         s_aux: Optional[torch.Tensor] = s_aux_raw if isinstance(s_aux_raw, torch.Tensor) else None
         weights: Optional[torch.Tensor] = None
+        # a masker of this call scored every key exactly (OracleTopK, AdaptiveSampling): the attention takes its
+        # logits from those scores instead of reading K again
+        kwargs["_score_keys"] = (call_scratch.get("qk_score_keys"), call_scratch.get("qk_score_resid"))
         if self.return_attention_weights:
             out, weights = get_masked_attention_output(
                 module=module, queries=queries, keys=keys, values=values, attention_mask=attention_mask,

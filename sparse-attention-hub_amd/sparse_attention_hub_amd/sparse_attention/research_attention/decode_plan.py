@@ -82,6 +82,7 @@ class DecodePlan:
         self.cols = self.cnt = self.bitmap = None
         self.qcodes = None
         self.keybuf = None
+        self.residbuf = None
         self.keybuf_pitch = 0
         self.layers: Dict[int, _LayerBlocks] = {}
         self.sink_local = N.SinkLocalArgs()
@@ -123,6 +124,10 @@ class DecodePlan:
             self.keybuf_pitch = (n_cols + 4096 + 63) // 64 * 64
             kdt = torch.int32 if self.dtype == torch.float32 else torch.int16
             self.keybuf = torch.empty((self.n_rows, self.keybuf_pitch), dtype=kdt, device=self.device)
+            # exact scores (OracleTopK) of 16-bit tensors: what their rounding took away goes beside the keys, and the
+            # attention takes its logits from the two instead of reading K again
+            self.residbuf = (torch.empty_like(self.keybuf)
+                             if self.kind == "oracle" and kdt == torch.int16 and self.D in (64, 128) else None)
 
     # --------------------------------------------------------------------- run
     def run(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scaling: float,
@@ -242,6 +247,7 @@ class DecodePlan:
             qa.amask = None
             qa.dtype, qa.B, qa.Hq, qa.Hkv, qa.Lq, qa.Lk, qa.D = self.dt, self.B, self.Hq, self.Hkv, Lq, Lk, self.D
             qa.keys_out, qa.key_pitch, qa.stream = self.keybuf.data_ptr(), self.keybuf_pitch, stream
+            qa.resid_out = None if self.residbuf is None else self.residbuf.data_ptr()
             chain.qk = C.addressof(qa)
             se = self.select
             se.rows, se.keys, se.key_pitch, se.key_bits = rows, self.keybuf.data_ptr(), self.keybuf_pitch, self.key_bits
@@ -324,6 +330,10 @@ class DecodePlan:
         at.out, at.work, at.work_floats = out.data_ptr(), work.data_ptr(), work.numel()
         at.logits_out = at.stats_out = None
         at.closed_form = 0
+        # an exact scoring pass came before: its 16-bit keys are the attention's logits, K is not read again
+        at.score_keys, at.score_resid, at.score_pitch = None, None, 0
+        if self.kind == "oracle" and self.residbuf is not None:
+            at.score_keys, at.score_resid, at.score_pitch = self.keybuf.data_ptr(), self.residbuf.data_ptr(), self.keybuf_pitch
         if self.kind == "fixed" and Lq == 1:
             # Sink + Local alone: the attention kernel takes the columns in closed form, no row is ever written
             at.closed_form, at.closed_sink, at.closed_window = 1, sink, window

@@ -46,6 +46,15 @@ def score_key_buffer(n_rows: int, n_cols: int, dtype: torch.dtype, device: torch
     return torch.empty((n_rows, pitch), dtype=kdt, device=device)
 
 
+def score_remainder_buffer(keybuf: torch.Tensor, head_dim: int, masked: bool) -> Optional[torch.Tensor]:
+    """Beside 16-bit score keys of an unmasked scoring pass: room for what the scores' rounding took away
+    (`sah_qk_scores_args.resid_out`), with which the attention of the same call need not read K again. None where the
+    kernels have no use for it (fp32 tensors, an additive mask in the scores, head_dim other than 64 / 128)."""
+    if masked or keybuf.dtype != torch.int16 or head_dim not in (64, 128):
+        return None
+    return torch.empty_like(keybuf)
+
+
 @MaskerRegistry.register(OracleTopKConfig)
 class OracleTopK(TopKMasker):
     heavy_size: Union[float, int]
@@ -83,17 +92,20 @@ class OracleTopK(TopKMasker):
         rows = previous_mask.to_rows(extra=k_eff)
         keybuf = score_key_buffer(rows.n_rows, Lk, q.dtype, q.device)
         am_keep, am_ptr, ms_b, ms_h, ms_l = additive_mask_args(attention_mask, q, Lk)
+        shared = kwargs.get("_call_scratch")
+        resid = score_remainder_buffer(keybuf, D, am_ptr is not None) if isinstance(shared, dict) else None
         args = N.QkScoresArgs(
             q.data_ptr(), q.stride(0), q.stride(1), q.stride(2),
             k.data_ptr(), k.stride(0), k.stride(1), k.stride(2),
             am_ptr, ms_b, ms_h, ms_l,
             N.dtype_code(q.dtype), B, Hq, Hkv, Lq, Lk, D,
             keybuf.data_ptr(), keybuf.stride(0), N.stream_ptr(q.device),
+            None if resid is None else resid.data_ptr(),
         )
         N.call("sah_qk_scores", args)
-        shared = kwargs.get("_call_scratch")
         if am_ptr is None and isinstance(shared, dict):
             shared["qk_score_keys"] = keybuf  # later maskers of this call can skip their own scoring pass
+            shared["qk_score_resid"] = resid  # ... and the attention its reading of K
             # ... and know that the largest key of every row now belongs to a column of the row: the k_eff >= 1
             # largest keys outside the previous mask were just added
             shared["qk_top_in_rows"] = True

@@ -32,7 +32,7 @@ from .....utils.mask import Mask
 from .....utils.mask_attention_utils import _inner_contiguous, additive_mask_args
 from ...... import _native as N
 from ...base import AttentionTensorDimensions, MaskerConfig, MaskerRegistry
-from ...fixed.implementations.oracle_top_k import score_key_buffer
+from ...fixed.implementations.oracle_top_k import score_key_buffer, score_remainder_buffer
 from ..base import SamplingMasker, SamplingMaskerConfig
 
 _RATE_GRID = [0.01, 0.02, 0.03]
@@ -177,16 +177,19 @@ class AdaptiveSamplingMasker(SamplingMasker):
         if keybuf is None:
             k = _inner_contiguous(keys)
             keybuf = score_key_buffer(n_rows, Lk, q.dtype, q.device)
+            resid = score_remainder_buffer(keybuf, D, False) if isinstance(shared, dict) else None
             args = N.QkScoresArgs(
                 q.data_ptr(), q.stride(0), q.stride(1), q.stride(2),
                 k.data_ptr(), k.stride(0), k.stride(1), k.stride(2),
                 None, 0, 0, 0,
                 N.dtype_code(q.dtype), B, Hq, Hkv, Lq, Lk, D,
                 keybuf.data_ptr(), keybuf.stride(0), N.stream_ptr(q.device),
+                None if resid is None else resid.data_ptr(),
             )
             N.call("sah_qk_scores", args)
             if isinstance(shared, dict):
                 shared["qk_score_keys"] = keybuf
+                shared["qk_score_resid"] = resid
 
         nb = self._get_base_sample_count(n)
         prev_empty = previous_mask.is_empty_mask()

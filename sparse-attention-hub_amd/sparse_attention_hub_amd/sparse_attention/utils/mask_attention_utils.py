@@ -112,10 +112,13 @@ def _run_attention(
     return_stats: bool = False,
     dropout: Tuple[float, int, int] = (0.0, 0, 0),
     dropout_numerator_only: bool = False,
+    score_keys: Optional[Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]] = None,
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """rows=None => dense attention over all keys. `return_stats`: the second value is the kernel's
     fp32 (n_rows, 2) tensor of (largest logit among the row's entries, softmax denominator relative to it)
-    instead of the dense probabilities."""
+    instead of the dense probabilities. `score_keys`: the (n_rows, >= Lk) 16-bit keys and remainders
+    `sah_qk_scores` wrote for these queries and keys without an additive mask, when a masker of this call has scored
+    every key already - the kernel then takes its logits from there and does not read K."""
     N.require_device(queries, "queries")
     N.require_device(keys, "keys")
     N.require_device(values, "values")
@@ -174,6 +177,11 @@ def _run_attention(
         N.stream_ptr(dev),
         dropout[0], dropout[1], dropout[2], int(dropout_numerator_only),
     )
+    sk, sr = score_keys if score_keys is not None else (None, None)
+    if (sk is not None and sr is not None and not dense and sk.dtype == torch.int16 and sk.device == dev
+            and sk.ndim == 2 and sk.shape[0] == n_rows and sk.stride(1) == 1 and sk.stride(0) >= Lk
+            and sr.dtype == sk.dtype and sr.shape == sk.shape and sr.stride() == sk.stride()):
+        args.score_keys, args.score_resid, args.score_pitch = sk.data_ptr(), sr.data_ptr(), sk.stride(0)
     N.call("sah_sparse_attention", args)
     if return_stats:
         return out, stats
@@ -251,7 +259,7 @@ def get_masked_attention_output(
         rows = mask.to_rows(0)
     out, weights = _run_attention(
         queries, keys, values, attention_mask, sinks, scaling, rows, return_attention_weights,
-        dropout=_training_dropout(module, dropout),
+        dropout=_training_dropout(module, dropout), score_keys=kwargs.get("_score_keys"),
     )
     if return_attention_weights:
         return out, weights

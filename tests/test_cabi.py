@@ -129,6 +129,10 @@ def test_bad_argument_blocks_are_refused_with_the_documented_codes():
     assert lib.sah_select_topk(ctypes.byref(sel)) == -1
     # what the no-allocation attention refuses is more than its built-in buffer holds
     assert N.work_floats(1024, 131072, 128) > 4 * 1024 * 1024 >= N.work_floats(512, 131072, 128)
+    # the remainders of a scoring pass: 16-bit scores only
+    al = (ptr + 63) // 64 * 64
+    qk = N.QkScoresArgs(al, 128, 128, 128, al, 128, 128, 128, None, 0, 0, 0, 0, 1, 1, 1, 1, 8, 128, al, 64, None, al)
+    assert lib.sah_qk_scores(ctypes.byref(qk)) == -1 and b"resid_out" in lib.sah_last_error()
     # additive-mask classification: empty shape, too many rows, unknown dtype
     amc = N.AmaskClassifyArgs(ptr, 0, 0, 0, 1, 2, 1, 1, 0, ptr, None)
     assert lib.sah_amask_classify(ctypes.byref(amc)) == -1

@@ -1376,3 +1376,84 @@ def test_composite_sampling_stacks(cuda, base):
     oo, ow, om = O.research_attention(specs, q, k, v, None, scaling, None, state)
     assert torch.equal(w.cpu() != 0, ow != 0)
     assert rel_err(out, oo) < TOL[dtype]
+
+
+# ------------------------------------------------------------------------ logits from the scoring pass
+def _key_scores(keys16, resid16, dtype):
+    """fp32 (score, remainder) from the 16-bit score keys (the inverse of the order-preserving map) and the remainder
+    words, both (rows, n) int16 tensors on the host."""
+    k = keys16.to(torch.int32) & 0xFFFF
+    bits = torch.where((k & 0x8000) != 0, k & 0x7FFF, (~k) & 0xFFFF).to(torch.int16)
+    return bits.view(dtype).float(), resid16.view(dtype).float()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(1, 8, 2, 1, 6000, 128, 900), (8, 32, 8, 1, 1500, 64, 300), (2, 4, 4, 2, 700, 128, 64)])
+def test_attention_takes_its_logits_from_the_scoring_pass(cuda, dtype, shape):
+    """`sah_qk_scores` with `resid_out`: the keys are unchanged and key + remainder reproduce the fp32 dot product to
+    about 16 mantissa bits. `sah_sparse_attention` with `score_keys` / `score_resid`: the same output as from K (to the
+    rounding of the 16-bit result), and K is not read at all - the call gives the same bits when K holds garbage."""
+    from sparse_attention_hub_amd import _native as N
+    from sparse_attention_hub_amd.sparse_attention.utils.mask_attention_utils import unit_inverse_weight
+
+    B, Hq, Hkv, Lq, Lk, D, n_sel = shape
+    q, k, v = make_qkv(B, Hq, Hkv, Lq, Lk, D, dtype, seed=31, outliers=True, device=cuda)
+    n_rows = B * Hq * Lq
+    pitch = (Lk + 63) // 64 * 64
+    keys = torch.zeros((n_rows, pitch), dtype=torch.int16, device=cuda)
+    keys_plain = torch.zeros_like(keys)
+    resid = torch.zeros_like(keys)
+
+    def score(keys_out, resid_out):
+        N.call("sah_qk_scores", N.QkScoresArgs(
+            q.data_ptr(), q.stride(0), q.stride(1), q.stride(2), k.data_ptr(), k.stride(0), k.stride(1), k.stride(2),
+            None, 0, 0, 0, N.dtype_code(dtype), B, Hq, Hkv, Lq, Lk, D, keys_out.data_ptr(), pitch, N.stream_ptr(cuda),
+            None if resid_out is None else resid_out.data_ptr()))
+
+    score(keys, resid)
+    score(keys_plain, None)
+    torch.cuda.synchronize()
+    assert torch.equal(keys, keys_plain)
+    G = Hq // Hkv
+    exact = torch.einsum("bhqd,bhkd->bhqk", q.double().cpu(), k.double().cpu().repeat_interleave(G, dim=1)).reshape(n_rows, Lk)
+    s, rem = _key_scores(keys[:, :Lk].cpu(), resid[:, :Lk].cpu(), dtype)
+    assert bool(torch.isfinite(s).all())
+    scale = exact.abs().clamp_min(1.0)
+    # the key alone is the score rounded to the tensor type (8 or 11 mantissa bits); with the remainder 2^-15 or better
+    assert float(((s.double() - exact).abs() / scale).max()) > 2.0 ** -12
+    assert float((((s + rem).double() - exact).abs() / scale).max()) < 2.0 ** -15
+
+    g = torch.Generator().manual_seed(5)
+    cols = torch.stack([torch.randperm(Lk, generator=g)[:n_sel] for _ in range(n_rows)]).to(torch.int32).to(cuda)
+    cnt = torch.full((n_rows,), n_sel, dtype=torch.int32, device=cuda)
+    cnt[0] = n_sel // 3
+    w = (torch.rand((n_rows, n_sel), generator=g) * 0.9 + 0.1).to(cuda)
+    bitmap = torch.zeros((n_rows, (Lk + 31) // 32), dtype=torch.int32, device=cuda)
+    rows = N.Rows(cols.data_ptr(), cnt.data_ptr(), w.data_ptr(), bitmap.data_ptr(), n_rows, n_sel, Lk, (Lk + 31) // 32)
+    work = torch.zeros((max(1, N.work_floats(n_rows, n_sel, D)),), dtype=torch.float32, device=cuda)
+    sinks = torch.linspace(-1.0, 1.0, Hq, device=cuda)
+
+    def attend(k_tensor, with_keys):
+        out = torch.zeros((B, Lq, Hq, D), dtype=dtype, device=cuda)
+        stats = torch.zeros((n_rows, 2), dtype=torch.float32, device=cuda)
+        a = N.AttentionArgs(
+            rows, q.data_ptr(), q.stride(0), q.stride(1), q.stride(2),
+            k_tensor.data_ptr(), k_tensor.stride(0), k_tensor.stride(1), k_tensor.stride(2),
+            v.data_ptr(), v.stride(0), v.stride(1), v.stride(2), None, 0, 0, 0, sinks.data_ptr(),
+            N.dtype_code(dtype), B, Hq, Hkv, Lq, Lk, D, float(D ** -0.5), unit_inverse_weight(dtype), 0, 0, 0, 0, n_sel,
+            out.data_ptr(), work.data_ptr(), work.numel(), None, stats.data_ptr(), N.stream_ptr(cuda))
+        if with_keys:
+            a.score_keys, a.score_resid, a.score_pitch = keys.data_ptr(), resid.data_ptr(), pitch
+        N.call("sah_sparse_attention", a)
+        torch.cuda.synchronize()
+        return out, stats
+
+    from_k, st_k = attend(k, False)
+    from_keys, st_keys = attend(k, True)
+    garbage = torch.full_like(k, 3.0)
+    from_keys_no_k, _ = attend(garbage, True)
+    wrong, _ = attend(garbage, False)
+    assert torch.equal(from_keys, from_keys_no_k)             # K is not read
+    assert rel_err(wrong, from_k) > 0.1                       # ... which the plain call would have noticed
+    assert rel_err(from_keys, from_k) < (4e-3 if dtype == torch.bfloat16 else 1e-3)
+    assert float((st_keys - st_k).abs().max() / st_k.abs().max()) < 1e-3
