@@ -43,7 +43,7 @@ extern "C" {
  * entry point changes its signature, and never otherwise: a caller compares sah_version() with the SAH_VERSION it was
  * compiled (or, for a ctypes binding, written) against before its first call and refuses a library that differs,
  * because a struct of another generation would be read past its end. */
-#define SAH_VERSION 3
+#define SAH_VERSION 4
 
 enum {
   SAH_OK = 0,

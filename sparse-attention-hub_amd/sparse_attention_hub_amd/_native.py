@@ -18,7 +18,7 @@ _PKG_ROOT = Path(__file__).resolve().parent.parent  # sparse-attention-hub_amd/
 _DEFAULT_LIB = _PKG_ROOT / "lib" / "libsah_mi355.so"
 
 # SAH_VERSION of the include/sah.h the structures below were written against
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 SAH_F32, SAH_BF16, SAH_F16 = 0, 1, 2
 SAH_ACT = {"relu": 0, "silu": 1, "gelu": 2, "tanh": 3}

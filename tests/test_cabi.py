@@ -19,7 +19,7 @@ def _declared_functions():
 def test_library_is_built_and_loads():
     assert N.library_path().exists(), "build it with python sparse-attention-hub_amd/build.py"
     lib = N.lib()
-    assert lib.sah_version() == N.ABI_VERSION == 3
+    assert lib.sah_version() == N.ABI_VERSION == 4
 
 
 def test_a_library_of_another_layout_generation_is_refused(monkeypatch):
