@@ -484,3 +484,46 @@ def test_config3_chain_at_other_batch_sizes_matches_the_oracle(cuda, B):
         oo, _, om = O.research_attention(specs, q[b:b + 1], k[b:b + 1], v[b:b + 1], None, scaling, state=state)
         assert torch.equal(member[b], om.to_dense()[0, :, 0] != 0), f"batch row {b}: selected sets differ"
         assert rel_err(out[b], oo[0]) < 2e-2
+
+
+@pytest.mark.parametrize("kind", ["hash", "oracle", "pq"])
+def test_rows_shared_by_several_workgroups_give_the_same_bits_every_time(cuda, kind):
+    """Batch 1 at 32768 keys: 32 mask rows, 8 workgroups per row, the one that arrives last merges. The order of arrival
+    changes from launch to launch, the result must not: 40 repetitions of the same decode step (same queries, same keys)
+    through the plan give the same output bits and the same rows, and the arrival counters are back at zero after each."""
+    from sparse_attention_hub_amd.sparse_attention.utils.hashattention_utils import random_hat_weights
+
+    sa = _sa()
+    B, Hq, Hkv, Lk, D = 1, 32, 8, 32768, 128
+    sink, window, heavy = 128, 256, 1024
+    dtype = torch.bfloat16
+    q, k, v = make_qkv(B, Hq, Hkv, 1, Lk, D, dtype, seed=91, outliers=(kind != "hash"), device=cuda)
+    if kind == "hash":
+        wts = random_hat_weights(1, Hq, D, 32, 3, 128, dtype=dtype, seed=1)
+        top = sa.HashAttentionTopKMaskerConfig(heavy_size=heavy, hat_bits=32, hat_mlp_layers=3, hat_mlp_hidden_size=128,
+                                               hat_mlp_activation="silu", hat_weights=wts)
+    elif kind == "oracle":
+        top = sa.OracleTopKConfig(heavy_size=heavy)
+    else:
+        top = sa.PQCacheConfig(heavy_size=heavy, pq_group_factor=16, pq_bits=8, kmeans_iter=2, init_offset=sink, metric="euclidean")
+    ra = sa.ResearchAttention.create_from_config(sa.ResearchAttentionConfig(
+        masker_configs=[sa.SinkMaskerConfig(sink_size=sink), sa.LocalMaskerConfig(window_size=window), top]))
+    ra.return_attention_weights = False
+    meta = {}
+    scaling = D ** -0.5
+    # the caches are built on the first call (one key short), the plan takes over from the second
+    ra.custom_attention(None, q, k[:, :, :Lk - 1], v[:, :, :Lk - 1], None, scaling, 0.0, sparse_meta_data=meta, layer_idx=0)
+    first, first_rows = None, None
+    for rep in range(40):
+        out, _ = ra.custom_attention(None, q, k, v, None, scaling, 0.0, sparse_meta_data=meta, layer_idx=0)
+        plan = next(iter(ra._plans.values()))
+        torch.cuda.synchronize()
+        assert int(plan.tickets.abs().max()) == 0, rep
+        rows = torch.sort(plan.cols[:, :sink + window + heavy], dim=1).values
+        if first is None:
+            first, first_rows = out.clone(), rows.clone()
+            assert plan.kind == kind and bool((plan.cnt == sink + window + heavy).all())
+            assert bool(torch.isfinite(out.float()).all()) and float(out.float().abs().max()) > 0
+        else:
+            assert torch.equal(out, first), f"repetition {rep}: output bits differ"
+            assert torch.equal(rows, first_rows), f"repetition {rep}: rows differ"

@@ -2,6 +2,7 @@
 seeded inputs. Bars: index sets bit-exact (ties to the lowest column); attention outputs
 within 1e-5 relative error for fp32 and 2e-2 for bf16."""
 import copy
+import ctypes as C
 import math
 
 import pytest
@@ -1457,3 +1458,74 @@ def test_attention_takes_its_logits_from_the_scoring_pass(cuda, dtype, shape):
     assert rel_err(wrong, from_k) > 0.1                       # ... which the plain call would have noticed
     assert rel_err(from_keys, from_k) < (4e-3 if dtype == torch.bfloat16 else 1e-3)
     assert float((st_keys - st_k).abs().max() / st_k.abs().max()) < 1e-3
+
+
+@pytest.mark.parametrize("case", ["one_per_row", "parts", "parts_keyed", "one_per_row_keyed", "not_fresh", "fallback_f32"])
+def test_select_topk_attention_entry_point_against_the_two_calls(cuda, case):
+    """`sah_select_topk_attention` through the C ABI (no plan in between): rows (column sets, counts, bitmap) and output
+    of the one call against `sah_select_topk` followed by `sah_sparse_attention`, with one workgroup per row, with
+    several (their partial results merged by the last arrival, the tickets left at zero), with the logits taken from the
+    scoring pass, on rows that already hold sink and local columns, and where the one-kernel form does not apply."""
+    from sparse_attention_hub_amd import _native as N
+    from sparse_attention_hub_amd.sparse_attention.utils.mask_attention_utils import unit_inverse_weight
+    from sparse_attention_hub_amd.sparse_attention.utils.native_rows import NativeRows
+
+    dtype = torch.float32 if case == "fallback_f32" else torch.bfloat16
+    B, Hq, Hkv, Lk, D = (8, 32, 8, 2500, 128) if case in ("one_per_row", "one_per_row_keyed", "not_fresh") else (1, 8, 2, 5000, 64)
+    sink, window, k = 16, 48, 200
+    keyed = case.endswith("keyed")
+    fresh = case != "not_fresh"
+    q, kk, v = make_qkv(B, Hq, Hkv, 1, Lk, D, dtype, seed=17, outliers=True, device=cuda)
+    n_rows = B * Hq
+    pitch = (Lk + 63) // 64 * 64
+    kdt = torch.int32 if dtype == torch.float32 else torch.int16
+    keys = torch.zeros((n_rows, pitch), dtype=kdt, device=cuda)
+    resid = torch.zeros_like(keys) if keyed else None
+    N.call("sah_qk_scores", N.QkScoresArgs(
+        q.data_ptr(), q.stride(0), q.stride(1), q.stride(2), kk.data_ptr(), kk.stride(0), kk.stride(1), kk.stride(2),
+        None, 0, 0, 0, N.dtype_code(dtype), B, Hq, Hkv, 1, Lk, D, keys.data_ptr(), pitch, N.stream_ptr(cuda),
+        None if resid is None else resid.data_ptr()))
+    cap = sink + window + k
+    work = torch.zeros((max(1, N.work_floats(n_rows, cap, D)),), dtype=torch.float32, device=cuda)
+    tickets = torch.zeros((n_rows,), dtype=torch.int32, device=cuda)
+    excluded = 0  # the lowest key: active columns rank last
+
+    def run(one_call):
+        rows = NativeRows(n_rows, Lk, cap, cuda)
+        if not fresh:
+            N.call("sah_sink_local_indices", N.SinkLocalArgs(rows.as_struct(), 1, sink, window, 1, 0, N.stream_ptr(cuda)))
+        sel = N.SelectTopkArgs(rows.as_struct(), keys.data_ptr(), pitch, 32 if dtype == torch.float32 else 16, Lk, 0, k, excluded,
+                               1 if fresh else 0, sink if fresh else 0, window if fresh else 0, N.stream_ptr(cuda))
+        out = torch.zeros((B, 1, Hq, D), dtype=dtype, device=cuda)
+        att = N.AttentionArgs(
+            rows.as_struct(), q.data_ptr(), q.stride(0), q.stride(1), q.stride(2),
+            kk.data_ptr(), kk.stride(0), kk.stride(1), kk.stride(2), v.data_ptr(), v.stride(0), v.stride(1), v.stride(2),
+            None, 0, 0, 0, None, N.dtype_code(dtype), B, Hq, Hkv, 1, Lk, D, float(D ** -0.5), unit_inverse_weight(dtype),
+            0, 0, 0, 0, cap, out.data_ptr(), work.data_ptr(), work.numel(), None, None, N.stream_ptr(cuda))
+        if keyed and one_call:
+            att.score_keys, att.score_resid, att.score_pitch = keys.data_ptr(), resid.data_ptr(), pitch
+        N.timing_enable(True)
+        if one_call:
+            rc = N.lib().sah_select_topk_attention(C.byref(sel), C.byref(att), C.c_void_p(tickets.data_ptr()))
+            assert rc == 0, N.lib().sah_last_error()
+        else:
+            N.call("sah_select_topk", sel)
+            N.call("sah_sparse_attention", att)
+        torch.cuda.synchronize()
+        names = set(N.timing_collect())
+        N.timing_enable(False)
+        return rows.cnt.cpu(), torch.sort(rows.cols.cpu(), dim=1).values, rows.bitmap.cpu(), out, names
+
+    c1, s1, b1, o1, names1 = run(True)
+    c2, s2, b2, o2, names2 = run(False)
+    one_kernel = case not in ("fallback_f32",) and (fresh or n_rows >= 192)
+    assert ("k_select16_attn" in names1) == one_kernel, names1
+    assert "k_select16_attn" not in names2
+    assert bool((c1 == cap).all()) and torch.equal(c1, c2)
+    assert torch.equal(s1, s2) and torch.equal(b1, b2)          # skip_bitmap = 0: the bitmap rows are brought up to date
+    assert int(tickets.abs().max()) == 0                         # the last arrival of every row has reset its ticket
+    several = n_rows < 192
+    if keyed or several:
+        assert rel_err(o1, o2) < 4e-3
+    else:
+        assert torch.equal(o1, o2)
