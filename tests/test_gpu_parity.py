@@ -1529,3 +1529,25 @@ def test_select_topk_attention_entry_point_against_the_two_calls(cuda, case):
         assert rel_err(o1, o2) < 4e-3
     else:
         assert torch.equal(o1, o2)
+
+
+@pytest.mark.parametrize("case", ["bf16_decode_d64", "bf16_three_queries", "bf16_sinks_and_mask"])
+def test_oracle_topk_chain_with_logits_from_the_scoring_pass(cuda, case):
+    """Sink + Local + OracleTopK masker by masker (attention weights wanted, so no plan): the attention takes its logits
+    from the scoring pass's keys and remainders - with head_dim 64, with several queries per head (mask rows =
+    B x heads x queries), with sink logits, and with an additive mask (then the selection's scores carry the mask, are
+    not shared, and the attention reads K as ever). Index sets, dense probabilities and outputs against the oracle.
+    (bf16 only: in fp16 the reference's inverse-mask formula, 1 / (mask + 1e-6) * (mask != 0), is inf * 0 = NaN on every
+    entry outside the mask, so there is nothing to compare with.)"""
+    sa = _sa()
+    cfgs = [sa.SinkMaskerConfig(sink_size=16), sa.LocalMaskerConfig(window_size=32), sa.OracleTopKConfig(heavy_size=0.05)]
+    specs = [("sink", 16), ("local", 32), ("oracle_topk", 0.05)]
+    if case == "bf16_decode_d64":
+        _run_chain(cuda, cfgs, specs, 2, 8, 2, 1, 3000, 64, torch.bfloat16, seed=3)
+    elif case == "bf16_three_queries":
+        _run_chain(cuda, cfgs, specs, 1, 8, 4, 3, 2000, 128, torch.bfloat16, outliers=True, seed=4)
+    else:
+        am = torch.zeros(2, 1, 1, 2500)
+        am[1, :, :, 700:900] = torch.finfo(torch.float32).min
+        _run_chain(cuda, cfgs, specs, 2, 8, 2, 1, 2500, 128, torch.bfloat16, amask=am.to(torch.bfloat16),
+                   sinks=torch.linspace(-1.0, 1.0, 8), outliers=True, seed=5)
